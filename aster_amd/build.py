@@ -1,0 +1,69 @@
+"""Ahead-of-time build of libastergemm.so for gfx950 with hipcc.
+
+The reference JIT-compiles every GEMM through its MLIR pipeline
+(`compile_mlir_module_to_asm` + `assemble_to_hsaco`,
+python/aster/compiler/core.py:100-345); here the kernels are hand-written HIP
+and are compiled once, in-tree, so the shared library travels with the source
+tree.  `python -m aster_amd.build` rebuilds it.
+"""
+
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(PKG_DIR)
+CSRC = os.path.join(PKG_DIR, "csrc")
+LIB_DIR = os.path.join(PKG_DIR, "lib")
+LIB_PATH = os.path.join(LIB_DIR, "libastergemm.so")
+OBJ_DIR = os.path.join(ROOT, "build", "obj")
+
+SOURCES = ["gemm_tile.hip", "gemm_skinny.hip", "astergemm_api.hip"]
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+
+# -packed-fp32-ops off: hipcc must not form v_pk_{add,mul,fma}_f32 from the
+# epilogue float math.
+COMMON_FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+    "-I" + os.path.join(ROOT, "include"),
+    "-I" + CSRC,
+]
+
+
+def _compile(src: str) -> str:
+    obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
+    cmd = [HIPCC, *COMMON_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed on {src}:\n{proc.stdout}\n{proc.stderr}")
+    return obj
+
+
+def build_library(verbose: bool = False) -> str:
+    """Compile every HIP source and link libastergemm.so; returns its path."""
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    os.makedirs(LIB_DIR, exist_ok=True)
+    with ThreadPoolExecutor(max_workers=min(4, len(SOURCES))) as pool:
+        objs = list(pool.map(_compile, SOURCES))
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC",
+           "-Wno-unused-command-line-argument", *objs, "-o", LIB_PATH]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"link failed:\n{proc.stdout}\n{proc.stderr}")
+    if verbose:
+        print(f"built {LIB_PATH}")
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    build_library(verbose=True)
+    sys.exit(0)

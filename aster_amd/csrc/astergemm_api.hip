@@ -1,0 +1,508 @@
+// Host side of libastergemm: variant selection, launch, event timing, and the
+// thin HIP runtime seam.  Everything exported is declared in include/astergemm.h.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <vector>
+
+#include "astergemm_internal.h"
+
+namespace astergemm {
+
+static thread_local char g_err[512] = "";
+
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+
+// Same message shape as the reference's HIP error exceptions
+// ("file:line - hipGetErrorString", python/lib/RuntimeModule.cpp:126-134).
+int hip_fail(hipError_t e, const char* what, const char* file, int line) {
+  set_error("%s:%d - %s (%s)", file, line, hipGetErrorString(e), what);
+  return ASTERGEMM_EHIP;
+}
+
+namespace {
+
+int total_variants() { return num_tile_variants() + num_skinny_variants(); }
+
+const Variant* variant_at(int index) {
+  if (index < 0) return nullptr;
+  if (index < num_tile_variants()) return tile_variants() + index;
+  index -= num_tile_variants();
+  if (index < num_skinny_variants()) return skinny_variants() + index;
+  return nullptr;
+}
+
+bool variant_matches_types(const Variant& v, const astergemm_config& c) {
+  return v.dtype_ab == c.dtype_ab && v.dtype_c == c.dtype_c;
+}
+
+const char* validate_problem(const astergemm_config& c) {
+  if (c.M < 0 || c.N < 0 || c.K <= 0) return "M, N must be >= 0 and K > 0";
+  if (c.M > INT32_MAX || c.N > INT32_MAX || c.K > INT32_MAX) return "dimension exceeds int32";
+  if (c.dtype_ab < ASTERGEMM_F16 || c.dtype_ab > ASTERGEMM_MXFP4) return "bad dtype_ab";
+  if (c.dtype_c != ASTERGEMM_F32 && c.dtype_c != ASTERGEMM_BF16 && c.dtype_c != ASTERGEMM_F16)
+    return "dtype_c must be F32, BF16 or F16";
+  if (c.scale_mode < ASTERGEMM_SCALE_NONE || c.scale_mode > ASTERGEMM_SCALE_MX32)
+    return "bad scale_mode";
+  if ((c.dtype_ab == ASTERGEMM_MXFP4) != (c.scale_mode == ASTERGEMM_SCALE_MX32))
+    return "MXFP4 operands and SCALE_MX32 go together";
+  if (c.dtype_ab == ASTERGEMM_MXFP4 && c.K % 32 != 0) return "MXFP4 needs K % 32 == 0";
+  const int64_t lda = c.lda ? c.lda : c.K, ldb = c.ldb ? c.ldb : c.K, ldc = c.ldc ? c.ldc : c.N;
+  if (lda < c.K || ldb < c.K || ldc < c.N) return "leading dimension smaller than the row";
+  if (row_bytes(c.dtype_ab, lda) % 16 != 0 || row_bytes(c.dtype_ab, ldb) % 16 != 0)
+    return "row pitch of A and B must be a multiple of 16 bytes";
+  if (row_bytes(c.dtype_ab, lda) * 256 >= (int64_t)1 << 31 ||
+      row_bytes(c.dtype_ab, ldb) * 256 >= (int64_t)1 << 31)
+    return "row pitch too large for 32-bit tile offsets";
+  return nullptr;
+}
+
+// Picks the variant for cfg; on failure returns nullptr with the error set.
+const Variant* choose(const astergemm_config& c, int* index_out) {
+  if (const char* why = validate_problem(c)) {
+    set_error("astergemm: invalid config: %s", why);
+    return nullptr;
+  }
+  if (c.variant != 0) {
+    const Variant* v = variant_at(c.variant - 1);
+    if (!v || !variant_matches_types(*v, c)) {
+      set_error("astergemm: variant %d does not exist for these dtypes", c.variant);
+      return nullptr;
+    }
+    if (const char* why = v->check(c)) {
+      set_error("astergemm: variant %s: %s", v->name, why);
+      return nullptr;
+    }
+    if (index_out) *index_out = c.variant - 1;
+    return v;
+  }
+  const bool is16 = c.dtype_ab == ASTERGEMM_F16 || c.dtype_ab == ASTERGEMM_BF16;
+  int family = c.family;
+  if (family == ASTERGEMM_KERNEL_AUTO)
+    family = (is16 && c.M <= 64 && c.K % 32 == 0) ? ASTERGEMM_KERNEL_SKINNY : ASTERGEMM_KERNEL_TILE;
+
+  const Variant* best = nullptr;
+  int best_index = -1;
+  const char* last_why = "no variant with these dtypes";
+  for (int i = 0; i < total_variants(); ++i) {
+    const Variant* v = variant_at(i);
+    if (v->family != family || !variant_matches_types(*v, c)) continue;
+    if (const char* why = v->check(c)) {
+      last_why = why;
+      continue;
+    }
+    if (c.wg_tile_m && c.wg_tile_m != v->tile_m) continue;
+    if (c.wg_tile_n && c.wg_tile_n != v->tile_n) continue;
+    if (c.waves_m && c.waves_m != v->waves_m) continue;
+    if (c.waves_n && c.waves_n != v->waves_n) continue;
+    bool better = false;
+    if (!best) {
+      better = true;
+    } else if (family == ASTERGEMM_KERNEL_SKINNY) {
+      // smallest activation tile that still covers M
+      const bool fits = v->tile_m >= c.M, best_fits = best->tile_m >= c.M;
+      better = (fits && !best_fits) || (fits == best_fits && fits && v->tile_m < best->tile_m) ||
+               (!fits && !best_fits && v->tile_m > best->tile_m);
+    } else {
+      // largest tile that still yields at least one workgroup per CU (256)
+      auto wgs = [&](const Variant* x) {
+        return ((c.M + x->tile_m - 1) / x->tile_m) * ((c.N + x->tile_n - 1) / x->tile_n);
+      };
+      const bool big_ok = wgs(v) >= 256, best_big_ok = wgs(best) >= 256;
+      const int area = v->tile_m * v->tile_n, best_area = best->tile_m * best->tile_n;
+      better = (big_ok && !best_big_ok) || (big_ok == best_big_ok &&
+                                            (big_ok ? area > best_area : area < best_area));
+    }
+    if (better) {
+      best = v;
+      best_index = i;
+    }
+  }
+  if (!best) {
+    set_error("astergemm: no kernel variant for this config (%s)", last_why);
+    return nullptr;
+  }
+  if (family == ASTERGEMM_KERNEL_SKINNY && best->tile_m < c.M) {
+    set_error("astergemm: skinny path covers M <= %d, got M=%lld", best->tile_m, (long long)c.M);
+    return nullptr;
+  }
+  if (index_out) *index_out = best_index;
+  return best;
+}
+
+int grid_of(const Variant& v, const astergemm_config& c) {
+  if (v.family == ASTERGEMM_KERNEL_SKINNY) return (int)((c.N + v.tile_n - 1) / v.tile_n);
+  return (int)(((c.M + v.tile_m - 1) / v.tile_m) * ((c.N + v.tile_n - 1) / v.tile_n));
+}
+
+int64_t algorithmic_bytes(const astergemm_config& c) {
+  int64_t b = row_bytes(c.dtype_ab, c.K) * (c.M + c.N) + c.M * c.N * out_elt_bytes(c.dtype_c);
+  if (c.scale_mode == ASTERGEMM_SCALE_MX32) b += (c.M + c.N) * (c.K / 32);
+  if (c.scale_mode == ASTERGEMM_SCALE_TENSOR) b += 8;
+  if (c.has_bias) b += c.N * 4;
+  return b;
+}
+
+void describe(const Variant& v, int index, const astergemm_config& c, astergemm_kernel_info* o) {
+  memset(o, 0, sizeof(*o));
+  o->variant = index + 1;
+  o->family = v.family;
+  o->grid_x = grid_of(v, c);
+  o->block_x = v.waves_m * v.waves_n * 64;
+  o->lds_bytes = v.lds_bytes;
+  o->wg_tile_m = v.tile_m;
+  o->wg_tile_n = v.tile_n;
+  const int eb2 = (int)row_bytes(c.dtype_ab, 2);  // bytes of two elements (fp4-safe)
+  o->wg_tile_k = eb2 ? v.tile_k_bytes * 2 / eb2 : 0;
+  o->waves_m = v.waves_m;
+  o->waves_n = v.waves_n;
+  o->pipeline_stages = v.stages;
+  o->flops = 2 * c.M * c.N * c.K;
+  o->bytes = algorithmic_bytes(c);
+  snprintf(o->name, sizeof(o->name), "%s", v.name);
+  hipFuncAttributes fa;
+  if (hipFuncGetAttributes(&fa, v.func) == hipSuccess) {
+    o->vgprs = fa.numRegs;
+    o->agprs = 0;
+  } else {
+    (void)hipGetLastError();
+  }
+}
+
+int build_args(const Variant& v, const astergemm_config& c, const astergemm_operands& ops,
+               GemmArgs* a) {
+  if (!ops.dA || !ops.dB || !ops.dC) {
+    set_error("astergemm: dA, dB and dC must be non-null");
+    return ASTERGEMM_EINVAL;
+  }
+  if ((((uintptr_t)ops.dA) | ((uintptr_t)ops.dB)) & 15) {
+    set_error("astergemm: dA and dB must be 16-byte aligned");
+    return ASTERGEMM_EINVAL;
+  }
+  if (((uintptr_t)ops.dC) & 15) {
+    set_error("astergemm: dC must be 16-byte aligned");
+    return ASTERGEMM_EINVAL;
+  }
+  if (c.scale_mode == ASTERGEMM_SCALE_MX32 && (!ops.dMxA || !ops.dMxB)) {
+    set_error("astergemm: SCALE_MX32 needs dMxA and dMxB");
+    return ASTERGEMM_EINVAL;
+  }
+  if (c.scale_mode == ASTERGEMM_SCALE_MX32 && ((((uintptr_t)ops.dMxA) | ((uintptr_t)ops.dMxB)) & 7)) {
+    set_error("astergemm: dMxA and dMxB must be 8-byte aligned");
+    return ASTERGEMM_EINVAL;
+  }
+  if (c.scale_mode == ASTERGEMM_SCALE_TENSOR && (!ops.dScaleA || !ops.dScaleB)) {
+    set_error("astergemm: SCALE_TENSOR needs dScaleA and dScaleB");
+    return ASTERGEMM_EINVAL;
+  }
+  if (c.has_bias && !ops.dBias) {
+    set_error("astergemm: has_bias set but dBias is null");
+    return ASTERGEMM_EINVAL;
+  }
+  memset(a, 0, sizeof(*a));
+  a->A = (const uint8_t*)ops.dA;
+  a->B = (const uint8_t*)ops.dB;
+  a->C = ops.dC;
+  if (c.scale_mode == ASTERGEMM_SCALE_TENSOR) {
+    a->scale_a = ops.dScaleA;
+    a->scale_b = ops.dScaleB;
+  }
+  if (c.scale_mode == ASTERGEMM_SCALE_MX32) {
+    a->mx_a = ops.dMxA;
+    a->mx_b = ops.dMxB;
+    a->mx_ld = (int32_t)(c.K / 32);
+  }
+  a->bias = c.has_bias ? ops.dBias : nullptr;
+  a->lda_bytes = row_bytes(c.dtype_ab, c.lda ? c.lda : c.K);
+  a->ldb_bytes = row_bytes(c.dtype_ab, c.ldb ? c.ldb : c.K);
+  a->ldc = c.ldc ? c.ldc : c.N;
+  a->M = (int32_t)c.M;
+  a->N = (int32_t)c.N;
+  a->K = (int32_t)c.K;
+  a->ksteps = (int32_t)(row_bytes(c.dtype_ab, c.K) / 128);
+  a->tiles_m = (int32_t)((c.M + v.tile_m - 1) / v.tile_m);
+  a->tiles_n = (int32_t)((c.N + v.tile_n - 1) / v.tile_n);
+  a->group_m = 8;
+  a->split_k = 1;
+  return 0;
+}
+
+// Streams a scratch buffer so the next launch finds the last-level cache cold;
+// the reference's flush kernel does the same with a global_load_dword loop
+// (python/aster/execution/flush_llc.py:25-120).
+__global__ void flush_llc_kernel(uint32_t* buf, size_t words) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < words; i += stride) buf[i] = buf[i] + 1u;
+}
+
+}  // namespace
+}  // namespace astergemm
+
+using namespace astergemm;
+
+extern "C" {
+
+int astergemm_abi_version(void) { return ASTERGEMM_ABI_VERSION; }
+const char* astergemm_last_error(void) { return g_err; }
+
+int astergemm_variant_count(void) { return total_variants(); }
+
+int astergemm_variant_info(int index, const astergemm_config* cfg, astergemm_kernel_info* out) {
+  if (!cfg || !out) {
+    set_error("astergemm_variant_info: null argument");
+    return ASTERGEMM_EINVAL;
+  }
+  const Variant* v = variant_at(index);
+  if (!v) {
+    set_error("astergemm_variant_info: index %d out of range", index);
+    return ASTERGEMM_EINVAL;
+  }
+  describe(*v, index, *cfg, out);
+  return 0;
+}
+
+int astergemm_select(const astergemm_config* cfg, astergemm_kernel_info* out) {
+  if (!cfg || !out) {
+    set_error("astergemm_select: null argument");
+    return ASTERGEMM_EINVAL;
+  }
+  int index = -1;
+  const Variant* v = choose(*cfg, &index);
+  if (!v) return ASTERGEMM_ENOTSUP;
+  describe(*v, index, *cfg, out);
+  return 0;
+}
+
+int astergemm_run(const astergemm_config* cfg, const astergemm_operands* ops, void* stream) {
+  if (!cfg || !ops) {
+    set_error("astergemm_run: null argument");
+    return ASTERGEMM_EINVAL;
+  }
+  int index = -1;
+  const Variant* v = choose(*cfg, &index);
+  if (!v) return ASTERGEMM_ENOTSUP;
+  if (cfg->M == 0 || cfg->N == 0) return 0;
+  GemmArgs a;
+  if (int rc = build_args(*v, *cfg, *ops, &a)) return rc;
+  const int e = v->launch(a, grid_of(*v, *cfg), (hipStream_t)stream);
+  if (e != 0) return hip_fail((hipError_t)e, v->name, __FILE__, __LINE__);
+  return 0;
+}
+
+int astergemm_bench(const astergemm_config* cfg, const astergemm_operands* ops, int iters,
+                    int64_t* times_ns, int64_t flush_bytes, void* stream) {
+  if (!cfg || !ops || !times_ns || iters <= 0) {
+    set_error("astergemm_bench: bad argument");
+    return ASTERGEMM_EINVAL;
+  }
+  int index = -1;
+  const Variant* v = choose(*cfg, &index);
+  if (!v) return ASTERGEMM_ENOTSUP;
+  if (cfg->M == 0 || cfg->N == 0) {
+    for (int i = 0; i < iters; ++i) times_ns[i] = 0;
+    return 0;
+  }
+  GemmArgs a;
+  if (int rc = build_args(*v, *cfg, *ops, &a)) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  const int grid = grid_of(*v, *cfg);
+
+  uint32_t* flush = nullptr;
+  if (flush_bytes > 0) {
+    AG_HIP(hipMalloc((void**)&flush, (size_t)flush_bytes));
+    AG_HIP(hipMemsetAsync(flush, 0, (size_t)flush_bytes, s));
+  }
+  hipEvent_t e0, e1;
+  AG_HIP(hipEventCreate(&e0));
+  AG_HIP(hipEventCreate(&e1));
+  int rc = 0;
+  for (int i = 0; i < iters && rc == 0; ++i) {
+    if (flush)
+      hipLaunchKernelGGL(flush_llc_kernel, dim3(2048), dim3(256), 0, s, flush,
+                         (size_t)flush_bytes / 4);
+    hipError_t e = hipEventRecord(e0, s);
+    int le = (e == hipSuccess) ? v->launch(a, grid, s) : (int)e;
+    if (le == 0) le = (int)hipEventRecord(e1, s);
+    if (le == 0) le = (int)hipEventSynchronize(e1);
+    float ms = 0.f;
+    if (le == 0) le = (int)hipEventElapsedTime(&ms, e0, e1);
+    if (le != 0) {
+      rc = hip_fail((hipError_t)le, v->name, __FILE__, __LINE__);
+      break;
+    }
+    times_ns[i] = (int64_t)((double)ms * 1e6);
+  }
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  if (flush) (void)hipFree(flush);
+  return rc;
+}
+
+int astergemm_shuffle_weight_16(const uint16_t* src, uint16_t* dst, int64_t N, int64_t K) {
+  if (!src || !dst || N < 0 || K < 0 || N % 16 != 0 || K % 32 != 0) {
+    set_error("astergemm_shuffle_weight_16: need N %% 16 == 0 and K %% 32 == 0");
+    return ASTERGEMM_EINVAL;
+  }
+  // dst index order (nb, kb, lane_group, n_lane, kh, k_within) <- src (nb, n_lane, kb, kh,
+  // lane_group, k_within): each lane's 8 contiguous elements are its two 16x16x16 K-steps.
+  const int64_t kblocks = K / 32;
+  int64_t o = 0;
+  for (int64_t nb = 0; nb < N / 16; ++nb)
+    for (int64_t kb = 0; kb < kblocks; ++kb)
+      for (int g = 0; g < 4; ++g)
+        for (int nl = 0; nl < 16; ++nl)
+          for (int kh = 0; kh < 2; ++kh)
+            for (int kw = 0; kw < 4; ++kw)
+              dst[o++] = src[(nb * 16 + nl) * K + kb * 32 + kh * 16 + g * 4 + kw];
+  return 0;
+}
+
+/* ---- runtime seam --------------------------------------------------------- */
+
+int aster_rt_init(void) {
+  int n = 0;
+  AG_HIP(hipGetDeviceCount(&n));
+  if (n <= 0) {
+    set_error("aster_rt_init: no HIP device");
+    return ASTERGEMM_ENODEV;
+  }
+  return 0;
+}
+int aster_rt_peek_at_last_error(void) { return (int)hipPeekAtLastError(); }
+int aster_rt_clear_last_error(void) { return (int)hipGetLastError(); }
+int aster_rt_get_device_count(int* count) {
+  AG_HIP(hipGetDeviceCount(count));
+  return 0;
+}
+int aster_rt_set_device(int device) {
+  AG_HIP(hipSetDevice(device));
+  return 0;
+}
+int aster_rt_get_device(int* device) {
+  AG_HIP(hipGetDevice(device));
+  return 0;
+}
+int aster_rt_device_reset(void) {
+  AG_HIP(hipDeviceReset());
+  return 0;
+}
+int aster_rt_device_synchronize(void) {
+  AG_HIP(hipDeviceSynchronize());
+  return 0;
+}
+int aster_rt_get_device_props(int device, astergemm_device_props* out) {
+  if (!out) {
+    set_error("aster_rt_get_device_props: null out");
+    return ASTERGEMM_EINVAL;
+  }
+  hipDeviceProp_t p;
+  AG_HIP(hipGetDeviceProperties(&p, device));
+  memset(out, 0, sizeof(*out));
+  snprintf(out->name, sizeof(out->name), "%s", p.name);
+  snprintf(out->gcn_arch_name, sizeof(out->gcn_arch_name), "%s", p.gcnArchName);
+  out->warp_size = p.warpSize;
+  out->lds_per_cu = (int32_t)p.sharedMemPerBlock;
+  out->regs_per_multiprocessor = p.regsPerMultiprocessor;
+  out->multiprocessor_count = p.multiProcessorCount;
+  out->max_threads_per_block = p.maxThreadsPerBlock;
+  out->max_threads_per_multiprocessor = p.maxThreadsPerMultiProcessor;
+  out->asic_revision = p.asicRevision;
+  out->cluster_launch = 0;
+  out->total_global_mem = (int64_t)p.totalGlobalMem;
+  out->clock_rate_khz = p.clockRate;
+  out->l2_cache_bytes = p.l2CacheSize;
+  return 0;
+}
+int aster_rt_malloc(void** dptr, size_t bytes) {
+  AG_HIP(hipMalloc(dptr, bytes));
+  return 0;
+}
+int aster_rt_free(void* dptr) {
+  AG_HIP(hipFree(dptr));
+  return 0;
+}
+int aster_rt_memcpy_h2d(void* dst, const void* src, size_t bytes) {
+  AG_HIP(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice));
+  return 0;
+}
+int aster_rt_memcpy_d2h(void* dst, const void* src, size_t bytes) {
+  AG_HIP(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost));
+  return 0;
+}
+int aster_rt_memcpy_d2d(void* dst, const void* src, size_t bytes) {
+  AG_HIP(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToDevice));
+  return 0;
+}
+int aster_rt_memset(void* dst, int value, size_t bytes) {
+  AG_HIP(hipMemset(dst, value, bytes));
+  return 0;
+}
+int aster_rt_module_load_data(const void* image, size_t bytes, void** module) {
+  (void)bytes;
+  hipModule_t m;
+  AG_HIP(hipModuleLoadData(&m, image));
+  *module = (void*)m;
+  return 0;
+}
+int aster_rt_module_get_function(void* module, const char* name, void** fn) {
+  hipFunction_t f;
+  AG_HIP(hipModuleGetFunction(&f, (hipModule_t)module, name));
+  *fn = (void*)f;
+  return 0;
+}
+int aster_rt_module_unload(void* module) {
+  AG_HIP(hipModuleUnload((hipModule_t)module));
+  return 0;
+}
+int aster_rt_module_launch_kernel(void* fn, unsigned gx, unsigned gy, unsigned gz, unsigned bx,
+                                  unsigned by, unsigned bz, unsigned shared_bytes, void* stream,
+                                  void** kernel_params) {
+  AG_HIP(hipModuleLaunchKernel((hipFunction_t)fn, gx, gy, gz, bx, by, bz, shared_bytes,
+                               (hipStream_t)stream, kernel_params, nullptr));
+  return 0;
+}
+int aster_rt_event_create(void** event) {
+  hipEvent_t e;
+  AG_HIP(hipEventCreate(&e));
+  *event = (void*)e;
+  return 0;
+}
+int aster_rt_event_destroy(void* event) {
+  AG_HIP(hipEventDestroy((hipEvent_t)event));
+  return 0;
+}
+int aster_rt_event_record(void* event, void* stream) {
+  AG_HIP(hipEventRecord((hipEvent_t)event, (hipStream_t)stream));
+  return 0;
+}
+int aster_rt_event_synchronize(void* event) {
+  AG_HIP(hipEventSynchronize((hipEvent_t)event));
+  return 0;
+}
+int aster_rt_event_elapsed_ms(void* start, void* stop, float* ms) {
+  AG_HIP(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+  return 0;
+}
+int aster_rt_stream_create(void** stream) {
+  hipStream_t s;
+  AG_HIP(hipStreamCreate(&s));
+  *stream = (void*)s;
+  return 0;
+}
+int aster_rt_stream_destroy(void* stream) {
+  AG_HIP(hipStreamDestroy((hipStream_t)stream));
+  return 0;
+}
+int aster_rt_stream_synchronize(void* stream) {
+  AG_HIP(hipStreamSynchronize((hipStream_t)stream));
+  return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,75 @@
+// Internal declarations shared by the HIP translation units of libastergemm.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "astergemm.h"
+
+namespace astergemm {
+
+// Arguments of every GEMM kernel (passed by value as one kernarg struct).
+struct GemmArgs {
+  const uint8_t* A;      // [M, lda_bytes]
+  const uint8_t* B;      // [N, ldb_bytes]
+  void* C;               // [M, ldc] elements of the output type
+  const float* scale_a;  // per-tensor scales (device) or nullptr
+  const float* scale_b;
+  const float* bias;     // [N] or nullptr
+  const uint8_t* mx_a;   // e8m0 [M, mx_ld] or nullptr
+  const uint8_t* mx_b;   // e8m0 [N, mx_ld]
+  int64_t lda_bytes, ldb_bytes;
+  int64_t ldc;           // elements
+  int32_t mx_ld;         // bytes per row of the e8m0 planes (= K/32)
+  int32_t M, N, K;       // K in elements
+  int32_t ksteps;        // K-loop trip count (128 bytes of a row per step)
+  int32_t tiles_m, tiles_n;
+  int32_t group_m;       // tile rows per rasterisation group
+  int32_t split_k;       // skinny path: K slices per output row block
+  float* workspace;      // skinny path: fp32 partials when split_k > 1
+};
+
+// Bytes of one operand row covering `k` elements.
+__host__ __device__ inline int64_t row_bytes(int dtype, int64_t k) {
+  switch (dtype) {
+    case ASTERGEMM_F16:
+    case ASTERGEMM_BF16: return k * 2;
+    case ASTERGEMM_FP8_E4M3: return k;
+    case ASTERGEMM_MXFP4: return k / 2;
+    default: return k * 4;
+  }
+}
+
+inline int out_elt_bytes(int dtype) { return dtype == ASTERGEMM_F32 ? 4 : 2; }
+
+// One entry of the variant table (filled in by gemm_tile.hip / gemm_skinny.hip).
+struct Variant {
+  const char* name;
+  int family;
+  int dtype_ab;      // -1 = any 16-bit float (F16 and BF16 share a kernel body)
+  int dtype_c;
+  int tile_m, tile_n, tile_k_bytes;
+  int waves_m, waves_n;
+  int stages;
+  int lds_bytes;
+  const void* func;  // device function symbol, for hipFuncGetAttributes
+  // Launches the kernel; returns a hipError_t as int.
+  int (*launch)(const GemmArgs& a, int grid, hipStream_t s);
+  // Host-side shape check: nullptr when ok, else a reason.
+  const char* (*check)(const astergemm_config& c);
+};
+
+int num_tile_variants();
+const Variant* tile_variants();
+int num_skinny_variants();
+const Variant* skinny_variants();
+
+void set_error(const char* fmt, ...);
+int hip_fail(hipError_t e, const char* what, const char* file, int line);
+
+#define AG_HIP(expr)                                                   \
+  do {                                                                 \
+    hipError_t _e = (expr);                                            \
+    if (_e != hipSuccess) return hip_fail(_e, #expr, __FILE__, __LINE__); \
+  } while (0)
+
+}  // namespace astergemm

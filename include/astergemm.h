@@ -1,0 +1,207 @@
+/*
+ * astergemm.h -- C-ABI of the MI355X (gfx950) GEMM hot path.
+ *
+ * One shared library (libastergemm.so) exports everything below with C
+ * linkage: plain pointers, sizes and PODs only.  It replaces two seams of the
+ * reference:
+ *
+ *   1. the nanobind HIP wrapper `_runtime_module`
+ *      (reference: python/lib/RuntimeModule.cpp:140-418) -- the `aster_rt_*`
+ *      functions are its hip_* functions one for one, so the reference's
+ *      `execute_hsaco` (python/aster/execution/core.py:605-717) can be bound
+ *      to them unchanged;
+ *   2. the per-config `compile_*` / `execute_*_hsaco` pair of every GEMM
+ *      generator (reference: contrib/kittens/test/
+ *      test_102_gemm_python_multitile_g2s_directb_cdna4.py:420-467) -- the
+ *      `astergemm_*` functions select a pre-built hand-written kernel for a
+ *      problem + mapping and launch / time it.
+ *
+ * Conventions: every function returns 0 on success and a negative
+ * ASTERGEMM_E* code on failure; nothing throws; the message of the last
+ * failure on the calling thread is returned by astergemm_last_error().
+ * All buffers are owned by the caller.  Pointers named d* are device
+ * pointers.  Launches go to the stream that is passed (NULL = the null
+ * stream, which is what the reference uses everywhere).
+ */
+#ifndef ASTERGEMM_H_
+#define ASTERGEMM_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ASTERGEMM_ABI_VERSION 1
+
+/* ---- error codes ------------------------------------------------------ */
+#define ASTERGEMM_OK 0
+#define ASTERGEMM_EINVAL (-22)   /* bad argument / unsupported shape       */
+#define ASTERGEMM_ENOTSUP (-95)  /* no kernel variant for this config      */
+#define ASTERGEMM_EHIP (-5)      /* a HIP runtime call failed              */
+#define ASTERGEMM_ENODEV (-19)   /* no gfx950 device                       */
+
+/* ---- element types ----------------------------------------------------- */
+/* The reference's GemmSpec carries only elt_bytes_a/b/c (f16 x f16 -> f32,
+ * contrib/kittens/gemm_config.py:115-118); the build adds the storage types
+ * of the other four configurations. */
+typedef enum astergemm_dtype {
+  ASTERGEMM_F16 = 0,      /* IEEE binary16                                  */
+  ASTERGEMM_BF16 = 1,     /* bfloat16                                       */
+  ASTERGEMM_FP8_E4M3 = 2, /* OCP e4m3 (bias 7, max 448, NaN 0x7F)           */
+  ASTERGEMM_MXFP4 = 3,    /* OCP e2m1, two per byte (low nibble first), with
+                             one e8m0 scale byte per 32 K-elements          */
+  ASTERGEMM_F32 = 4       /* output only                                    */
+} astergemm_dtype;
+
+typedef enum astergemm_scale_mode {
+  ASTERGEMM_SCALE_NONE = 0,
+  ASTERGEMM_SCALE_TENSOR = 1, /* one fp32 per operand, read from device     */
+  ASTERGEMM_SCALE_MX32 = 2    /* e8m0 byte per (row, 32-wide K block)       */
+} astergemm_scale_mode;
+
+typedef enum astergemm_kernel_family {
+  ASTERGEMM_KERNEL_AUTO = 0,
+  ASTERGEMM_KERNEL_TILE = 1,  /* LDS-staged MFMA tile kernel                */
+  ASTERGEMM_KERNEL_SKINNY = 2 /* weight-streaming kernel for M <= 64        */
+} astergemm_kernel_family;
+
+/* ---- problem + mapping --------------------------------------------------
+ * C[M,N] = epilogue( sum_k A[M,K] * B[N,K] )      (B is stored N x K, i.e.
+ * "column-major K x N"; reference: gemm_config.py:94, 109).
+ * Mirrors GemmSpec (gemm_config.py:90-205) and the subset of
+ * GemmMappingSpec (gemm_config.py:213-276) that selects a kernel variant.
+ * A zero in a mapping field means "library default".                      */
+typedef struct astergemm_config {
+  int64_t M, N, K;       /* K in elements (for MXFP4: e2m1 elements)        */
+  int64_t lda, ldb, ldc; /* row pitch in elements; 0 = packed (K, K, N)     */
+  int32_t dtype_ab;      /* astergemm_dtype of A and B                      */
+  int32_t dtype_c;       /* F32, BF16 or F16                                */
+  int32_t scale_mode;    /* astergemm_scale_mode                            */
+  int32_t has_bias;      /* fp32 bias[N] added after scaling                */
+  /* mapping (all optional) */
+  int32_t family;        /* astergemm_kernel_family                         */
+  int32_t wg_tile_m;     /* = num_tiles_per_workgroup[M] * mfma_m           */
+  int32_t wg_tile_n;     /* = num_tiles_per_workgroup[N] * mfma_n           */
+  int32_t waves_m;       /* num_waves_per_workgroup[M]                      */
+  int32_t waves_n;       /* num_waves_per_workgroup[N]                      */
+  int32_t variant;       /* explicit variant id from astergemm_variant_*,
+                            or 0                                             */
+  int32_t reserved[6];
+} astergemm_config;
+
+/* What astergemm_select() reports back; the reference gets the same facts by
+ * parsing the generated asm (`parse_asm_kernel_resources`,
+ * python/aster/compiler/metadata.py) and from cfg.num_workgroups/num_threads. */
+typedef struct astergemm_kernel_info {
+  int32_t variant;        /* id usable in astergemm_config.variant           */
+  int32_t family;
+  int32_t grid_x;         /* 1-D grid, like every reference GEMM             */
+  int32_t block_x;
+  int32_t lds_bytes;
+  int32_t vgprs, agprs;   /* from hipFuncGetAttributes; agprs is 0 when the
+                             runtime reports only the unified count          */
+  int32_t wg_tile_m, wg_tile_n, wg_tile_k;
+  int32_t waves_m, waves_n;
+  int32_t pipeline_stages;
+  int64_t flops;          /* 2*M*N*K                                         */
+  int64_t bytes;          /* algorithmic bytes: A + B (+ scales) + C         */
+  char name[64];
+} astergemm_kernel_info;
+
+/* Device operands of one GEMM call. Unused pointers are NULL. */
+typedef struct astergemm_operands {
+  const void* dA;          /* [M, lda]                                        */
+  const void* dB;          /* [N, ldb]                                        */
+  void* dC;                /* [M, ldc]                                        */
+  const float* dScaleA;    /* SCALE_TENSOR: 1 fp32 on device                  */
+  const float* dScaleB;
+  const uint8_t* dMxA;     /* SCALE_MX32: [M, K/32] e8m0 bytes, row-major     */
+  const uint8_t* dMxB;     /*             [N, K/32]                           */
+  const float* dBias;      /* [N] fp32                                        */
+} astergemm_operands;
+
+/* reference: hip_get_device_props dict (RuntimeModule.cpp:166-191) */
+typedef struct astergemm_device_props {
+  char name[128];
+  char gcn_arch_name[64];
+  int32_t warp_size;
+  int32_t lds_per_cu;
+  int32_t regs_per_multiprocessor;
+  int32_t multiprocessor_count;
+  int32_t max_threads_per_block;
+  int32_t max_threads_per_multiprocessor;
+  int32_t asic_revision;
+  int32_t cluster_launch;
+  int64_t total_global_mem;
+  int32_t clock_rate_khz;
+  int32_t l2_cache_bytes;
+} astergemm_device_props;
+
+/* ---- library ----------------------------------------------------------- */
+int astergemm_abi_version(void);
+const char* astergemm_last_error(void);
+
+/* ---- GEMM path ---------------------------------------------------------- */
+/* Replaces compile_fn: pick the kernel variant for cfg and describe it.     */
+int astergemm_select(const astergemm_config* cfg, astergemm_kernel_info* out);
+/* Number of built variants and a description of variant `index`
+ * (0 <= index < count) instantiated for cfg's problem.                      */
+int astergemm_variant_count(void);
+int astergemm_variant_info(int index, const astergemm_config* cfg,
+                           astergemm_kernel_info* out);
+/* One asynchronous launch on `stream` (hipStream_t, NULL = null stream).    */
+int astergemm_run(const astergemm_config* cfg, const astergemm_operands* ops,
+                  void* stream);
+/* Replaces execute_fn's timed loop (execution/core.py:690-703): `iters`
+ * launches, each bracketed by its own HIP event pair on `stream`;
+ * times_ns[i] = int(ms * 1e6).  If flush_bytes > 0 a streaming kernel over a
+ * scratch buffer of that size runs before every start event (the reference's
+ * FlushLLC hook, python/aster/execution/flush_llc.py:25-120).               */
+int astergemm_bench(const astergemm_config* cfg, const astergemm_operands* ops,
+                    int iters, int64_t* times_ns, int64_t flush_bytes,
+                    void* stream);
+
+/* Host pre-shuffle of B[N,K] 2-byte elements into per-lane MFMA order
+ * (reference: shuffle_weight, contrib/kittens/test/kittens_helpers.py:90-119). */
+int astergemm_shuffle_weight_16(const uint16_t* src, uint16_t* dst, int64_t N,
+                                int64_t K);
+
+/* ---- runtime seam: 1:1 with RuntimeModule.cpp:140-418 -------------------- */
+int aster_rt_init(void);
+int aster_rt_peek_at_last_error(void);
+int aster_rt_clear_last_error(void);
+int aster_rt_get_device_count(int* count);
+int aster_rt_set_device(int device);
+int aster_rt_get_device(int* device);
+int aster_rt_device_reset(void);
+int aster_rt_device_synchronize(void);
+int aster_rt_get_device_props(int device, astergemm_device_props* out);
+int aster_rt_malloc(void** dptr, size_t bytes);
+int aster_rt_free(void* dptr);
+int aster_rt_memcpy_h2d(void* dst, const void* src, size_t bytes);
+int aster_rt_memcpy_d2h(void* dst, const void* src, size_t bytes);
+int aster_rt_memcpy_d2d(void* dst, const void* src, size_t bytes);
+int aster_rt_memset(void* dst, int value, size_t bytes);
+int aster_rt_module_load_data(const void* image, size_t bytes, void** module);
+int aster_rt_module_get_function(void* module, const char* name, void** fn);
+int aster_rt_module_unload(void* module);
+/* kernel_params: array of pointers to each argument, kept alive by caller. */
+int aster_rt_module_launch_kernel(void* fn, unsigned gx, unsigned gy,
+                                  unsigned gz, unsigned bx, unsigned by,
+                                  unsigned bz, unsigned shared_bytes,
+                                  void* stream, void** kernel_params);
+int aster_rt_event_create(void** event);
+int aster_rt_event_destroy(void* event);
+int aster_rt_event_record(void* event, void* stream);
+int aster_rt_event_synchronize(void* event);
+int aster_rt_event_elapsed_ms(void* start, void* stop, float* ms);
+int aster_rt_stream_create(void** stream);
+int aster_rt_stream_destroy(void* stream);
+int aster_rt_stream_synchronize(void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ASTERGEMM_H_ */
