@@ -1,0 +1,266 @@
+"""Measurement contract of the GEMM benches: input init, stats, single-config run,
+result lines.
+
+Mirrors the parts of the reference's bench harness that define what is measured
+(contrib/kittens/test/bench/bench_harness.py: peak table :31-41, `InitMode` /
+`init_array` :44-90, iteration counts :93-94, `PerfStats` :100-172,
+`_percentile_ns` / `_compute_stats` :174-198, `make_inputs` :1655-1662,
+`run_single` :1738-1850) and the `BENCH_RESULT_JSON:` line
+(tools/perf_bench_results_io.py:15, 113-144).  The compile pool, GPU workers and
+tiered config search of that file drive the reference's compiler and have no
+counterpart here.
+"""
+
+from __future__ import annotations
+
+import enum
+import json
+import statistics
+import sys
+from dataclasses import dataclass
+from typing import Optional, Sequence
+
+import numpy as np
+
+from .gemm_config import A as OP_A, B as OP_B
+
+# Dense peak TFLOP/s per target and operand type.  The f16 column is the
+# reference's table (:31-37); the others are MI355X's published dense peaks.
+_PEAK_TFLOPS_F16_BY_MCPU = {"gfx940": 980.6, "gfx942": 1307.0, "gfx950": 2500.0, "gfx1201": 100.0}
+PEAK_TFLOPS_GFX950 = {"f16": 2500.0, "bf16": 2500.0, "fp8_e4m3": 5000.0, "mxfp4": 10100.0}
+PEAK_HBM_GBPS_GFX950 = 8000.0
+
+
+def peak_tflops_f16(mcpu: str) -> float:
+    return _PEAK_TFLOPS_F16_BY_MCPU[mcpu]
+
+
+def peak_tflops(mcpu: str, dtype_ab: str = "f16") -> float:
+    if mcpu == "gfx950":
+        return PEAK_TFLOPS_GFX950[dtype_ab]
+    return peak_tflops_f16(mcpu)
+
+
+class InitMode(str, enum.Enum):
+    """Input init modes (hipblas names): HPL uniform[-0.5, 0.5]; TRIG_FLOAT
+    A=sin(i), B=cos(i); RAND_INT integers in {-2..2}; ZERO; SPECIAL fp16 extremes
+    (A = 65280, B = 6.07967e-5); NORM_DIST N(0, 1)."""
+
+    HPL = "hpl"
+    TRIG_FLOAT = "trig_float"
+    RAND_INT = "rand_int"
+    ZERO = "zero"
+    SPECIAL = "special"
+    NORM_DIST = "norm_dist"
+
+    def __str__(self) -> str:
+        return self.value
+
+
+INIT_DEFAULT = InitMode.HPL
+_SPECIAL = {"A": np.float16(65280.0), "B": np.float16(6.07967376708984375e-5)}
+
+NUM_ITERATIONS = 100
+WARMUP_ITERATIONS = 20
+
+
+def init_array(shape, mode, role: str, dtype=np.float16, seed: int = 42) -> np.ndarray:
+    """Deterministic input of the given mode; B uses stream `seed + 1`."""
+    mode = InitMode(mode)
+    flat = int(np.prod(shape))
+    if mode is InitMode.ZERO:
+        return np.zeros(shape, dtype=dtype)
+    if mode is InitMode.TRIG_FLOAT:
+        idx = np.arange(flat, dtype=np.float64)
+        return (np.sin(idx) if role == "A" else np.cos(idx)).astype(dtype).reshape(shape)
+    if mode is InitMode.SPECIAL:
+        return np.full(shape, _SPECIAL["A" if role == "A" else "B"], dtype=dtype)
+    rng = np.random.default_rng(seed + (1 if role == "B" else 0))
+    if mode is InitMode.HPL:
+        vals = rng.uniform(-0.5, 0.5, size=flat)
+    elif mode is InitMode.RAND_INT:
+        vals = rng.integers(-2, 3, size=flat)
+    else:
+        vals = rng.standard_normal(size=flat)
+    return vals.astype(dtype).reshape(shape)
+
+
+@dataclass(frozen=True)
+class PerfStats:
+    p0_ns: float
+    p10_ns: float
+    p25_ns: float
+    p50_ns: float
+    p90_ns: float
+    mean_ns: float
+    stddev_ns: float
+    stddev_tf: float
+    total_flops: int
+    peak_tflops: float
+
+    def _tf(self, ns: float) -> float:
+        return self.total_flops / ns * 1e-3
+
+    p0_ms = property(lambda s: s.p0_ns / 1e6)
+    p10_ms = property(lambda s: s.p10_ns / 1e6)
+    p25_ms = property(lambda s: s.p25_ns / 1e6)
+    p50_ms = property(lambda s: s.p50_ns / 1e6)
+    p90_ms = property(lambda s: s.p90_ns / 1e6)
+    mean_ms = property(lambda s: s.mean_ns / 1e6)
+    p0_tf = property(lambda s: s._tf(s.p0_ns))
+    p10_tf = property(lambda s: s._tf(s.p10_ns))
+    p25_tf = property(lambda s: s._tf(s.p25_ns))
+    p50_tf = property(lambda s: s._tf(s.p50_ns))
+    p90_tf = property(lambda s: s._tf(s.p90_ns))
+    mean_tf = property(lambda s: s._tf(s.mean_ns))
+    p0_pct = property(lambda s: s.p0_tf / s.peak_tflops * 100)
+    p50_pct = property(lambda s: s.p50_tf / s.peak_tflops * 100)
+    mean_pct = property(lambda s: s.mean_tf / s.peak_tflops * 100)
+
+
+def _percentile_ns(sorted_times: Sequence[float], pct: float) -> float:
+    """Nearest-rank percentile of an ascending list."""
+    n = len(sorted_times)
+    return float(sorted_times[max(0, min(n - 1, int(round(pct / 100.0 * (n - 1)))))])
+
+
+def _compute_stats(post_warmup: Sequence[float], total_flops: int,
+                   peak_tflops: float) -> Optional[PerfStats]:
+    """Post-warm-up launch times (ns) -> percentiles, mean, stddev; None when a
+    time is not positive."""
+    if not post_warmup or min(post_warmup) <= 0:
+        return None
+    times = sorted(float(t) for t in post_warmup)
+    tfs = [int(total_flops) / t * 1e-3 for t in times]
+    many = len(times) > 1
+    return PerfStats(
+        p0_ns=times[0], p10_ns=_percentile_ns(times, 10), p25_ns=_percentile_ns(times, 25),
+        p50_ns=_percentile_ns(times, 50), p90_ns=_percentile_ns(times, 90),
+        mean_ns=float(statistics.fmean(times)),
+        stddev_ns=float(statistics.stdev(times)) if many else 0.0,
+        stddev_tf=float(statistics.stdev(tfs)) if many else 0.0,
+        total_flops=int(total_flops), peak_tflops=peak_tflops)
+
+
+RESULT_SENTINEL = "BENCH_RESULT_JSON:"
+
+
+def emit_one_result(stream, bench: str, cfg, stats: PerfStats) -> None:
+    """One `BENCH_RESULT_JSON:{...}` line; `stream=None` discards."""
+    if stream is None:
+        return
+    m, n, k = cfg.spec.gemm_size
+    rec = {"mcpu": cfg.mapping.mcpu, "bench": bench, "M": m, "N": n, "K": k, "label": cfg.label,
+           "tflops_median": stats.p50_tf, "tflops_p10": stats.p10_tf, "tflops_p90": stats.p90_tf,
+           "tflops_mean": stats.mean_tf, "tflops_p0": stats.p0_tf, "tflops_p25": stats.p25_tf,
+           "tflops_stddev": stats.stddev_tf, "pct_peak_p50": stats.p50_pct, "sample_n": 1}
+    print(RESULT_SENTINEL + json.dumps(rec), file=stream)
+    stream.flush()
+
+
+def parse_result_lines(lines):
+    """Records of every `BENCH_RESULT_JSON:` line in `lines`; other text is skipped."""
+    out = []
+    for raw in lines:
+        i = raw.find(RESULT_SENTINEL)
+        if i < 0:
+            continue
+        try:
+            out.append(json.loads(raw[i + len(RESULT_SENTINEL):]))
+        except json.JSONDecodeError:
+            continue
+    return out
+
+
+def _storage(values: np.ndarray, dtype_ab: str) -> np.ndarray:
+    """fp16-valued init data in the operand's storage type."""
+    if dtype_ab == "f16":
+        return values.astype(np.float16)
+    if dtype_ab == "bf16":
+        u = values.astype(np.float32).view(np.uint32).astype(np.uint64)
+        return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+    raise ValueError(f"make_inputs covers f16 and bf16, not {dtype_ab}")
+
+
+def make_inputs(cfg, init_mode=INIT_DEFAULT):
+    """A [M, K] and B [N, K] for `cfg`, seeds 42 / 43."""
+    a = init_array(cfg.spec.operand_shape(OP_A), init_mode, "A")
+    b = init_array(cfg.spec.operand_shape(OP_B), init_mode, "B")
+    dt = cfg.spec.dtype_ab
+    return _storage(a, dt), _storage(b, dt)
+
+
+def _as_f32(arr: np.ndarray, dtype: str) -> np.ndarray:
+    if dtype == "bf16":
+        return (arr.astype(np.uint32) << 16).view(np.float32)
+    return arr.astype(np.float32)
+
+
+def run_single(cfg, compile_fn, args, execute_fn, *, bench: str = "unknown", out=sys.stdout):
+    """Compile (select), time `iterations` launches, print the summary table, then
+    a one-launch correctness check against `A.f32 @ B.f32.T` with rtol = atol =
+    1e-2, as the reference does.  Returns the PerfStats (None without a GPU)."""
+    import tempfile
+
+    from .execution import system_has_gpu
+
+    iterations = getattr(args, "iterations", None) or NUM_ITERATIONS
+    hsaco = getattr(args, "hsaco", None)
+    tmp = None
+    if not hsaco:
+        tmp = tempfile.NamedTemporaryFile(suffix=".hsaco", delete=False)
+        tmp.close()
+        hsaco = tmp.name
+    try:
+        _, asm = compile_fn(cfg, hsaco)
+        print(f"Config: {cfg.label}", file=out)
+        print(asm, file=out)
+        if getattr(args, "compile_only", False):
+            return None
+        if not system_has_gpu("gfx950"):
+            print("No GPUs detected -- skipping execution.", file=out)
+            return None
+        init_mode = getattr(args, "init", INIT_DEFAULT)
+        A, B = make_inputs(cfg, init_mode)
+        _, times_ns = execute_fn(cfg, hsaco, iterations, A, B, skip_gpu_check=True)
+        measured = times_ns[WARMUP_ITERATIONS:]
+        if not measured:
+            print(f"\nNo measurements after warmup ({iterations} iterations), use a number > "
+                  f"{WARMUP_ITERATIONS} e.g. --iterations=100", file=out)
+            return None
+        s = _compute_stats(measured, cfg.total_flops,
+                           peak_tflops(cfg.mapping.mcpu, cfg.spec.dtype_ab))
+        if s is None:
+            print(f"\nInvalid timings (min={min(measured)} ns)", file=out)
+            return None
+        results_path = getattr(args, "results_file", None)
+        if results_path:
+            with open(results_path, "a") as rs:
+                emit_one_result(rs, bench, cfg, s)
+        print("\n--- Summary ---", file=out)
+        print(f"  {'metric':<8s}  {'ms':>10s}  {'TFLOPS':>10s}  {'% peak':>8s}", file=out)
+        for name, ms, tf, pct in (("p0", s.p0_ms, s.p0_tf, s.p0_pct), ("p10", s.p10_ms, s.p10_tf, None),
+                                  ("p25", s.p25_ms, s.p25_tf, None), ("p50", s.p50_ms, s.p50_tf, s.p50_pct),
+                                  ("p90", s.p90_ms, s.p90_tf, None), ("mean", s.mean_ms, s.mean_tf, s.mean_pct)):
+            tail = f"{pct:>7.1f}%" if pct is not None else ""
+            print(f"  {name:<8s}  {ms:>10.4f}  {tf:>10.1f}  {tail:>8s}", file=out)
+        print(f"  {'stddev':<8s}  {'':>10s}  {s.stddev_tf:>10.1f}", file=out)
+
+        print("\n--- Correctness check ---", file=out)
+        expected = (_as_f32(A, cfg.spec.dtype_ab) @ _as_f32(B, cfg.spec.dtype_ab).T).flatten()
+        C_output, _ = execute_fn(cfg, hsaco, 1, A, B, skip_gpu_check=True)
+        got = _as_f32(C_output, cfg.spec.dtype_c)
+        try:
+            np.testing.assert_allclose(got, expected, rtol=1e-2, atol=1e-2)
+            print("PASS", file=out)
+        except AssertionError:
+            print(f"FAIL: max_abs_diff={float(np.max(np.abs(got - expected))):.6g}", file=out)
+        return s
+    finally:
+        if tmp is not None:
+            import os
+
+            try:
+                os.unlink(tmp.name)
+            except OSError:
+                pass

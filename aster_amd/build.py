@@ -22,6 +22,8 @@ LIB_PATH = os.path.join(LIB_DIR, "libastergemm.so")
 OBJ_DIR = os.path.join(ROOT, "build", "obj")
 
 SOURCES = ["gemm_tile.hip", "gemm_skinny.hip", "astergemm_api.hip"]
+HSACO_SOURCE = "hsaco_kernels.hip"
+HSACO_PATH = os.path.join(LIB_DIR, "astergemm_kernels.hsaco")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
@@ -48,12 +50,25 @@ def _compile(src: str) -> str:
     return obj
 
 
+def _genco(src: str) -> str:
+    """Device-only code object for module launchers (hipModuleLoadData)."""
+    flags = [f for f in COMMON_FLAGS if f != "-fPIC"]
+    cmd = [HIPCC, "--genco", *flags, os.path.join(CSRC, src), "-o", HSACO_PATH]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc --genco failed on {src}:\n{proc.stdout}\n{proc.stderr}")
+    return HSACO_PATH
+
+
 def build_library(verbose: bool = False) -> str:
-    """Compile every HIP source and link libastergemm.so; returns its path."""
+    """Compile every HIP source, link libastergemm.so and build the code object
+    astergemm_kernels.hsaco; returns the library path."""
     os.makedirs(OBJ_DIR, exist_ok=True)
     os.makedirs(LIB_DIR, exist_ok=True)
-    with ThreadPoolExecutor(max_workers=min(4, len(SOURCES))) as pool:
+    with ThreadPoolExecutor(max_workers=4) as pool:
+        hsaco = pool.submit(_genco, HSACO_SOURCE)
         objs = list(pool.map(_compile, SOURCES))
+        hsaco.result()
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC",
            "-Wno-unused-command-line-argument", *objs, "-o", LIB_PATH]
     proc = subprocess.run(cmd, capture_output=True, text=True)

@@ -11,6 +11,7 @@
 namespace astergemm {
 
 static thread_local char g_err[512] = "";
+static thread_local int g_choose_rc = 0;  // why choose() returned nullptr
 
 void set_error(const char* fmt, ...) {
   va_list ap;
@@ -65,8 +66,10 @@ const char* validate_problem(const astergemm_config& c) {
 
 // Picks the variant for cfg; on failure returns nullptr with the error set.
 const Variant* choose(const astergemm_config& c, int* index_out) {
+  g_choose_rc = ASTERGEMM_ENOTSUP;
   if (const char* why = validate_problem(c)) {
     set_error("astergemm: invalid config: %s", why);
+    g_choose_rc = ASTERGEMM_EINVAL;
     return nullptr;
   }
   if (c.variant != 0) {
@@ -225,7 +228,8 @@ int build_args(const Variant& v, const astergemm_config& c, const astergemm_oper
   a->M = (int32_t)c.M;
   a->N = (int32_t)c.N;
   a->K = (int32_t)c.K;
-  a->ksteps = (int32_t)(row_bytes(c.dtype_ab, c.K) / 128);
+  a->ksteps = (int32_t)((row_bytes(c.dtype_ab, c.K) + 127) / 128);
+  a->tail_granules = (int32_t)((row_bytes(c.dtype_ab, c.K) % 128) / 16);
   a->tiles_m = (int32_t)((c.M + v.tile_m - 1) / v.tile_m);
   a->tiles_n = (int32_t)((c.N + v.tile_n - 1) / v.tile_n);
   a->group_m = 8;
@@ -275,7 +279,7 @@ int astergemm_select(const astergemm_config* cfg, astergemm_kernel_info* out) {
   }
   int index = -1;
   const Variant* v = choose(*cfg, &index);
-  if (!v) return ASTERGEMM_ENOTSUP;
+  if (!v) return g_choose_rc;
   describe(*v, index, *cfg, out);
   return 0;
 }
@@ -287,7 +291,7 @@ int astergemm_run(const astergemm_config* cfg, const astergemm_operands* ops, vo
   }
   int index = -1;
   const Variant* v = choose(*cfg, &index);
-  if (!v) return ASTERGEMM_ENOTSUP;
+  if (!v) return g_choose_rc;
   if (cfg->M == 0 || cfg->N == 0) return 0;
   GemmArgs a;
   if (int rc = build_args(*v, *cfg, *ops, &a)) return rc;
@@ -304,7 +308,7 @@ int astergemm_bench(const astergemm_config* cfg, const astergemm_operands* ops, 
   }
   int index = -1;
   const Variant* v = choose(*cfg, &index);
-  if (!v) return ASTERGEMM_ENOTSUP;
+  if (!v) return g_choose_rc;
   if (cfg->M == 0 || cfg->N == 0) {
     for (int i = 0; i < iters; ++i) times_ns[i] = 0;
     return 0;

@@ -22,6 +22,7 @@ struct GemmArgs {
   int32_t mx_ld;         // bytes per row of the e8m0 planes (= K/32)
   int32_t M, N, K;       // K in elements
   int32_t ksteps;        // K-loop trip count (128 bytes of a row per step)
+  int32_t tail_granules; // valid 16-byte granules of the last step, 0 = all 8
   int32_t tiles_m, tiles_n;
   int32_t group_m;       // tile rows per rasterisation group
   int32_t split_k;       // skinny path: K slices per output row block

@@ -1,0 +1,71 @@
+"""Host helpers of the GEMM family: B pre-shuffle and pipeline-strategy table.
+
+Mirrors contrib/kittens/test/kittens_helpers.py:90-169 of the reference.  The
+MLIR-template plumbing of that file (library paths, `run_kittens_kernel`,
+`{{...}}` substitutions) belongs to the compiler path that this build does not
+have.
+"""
+
+from __future__ import annotations
+
+import numpy as np
+
+_STAGE_KEYS = ("A_LOAD", "A_LDS_WRITE", "A_LDS_READ", "B_LOAD", "B_LDS_WRITE", "B_LDS_READ",
+               "COMPUTE")
+
+# Stage index of every op class, one row per strategy, columns as _STAGE_KEYS
+# (reference: PIPELINE_STRATEGIES, kittens_helpers.py:137-157).  The reference
+# feeds these to its SCF pipeliner; here they only describe prefetch distance
+# for the resource estimators and for labels.
+_STAGE_ROWS = (
+    (0, 0, 0, 0, 0, 0, 0),
+    (0, 1, 1, 1, 1, 1, 1),
+    (0, 0, 1, 0, 1, 1, 1),
+    (0, 1, 2, 0, 1, 2, 2),
+    (0, 2, 2, 0, 1, 2, 2),
+    (0, 1, 2, 2, 2, 2, 3),
+    (0, 2, 2, 1, 1, 2, 3),
+    (0, 2, 3, 0, 2, 3, 4),
+    (0, 1, 3, 0, 2, 3, 4),
+    (0, 3, 4, 0, 3, 4, 5),
+    (0, 2, 4, 0, 3, 4, 5),
+    (0, 1, 3, 0, 1, 4, 4),
+    (0, 1, 3, 1, 2, 4, 4),
+    (0, 1, 3, 0, 2, 4, 4),
+)
+PIPELINE_STRATEGIES = {i: dict(zip(_STAGE_KEYS, row)) for i, row in enumerate(_STAGE_ROWS)}
+
+
+def pipeline_strategy_stages(strategy: int):
+    """(a_stages, b_stages): deepest stage index + 1 on each operand's chain
+    (reference: kittens_helpers.py:161-169)."""
+    s = PIPELINE_STRATEGIES[strategy]
+    a = max(s["A_LOAD"], s["A_LDS_WRITE"], s["A_LDS_READ"], s["COMPUTE"]) + 1
+    b = max(s["B_LOAD"], s["B_LDS_WRITE"], s["B_LDS_READ"], s["COMPUTE"]) + 1
+    return a, b
+
+
+def shuffle_weight(B: np.ndarray) -> np.ndarray:
+    """Pre-shuffle B[N, K] (2-byte elements) so that each lane's 16-byte load is
+    its MFMA operand for two 16x16x16 K-steps.
+
+    Same result as the reference's `shuffle_weight` (kittens_helpers.py:90-119):
+    view B as (n_block, n_lane=16, k_block, k_half=2, lane_group=4, k_within=4)
+    and store it in the order (n_block, k_block, lane_group, n_lane, k_half,
+    k_within).  Lane d of block (nb, kb) then finds
+    B[nb*16 + d%16, kb*32 + kh*16 + (d//16)*4 + 0..3] for kh = 0, 1 contiguous.
+    """
+    N, K = B.shape
+    if N % 16 != 0:
+        raise AssertionError(f"N={N} must be multiple of 16")
+    if K % 32 != 0:
+        raise AssertionError(f"K={K} must be multiple of 32")
+    view = B.reshape(N // 16, 16, K // 32, 2, 4, 4)
+    return np.ascontiguousarray(np.moveaxis(view, (0, 2, 4, 1, 3, 5), (0, 1, 2, 3, 4, 5))).reshape(N, K)
+
+
+def unshuffle_weight(Bs: np.ndarray) -> np.ndarray:
+    """Inverse of `shuffle_weight`."""
+    N, K = Bs.shape
+    view = Bs.reshape(N // 16, K // 32, 4, 16, 2, 4)
+    return np.ascontiguousarray(view.transpose(0, 3, 1, 4, 2, 5)).reshape(N, K)

@@ -1,0 +1,342 @@
+"""GPU parity: the HIP kernels, called through the C-ABI, against the CPU oracle on
+the same seeded inputs.
+
+Bars: rel-L2 <= 1e-3 against the fp32-accumulated oracle for every floating
+output (bf16 / f16 outputs are compared with the oracle's output rounded the
+same way); the reference's own bar `assert_allclose(rtol=1e-2, atol=1e-2)` on
+its own test shapes; bit-exact where the arithmetic is exact (known answers,
+power-of-two scaling, identity operand, run-to-run determinism).
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from aster_amd import _capi, gemm as AG
+from aster_amd.execution import GpuBuffer
+from aster_amd.gemm_config import (Cdna4GemmInstance, GemmMappingSpec, GemmSpec, OperandPath,
+                                   make_instance)
+from oracle import cgemm, formats as F, gemm as G
+
+pytestmark = pytest.mark.gpu
+
+REL_L2_BAR = 1e-3
+_DT = {"f16": G.F16, "bf16": G.BF16, "fp8_e4m3": G.FP8_E4M3, "mxfp4": G.MXFP4, "f32": G.F32}
+_OUT_NP = {"f32": np.float32, "bf16": np.uint16, "f16": np.uint16}
+
+
+def run_gemm(a, b, M, N, K, dtype_ab, dtype_c, *, scale_a=None, scale_b=None, mx_a=None, mx_b=None,
+             bias=None, lda=0, ldb=0, ldc=0, family=_capi.KERNEL_AUTO, wg_tile=(0, 0)):
+    """Upload, launch once through astergemm_run, download.  Returns the raw
+    output storage [M, ldc or N] and the kernel name."""
+    plan = AG.GemmPlan.create(M, N, K, dtype_ab, dtype_c, has_bias=bias is not None, lda=lda,
+                              ldb=ldb, ldc=ldc, family=family, wg_tile=wg_tile)
+    ldc_eff = ldc or N
+    out = np.full((M, ldc_eff), 0x7FC1 if dtype_c != "f32" else np.nan, dtype=_OUT_NP[dtype_c])
+    bufs = []
+
+    def up(x):
+        if x is None:
+            return None
+        x = np.ascontiguousarray(x)
+        buf = GpuBuffer(x.nbytes)
+        buf.copy_from_host(x)
+        bufs.append(buf)
+        return buf.ptr_value
+
+    dA, dB, dC = up(a), up(b), up(out)
+    kw = {}
+    if scale_a is not None:
+        kw["scale_a"] = up(np.array([scale_a], np.float32))
+        kw["scale_b"] = up(np.array([scale_b], np.float32))
+    if mx_a is not None:
+        kw["mx_a"], kw["mx_b"] = up(mx_a), up(mx_b)
+    if bias is not None:
+        kw["bias"] = up(np.asarray(bias, np.float32))
+    print(f"launch {plan.info.name.decode()} M={M} N={N} K={K}", flush=True)
+    plan.run(dA, dB, dC, **kw)
+    bufs[2].copy_to_host(out)
+    for bf in bufs:
+        bf.free()
+    return out, plan.info.name.decode()
+
+
+def check(out_raw, want_raw, dtype_c, N, bar=REL_L2_BAR):
+    got = G.output_to_f32(out_raw[:, :N], _DT[dtype_c])
+    want = G.output_to_f32(want_raw, _DT[dtype_c])
+    assert not np.isnan(got).any()
+    rel = G.rel_l2(got, want)
+    assert rel <= bar, f"rel-L2 {rel:.3e} > {bar}"
+    return rel
+
+
+def operands(M, N, K, dtype_ab, seed=42, a_std=1.0, b_std=0.02, dist="normal"):
+    """Seeded operands in storage form: seeds `seed` (A) and `seed + 1` (B)."""
+    ra, rb = np.random.default_rng(seed), np.random.default_rng(seed + 1)
+    if dist == "uniform":
+        xa = ra.uniform(-1, 1, (M, K)).astype(np.float32)
+        xb = rb.uniform(-1, 1, (N, K)).astype(np.float32)
+    else:
+        xa = (ra.standard_normal((M, K)) * a_std).astype(np.float32)
+        xb = (rb.standard_normal((N, K)) * b_std).astype(np.float32)
+    extra = {}
+    if dtype_ab == "f16":
+        a, b = xa.astype(np.float16), xb.astype(np.float16)
+    elif dtype_ab == "bf16":
+        a, b = F.f32_to_bf16_bits(xa), F.f32_to_bf16_bits(xb)
+    elif dtype_ab == "fp8_e4m3":
+        a, sa = F.quantize_fp8_tensor(xa)
+        b, sb = F.quantize_fp8_tensor(xb)
+        extra = dict(scale_a=sa, scale_b=sb)
+    else:
+        a, mxa = F.quantize_mxfp4(xa)
+        b, mxb = F.quantize_mxfp4(xb)
+        extra = dict(mx_a=mxa, mx_b=mxb)
+    return a, b, extra
+
+
+# ---- configuration 1 of the baseline: fp16 256^3, uniform[-1,1], fp32 out ---------
+
+def test_config1_fp16_256(gpu):
+    a, b, _ = operands(256, 256, 256, "f16", dist="uniform")
+    out, _ = run_gemm(a, b, 256, 256, 256, "f16", "f32")
+    want = G.gemm(a, b, G.F16, G.F32)
+    check(out, want, "f32", 256)
+    assert G.rel_l2(out, cgemm.gemm_raw(a, b, G.F16, 256, 256, 256)) <= REL_L2_BAR
+    np.testing.assert_allclose(out, want, rtol=1e-2, atol=1e-2)
+
+
+# ---- the reference's own GEMM test shapes (f16 x f16 -> f32) -------------------------
+# TestCdna4GemmG2S / MultiWG / Coop8Waves / Pipelined8Wave of
+# contrib/kittens/test/test_102_gemm_python_multitile_g2s_directb_cdna4.py:493-570:
+# M = wg_m * twg_m * 16, N = wg_n * twg_n * 16, K = 32 * k_mult,
+# inputs np.random.seed(42 + M + N + K); randn * 0.1 -> f16.
+REFERENCE_SHAPES = (
+    [((1, 1), twg, km) for twg in ((2, 2), (2, 1), (1, 2)) for km in (1, 2, 4, 8)]
+    + [((2, 2), (2, 2), 4)]
+    + [((1, 1), twg, 4) for twg in ((4, 16), (16, 4), (2, 32), (32, 2))]
+    + [((1, 1), (8, 8), 8), ((1, 1), (8, 8), 5)]
+)
+
+
+@pytest.mark.parametrize("wg,twg,k_mult", REFERENCE_SHAPES)
+def test_reference_test_shapes_f16(gpu, wg, twg, k_mult):
+    M, N, K = wg[0] * twg[0] * 16, wg[1] * twg[1] * 16, 32 * k_mult
+    np.random.seed(42 + M + N + K)
+    a = (np.random.randn(M, K) * 0.1).astype(np.float16)
+    b = (np.random.randn(N, K) * 0.1).astype(np.float16)
+    spec = GemmSpec.from_sizes(M, N, K, mfma_shape=[16, 16, 32])
+    mapping = GemmMappingSpec([wg[0], wg[1], 1], [1, 1, 1], [twg[0], twg[1], 1],
+                              operand_path=OperandPath.DIRECT_B, mcpu="gfx950")
+    cfg = Cdna4GemmInstance(spec, mapping)
+    import tempfile
+    with tempfile.NamedTemporaryFile(suffix=".hsaco") as tmp:
+        AG.compile_gemm(cfg, tmp.name)
+        c_flat, times = AG.execute_gemm_hsaco(cfg, tmp.name, 1, a, b)
+    expected = (a.astype(np.float32) @ b.astype(np.float32).T).flatten()
+    np.testing.assert_allclose(c_flat, expected, rtol=1e-2, atol=1e-2)   # the reference's bar
+    assert G.rel_l2(c_flat, expected) <= REL_L2_BAR                      # this build's bar
+    assert len(times) == 1 and times[0] > 0
+    # the same problem through the LDS-staged tile kernel
+    out, name = run_gemm(a, b, M, N, K, "f16", "f32", family=_capi.KERNEL_TILE)
+    assert name.startswith("tile")
+    np.testing.assert_allclose(out.flatten(), expected, rtol=1e-2, atol=1e-2)
+    assert G.rel_l2(out.flatten(), expected) <= REL_L2_BAR
+
+
+# ---- scaled-down versions of configurations 2-5, same distributions and seeds --------
+
+@pytest.mark.parametrize("M,N,K,tile", [(512, 512, 512, 256), (384, 640, 448, 128), (256, 256, 64, 128)])
+@pytest.mark.parametrize("dtype_c", ["bf16", "f32"])
+def test_config2_bf16(gpu, M, N, K, tile, dtype_c):
+    a, b, _ = operands(M, N, K, "bf16")
+    out, name = run_gemm(a, b, M, N, K, "bf16", dtype_c, family=_capi.KERNEL_TILE, wg_tile=(tile, tile))
+    assert f"{tile}x{tile}" in name
+    check(out, G.gemm(a, b, G.BF16, _DT[dtype_c]), dtype_c, N)
+
+
+@pytest.mark.parametrize("M,N,K,tile", [(512, 512, 512, 256), (256, 384, 640, 128)])
+def test_config3_fp8_per_tensor_scales(gpu, M, N, K, tile):
+    a, b, ex = operands(M, N, K, "fp8_e4m3", a_std=1.0, b_std=1.0)
+    out, _ = run_gemm(a, b, M, N, K, "fp8_e4m3", "bf16", wg_tile=(tile, tile), **ex)
+    want = G.gemm_fp8(a, b, ex["scale_a"], ex["scale_b"], out_dtype=G.BF16)
+    check(out, want, "bf16", N)
+    # against the float64-accumulated product: the fp8 matrix-core path sums each
+    # 128-wide block of products in a fixed-point adder tree that is a little
+    # narrower than fp32 (measured rel-L2 ~1.3e-5 on fp32 outputs), so a handful
+    # of bf16 outputs land 2 ulp away; none further.
+    w64 = G.gemm_fp8(a, b, ex["scale_a"], ex["scale_b"], out_dtype=G.BF16, accumulate="f64")
+    # (entries that cancel to almost nothing are judged by rel-L2 above, not in ulps)
+    w64f = F.bf16_bits_to_f32(w64)
+    solid = np.abs(w64f) > 1e-2 * np.sqrt(np.mean(w64f.astype(np.float64) ** 2))
+    ulp = np.abs(out.astype(np.int32) - w64.astype(np.int32))
+    assert ulp[solid].max() <= 2 and np.mean(ulp[solid] > 1) < 1e-3
+    out32, _ = run_gemm(a, b, M, N, K, "fp8_e4m3", "f32", wg_tile=(tile, tile), **ex)
+    check(out32, G.gemm_fp8(a, b, ex["scale_a"], ex["scale_b"], out_dtype=G.F32), "f32", N, bar=1e-4)
+
+
+@pytest.mark.parametrize("M,N,K,tile", [(512, 512, 512, 256), (256, 384, 768, 128)])
+def test_config5_mxfp4(gpu, M, N, K, tile):
+    a, b, ex = operands(M, N, K, "mxfp4", a_std=1.0, b_std=1.0)
+    out, _ = run_gemm(a, b, M, N, K, "mxfp4", "bf16", wg_tile=(tile, tile), **ex)
+    check(out, G.gemm_mxfp4(a, ex["mx_a"], b, ex["mx_b"], out_dtype=G.BF16), "bf16", N)
+    out32, _ = run_gemm(a, b, M, N, K, "mxfp4", "f32", wg_tile=(tile, tile), **ex)
+    check(out32, G.gemm_mxfp4(a, ex["mx_a"], b, ex["mx_b"], out_dtype=G.F32), "f32", N, bar=1e-5)
+
+
+def test_mxfp4_nonuniform_scales_pin_the_lane_to_k_block_mapping(gpu):
+    # every (row, K-block) gets its own e8m0 byte and every element its own code:
+    # a wrong lane <-> K-block pairing cannot cancel.
+    M = N = 128
+    K = 512
+    rng = np.random.default_rng(5)
+    a = rng.integers(0, 256, (M, K // 2)).astype(np.uint8)
+    b = rng.integers(0, 256, (N, K // 2)).astype(np.uint8)
+    mxa = rng.integers(118, 134, (M, K // 32)).astype(np.uint8)
+    mxb = rng.integers(118, 134, (N, K // 32)).astype(np.uint8)
+    out, _ = run_gemm(a, b, M, N, K, "mxfp4", "f32", mx_a=mxa, mx_b=mxb)
+    check(out, G.gemm_mxfp4(a, mxa, b, mxb, out_dtype=G.F32), "f32", N, bar=1e-5)
+
+
+@pytest.mark.parametrize("M", [1, 16, 64])
+def test_config4_skinny_full_size(gpu, M):
+    N, K = 14336, 4096
+    a, b, _ = operands(M, N, K, "bf16", a_std=1.0, b_std=0.02)
+    out, name = run_gemm(a, b, M, N, K, "bf16", "bf16")
+    assert name.startswith("skinny")
+    check(out, G.gemm(a, b, G.BF16, G.BF16), "bf16", N)
+
+
+@pytest.mark.parametrize("M,N,K", [(3, 100, 64), (17, 264, 1056), (33, 48, 32), (64, 1032, 4096)])
+@pytest.mark.parametrize("dtype_ab", ["bf16", "f16"])
+def test_skinny_ragged(gpu, M, N, K, dtype_ab):
+    a, b, _ = operands(M, N, K, dtype_ab, seed=7, b_std=0.05)
+    bias = np.random.default_rng(9).standard_normal(N).astype(np.float32)
+    out, name = run_gemm(a, b, M, N, K, dtype_ab, "f32", bias=bias)
+    assert name.startswith("skinny")
+    check(out, G.gemm(a, b, _DT[dtype_ab], G.F32, bias=bias), "f32", N, bar=1e-5)
+
+
+# ---- edge cases: ragged M / N, K tails, leading dimensions, epilogue -----------------
+
+@pytest.mark.parametrize("M,N,K", [(1, 1, 8), (65, 16, 8), (130, 257, 72), (300, 520, 776), (129, 1, 64)])
+@pytest.mark.parametrize("dtype_ab", ["bf16", "f16"])
+def test_tile_ragged_shapes_and_k_tails(gpu, M, N, K, dtype_ab):
+    a, b, _ = operands(M, N, K, dtype_ab, seed=3, b_std=0.1)
+    out, name = run_gemm(a, b, M, N, K, dtype_ab, "f32", family=_capi.KERNEL_TILE)
+    assert name.startswith("tile")
+    check(out, G.gemm(a, b, _DT[dtype_ab], G.F32), "f32", N, bar=1e-5)
+
+
+def test_tile_fp8_k_tail(gpu):
+    M, N, K = 100, 200, 16 * 13
+    a, b, ex = operands(M, N, K, "fp8_e4m3", seed=4, b_std=1.0)
+    out, _ = run_gemm(a, b, M, N, K, "fp8_e4m3", "f32", **ex)
+    check(out, G.gemm_fp8(a, b, ex["scale_a"], ex["scale_b"], out_dtype=G.F32), "f32", N, bar=1e-4)
+
+
+def test_leading_dimensions(gpu):
+    M, N, K, lda, ldb, ldc = 200, 136, 96, 128, 104, 160
+    rng = np.random.default_rng(6)
+    a = F.f32_to_bf16_bits(rng.standard_normal((M, lda)).astype(np.float32))
+    b = F.f32_to_bf16_bits((rng.standard_normal((N, ldb)) * 0.1).astype(np.float32))
+    out, _ = run_gemm(a, b, M, N, K, "bf16", "bf16", lda=lda, ldb=ldb, ldc=ldc,
+                      family=_capi.KERNEL_TILE)
+    check(out, G.gemm(a[:, :K], b[:, :K], G.BF16, G.BF16), "bf16", N)
+    assert np.all(out[:, N:] == 0x7FC1)  # padding columns of C are not written
+
+
+@pytest.mark.parametrize("ldc", [0, 203])
+def test_bias_scale_and_output_types(gpu, ldc):
+    M, N, K = 140, 200, 128
+    a, b, ex = operands(M, N, K, "fp8_e4m3", seed=8, b_std=1.0)
+    bias = np.random.default_rng(10).standard_normal(N).astype(np.float32)
+    for dtype_c in ("f32", "bf16", "f16"):
+        out, _ = run_gemm(a, b, M, N, K, "fp8_e4m3", dtype_c, bias=bias, ldc=ldc, **ex)
+        want = G.gemm_fp8(a, b, ex["scale_a"], ex["scale_b"], out_dtype=_DT[dtype_c], bias=bias)
+        check(out, want, dtype_c, N)
+
+
+# ---- known answers of the reference's MFMA tests ---------------------------------------
+
+@pytest.fixture(scope="module")
+def kat(golden_dir):
+    with open(os.path.join(golden_dir, "kat.json")) as f:
+        return {c["name"]: c for c in json.load(f)["cases"]}
+
+
+def test_kat_bf16_all_ones(gpu, kat):
+    c = kat["bf16_16x16x32_all_ones"]
+    a = np.full((16, 32), int(c["a_bits"], 16), np.uint16)
+    out, _ = run_gemm(a, a, 16, 16, 32, "bf16", "f32", family=_capi.KERNEL_TILE)
+    assert np.all(out == c["expected"])
+    out, _ = run_gemm(a, a, 16, 16, 32, "bf16", "f32", family=_capi.KERNEL_SKINNY)
+    assert np.all(out == c["expected"])
+
+
+def test_kat_fp8_scaled(gpu, kat):
+    c = kat["fp8_scaled_nonidentity"]
+    a = np.full((16, 128), int(c["a_byte"], 16), np.uint8)
+    b = np.full((16, 128), int(c["b_byte"], 16), np.uint8)
+    out, _ = run_gemm(a, b, 16, 16, 128, "fp8_e4m3", "f32", scale_a=c["scale_a"], scale_b=c["scale_b"])
+    assert np.all(out == c["expected"])
+
+
+def test_kat_fp8_split_k_accumulate(gpu, kat):
+    c = kat["fp8_split_k_accum"]
+    a = np.empty((16, 128), np.uint8)
+    b = np.empty((16, 128), np.uint8)
+    a[:, :64], a[:, 64:] = (int(v, 16) for v in c["a_bytes_halves"])
+    b[:, :64], b[:, 64:] = (int(v, 16) for v in c["b_bytes_halves"])
+    out, _ = run_gemm(a, b, 16, 16, 128, "fp8_e4m3", "f32", scale_a=1.0, scale_b=1.0,
+                      bias=np.full(16, c["c_init"], np.float32))
+    assert np.all(out == c["expected"])
+
+
+def test_kat_mxfp4_block_scales(gpu):
+    # e2m1 code 2 = 1.0, code 3 = 1.5; e8m0 0x81 = 4, 0x80 = 2: 256 * 1.0 * 1.5 * 8 = 3072
+    a = np.full((16, 128), 0x22, np.uint8)
+    b = np.full((16, 128), 0x33, np.uint8)
+    out, _ = run_gemm(a, b, 16, 16, 256, "mxfp4", "f32", mx_a=np.full((16, 8), 0x81, np.uint8),
+                      mx_b=np.full((16, 8), 0x80, np.uint8))
+    assert np.all(out == 3072.0)
+
+
+# ---- full-size properties (configuration 2: bf16 8192^3) -------------------------------
+
+@pytest.fixture(scope="module")
+def big():
+    M = N = K = 8192
+    a, b, _ = operands(M, N, K, "bf16")
+    return M, N, K, a, b
+
+
+def test_config2_full_size_row_sample_determinism_and_scaling(gpu, big):
+    M, N, K, a, b = big
+    out, name = run_gemm(a, b, M, N, K, "bf16", "bf16")
+    assert "256x256" in name
+    rows = np.random.default_rng(0).choice(M, 48, replace=False)
+    rows = np.concatenate([rows, [0, 255, 256, M - 1]])
+    want = G.gemm(a[rows], b, G.BF16, G.BF16)
+    check(out[rows], want, "bf16", N)
+    cols = np.random.default_rng(1).choice(N, 32, replace=False)
+    want_c = G.gemm(a, b[cols], G.BF16, G.BF16)
+    check(out[:, cols], want_c, "bf16", 32)
+    # run-to-run determinism
+    out2, _ = run_gemm(a, b, M, N, K, "bf16", "bf16")
+    assert np.array_equal(out, out2)
+    # scaling A by 4 is exact in bf16 and in the fp32 accumulator
+    a4 = F.f32_to_bf16_bits(F.bf16_bits_to_f32(a) * 4.0)
+    out4, _ = run_gemm(a4, b, M, N, K, "bf16", "bf16")
+    assert np.array_equal(F.bf16_bits_to_f32(out4), F.bf16_bits_to_f32(out) * 4.0)
+
+
+def test_identity_operand_is_exact_at_full_width(gpu):
+    # B = I: every output is one product plus zeros, so C == A bit for bit.
+    M, N = 512, 8192
+    a = F.f32_to_bf16_bits(np.random.default_rng(2).standard_normal((M, N)).astype(np.float32))
+    eye = np.zeros((N, N), np.uint16)
+    eye[np.arange(N), np.arange(N)] = 0x3F80
+    out, _ = run_gemm(a, eye, M, N, N, "bf16", "bf16", family=_capi.KERNEL_TILE)
+    assert np.array_equal(out, a)

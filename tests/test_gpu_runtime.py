@@ -1,0 +1,116 @@
+"""Runtime seam on the GPU: buffers, events, memory manager, and `execute_hsaco`
+on the code object built from the same kernels (contracts of the reference's
+test/integration/test_execution_core.py:198-500)."""
+import os
+
+import numpy as np
+import pytest
+
+from aster_amd import build as B
+from aster_amd.execution import (FlushLLC, GpuBuffer, GpuEvent, GpuStream, InOutArray, InputArray,
+                                 MemoryManager, OutputArray, execute_hsaco, system_has_gpu)
+from oracle import gemm as G
+
+pytestmark = pytest.mark.gpu
+
+
+def test_system_has_gpu(gpu):
+    assert system_has_gpu("gfx950") and not system_has_gpu("gfx942")
+
+
+def test_gpu_buffer_roundtrip_and_contracts(gpu):
+    for dt in (np.float32, np.float16, np.int32, np.uint8, np.float64):
+        x = (np.arange(1000) % 251).astype(dt)
+        buf = GpuBuffer(x.nbytes)
+        buf.copy_from_host(x)
+        y = np.zeros_like(x)
+        buf.copy_to_host(y)
+        assert np.array_equal(x, y)
+        buf.free()
+        buf.free()  # idempotent
+    buf = GpuBuffer(16)
+    assert buf.size_bytes == 16 and buf.ptr_value
+    with pytest.raises(TypeError):
+        buf.copy_from_host([1, 2, 3])
+    with pytest.raises(TypeError):
+        buf.copy_to_host("x")
+    with pytest.raises(ValueError):
+        buf.copy_from_host(np.zeros(100, np.float32))
+    with pytest.raises(ValueError):
+        buf.copy_to_host(np.zeros(100, np.float32))
+
+
+def test_events_and_streams(gpu):
+    s = GpuStream()
+    s.synchronize()
+    s.destroy()
+    s.destroy()
+    e0, e1 = GpuEvent(), GpuEvent()
+    e0.record()
+    e1.record()
+    e1.synchronize()
+    assert e1.elapsed_ms(e0) >= 0.0
+    ns = e1.elapsed_ns(e0)
+    assert isinstance(ns, int) and ns >= 0
+    e0.destroy()
+    e0.destroy()
+
+
+def test_memory_manager_contracts(gpu):
+    mm = MemoryManager()
+    a = np.arange(64, dtype=np.float32)
+    b = np.zeros(64, dtype=np.float32)
+    buf = mm.register(a)
+    assert isinstance(buf, GpuBuffer) and mm.register(a) is buf
+    with pytest.raises(TypeError):
+        mm.register([1, 2])
+    mm.register(b, upload=False)
+    assert mm.get_buffer(b) is not buf
+    a[:] = 5
+    mm.sync_to_gpu(a)
+    a[:] = 0
+    mm.sync_from_gpu(a)
+    assert np.all(a == 5)
+    other = np.zeros(4, np.float32)
+    for fn in (mm.get_buffer, mm.sync_to_gpu, mm.sync_from_gpu, mm.release):
+        with pytest.raises(KeyError):
+            fn(other)
+    mm.release(a)
+    with pytest.raises(KeyError):
+        mm.get_buffer(a)
+    mm.release_all()
+    mm.release_all()
+    with pytest.raises(KeyError):
+        mm.get_buffer(b)
+
+
+def test_execute_hsaco_runs_the_code_object(gpu):
+    assert os.path.exists(B.HSACO_PATH), "run python -m aster_amd.build"
+    M, N, K = 160, 96, 72
+    np.random.seed(42 + M + N + K)
+    a = (np.random.randn(M, K) * 0.1).astype(np.float16)
+    b = (np.random.randn(N, K) * 0.1).astype(np.float16)
+    c = np.zeros(M * N, dtype=np.float32)
+    seen = []
+    grid = ((M + 127) // 128) * ((N + 127) // 128)
+    times = execute_hsaco(B.HSACO_PATH, "gemm_cdna4",
+                          [InputArray(a.flatten()), InputArray(b.flatten()), OutputArray(c), M, N, K],
+                          grid_dim=(grid, 1, 1), block_dim=(256, 1, 1), num_iterations=3,
+                          shared_bytes=65536, verify_fn=lambda args: seen.append(len(args)),
+                          flush_llc=FlushLLC(1 << 20))
+    assert len(times) == 3 and all(isinstance(t, int) and t > 0 for t in times)
+    assert seen == [6]
+    expected = (a.astype(np.float32) @ b.astype(np.float32).T).flatten()
+    np.testing.assert_allclose(c, expected, rtol=1e-2, atol=1e-2)
+    assert G.rel_l2(c, expected) <= 1e-3
+
+
+def test_execute_hsaco_inout_and_missing_kernel(gpu):
+    M = N = K = 128
+    a = np.full((M, K), 0x3F80, np.uint16)
+    c = np.zeros((M, N), dtype=np.uint16)
+    execute_hsaco(B.HSACO_PATH, "gemm_cdna4_bf16", [InputArray(a), InputArray(a), c, M, N, K],
+                  grid_dim=(1, 1, 1), block_dim=(256, 1, 1), shared_bytes=65536)
+    assert np.all(c == 0x4300)  # 128.0 in bf16
+    with pytest.raises(RuntimeError):
+        execute_hsaco(B.HSACO_PATH, "no_such_kernel", [InOutArray(c)])

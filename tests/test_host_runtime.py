@@ -1,0 +1,205 @@
+"""Host-side contracts that need no GPU: C-ABI exports, config validation and
+variant selection, kernel-argument packing, array roles, bench statistics."""
+import ctypes
+import io
+import json
+import os
+import re
+
+import numpy as np
+import pytest
+
+from aster_amd import _capi, bench_harness as BH, gemm, make_instance
+from aster_amd.execution import (InOutArray, InputArray, OutputArray, create_kernel_args,
+                                 create_kernel_args_capsule)
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    text = open(os.path.join(ROOT, "include", "astergemm.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    declared = set(re.findall(r"\b(astergemm_[a-z0-9_]+|aster_rt_[a-z0-9_]+)\s*\(", text))
+    assert len(declared) >= 35
+    lib = _capi.load()
+    for name in declared:
+        assert hasattr(lib, name), f"{name} declared in astergemm.h but not exported"
+    assert declared == set(_capi.SIGNATURES), declared ^ set(_capi.SIGNATURES)
+    assert lib.astergemm_abi_version() == 1
+
+
+def test_struct_sizes_match_header_layout():
+    # 6 x int64 + 16 x int32 ; pointers ; see include/astergemm.h
+    assert ctypes.sizeof(_capi.Config) == 6 * 8 + 16 * 4
+    assert ctypes.sizeof(_capi.Operands) == 8 * 8
+    assert ctypes.sizeof(_capi.KernelInfo) == 13 * 4 + 4 + 2 * 8 + 64
+
+
+def test_select_headline_configs():
+    p = gemm.GemmPlan.create(8192, 8192, 8192, "bf16", "bf16")
+    assert p.info.family == _capi.KERNEL_TILE
+    assert p.info.flops == 2 * 8192 ** 3 and p.info.bytes == 402653184
+    assert p.info.grid_x * p.info.wg_tile_m * p.info.wg_tile_n == 8192 * 8192
+    p = gemm.GemmPlan.create(8192, 8192, 8192, "fp8_e4m3", "bf16")
+    assert p.info.bytes == 268435464 and p.info.wg_tile_k == 128
+    p = gemm.GemmPlan.create(4096, 14336, 4096, "mxfp4", "bf16")
+    assert p.info.bytes == 157548544 and p.info.wg_tile_k == 256
+    for M, want in ((1, 117477376), (16, 118030336), (64, 119799808)):
+        p = gemm.GemmPlan.create(M, 14336, 4096, "bf16", "bf16")
+        assert p.info.family == _capi.KERNEL_SKINNY and p.info.bytes == want
+    p = gemm.GemmPlan.create(256, 256, 256, "f16", "f32")
+    assert p.info.family == _capi.KERNEL_TILE and p.info.wg_tile_m == 128
+
+
+def test_explicit_variant_and_enumeration():
+    lib = _capi.load()
+    n = lib.astergemm_variant_count()
+    assert n >= 24
+    c = _capi.Config()
+    c.M = c.N = c.K = 1024
+    c.dtype_ab, c.dtype_c = _capi.BF16, _capi.BF16
+    names = set()
+    for i in range(n):
+        info = _capi.KernelInfo()
+        _capi.check(lib.astergemm_variant_info(i, ctypes.byref(c), ctypes.byref(info)))
+        assert info.variant == i + 1
+        names.add(info.name.decode())
+    assert len(names) == n
+    info = _capi.KernelInfo()
+    assert lib.astergemm_variant_info(n, ctypes.byref(c), ctypes.byref(info)) == -22
+
+
+@pytest.mark.parametrize("kw,msg", [
+    (dict(M=128, N=128, K=0), "K > 0"),
+    (dict(M=-1, N=128, K=64), ">= 0"),
+    (dict(M=128, N=128, K=100), "16 bytes"),
+    (dict(M=128, N=128, K=64, lda=32), "leading dimension"),
+    (dict(M=128, N=128, K=64, dtype_ab="mxfp4", dtype_c="bf16", scale_mode="none"), "go together"),
+    (dict(M=128, N=128, K=128, dtype_ab="mxfp4", dtype_c="bf16"), "K % 256"),
+    (dict(M=128, N=128, K=64, family=_capi.KERNEL_SKINNY), "M <= 64"),
+    (dict(M=16, N=128, K=64, dtype_ab="fp8_e4m3", family=_capi.KERNEL_SKINNY), "no variant"),
+])
+def test_invalid_configs_are_refused_with_a_reason(kw, msg):
+    kw = dict(kw)
+    M, N, K = kw.pop("M"), kw.pop("N"), kw.pop("K")
+    with pytest.raises(_capi.AsterGemmError) as e:
+        gemm.GemmPlan.create(M, N, K, kw.pop("dtype_ab", "bf16"), kw.pop("dtype_c", "bf16"), **kw)
+    assert msg in str(e.value)
+    assert e.value.code in (-22, -95)
+
+
+def test_run_refuses_null_and_misaligned_pointers_before_touching_the_gpu():
+    p = gemm.GemmPlan.create(256, 256, 256)
+    with pytest.raises(_capi.AsterGemmError, match="non-null"):
+        p.run(None, None, None)
+    with pytest.raises(_capi.AsterGemmError, match="16-byte aligned"):
+        p.run(4096 + 8, 4096, 4096)
+    q = gemm.GemmPlan.create(256, 256, 256, "fp8_e4m3", "bf16")
+    with pytest.raises(_capi.AsterGemmError, match="dScaleA"):
+        q.run(4096, 4096, 4096)
+    b = gemm.GemmPlan.create(256, 256, 256, has_bias=True)
+    with pytest.raises(_capi.AsterGemmError, match="dBias"):
+        b.run(4096, 4096, 4096)
+    # empty problems are a no-op
+    gemm.GemmPlan.create(0, 256, 256).run(4096, 4096, 4096)
+
+
+def test_compile_gemm_writes_descriptor(tmp_path):
+    cfg = make_instance(512, 512, 256)
+    path, asm = gemm.compile_gemm(cfg, str(tmp_path / "k.hsaco"), num_vgprs=256, num_agprs=256)
+    desc = json.load(open(path))
+    assert desc["kernel"] == "tile_bf16_256x256_w2x4_bf16" and desc["grid"] == 4
+    assert desc["label"] == cfg.label and desc["lds_bytes"] == 131072
+    assert ".group_segment_fixed_size: 131072" in asm
+    (tmp_path / "bad.hsaco").write_text("{}")
+    with pytest.raises(ValueError):
+        gemm._read_descriptor(str(tmp_path / "bad.hsaco"))
+
+
+# ---- array roles and kernel-argument packing (reference:
+# test/integration/test_execution_core.py:51-189) ---------------------------------
+
+def test_array_role_wrappers():
+    a = np.zeros(4, np.float32)
+    assert InputArray(a).array is a and OutputArray(a).array is a and InOutArray(a).array is a
+    assert len({InputArray, OutputArray, InOutArray}) == 3
+    assert create_kernel_args_capsule is create_kernel_args
+
+
+def test_kernel_args_packing():
+    assert create_kernel_args() == (None, None, None)
+    ptrs, packed, _ = create_kernel_args(7, -3, 1.5, np.int64(9), np.float64(2.25),
+                                         ctypes.c_int64(1 << 40), ctypes.c_void_p(0x1234))
+    kinds = [t for _, t in packed._fields_]
+    assert kinds == [ctypes.c_int32, ctypes.c_int32, ctypes.c_float, ctypes.c_int32, ctypes.c_float,
+                     ctypes.c_int64, ctypes.c_void_p]
+    assert (packed._field0, packed._field1, packed._field2) == (7, -3, 1.5)
+    assert packed._field3 == 9 and packed._field4 == 2.25 and packed._field5 == 1 << 40
+    base, size = ctypes.addressof(packed), ctypes.sizeof(packed)
+    assert all(base <= p < base + size for p in ptrs)
+    arr = np.arange(4, dtype=np.float32)
+    ptrs, packed, _ = create_kernel_args(arr)
+    assert packed._field0 == arr.ctypes.data
+    with pytest.raises(TypeError, match="unsupported argument type"):
+        create_kernel_args("nope")
+
+
+# ---- bench statistics (reference: bench_harness.py:44-90, 174-198) ----------------
+
+def test_init_array_modes_are_deterministic():
+    a = BH.init_array((4, 8), "hpl", "A")
+    b = BH.init_array((4, 8), BH.InitMode.HPL, "B")
+    assert a.dtype == np.float16 and a.shape == (4, 8)
+    assert np.array_equal(a.reshape(-1), np.random.default_rng(42).uniform(-0.5, 0.5, 32).astype(np.float16))
+    assert np.array_equal(b.reshape(-1), np.random.default_rng(43).uniform(-0.5, 0.5, 32).astype(np.float16))
+    t = BH.init_array((8,), "trig_float", "B")
+    assert np.array_equal(t, np.cos(np.arange(8, dtype=np.float64)).astype(np.float16))
+    assert set(np.unique(BH.init_array((64,), "rand_int", "A")).tolist()) <= {-2, -1, 0, 1, 2}
+    assert not BH.init_array((4,), "zero", "A").any()
+    assert BH.init_array((2,), "special", "A")[0] == np.float16(65280.0)
+    assert BH.init_array((2,), "special", "B")[0] == np.float16(6.07967376708984375e-5)
+    n = BH.init_array((16,), "norm_dist", "A", dtype=np.float32)
+    assert np.array_equal(n, np.random.default_rng(42).standard_normal(16).astype(np.float32))
+    with pytest.raises(ValueError):
+        BH.init_array((2,), "nope", "A")
+    assert str(BH.INIT_DEFAULT) == "hpl" and BH.NUM_ITERATIONS == 100 and BH.WARMUP_ITERATIONS == 20
+
+
+def test_percentiles_and_stats():
+    times = [float(t) for t in range(100, 200)]          # 100 samples, ns
+    assert BH._percentile_ns(times, 0) == 100 and BH._percentile_ns(times, 100) == 199
+    assert BH._percentile_ns(times, 50) == 150 and BH._percentile_ns(times, 10) == 110
+    s = BH._compute_stats(list(reversed(times)), total_flops=3_000_000, peak_tflops=2500.0)
+    assert (s.p0_ns, s.p10_ns, s.p25_ns, s.p50_ns, s.p90_ns) == (100, 110, 125, 150, 189)
+    assert s.mean_ns == 149.5 and s.p50_tf == 3_000_000 / 150 * 1e-3
+    assert s.p50_pct == s.p50_tf / 2500.0 * 100 and s.p0_ms == 1e-4
+    assert BH._compute_stats([], 1, 1.0) is None and BH._compute_stats([5, 0], 1, 1.0) is None
+    one = BH._compute_stats([10], 1000, 1.0)
+    assert one.stddev_ns == 0.0 and one.stddev_tf == 0.0
+    assert BH.peak_tflops_f16("gfx950") == 2500.0 and BH.peak_tflops_f16("gfx942") == 1307.0
+    assert BH.peak_tflops("gfx950", "fp8_e4m3") == 5000.0
+
+
+def test_result_line_roundtrip():
+    cfg = make_instance(512, 512, 256)
+    s = BH._compute_stats([1000.0, 1100.0, 900.0], cfg.total_flops, 2500.0)
+    buf = io.StringIO()
+    BH.emit_one_result(buf, "bench_gemm", cfg, s)
+    BH.emit_one_result(None, "bench_gemm", cfg, s)
+    line = buf.getvalue()
+    assert line.startswith("BENCH_RESULT_JSON:")
+    rec, = BH.parse_result_lines(["noise", "x " + line, "BENCH_RESULT_JSON:{bad"])
+    assert rec["label"] == cfg.label and rec["mcpu"] == "gfx950" and rec["M"] == 512
+    assert rec["tflops_median"] == s.p50_tf and rec["sample_n"] == 1
+    assert set(rec) == {"mcpu", "bench", "M", "N", "K", "label", "tflops_median", "tflops_p10",
+                        "tflops_p90", "tflops_mean", "tflops_p0", "tflops_p25", "tflops_stddev",
+                        "pct_peak_p50", "sample_n"}
+
+
+def test_make_inputs_storage_types():
+    cfg = make_instance(256, 256, 64, dtype_ab="bf16")
+    a, b = BH.make_inputs(cfg)
+    assert a.dtype == np.uint16 and a.shape == (256, 64) and b.shape == (256, 64)
+    from oracle import formats as F
+    want = F.f32_to_bf16_bits(BH.init_array((256, 64), "hpl", "A").astype(np.float32))
+    assert np.array_equal(a, want)

@@ -1,0 +1,145 @@
+"""Layout algebra, swizzles, B pre-shuffle and the cooperative split."""
+import ctypes
+import itertools
+import math
+
+import numpy as np
+import pytest
+
+from aster_amd import _capi
+from aster_amd.coop import coop_2d_split, coop_wave_start
+from aster_amd.kittens_helpers import shuffle_weight, unshuffle_weight
+from aster_amd.layout import (TILE_LDS_SWIZZLE, Layout, Swizzle, delinearize, flatten_nested,
+                              linearize, make_layout, product, suffix_product, tile)
+from oracle import layouts as OL
+
+
+def test_int_tuple_helpers():
+    assert flatten_nested(((1, 2), 3, [4, (5,)])) == (1, 2, 3, 4, 5)
+    assert flatten_nested(7) == (7,)
+    assert product((2, 3, 4)) == 24 and product(5) == 5
+    assert suffix_product((2, 3, 4)) == (12, 4, 1) and suffix_product(9) == 1
+    assert delinearize(7, (4, 3)) == (2, 1)
+    assert linearize((3, 1), (1, 4)) == 7
+    for idx in range(24):
+        assert linearize(delinearize(idx, (2, 3, 4)), suffix_product((2, 3, 4))) == idx
+
+
+def test_layout_call_and_properties():
+    l = Layout((4, 16), (16, 64))
+    assert l(0) == 0 and l(1) == 64 and l(16) == 16 and l(17) == 80
+    assert Layout((4, 16)).strides == (16, 1)
+    assert Layout(8)(3) == 3
+    assert l.size() == 64 and len(l) == 2 and l.is_flat and l.flat_sizes == (4, 16)
+    assert not Layout(((2, 2), 4), ((1, 2), 4)).is_flat
+    assert l == Layout((4, 16), (16, 64)) and l != Layout((4, 16))
+    assert make_layout(Layout(4, 1), Layout(8, 4)) == Layout((4, 8), (1, 4))
+
+
+def test_tile():
+    t = tile(Layout((64, 32), (64, 2)), (16, 8))
+    assert t.sizes == (4, 4, 16, 8) and t.strides == (1024, 16, 64, 2)
+    h = tile(Layout((64,), (2,)), ((4, 2),))
+    assert h.sizes == (2, 8, 4) and h.strides == (8, 16, 2)
+    with pytest.raises(AssertionError):
+        tile(Layout((10,), (1,)), (4,))
+
+
+@pytest.mark.parametrize("sw", [Swizzle(3, 3, 4), Swizzle(2, 4, 4), TILE_LDS_SWIZZLE])
+def test_swizzle_is_an_involution_and_keeps_low_bits(sw):
+    span = 1 << (sw.base + sw.shift + sw.bits)
+    image = [sw(o) for o in range(span)]
+    assert sorted(image) == list(range(span))
+    assert all(sw(sw(o)) == o for o in range(span))
+    assert all((sw(o) ^ o) & ((1 << sw.base) - 1) == 0 for o in range(span))
+    assert all(sw(o) == OL.swizzle(o, sw.bits, sw.base, sw.shift) for o in range(span))
+
+
+def test_swizzle_3_3_4_is_the_mlir_16x64_formula():
+    sw = Swizzle(3, 3, 4)
+    for row in range(16):
+        for byte in range(64):
+            assert sw(row * 64 + byte) == OL.lds_swizzled_addr_16x64_b(0, row, byte)
+
+
+def test_tile_lds_swizzle_matches_kernel_formula_and_is_conflict_free():
+    for row in range(32):
+        for g in range(8):
+            assert TILE_LDS_SWIZZLE(row * 128 + g * 16) == OL.tile_lds_offset(row, g)
+    # A ds_read_b128 serves 16 lanes at a time: 16 rows x one K granule must land
+    # in 16 distinct 16-byte bank groups (64 banks x 4 B).
+    for row0 in (0, 16):
+        for g in range(8):
+            offs = [OL.tile_lds_offset(row0 + i, g) for i in range(16)]
+            assert len(set(OL.bank_groups_16B(offs))) == 16
+    # without the swizzle the same access is an 8-way conflict
+    assert len(set(OL.bank_groups_16B([i * 128 for i in range(16)]))) == 2
+
+
+def test_mfma_fragment_maps_cover_the_tile():
+    a = {(OL.mfma_index_a_16x16_f16(l)[0], OL.mfma_index_a_16x16_f16(l)[1] + e)
+         for l in range(64) for e in range(4)}
+    assert a == set(itertools.product(range(16), range(16)))
+    f8 = {(OL.mfma_index_a_16x16_fp8(l)[0], OL.mfma_index_a_16x16_fp8(l)[1] + e)
+          for l in range(64) for e in range(8)}
+    assert f8 == set(itertools.product(range(16), range(32)))
+    c = {(OL.mfma_index_c_16x16_f32(l)[1] + r, OL.mfma_index_c_16x16_f32(l)[0])
+         for l in range(64) for r in range(4)}
+    assert c == set(itertools.product(range(16), range(16)))
+    # element (r, c) of the C tile is owned by lane 16 * (r // 4) + c
+    for l in range(64):
+        col, rb = OL.mfma_index_c_16x16_f32(l)
+        assert l == 16 * (rb // 4) + col
+
+
+@pytest.mark.parametrize("N,K", [(16, 32), (32, 64), (48, 96)])
+def test_shuffle_weight(N, K):
+    B = np.arange(N * K, dtype=np.uint16).reshape(N, K)
+    S = shuffle_weight(B)
+    assert np.array_equal(S, OL.shuffle_weight(B))
+    assert np.array_equal(np.sort(S.reshape(-1)), B.reshape(-1))
+    assert np.array_equal(unshuffle_weight(S), B)
+    # the docstring's lane property: lane d of block (nb, kb) reads 8 contiguous
+    # elements = B[nb*16 + d%16, kb*32 + kh*16 + (d//16)*4 + 0..3], kh = 0, 1
+    flat = S.reshape(-1)
+    for nb in range(N // 16):
+        for kb in range(K // 32):
+            for d in range(64):
+                base = (nb * (K // 32) + kb) * 512 + d * 8
+                for kh in range(2):
+                    want = B[nb * 16 + d % 16, kb * 32 + kh * 16 + (d // 16) * 4:][:4]
+                    assert np.array_equal(flat[base + kh * 4: base + kh * 4 + 4], want)
+    # the C-ABI host routine gives the same bytes
+    out = np.empty_like(B)
+    _capi.check(_capi.load().astergemm_shuffle_weight_16(B.ctypes.data, out.ctypes.data, N, K))
+    assert np.array_equal(out, S)
+
+
+def test_shuffle_weight_rejects_bad_shapes():
+    with pytest.raises(AssertionError):
+        shuffle_weight(np.zeros((15, 32), np.float16))
+    with pytest.raises(AssertionError):
+        shuffle_weight(np.zeros((16, 48), np.float16))
+    z = np.zeros((15, 32), np.uint16)
+    assert _capi.load().astergemm_shuffle_weight_16(z.ctypes.data, z.ctypes.data, 15, 32) == -22
+
+
+def test_coop_2d_split_bruteforce():
+    for num_tiles in range(1, 33):
+        for num_waves in (1, 2, 4, 8):
+            for kt in range(1, 5):
+                ws, wk, cs, ck = coop_2d_split(num_tiles, num_waves, kt)
+                assert ws * wk == num_waves
+                assert cs == math.ceil(num_tiles / ws) and ck == math.ceil(kt / wk)
+                waste = ws * wk * cs * ck - num_tiles * kt
+                for d in (d for d in range(1, num_waves + 1) if num_waves % d == 0):
+                    other = num_waves * math.ceil(num_tiles / d) * math.ceil(kt / (num_waves // d))
+                    assert waste <= other - num_tiles * kt
+                covered = set()
+                for w in range(num_waves):
+                    s0 = coop_wave_start(w // wk, cs, num_tiles)
+                    k0 = coop_wave_start(w % wk, ck, kt)
+                    covered |= {(s, k) for s in range(s0, s0 + cs) for k in range(k0, k0 + ck)}
+                assert covered >= set(itertools.product(range(num_tiles), range(kt)))
+    assert coop_2d_split(8, 4, 1) == (4, 1, 2, 1)
+    assert coop_2d_split(2, 8, 2) == (4, 2, 1, 1)
