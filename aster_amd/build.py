@@ -24,6 +24,7 @@ OBJ_DIR = os.path.join(ROOT, "build", "obj")
 SOURCES = ["gemm_tile.hip", "gemm_skinny.hip", "astergemm_api.hip"]
 HSACO_SOURCE = "hsaco_kernels.hip"
 HSACO_PATH = os.path.join(LIB_DIR, "astergemm_kernels.hsaco")
+REPLAY_PATH = os.path.join(LIB_DIR, "astergemm_replay")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
@@ -74,6 +75,13 @@ def build_library(verbose: bool = False) -> str:
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError(f"link failed:\n{proc.stdout}\n{proc.stderr}")
+    # astergemm_replay: host-only program on top of the C-ABI, for profilers.
+    cmd = ["g++", "-O2", "-std=c++17", "-I" + os.path.join(ROOT, "include"),
+           os.path.join(CSRC, "astergemm_replay.cpp"), "-o", REPLAY_PATH,
+           "-L" + LIB_DIR, "-lastergemm", "-Wl,-rpath,$ORIGIN"]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"replay tool build failed:\n{proc.stdout}\n{proc.stderr}")
     if verbose:
         print(f"built {LIB_PATH}")
     return LIB_PATH

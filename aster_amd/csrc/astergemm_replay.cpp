@@ -1,0 +1,199 @@
+// astergemm_replay: launch one GEMM configuration N times through the C-ABI and
+// print per-launch timing statistics.  A plain executable with no interpreter in
+// front of it, so it can sit directly after `rocprofv3 ... --`.
+//
+// The reference profiles its kernels by replaying a pre-compiled code object
+// under rocprofv3 (contrib/kittens/rocprof-kittens-bench.sh:44, 103-112; two
+// phases because its compiler cannot run under the profiler).  Nothing is
+// compiled at run time here, so the replay is this one program.
+//
+//   astergemm_replay --m 8192 --n 8192 --k 8192 --ab bf16 --c bf16 --iters 100
+//                    [--warmup 20] [--tile 256] [--family tile|skinny|auto]
+//                    [--variant ID] [--flush BYTES] [--bias] [--json]
+#include <math.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <algorithm>
+#include <string>
+#include <vector>
+
+#include "astergemm.h"
+
+static int dtype_of(const char* s) {
+  if (!strcmp(s, "f16")) return ASTERGEMM_F16;
+  if (!strcmp(s, "bf16")) return ASTERGEMM_BF16;
+  if (!strcmp(s, "fp8") || !strcmp(s, "fp8_e4m3")) return ASTERGEMM_FP8_E4M3;
+  if (!strcmp(s, "mxfp4") || !strcmp(s, "fp4")) return ASTERGEMM_MXFP4;
+  if (!strcmp(s, "f32")) return ASTERGEMM_F32;
+  fprintf(stderr, "unknown dtype %s\n", s);
+  exit(2);
+}
+
+#define CHECK(call)                                                          \
+  do {                                                                       \
+    int _rc = (call);                                                        \
+    if (_rc != 0) {                                                          \
+      fprintf(stderr, "%s failed: %d %s\n", #call, _rc, astergemm_last_error()); \
+      return 1;                                                              \
+    }                                                                        \
+  } while (0)
+
+// xorshift bytes; for 16-bit floats keep exponents near 1.0 * 2^-6 so nothing
+// overflows: sign random, exponent in a narrow band, mantissa random.
+static void fill(std::vector<uint8_t>& buf, int dtype, uint64_t seed) {
+  uint64_t x = seed * 0x9E3779B97F4A7C15ull + 1;
+  auto next = [&]() {
+    x ^= x << 13;
+    x ^= x >> 7;
+    x ^= x << 17;
+    return x;
+  };
+  if (dtype == ASTERGEMM_BF16 || dtype == ASTERGEMM_F16) {
+    uint16_t* p = (uint16_t*)buf.data();
+    const size_t n = buf.size() / 2;
+    for (size_t i = 0; i < n; ++i) {
+      const uint64_t r = next();
+      if (dtype == ASTERGEMM_BF16) {
+        const uint16_t e = (uint16_t)(118 + (r & 3));  // 2^-9 .. 2^-6
+        p[i] = (uint16_t)(((r >> 8) & 1) << 15 | e << 7 | ((r >> 16) & 0x7F));
+      } else {
+        const uint16_t e = (uint16_t)(6 + (r & 3));
+        p[i] = (uint16_t)(((r >> 8) & 1) << 15 | e << 10 | ((r >> 16) & 0x3FF));
+      }
+    }
+  } else if (dtype == ASTERGEMM_FP8_E4M3) {
+    for (size_t i = 0; i < buf.size(); ++i) {
+      uint8_t b = (uint8_t)next();
+      if ((b & 0x7F) == 0x7F) b &= 0xFE;  // no NaN codes
+      buf[i] = b;
+    }
+  } else {
+    for (size_t i = 0; i < buf.size(); ++i) buf[i] = (uint8_t)next();
+  }
+}
+
+int main(int argc, char** argv) {
+  astergemm_config cfg;
+  memset(&cfg, 0, sizeof(cfg));
+  cfg.M = cfg.N = cfg.K = 8192;
+  cfg.dtype_ab = ASTERGEMM_BF16;
+  cfg.dtype_c = ASTERGEMM_BF16;
+  int iters = 100, warmup = 20, json = 0;
+  long long flush = 0;
+  for (int i = 1; i < argc; ++i) {
+    std::string a = argv[i];
+    auto val = [&]() -> const char* {
+      if (i + 1 >= argc) {
+        fprintf(stderr, "%s needs a value\n", a.c_str());
+        exit(2);
+      }
+      return argv[++i];
+    };
+    if (a == "--m") cfg.M = atoll(val());
+    else if (a == "--n") cfg.N = atoll(val());
+    else if (a == "--k") cfg.K = atoll(val());
+    else if (a == "--ab") cfg.dtype_ab = dtype_of(val());
+    else if (a == "--c") cfg.dtype_c = dtype_of(val());
+    else if (a == "--iters") iters = atoi(val());
+    else if (a == "--warmup") warmup = atoi(val());
+    else if (a == "--tile") cfg.wg_tile_m = cfg.wg_tile_n = atoi(val());
+    else if (a == "--variant") cfg.variant = atoi(val());
+    else if (a == "--flush") flush = atoll(val());
+    else if (a == "--bias") cfg.has_bias = 1;
+    else if (a == "--json") json = 1;
+    else if (a == "--family") {
+      const char* f = val();
+      cfg.family = !strcmp(f, "tile") ? ASTERGEMM_KERNEL_TILE
+                   : !strcmp(f, "skinny") ? ASTERGEMM_KERNEL_SKINNY : ASTERGEMM_KERNEL_AUTO;
+    } else {
+      fprintf(stderr, "unknown argument %s\n", a.c_str());
+      return 2;
+    }
+  }
+  if (cfg.dtype_ab == ASTERGEMM_FP8_E4M3) cfg.scale_mode = ASTERGEMM_SCALE_TENSOR;
+  if (cfg.dtype_ab == ASTERGEMM_MXFP4) cfg.scale_mode = ASTERGEMM_SCALE_MX32;
+  if (iters <= warmup) {
+    fprintf(stderr, "--iters must exceed --warmup\n");
+    return 2;
+  }
+
+  CHECK(aster_rt_init());
+  astergemm_kernel_info info;
+  CHECK(astergemm_select(&cfg, &info));
+
+  const int bits = cfg.dtype_ab == ASTERGEMM_MXFP4 ? 4 : cfg.dtype_ab == ASTERGEMM_FP8_E4M3 ? 8 : 16;
+  const size_t a_bytes = (size_t)cfg.M * cfg.K * bits / 8, b_bytes = (size_t)cfg.N * cfg.K * bits / 8;
+  const size_t c_bytes = (size_t)cfg.M * cfg.N * (cfg.dtype_c == ASTERGEMM_F32 ? 4 : 2);
+  std::vector<uint8_t> ha(a_bytes), hb(b_bytes);
+  fill(ha, cfg.dtype_ab, 42);
+  fill(hb, cfg.dtype_ab, 43);
+
+  astergemm_operands ops;
+  memset(&ops, 0, sizeof(ops));
+  void *dA, *dB, *dC;
+  CHECK(aster_rt_malloc(&dA, a_bytes));
+  CHECK(aster_rt_malloc(&dB, b_bytes));
+  CHECK(aster_rt_malloc(&dC, c_bytes));
+  CHECK(aster_rt_memcpy_h2d(dA, ha.data(), a_bytes));
+  CHECK(aster_rt_memcpy_h2d(dB, hb.data(), b_bytes));
+  ops.dA = dA;
+  ops.dB = dB;
+  ops.dC = dC;
+  if (cfg.scale_mode == ASTERGEMM_SCALE_TENSOR) {
+    const float s[2] = {0.01f, 0.02f};
+    void* ds;
+    CHECK(aster_rt_malloc(&ds, 256));
+    CHECK(aster_rt_memcpy_h2d(ds, s, sizeof(s)));
+    ops.dScaleA = (const float*)ds;
+    ops.dScaleB = (const float*)ds + 1;
+  }
+  if (cfg.scale_mode == ASTERGEMM_SCALE_MX32) {
+    std::vector<uint8_t> sa((size_t)cfg.M * cfg.K / 32, 122), sb((size_t)cfg.N * cfg.K / 32, 123);
+    void *da, *db;
+    CHECK(aster_rt_malloc(&da, sa.size()));
+    CHECK(aster_rt_malloc(&db, sb.size()));
+    CHECK(aster_rt_memcpy_h2d(da, sa.data(), sa.size()));
+    CHECK(aster_rt_memcpy_h2d(db, sb.data(), sb.size()));
+    ops.dMxA = (const uint8_t*)da;
+    ops.dMxB = (const uint8_t*)db;
+  }
+  if (cfg.has_bias) {
+    std::vector<float> hbias((size_t)cfg.N, 0.5f);
+    void* dbias;
+    CHECK(aster_rt_malloc(&dbias, hbias.size() * 4));
+    CHECK(aster_rt_memcpy_h2d(dbias, hbias.data(), hbias.size() * 4));
+    ops.dBias = (const float*)dbias;
+  }
+
+  std::vector<int64_t> t((size_t)iters);
+  CHECK(astergemm_bench(&cfg, &ops, iters, t.data(), flush, nullptr));
+  std::vector<int64_t> m(t.begin() + warmup, t.end());
+  std::sort(m.begin(), m.end());
+  auto pct = [&](double p) {
+    long idx = lround(p / 100.0 * (double)(m.size() - 1));
+    return (double)m[(size_t)std::max(0l, std::min((long)m.size() - 1, idx))];
+  };
+  double mean = 0;
+  for (int64_t v : m) mean += (double)v;
+  mean /= (double)m.size();
+  const double p50 = pct(50);
+  const double tflops = (double)info.flops / p50 * 1e-3, gbps = (double)info.bytes / p50;
+  if (json) {
+    printf("{\"kernel\": \"%s\", \"M\": %lld, \"N\": %lld, \"K\": %lld, \"grid\": %d, \"block\": %d, "
+           "\"lds_bytes\": %d, \"regs\": %d, \"iters\": %d, \"warmup\": %d, \"p0_us\": %.2f, "
+           "\"p10_us\": %.2f, \"p50_us\": %.2f, \"p90_us\": %.2f, \"mean_us\": %.2f, "
+           "\"tflops_p50\": %.1f, \"gbps_p50\": %.1f, \"flush_bytes\": %lld}\n",
+           info.name, (long long)cfg.M, (long long)cfg.N, (long long)cfg.K, info.grid_x, info.block_x,
+           info.lds_bytes, info.vgprs, iters, warmup, pct(0) / 1e3, pct(10) / 1e3, p50 / 1e3,
+           pct(90) / 1e3, mean / 1e3, tflops, gbps, flush);
+  } else {
+    printf("%s  M=%lld N=%lld K=%lld grid=%d block=%d lds=%d regs=%d\n", info.name, (long long)cfg.M,
+           (long long)cfg.N, (long long)cfg.K, info.grid_x, info.block_x, info.lds_bytes, info.vgprs);
+    printf("  p0 %.2f us  p10 %.2f  p50 %.2f  p90 %.2f  mean %.2f   p50: %.1f TFLOP/s  %.1f GB/s\n",
+           pct(0) / 1e3, pct(10) / 1e3, p50 / 1e3, pct(90) / 1e3, mean / 1e3, tflops, gbps);
+  }
+  return 0;
+}
