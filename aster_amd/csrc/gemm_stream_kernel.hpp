@@ -1,0 +1,322 @@
+// MFMA tile kernel with whole-cache-line staging and register double-buffered
+// fragments, for gfx950: C[M,N] = epi(A[M,K] * B[N,K]^T), 16-bit operands.
+//
+// What measurement on MI355X says this kernel has to respect:
+//   * the vector L1 moves 64 B/clk/CU and is charged per cache line touched, so
+//     a global->LDS transfer should cover whole 128-byte lines (8 rows x 128 B per
+//     wave instruction); 64-byte row slices cost twice the L1 time per byte;
+//   * with realistic operand bits the matrix cores are power limited: back-to-back
+//     v_mfma_f32_16x16x32_bf16 on random data sustain ~1.75 PFLOP/s when srcA
+//     changes on every instruction and ~1.92 PFLOP/s when srcA is held for eight
+//     instructions in a row, so the inner loop is ordered n-outer / m-inner with
+//     the B-row fragment as srcA;
+//   * ds_read_b128 serves 16 lanes per cycle (256 B/clk) when conflict-free,
+//     ds_read_b64 only a quarter of that.
+//   * a 64 KiB K-step of transfers issued at once needs ~2150 shader clocks until
+//     the last byte is in LDS (about half latency, half L1 transfer time), more
+//     than the 2048 clocks the matrix cores need for that K-step; and under MFMA
+//     load the shader clock, which also clocks L1 and L2, drops to ~1.7 GHz.
+// Structure: 256x256 workgroup tile, K-step = 128 bytes of a row.  LDS is a ring of
+// five 32 KiB slots (all 160 KiB), each holding the A half or the B half of one
+// K-step: A(k) in slot 2k mod 5, B(k) in slot (2k+1) mod 5.  When K-step k has been
+// read into registers its two slots are refilled with B(k+2) and A(k+3), so 96 KiB
+// are in flight and the half that is needed first, B(k+1), was the first in the
+// queue a whole K-step earlier.  Each K-step is two MFMA k-substeps; the fragments
+// of substep j+1 are read from LDS before the MFMAs of substep j are issued; one
+// barrier per K-step.  The reference's equivalent pieces: direct-to-LDS staging
+// (python/aster/dialects/kernel_builder_with_layouts.py:371-481), fragment reads
+// (contrib/kittens/library/lds_mfma_16x64_b.mlir), the (k, m, n) MFMA loop
+// (contrib/kittens/test/test_102_gemm_python_multitile_g2s_directb_cdna4.py:296-306).
+#pragma once
+#include <type_traits>
+
+#include "gemm_tile_kernel.hpp"
+
+namespace astergemm {
+namespace {
+
+template <int I, int N, class Fn>
+__device__ __forceinline__ void static_for(Fn&& f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<I + 1, N>(f);
+  }
+}
+
+template <int DT, int OUT, int BM, int BN, int WM, int WN>
+__device__ __forceinline__ void gemm_stream_body(const GemmArgs& p) {
+  constexpr int NW = WM * WN;
+  constexpr int TM = BM / WM / 16;
+  constexpr int TN = BN / WN / 16;
+  constexpr int SLOT = BM * kRowBytes;  // 32 KiB: one operand half of one K-step
+  constexpr int NSLOT = 5;
+  constexpr int LH = BM / 8 / NW;       // 1 KiB (8 rows x 128 B) transfers per wave and slot
+  static_assert(BM == BN, "the ring holds equal A and B halves");
+  static_assert(DT == ASTERGEMM_BF16 || DT == ASTERGEMM_F16, "16-bit operands");
+  static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "tile rows per wave");
+  static_assert((8 * NW) % 16 == 0, "swizzle phase must not depend on the transfer index");
+
+  extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WN, wn = wave % WN;
+
+  int tile_m, tile_n;
+  map_tile(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m, tile_m, tile_n);
+  const int row0 = tile_m * BM, col0 = tile_n * BN;
+
+  // ---- global -> LDS (same layout as gemm_tile_body: 128-byte rows, granule
+  // index XOR ((row >> 1) & 7)).  Only whole tiles and whole K-steps come here, so
+  // one per-lane offset serves every transfer and the row block of transfer j goes
+  // into the scalar base.
+  const int lrow = lane >> 3;
+  const int g_lane = (lane & 7) ^ (((wave * 8 + lrow) >> 1) & 7);
+  const unsigned a_off = (unsigned)(lrow * (int)p.lda_bytes + g_lane * 16);
+  const unsigned b_off = (unsigned)(lrow * (int)p.ldb_bytes + g_lane * 16);
+  const uint8_t* a_base = p.A + ((int64_t)row0 + wave * 8) * p.lda_bytes;
+  const uint8_t* b_base = p.B + ((int64_t)col0 + wave * 8) * p.ldb_bytes;
+  const int64_t a_jstride = (int64_t)8 * NW * p.lda_bytes;
+  const int64_t b_jstride = (int64_t)8 * NW * p.ldb_bytes;
+  const int nk = p.ksteps;
+
+  // 64 lanes x 16 bytes from (scalar base + per-lane offset) to LDS at M0 + lane*16.
+  // Written as asm to keep the scalar-base form; vmcnt is tracked by hand.
+  auto g2s = [&](const uint8_t* base, unsigned voff, uint8_t* dst) {
+#ifdef AG_DBG_BUILTIN_G2S
+    __builtin_amdgcn_global_load_lds(AG_GLOBAL(base + voff), AG_LDS(dst), 16, 0, 0);
+    return;
+#endif
+    const unsigned m0v = (unsigned)(size_t)AG_LDS(dst);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(m0v), "v"(voff), "s"(base)
+                 : "memory", "m0");
+  };
+  // transfer j (0..LH-1) of this wave for the A / B half of K-step k
+  auto issue_a1 = [&](int k, int slot, int j) {
+    g2s(a_base + (int64_t)k * kRowBytes + j * a_jstride, a_off,
+        lds + slot * SLOT + (j * NW + wave) * 8 * kRowBytes);
+  };
+  auto issue_b1 = [&](int k, int slot, int j) {
+    g2s(b_base + (int64_t)k * kRowBytes + j * b_jstride, b_off,
+        lds + slot * SLOT + (j * NW + wave) * 8 * kRowBytes);
+  };
+  auto issue_a = [&](int k, int slot) {
+#pragma unroll
+    for (int j = 0; j < LH; ++j) issue_a1(k, slot, j);
+  };
+  auto issue_b = [&](int k, int slot) {
+#pragma unroll
+    for (int j = 0; j < LH; ++j) issue_b1(k, slot, j);
+  };
+
+  // ---- LDS -> fragments -------------------------------------------------------------
+  const int li = lane & 15, lq = lane >> 4;
+  unsigned rd_off[2];
+#pragma unroll
+  for (int s = 0; s < 2; ++s)
+    rd_off[s] = (unsigned)(li * kRowBytes + (((s * 4 + lq) ^ (li >> 1)) << 4));
+  const unsigned a_rd = (unsigned)(wm * TM * 16 * kRowBytes);
+  const unsigned b_rd = (unsigned)(wn * TN * 16 * kRowBytes);
+
+  // KM = k mod 5 fixes the ring slots of K-step k at compile time.
+  i32x4 fa[2][TM], fb[2][TN];
+  auto read_frags = [&](auto kmod, auto sub) {
+    constexpr int KM = decltype(kmod)::value;
+    constexpr int S = decltype(sub)::value;
+    const uint8_t* sa = lds + ((2 * KM) % NSLOT) * SLOT;
+    const uint8_t* sb = lds + ((2 * KM + 1) % NSLOT) * SLOT;
+#pragma unroll
+    for (int n = 0; n < TN; ++n)
+      fb[S][n] = *(const i32x4*)(sb + b_rd + n * 16 * kRowBytes + rd_off[S]);
+#pragma unroll
+    for (int m = 0; m < TM; ++m)
+      fa[S][m] = *(const i32x4*)(sa + a_rd + m * 16 * kRowBytes + rd_off[S]);
+  };
+
+  f32x4 acc[TM][TN];
+#pragma unroll
+  for (int m = 0; m < TM; ++m)
+#pragma unroll
+    for (int n = 0; n < TN; ++n) acc[m][n] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // fragment I of substep S of the K-step with ring position KM: I < TN is B tile I,
+  // else A tile I - TN
+  auto read_one = [&](auto kmod, auto sub, auto idx) {
+    constexpr int KM = decltype(kmod)::value;
+    constexpr int S = decltype(sub)::value;
+    constexpr int I = decltype(idx)::value;
+    if constexpr (I < TN) {
+      const uint8_t* sb = lds + ((2 * KM + 1) % NSLOT) * SLOT;
+      fb[S][I] = *(const i32x4*)(sb + b_rd + I * 16 * kRowBytes + rd_off[S]);
+    } else {
+      const uint8_t* sa = lds + ((2 * KM) % NSLOT) * SLOT;
+      fa[S][I - TN] = *(const i32x4*)(sa + a_rd + (I - TN) * 16 * kRowBytes + rd_off[S]);
+    }
+  };
+
+  // srcA = B-row fragment, held for TM instructions in a row; lane owns
+  // C[m = lane % 16][4 consecutive n].
+  auto mfmas = [&](auto sub) {
+    constexpr int S = decltype(sub)::value;
+#ifdef AG_DBG_NO_MFMA
+#pragma unroll
+    for (int n = 0; n < TN; ++n) {
+      i32x4 t = fb[S][n];
+      asm volatile("" ::"v"(t));
+    }
+#pragma unroll
+    for (int m = 0; m < TM; ++m) {
+      i32x4 t = fa[S][m];
+      asm volatile("" ::"v"(t));
+    }
+#else
+#pragma unroll
+    for (int n = 0; n < TN; ++n)
+#pragma unroll
+      for (int m = 0; m < TM; ++m)
+        acc[m][n] = mfma_step<DT>(&fb[S][n], &fa[S][m], acc[m][n], 0, 0);
+#endif
+  };
+  using S0 = std::integral_constant<int, 0>;
+  using S1 = std::integral_constant<int, 1>;
+
+  // ---- prologue: A(0) B(0) A(1) B(1) A(2) in flight, both fragment sets of K-step 0
+  // read, first substep multiplied -----------------------------------------------------------
+  issue_a(0, 0);
+  issue_b(0, 1);
+  if (nk > 1) {
+    issue_a(1, 2);
+    issue_b(1, 3);
+  }
+  if (nk > 2) issue_a(2, 4);
+  if (nk > 2) __builtin_amdgcn_s_waitcnt(waitcnt_imm(3 * LH, 15));
+  else if (nk > 1) __builtin_amdgcn_s_waitcnt(waitcnt_imm(2 * LH, 15));
+  else __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+  using K0 = std::integral_constant<int, 0>;
+  read_frags(K0{}, S0{});
+  read_frags(K0{}, S1{});
+  __builtin_amdgcn_sched_barrier(0);
+  mfmas(S0{});
+  __builtin_amdgcn_sched_barrier(0);
+
+  // ---- K loop ------------------------------------------------------------------------------
+  // One trip finishes K-step k (substep 1) and starts K-step k+1 (substep 0).  It
+  // begins with a wait and a barrier: A(k+1) and B(k+1) have landed for everybody
+  // (only A(k+2) may still be in flight) and every fragment of K-step k is in
+  // registers, which frees its two slots for B(k+2) and A(k+3).
+  // Inside a trip nothing is issued in bursts: a wave that is stuck pushing loads
+  // into a full address queue, or reads into a full LDS queue, cannot issue MFMAs.
+  // So every MFMA is followed by at most one LDS read or one global->LDS transfer:
+  // block 1 (substep 1 of K-step k) carries the reads of substep 0 of K-step k+1 and
+  // the transfers of B(k+2), which is needed first; block 2 carries the reads of
+  // substep 1 and the transfers of A(k+3).
+  auto trip = [&](int k, auto kmod, auto steady) {
+    constexpr int KM = decltype(kmod)::value;
+    constexpr bool STEADY = decltype(steady)::value;
+    using KN = std::integral_constant<int, (KM + 1) % NSLOT>;
+    constexpr int NF = TM + TN;      // fragments per substep
+    constexpr int NMF = TM * TN;     // MFMAs per substep
+    static_assert(NF + LH <= NMF, "one side instruction per MFMA");
+    if constexpr (STEADY) __builtin_amdgcn_s_waitcnt(waitcnt_imm(LH, 0));
+    else __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    const bool do_b = STEADY || k + 2 < nk;
+    const bool do_a = STEADY || k + 3 < nk;
+    static_for<0, NMF>([&](auto ic) {
+      constexpr int I = decltype(ic)::value;
+      constexpr int n = I / TM, m = I % TM;
+#ifndef AG_DBG_NO_MFMA
+      acc[m][n] = mfma_step<DT>(&fb[1][n], &fa[1][m], acc[m][n], 0, 0);
+#endif
+#ifndef AG_DBG_NO_LOAD
+      if constexpr (I < LH) {
+        if (do_b) issue_b1(k + 2, (2 * KM) % NSLOT, I);
+      }
+#endif
+#ifndef AG_DBG_NO_READ
+      if constexpr (I >= LH && I < LH + NF) read_one(KN{}, S0{}, std::integral_constant<int, I - LH>{});
+#endif
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    static_for<0, NMF>([&](auto ic) {
+      constexpr int I = decltype(ic)::value;
+      constexpr int n = I / TM, m = I % TM;
+#ifndef AG_DBG_NO_MFMA
+      acc[m][n] = mfma_step<DT>(&fb[0][n], &fa[0][m], acc[m][n], 0, 0);
+#endif
+#ifndef AG_DBG_NO_READ
+      if constexpr (I < NF) read_one(KN{}, S1{}, std::integral_constant<int, I>{});
+#endif
+#ifndef AG_DBG_NO_LOAD
+      if constexpr (I >= NF && I < NF + LH) {
+        if (do_a) issue_a1(k + 3, (2 * KM + 1) % NSLOT, I - NF);
+      }
+#endif
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  };
+  using T = std::true_type;
+  using F = std::false_type;
+  int k = 0;
+  // steady: K-steps up to k+4+3 exist for the whole group of five trips
+  for (; k + 8 <= nk; k += 5) {
+    trip(k, std::integral_constant<int, 0>{}, T{});
+    trip(k + 1, std::integral_constant<int, 1>{}, T{});
+    trip(k + 2, std::integral_constant<int, 2>{}, T{});
+    trip(k + 3, std::integral_constant<int, 3>{}, T{});
+    trip(k + 4, std::integral_constant<int, 4>{}, T{});
+  }
+  for (; k + 1 < nk; k += 5) {
+    trip(k, std::integral_constant<int, 0>{}, F{});
+    if (k + 2 < nk) trip(k + 1, std::integral_constant<int, 1>{}, F{});
+    if (k + 3 < nk) trip(k + 2, std::integral_constant<int, 2>{}, F{});
+    if (k + 4 < nk) trip(k + 3, std::integral_constant<int, 3>{}, F{});
+    if (k + 5 < nk) trip(k + 4, std::integral_constant<int, 4>{}, F{});
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  mfmas(S1{});
+
+  // ---- epilogue ----------------------------------------------------------------------------
+  // The lane id is recomputed here (opaque to the optimiser) so that no lane-derived
+  // value has to stay in a VGPR across the K loop.
+  int lane_e;
+  asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lane_e));
+  const int li_e = lane_e & 15, lq_e = lane_e >> 4;
+  float scale = 1.0f;
+  if (p.scale_a) scale *= *p.scale_a;
+  if (p.scale_b) scale *= *p.scale_b;
+  const bool vec_ok = (p.ldc & 3) == 0;
+#pragma unroll
+  for (int m = 0; m < TM; ++m) {
+    const int row = row0 + (wm * TM + m) * 16 + li_e;
+#pragma unroll
+    for (int n = 0; n < TN; ++n) {
+      const int col = col0 + (wn * TN + n) * 16 + 4 * lq_e;
+      if (row < p.M && col < p.N) {
+        f32x4 v = acc[m][n] * scale;
+        const int ncols = (p.N - col) < 4 ? (p.N - col) : 4;
+        if (p.bias) {
+          for (int r = 0; r < ncols; ++r) v[r] += p.bias[col + r];
+        }
+#ifdef AG_DBG_NO_STORE
+        if (v[0] == 12345.678f)
+#endif
+        store4<OUT>(p.C, (int64_t)row * p.ldc + col, v, vec_ok, ncols);
+      }
+    }
+  }
+}
+
+template <int DT, int OUT, int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(WM* WN * 64) void gemm_stream_kernel(const GemmArgs p) {
+  gemm_stream_body<DT, OUT, BM, BN, WM, WN>(p);
+}
+
+}  // namespace
+}  // namespace astergemm
