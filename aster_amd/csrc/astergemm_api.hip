@@ -2,6 +2,7 @@
 // thin HIP runtime seam.  Everything exported is declared in include/astergemm.h.
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <vector>
@@ -119,8 +120,9 @@ const Variant* choose(const astergemm_config& c, int* index_out) {
       };
       const bool big_ok = wgs(v) >= 256, best_big_ok = wgs(best) >= 256;
       const int area = v->tile_m * v->tile_n, best_area = best->tile_m * best->tile_n;
-      better = (big_ok && !best_big_ok) || (big_ok == best_big_ok &&
-                                            (big_ok ? area > best_area : area < best_area));
+      if (big_ok != best_big_ok) better = big_ok;
+      else if (area != best_area) better = big_ok ? area > best_area : area < best_area;
+      else better = v->rank > best->rank;
     }
     if (better) {
       best = v;
@@ -233,6 +235,7 @@ int build_args(const Variant& v, const astergemm_config& c, const astergemm_oper
   a->tiles_m = (int32_t)((c.M + v.tile_m - 1) / v.tile_m);
   a->tiles_n = (int32_t)((c.N + v.tile_n - 1) / v.tile_n);
   a->group_m = 8;
+  if (const char* e = getenv("ASTERGEMM_GROUP_M")) a->group_m = atoi(e) > 0 ? atoi(e) : 8;
   a->split_k = 1;
   return 0;
 }

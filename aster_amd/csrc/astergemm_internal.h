@@ -51,6 +51,7 @@ struct Variant {
   int tile_m, tile_n, tile_k_bytes;
   int waves_m, waves_n;
   int stages;
+  int rank;          // preference among variants of equal tile size (higher wins)
   int lds_bytes;
   const void* func;  // device function symbol, for hipFuncGetAttributes
   // Launches the kernel; returns a hipError_t as int.

@@ -172,7 +172,7 @@ const char* check_skinny(const astergemm_config& c) {
 // tile_m = 16*MT (rows of A covered), tile_n = 16*NB, waves_n = KW (K split).
 #define AG_SKINNY(name, DT, OUT, MT, NB, KW, U)                                           \
   Variant {                                                                               \
-    name, ASTERGEMM_KERNEL_SKINNY, DT, OUT, 16 * MT, 16 * NB, 64 * U, 1, KW, 1,           \
+    name, ASTERGEMM_KERNEL_SKINNY, DT, OUT, 16 * MT, 16 * NB, 64 * U, 1, KW, 1, 0,        \
         KW * MT * NB * 1024, (const void*)gemm_skinny_kernel<DT, OUT, MT, NB, KW, U>,      \
         launch_skinny<DT, OUT, MT, NB, KW, U>, check_skinny                               \
   }

@@ -34,7 +34,7 @@ const char* check_tile(const astergemm_config& c) {
 
 #define AG_TILE(name, DT, OUT, BM, BN, WM, WN)                                   \
   Variant {                                                                      \
-    name, ASTERGEMM_KERNEL_TILE, DT, OUT, BM, BN, kRowBytes, WM, WN, 2,          \
+    name, ASTERGEMM_KERNEL_TILE, DT, OUT, BM, BN, kRowBytes, WM, WN, 2, 1,       \
         2 * (BM + BN) * kRowBytes,                                               \
         (const void*)gemm_tile_kernel<DT, OUT, BM, BN, WM, WN>,                  \
         launch_tile<DT, OUT, BM, BN, WM, WN>, check_tile                         \
@@ -70,7 +70,7 @@ int launch_pipe(const GemmArgs& a0, int grid, hipStream_t s) {
 
 #define AG_PIPE(name, DT, OUT, BM, BN, WM, WN)                                   \
   Variant {                                                                      \
-    name, ASTERGEMM_KERNEL_TILE, DT, OUT, BM, BN, kSubBytes, WM, WN, kStages,    \
+    name, ASTERGEMM_KERNEL_TILE, DT, OUT, BM, BN, kSubBytes, WM, WN, kStages, 0, \
         kStages * (BM + BN) * kSubBytes,                                         \
         (const void*)gemm_pipe_kernel<DT, OUT, BM, BN, WM, WN>,                  \
         launch_pipe<DT, OUT, BM, BN, WM, WN>, check_tile                         \
@@ -102,13 +102,14 @@ int launch_stream(const GemmArgs& a, int grid, hipStream_t s) {
 const char* check_stream(const astergemm_config& c) {
   if (c.M % 256 != 0 || c.N % 256 != 0) return "M and N must be multiples of 256";
   if (row_bytes(c.dtype_ab, c.K) % kRowBytes != 0) return "K must fill whole 128-byte row chunks";
+  if (c.ldc % 8 != 0) return "ldc must be a multiple of 8 elements";
   return nullptr;
 }
 
 #define AG_STREAM(name, DT, OUT, BM, BN, WM, WN)                                 \
   Variant {                                                                      \
     name, ASTERGEMM_KERNEL_TILE, DT, OUT, BM, BN, kRowBytes, WM, WN, 3,          \
-        5 * BM * kRowBytes,                                                      \
+        (WM * WN == 8) ? 2 : 0, 5 * BM * kRowBytes,                                                      \
         (const void*)gemm_stream_kernel<DT, OUT, BM, BN, WM, WN>,                \
         launch_stream<DT, OUT, BM, BN, WM, WN>, check_stream                     \
   }

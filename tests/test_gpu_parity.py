@@ -340,3 +340,64 @@ def test_identity_operand_is_exact_at_full_width(gpu):
     eye[np.arange(N), np.arange(N)] = 0x3F80
     out, _ = run_gemm(a, eye, M, N, N, "bf16", "bf16", family=_capi.KERNEL_TILE)
     assert np.array_equal(out, a)
+
+
+# ---- every pre-built tile variant, selected by its id ---------------------------------------
+
+def _tile_variants():
+    import ctypes
+    lib = _capi.load()
+    c = _capi.Config()
+    c.M = c.N = 512
+    c.K = 1024
+    out = []
+    for i in range(lib.astergemm_variant_count()):
+        info = _capi.KernelInfo()
+        _capi.check(lib.astergemm_variant_info(i, ctypes.byref(c), ctypes.byref(info)))
+        name = info.name.decode()
+        if info.family != _capi.KERNEL_TILE:
+            continue
+        kind, ab = name.split("_")[0], name.split("_")[1]
+        out.append((i + 1, name, {"fp8": "fp8_e4m3"}.get(ab, ab), name.rsplit("_", 1)[1]))
+    return out
+
+
+@pytest.mark.parametrize("vid,name,dtype_ab,dtype_c", _tile_variants(), ids=lambda v: str(v))
+def test_every_tile_variant(gpu, vid, name, dtype_ab, dtype_c):
+    M, N, K = 512, 768, 1280  # whole 256-tiles, ten 128-byte K-steps (two trips of the ring of five)
+    a, b, ex = operands(M, N, K, dtype_ab, seed=11, a_std=1.0, b_std=1.0 if dtype_ab != "bf16" else 0.05)
+    bias = np.random.default_rng(12).standard_normal(N).astype(np.float32)
+    plan = AG.GemmPlan.create(M, N, K, dtype_ab, dtype_c, has_bias=True, variant=vid)
+    assert plan.info.name.decode() == name
+    out = np.zeros((M, N), dtype=_OUT_NP[dtype_c])
+    bufs = {}
+    for key, arr in dict(a=a, b=b, c=out, bias=bias, **{k: np.asarray(v) for k, v in ex.items()}).items():
+        arr = np.ascontiguousarray(arr if arr.ndim else arr.reshape(1).astype(np.float32))
+        bufs[key] = GpuBuffer(arr.nbytes)
+        bufs[key].copy_from_host(arr)
+    kw = {k: bufs[k].ptr_value for k in ("scale_a", "scale_b", "mx_a", "mx_b") if k in bufs}
+    print(f"launch {name}", flush=True)
+    plan.run(bufs["a"].ptr_value, bufs["b"].ptr_value, bufs["c"].ptr_value, bias=bufs["bias"].ptr_value, **kw)
+    bufs["c"].copy_to_host(out)
+    for bf in bufs.values():
+        bf.free()
+    want = G.gemm(a, b, _DT[dtype_ab], _DT[dtype_c], bias=bias, **ex)
+    check(out, want, dtype_c, N, bar=1e-3 if dtype_c != "f32" else 1e-4)
+
+
+def test_stream_kernel_is_the_default_for_whole_tiles(gpu):
+    p = AG.GemmPlan.create(8192, 8192, 8192, "bf16", "bf16")
+    assert p.info.name.decode().startswith("stream_bf16_256x256")
+    assert p.info.lds_bytes == 163840
+    # shapes it does not take fall back to the general tile kernel
+    assert AG.GemmPlan.create(8192, 8192, 8200, "bf16", "bf16").info.name.decode().startswith("tile_")
+    assert AG.GemmPlan.create(8192, 8100, 8192, "bf16", "bf16").info.name.decode().startswith("tile_")
+
+
+@pytest.mark.parametrize("K", [64, 128, 192, 256, 320, 384, 448, 512, 576, 640, 704])
+def test_stream_kernel_every_ring_phase(gpu, K):
+    # K-steps 1..11: prologue only, partial rings, steady trips + every tail length
+    a, b, _ = operands(256, 512, K, "bf16", seed=13, b_std=0.1)
+    out, name = run_gemm(a, b, 256, 512, K, "bf16", "f32", family=_capi.KERNEL_TILE, wg_tile=(256, 256))
+    assert name.startswith("stream")
+    check(out, G.gemm(a, b, G.BF16, G.F32), "f32", 512, bar=1e-5)

@@ -108,9 +108,9 @@ def test_compile_gemm_writes_descriptor(tmp_path):
     cfg = make_instance(512, 512, 256)
     path, asm = gemm.compile_gemm(cfg, str(tmp_path / "k.hsaco"), num_vgprs=256, num_agprs=256)
     desc = json.load(open(path))
-    assert desc["kernel"] == "tile_bf16_256x256_w2x4_bf16" and desc["grid"] == 4
-    assert desc["label"] == cfg.label and desc["lds_bytes"] == 131072
-    assert ".group_segment_fixed_size: 131072" in asm
+    assert desc["kernel"] == "stream_bf16_256x256_w2x4_bf16" and desc["grid"] == 4
+    assert desc["label"] == cfg.label and desc["lds_bytes"] == 163840
+    assert ".group_segment_fixed_size: 163840" in asm
     (tmp_path / "bad.hsaco").write_text("{}")
     with pytest.raises(ValueError):
         gemm._read_descriptor(str(tmp_path / "bad.hsaco"))
