@@ -93,12 +93,12 @@ const Variant* choose(const astergemm_config& c, int* index_out) {
 
   const Variant* best = nullptr;
   int best_index = -1;
-  const char* last_why = "no variant with these dtypes";
+  const char* last_why = nullptr;  // reason given by the first variant that refused
   for (int i = 0; i < total_variants(); ++i) {
     const Variant* v = variant_at(i);
     if (v->family != family || !variant_matches_types(*v, c)) continue;
     if (const char* why = v->check(c)) {
-      last_why = why;
+      if (!last_why) last_why = why;
       continue;
     }
     if (c.wg_tile_m && c.wg_tile_m != v->tile_m) continue;
@@ -112,7 +112,8 @@ const Variant* choose(const astergemm_config& c, int* index_out) {
       // smallest activation tile that still covers M
       const bool fits = v->tile_m >= c.M, best_fits = best->tile_m >= c.M;
       better = (fits && !best_fits) || (fits == best_fits && fits && v->tile_m < best->tile_m) ||
-               (!fits && !best_fits && v->tile_m > best->tile_m);
+               (!fits && !best_fits && v->tile_m > best->tile_m) ||
+               (v->tile_m == best->tile_m && v->rank > best->rank);
     } else {
       // largest tile that still yields at least one workgroup per CU (256)
       auto wgs = [&](const Variant* x) {
@@ -130,7 +131,8 @@ const Variant* choose(const astergemm_config& c, int* index_out) {
     }
   }
   if (!best) {
-    set_error("astergemm: no kernel variant for this config (%s)", last_why);
+    set_error("astergemm: no kernel variant for this config (%s)",
+              last_why ? last_why : "no variant with these dtypes");
     return nullptr;
   }
   if (family == ASTERGEMM_KERNEL_SKINNY && best->tile_m < c.M) {
@@ -141,8 +143,27 @@ const Variant* choose(const astergemm_config& c, int* index_out) {
   return best;
 }
 
+// Compute units of the current device (0 when there is none), cached.
+int device_cus() {
+  static int cus = -1;
+  if (cus < 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+      cus = prop.multiProcessorCount;
+    else
+      (void)hipGetLastError(), cus = 0;
+  }
+  return cus;
+}
+
 int grid_of(const Variant& v, const astergemm_config& c) {
-  if (v.family == ASTERGEMM_KERNEL_SKINNY) return (int)((c.N + v.tile_n - 1) / v.tile_n);
+  if (v.family == ASTERGEMM_KERNEL_SKINNY) {
+    const int blocks = (int)((c.N + v.tile_n - 1) / v.tile_n);
+    // the resident-activation kernels (8 waves) are persistent: one workgroup per CU
+    if (v.waves_n == 8 && device_cus() > 0 && blocks > device_cus()) return device_cus();
+    return blocks;
+  }
   return (int)(((c.M + v.tile_m - 1) / v.tile_m) * ((c.N + v.tile_n - 1) / v.tile_n));
 }
 

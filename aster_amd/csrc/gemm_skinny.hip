@@ -11,6 +11,9 @@
 // activations take the same K positions as srcB, so the K permutation cancels.
 // It is HBM-bound: no LDS for weights, many 16-byte loads in flight per wave,
 // K split over the waves of a workgroup and reduced through LDS.
+#include <type_traits>
+#include <utility>
+
 #include "astergemm_internal.h"
 
 namespace astergemm {
@@ -27,6 +30,14 @@ __device__ __forceinline__ unsigned short sk_f32_to_bf16(float f) {
   if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)((u >> 16) | 0x40);
   u += 0x7fffu + ((u >> 16) & 1u);
   return (unsigned short)(u >> 16);
+}
+
+template <int I, int N, class Fn>
+__device__ __forceinline__ void static_for(Fn&& f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<I + 1, N>(f);
+  }
 }
 
 template <int DT>
@@ -156,6 +167,259 @@ __global__ __launch_bounds__(KW * 64) void gemm_skinny_kernel(const GemmArgs p) 
   }
 }
 
+// ---- M <= 16: activations resident in registers, one persistent workgroup per CU ----
+//
+// The kernel above re-reads the activation rows from L2 for every 16 weight rows and
+// fetches weights as 16 rows x 64 bytes per instruction (half cache lines), which
+// holds M = 16 near 2.9 TB/s.  Here the eight waves of a workgroup split K into
+// eight contiguous slices; a wave loads its slice of x once, straight into MFMA
+// operand registers, and then streams a contiguous range of weight rows (N is split
+// evenly over the grid in multiples of 8 rows, so no workgroup carries a whole extra
+// 16-row block).  Weights are fetched with non-temporal loads of 8 rows x 128 bytes
+// per instruction (whole cache lines), written to a wave-private LDS buffer and read
+// back in MFMA operand order; same-wave LDS operations execute in order, so the
+// transposition needs no barrier.  The partial 16x16 tiles of the eight waves are
+// summed through LDS once per four 16-row blocks.  All weight loads are unconditional
+// so that the wait counts stay exact: rows past the end of the range are clamped to
+// the last valid one (the same lines, in the same instruction), and the two units
+// prefetched past the last block read the first line of x instead, because weight
+// lines are fetched non-temporally and would come from HBM a second time.
+//
+// SPB = 128-byte steps per wave and block = K / 512; a unit of work is four steps
+// (eight loads, eight MFMAs) and two units are kept in flight per wave.
+template <int DT, int OUT, int SPB>
+__global__ __launch_bounds__(512) void gemm_skinny_reg_kernel(const GemmArgs p) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t slds[];
+  constexpr int KW = 8;
+  constexpr int UPB = SPB / 4;                   // units per block
+  constexpr int slice = SPB * 128;               // bytes of every row owned by one wave
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int li = lane & 15, lq = lane >> 4;
+  uint8_t* tbuf = slds + wave * 8192;            // 4 steps x 2 KiB, private to the wave
+  constexpr int NBS = 4;                         // blocks between workgroup barriers
+  f32x4* red = (f32x4*)(slds + KW * 8192);       // [2][NBS][KW][64]
+
+  // rows [r0, r1) of the weight matrix belong to this workgroup
+  const int g = gridDim.x;
+  const int per = (((p.N + g - 1) / g) + 7) & ~7;
+  const int r0 = blockIdx.x * per;
+  const int r1 = (r0 + per) < p.N ? (r0 + per) : p.N;
+  if (r0 >= p.N) return;
+  const int nblk = (r1 - r0 + 15) >> 4;
+  const int total = nblk * UPB;
+
+  // load: lane -> row (lane >> 3) of an 8-row half block, 16-byte piece (lane & 7)
+  const int lrow = lane >> 3, lpiece = lane & 7;
+  const uint8_t* wbase = p.B + wave * slice + lpiece * 16;
+  auto issue = [&](int j, i32x4(&dst)[8]) {      // flat index j = block * UPB + t
+    int blk = j / UPB;
+    const int t = j % UPB;
+    blk = blk < nblk ? blk : nblk - 1;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int nh = r0 + blk * 16 + h * 8;
+      int n = nh + lrow;
+      n = n < r1 ? n : r1 - 1;
+      const uint8_t* src = wbase + (int64_t)n * p.ldb_bytes + t * 512;
+      if (j >= total || nh >= r1) src = p.A + lpiece * 16;  // nothing to fetch: a line that stays in L2
+#pragma unroll
+      for (int s = 0; s < 4; ++s)
+        dst[s * 2 + h] = __builtin_nontemporal_load((const i32x4*)(src + s * 128));
+    }
+  };
+
+  // LDS transposition: 128-byte rows, 16-byte piece index XOR (row & 7)
+  const int wr_off = lrow * 128 + ((lpiece ^ lrow) << 4);          // + h * 1024 + s * 2048
+  const int rd_off = li * 128;                                     // + ((4u + lq) ^ (li & 7)) * 16
+  // stash: registers of one unit -> the wave's LDS buffer (frees the registers)
+  auto stash = [&](const i32x4(&src)[8]) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      *(i32x4*)(tbuf + (i >> 1) * 2048 + (i & 1) * 1024 + wr_off) = src[i];
+  };
+  auto operand = [&](int s, int u) {             // MFMA operand (row li, K piece 4u + lq) of step s
+    return *(const i32x4*)(tbuf + s * 2048 + rd_off + (((4 * u + lq) ^ (li & 7)) << 4));
+  };
+
+  // x: operand registers for the SPB*2 MFMAs of a block, fetched like the weights
+  // (whole lines, then through the LDS buffer) but cacheable: every workgroup reads
+  // them.  The loads of the first two units go out ahead of the first weight loads
+  // and are consumed while those are in flight.
+  i32x4 x[SPB * 2];
+  auto x_load = [&](int t, i32x4(&dst)[8]) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      int m = h * 8 + lrow;
+      m = m < p.M ? m : p.M - 1;
+      const uint8_t* src = p.A + (int64_t)m * p.lda_bytes + wave * slice + t * 512 + lpiece * 16;
+#pragma unroll
+      for (int s = 0; s < 4; ++s) dst[s * 2 + h] = *(const i32x4*)(src + s * 128);
+    }
+  };
+  auto x_keep = [&](auto T, const i32x4(&src)[8]) {
+    constexpr int t = decltype(T)::value;
+    stash(src);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x[t * 8 + i] = operand(i >> 1, i & 1);
+  };
+  i32x4 w0[8], w1[8];
+  {
+    i32x4 xa[8], xb[8];
+    x_load(0, xa);
+    if constexpr (UPB > 1) x_load(1, xb);
+    __builtin_amdgcn_sched_barrier(0);
+    issue(0, w0);
+    issue(1, w1);
+    __builtin_amdgcn_sched_barrier(0);
+    x_keep(std::integral_constant<int, 0>{}, xa);
+    if constexpr (UPB > 1) x_keep(std::integral_constant<int, 1>{}, xb);
+    static_for<2, UPB>([&](auto T) {
+      x_load(decltype(T)::value, xa);
+      x_keep(T, xa);
+    });
+  }
+  __builtin_amdgcn_sched_barrier(0);
+
+  float scale = 1.0f;
+  if (p.scale_a) scale *= *p.scale_a;
+  if (p.scale_b) scale *= *p.scale_b;
+
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  int parity = 0;
+
+  // Partial tiles go to red[parity][block % NBS][wave]; the workgroup meets only once
+  // per NBS blocks, then wave b sums and stores block b of the group.
+  auto block_end = [&](int blk) {
+    const int slot = blk & (NBS - 1);
+    red[((parity * NBS + slot) * KW + wave) * 64 + lane] = acc;
+    acc = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (slot != NBS - 1 && blk != nblk - 1) return;
+    __syncthreads();
+    if (wave <= slot) {
+      const f32x4* src = red + ((parity * NBS + wave) * KW) * 64 + lane;
+      f32x4 v = src[0];
+#pragma unroll
+      for (int k = 1; k < KW; ++k) v += src[k * 64];
+      const int m = li, n = r0 + (blk - slot + wave) * 16 + 4 * lq;
+      if (m < p.M && n < r1) {
+        v *= scale;
+        const int ncols = (r1 - n) < 4 ? (r1 - n) : 4;
+        if (p.bias)
+          for (int r = 0; r < ncols; ++r) v[r] += p.bias[n + r];
+        const int64_t idx = (int64_t)m * p.ldc + n;
+        const bool vec_ok = (p.ldc & 3) == 0 && ncols == 4;
+        if constexpr (OUT == ASTERGEMM_F32) {
+          float* o = (float*)p.C + idx;
+          if (vec_ok) *(f32x4*)o = v;
+          else
+            for (int r = 0; r < ncols; ++r) o[r] = v[r];
+        } else {
+          unsigned short h[4];
+          for (int r = 0; r < 4; ++r) {
+            if constexpr (OUT == ASTERGEMM_BF16) h[r] = sk_f32_to_bf16(v[r]);
+            else {
+              _Float16 hh = (_Float16)v[r];
+              h[r] = __builtin_bit_cast(unsigned short, hh);
+            }
+          }
+          unsigned short* o = (unsigned short*)p.C + idx;
+          if (vec_ok) *(u16x4*)o = u16x4{h[0], h[1], h[2], h[3]};
+          else
+            for (int r = 0; r < ncols; ++r) o[r] = h[r];
+        }
+      }
+    }
+    parity ^= 1;
+  };
+
+  // T = unit index inside the block (compile time: selects the x registers)
+  auto mma = [&](int blk, auto T) {
+    constexpr int t = decltype(T)::value;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      acc = sk_mfma<DT>(operand(i >> 1, i & 1), x[t * 8 + i], acc);
+    }
+    if (t == UPB - 1) block_end(blk);
+  };
+
+  // TRIP flat steps per trip so that register sets and x indices are static
+  constexpr int TRIP = UPB < 2 ? 2 : UPB;
+  int j = 0;
+  for (; j + TRIP <= total; j += TRIP) {
+    const int blk = j / UPB;
+    static_for<0, TRIP / 2>([&](auto I) {
+      constexpr int i = decltype(I)::value * 2;
+      // each register set is refilled as soon as its unit has been written to LDS;
+      // the scheduler must not move the loads across the units they overlap with
+      stash(w0);
+      __builtin_amdgcn_sched_barrier(0);
+      issue(j + i + 2, w0);
+      __builtin_amdgcn_sched_barrier(0);
+      mma(blk + i / UPB, std::integral_constant<int, i % UPB>{});
+      __builtin_amdgcn_sched_barrier(0);
+      stash(w1);
+      __builtin_amdgcn_sched_barrier(0);
+      issue(j + i + 3, w1);
+      __builtin_amdgcn_sched_barrier(0);
+      mma(blk + (i + 1) / UPB, std::integral_constant<int, (i + 1) % UPB>{});
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  }
+  if (j < total) {  // UPB == 1, odd block count
+    stash(w0);
+    mma(j / UPB, std::integral_constant<int, 0>{});
+  }
+}
+
+template <int DT, int OUT, int SPB>
+int launch_skinny_reg_t(const GemmArgs& a, hipStream_t s) {
+  auto k = gemm_skinny_reg_kernel<DT, OUT, SPB>;
+  constexpr int lds = 8 * 8192 + 2 * 4 * 8 * 64 * 16;
+  static bool attr_set = false;
+  static int cus = 0;
+  if (!attr_set) {
+    hipError_t e =
+        hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess) return (int)e;
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess)
+      return (int)hipGetLastError();
+    cus = prop.multiProcessorCount;
+    attr_set = true;
+  }
+  const int nblocks = (int)((a.N + 15) / 16);
+  const int g = nblocks < cus ? nblocks : cus;
+  hipLaunchKernelGGL(k, dim3(g), dim3(512), lds, s, a);
+  return (int)hipGetLastError();
+}
+
+template <int DT, int OUT>
+int launch_skinny_reg(const GemmArgs& a, int grid, hipStream_t s) {
+  (void)grid;
+  switch (a.K) {
+    case 2048: return launch_skinny_reg_t<DT, OUT, 4>(a, s);
+    case 4096: return launch_skinny_reg_t<DT, OUT, 8>(a, s);
+    case 8192: return launch_skinny_reg_t<DT, OUT, 16>(a, s);
+  }
+  return (int)hipErrorInvalidValue;
+}
+
+const char* check_skinny_reg(const astergemm_config& c) {
+  if (c.M > 16) return "resident-activation path needs M <= 16";
+  if (c.K != 2048 && c.K != 4096 && c.K != 8192)
+    return "resident-activation path needs K = 2048, 4096 or 8192";
+  return nullptr;
+}
+
+#define AG_SKINNY_LDS(name, DT, OUT)                                                       \
+  Variant {                                                                                \
+    name, ASTERGEMM_KERNEL_SKINNY, DT, OUT, 16, 16, 512, 1, 8, 1, 1, 8 * 8192 + 65536,      \
+        (const void*)gemm_skinny_reg_kernel<DT, OUT, 8>, launch_skinny_reg<DT, OUT>,       \
+        check_skinny_reg                                                                   \
+  }
+
 template <int DT, int OUT, int MT, int NB, int KW, int U>
 int launch_skinny(const GemmArgs& a, int grid, hipStream_t s) {
   hipLaunchKernelGGL((gemm_skinny_kernel<DT, OUT, MT, NB, KW, U>), dim3(grid), dim3(KW * 64), 0,
@@ -189,6 +453,12 @@ const Variant kSkinnyVariants[] = {
     AG_SKINNY_SET("skinny_f16", ASTERGEMM_F16, "bf16", ASTERGEMM_BF16),
     AG_SKINNY_SET("skinny_f16", ASTERGEMM_F16, "f32", ASTERGEMM_F32),
     AG_SKINNY_SET("skinny_f16", ASTERGEMM_F16, "f16", ASTERGEMM_F16),
+    AG_SKINNY_LDS("skinnyx_bf16_m16_bf16", ASTERGEMM_BF16, ASTERGEMM_BF16),
+    AG_SKINNY_LDS("skinnyx_bf16_m16_f32", ASTERGEMM_BF16, ASTERGEMM_F32),
+    AG_SKINNY_LDS("skinnyx_bf16_m16_f16", ASTERGEMM_BF16, ASTERGEMM_F16),
+    AG_SKINNY_LDS("skinnyx_f16_m16_bf16", ASTERGEMM_F16, ASTERGEMM_BF16),
+    AG_SKINNY_LDS("skinnyx_f16_m16_f32", ASTERGEMM_F16, ASTERGEMM_F32),
+    AG_SKINNY_LDS("skinnyx_f16_m16_f16", ASTERGEMM_F16, ASTERGEMM_F16),
 };
 
 }  // namespace

@@ -218,6 +218,25 @@ def test_skinny_ragged(gpu, M, N, K, dtype_ab):
     check(out, G.gemm(a, b, _DT[dtype_ab], G.F32, bias=bias), "f32", N, bar=1e-5)
 
 
+@pytest.mark.parametrize("M,N,K", [(16, 14337, 4096), (1, 8, 2048), (5, 777, 8192), (13, 6000, 2048),
+                                   (16, 24, 4096), (9, 4104, 8192), (16, 40, 2048)])
+@pytest.mark.parametrize("dtype_ab,dtype_c", [("bf16", "f32"), ("f16", "f16"), ("bf16", "bf16")])
+def test_skinny_resident_activations(gpu, M, N, K, dtype_ab, dtype_c):
+    """M <= 16 and K in {2048, 4096, 8192} take the persistent kernel that keeps x in
+    registers; row ranges that end inside a 16-row block, single-workgroup grids,
+    bias and a padded output pitch."""
+    a, b, _ = operands(M, N, K, dtype_ab, seed=11, b_std=0.05)
+    bias = np.random.default_rng(12).standard_normal(N).astype(np.float32)
+    ldc = (N + 11) & ~3
+    out, name = run_gemm(a, b, M, N, K, dtype_ab, dtype_c, bias=bias, ldc=ldc)
+    assert name.startswith("skinnyx")
+    want = G.gemm(a, b, _DT[dtype_ab], _DT[dtype_c], bias=bias)
+    check(out, want, dtype_c, N, bar=1e-5 if dtype_c == "f32" else REL_L2_BAR)
+    # the pad columns of every output row stay untouched
+    pad = out[:, N:]
+    assert np.isnan(pad).all() if dtype_c == "f32" else (pad == 0x7FC1).all()
+
+
 # ---- edge cases: ragged M / N, K tails, leading dimensions, epilogue -----------------
 
 @pytest.mark.parametrize("M,N,K", [(1, 1, 8), (65, 16, 8), (130, 257, 72), (300, 520, 776), (129, 1, 64)])
