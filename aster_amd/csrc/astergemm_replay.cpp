@@ -9,7 +9,11 @@
 //
 //   astergemm_replay --m 8192 --n 8192 --k 8192 --ab bf16 --c bf16 --iters 100
 //                    [--warmup 20] [--tile 256] [--family tile|skinny|auto]
-//                    [--variant ID] [--flush BYTES] [--bias] [--json]
+//                    [--variant ID] [--flush BYTES] [--bias] [--json] [--calib BYTES]
+//
+// --calib BYTES first copies BYTES device-to-device three times: a copy kernel that
+// reads and writes a known number of bytes, against which the counters of a
+// hardware-counter run (FETCH_SIZE, WRITE_SIZE) can be scaled.
 #include <math.h>
 #include <stdint.h>
 #include <stdio.h>
@@ -82,7 +86,7 @@ int main(int argc, char** argv) {
   cfg.dtype_ab = ASTERGEMM_BF16;
   cfg.dtype_c = ASTERGEMM_BF16;
   int iters = 100, warmup = 20, json = 0;
-  long long flush = 0;
+  long long flush = 0, calib = 0;
   for (int i = 1; i < argc; ++i) {
     std::string a = argv[i];
     auto val = [&]() -> const char* {
@@ -102,6 +106,7 @@ int main(int argc, char** argv) {
     else if (a == "--tile") cfg.wg_tile_m = cfg.wg_tile_n = atoi(val());
     else if (a == "--variant") cfg.variant = atoi(val());
     else if (a == "--flush") flush = atoll(val());
+    else if (a == "--calib") calib = atoll(val());
     else if (a == "--bias") cfg.has_bias = 1;
     else if (a == "--json") json = 1;
     else if (a == "--family") {
@@ -166,6 +171,16 @@ int main(int argc, char** argv) {
     CHECK(aster_rt_malloc(&dbias, hbias.size() * 4));
     CHECK(aster_rt_memcpy_h2d(dbias, hbias.data(), hbias.size() * 4));
     ops.dBias = (const float*)dbias;
+  }
+
+  if (calib > 0) {
+    void *src, *dst;
+    CHECK(aster_rt_malloc(&src, (size_t)calib));
+    CHECK(aster_rt_malloc(&dst, (size_t)calib));
+    CHECK(aster_rt_memset(src, 1, (size_t)calib));
+    for (int i = 0; i < 3; ++i) CHECK(aster_rt_memcpy_d2d(dst, src, (size_t)calib));
+    CHECK(aster_rt_free(src));
+    CHECK(aster_rt_free(dst));
   }
 
   std::vector<int64_t> t((size_t)iters);

@@ -29,6 +29,13 @@ sys.path.insert(0, ROOT)
 PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "fp8_e4m3": 5000.0, "mxfp4": 10100.0}
 PEAK_HBM_GBPS = 8000.0
 
+# Bytes moved past L2 per launch of the 8192^3 workload, by kernel, from two
+# `rocprofv3 --pmc` runs (FETCH_SIZE, WRITE_SIZE; KiB per dispatch, each scaled by what
+# the same counter reads for a 1 GiB device-to-device copy: x2.0 and x1.0); the figures
+# are in profiles/stream_bf16_8192x8192x8192_counters.txt.  A kernel that has not been
+# measured reports null.
+MEASURED_TRAFFIC_BYTES = {"stream_bf16_256x256_w2x4_bf16": 1.746e9}
+
 
 def _percentile(sorted_vals, pct):
     n = len(sorted_vals)
@@ -157,11 +164,7 @@ def main() -> int:
     value = flops * args.steps / wall / 1e12
     achieved = flops / (launch_ms * 1e-3) / 1e12
 
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
-    if os.path.exists(tpath):
-        with open(tpath) as f:
-            traffic = json.load(f).get(plan.info.name.decode() + "_8192x8192x8192")
+    traffic = MEASURED_TRAFFIC_BYTES.get(plan.info.name.decode())
 
     out = {
         "metric": "bf16 GEMM 8192^3 throughput (TFLOP/s; % of MI355X dense MFMA peak in roofline.frac)",
