@@ -43,6 +43,77 @@ __device__ __forceinline__ void static_for(Fn&& f) {
   }
 }
 
+// ---- epilogue shared by the stream kernels -------------------------------------------------
+// Scale, bias and cast in registers, then turn each 16-row slab of the wave tile
+// around in LDS so that every lane stores 16 contiguous bytes and every store
+// instruction covers whole 128-byte lines of C.  (A lane owns 4 consecutive
+// columns of one row per MFMA tile; stored directly that is 8 bytes per lane and
+// 32-byte pieces per row, which costs ~7 % of the kernel.)  The lane id is
+// recomputed here, opaque to the optimiser, so that no lane-derived value has to
+// stay in a VGPR across the K loop.
+template <int OUT, int BM, int BN, int WM, int WN>
+__device__ __forceinline__ void stream_epilogue(const GemmArgs& p,
+                                                f32x4 (&acc)[BM / WM / 16][BN / WN / 16],
+                                                uint8_t* lds, int wave, int row0, int col0) {
+  constexpr int NW = WM * WN;
+  constexpr int TM = BM / WM / 16;
+  constexpr int TN = BN / WN / 16;
+  constexpr int SLOT = BM * kRowBytes;
+  constexpr int NSLOT = 5;
+  const int wm = wave / WN, wn = wave % WN;
+  int lane_e;
+  asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lane_e));
+  const int li_e = lane_e & 15, lq_e = lane_e >> 4;
+  float scale = 1.0f;
+  if (p.scale_a) scale *= *p.scale_a;
+  if (p.scale_b) scale *= *p.scale_b;
+  constexpr int OB = (OUT == ASTERGEMM_F32) ? 4 : 2;  // bytes per output element
+  constexpr int WCOLS = TN * 16;                      // columns of the wave tile
+  constexpr int ROWB = WCOLS * OB;                    // bytes of one slab row
+  constexpr int PITCH = ROWB + 16;                    // padded LDS pitch
+  constexpr int SLAB = 16 * PITCH;
+  constexpr int CHUNKS = 16 * ROWB / 16;              // 16-byte chunks per slab
+  static_assert(CHUNKS % 64 == 0, "whole store instructions per slab");
+  static_assert(2 * SLAB * NW <= NSLOT * SLOT, "staging fits in the ring");
+  // every wave is done reading fragments before LDS is reused
+  __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+  uint8_t* stage = lds + wave * 2 * SLAB;
+  const int wrow0 = row0 + wm * TM * 16, wcol0 = col0 + wn * WCOLS;
+  float bias_v[TN][4];
+#pragma unroll
+  for (int n = 0; n < TN; ++n)
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      bias_v[n][e] = p.bias ? p.bias[wcol0 + n * 16 + 4 * lq_e + e] : 0.f;
+#pragma unroll
+  for (int m = 0; m < TM; ++m) {
+    uint8_t* slab = stage + (m & 1) * SLAB;
+#pragma unroll
+    for (int n = 0; n < TN; ++n) {
+      f32x4 v = acc[m][n] * scale;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] += bias_v[n][e];
+      uint8_t* dst = slab + li_e * PITCH + (n * 16 + 4 * lq_e) * OB;
+      if constexpr (OUT == ASTERGEMM_F32) {
+        *(f32x4*)dst = v;
+      } else {
+        const u16x4 h = cast4_16<OUT>(v);
+        *(u16x4*)dst = h;
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < CHUNKS / 64; ++t) {
+      const int c = t * 64 + lane_e;
+      const int r = c / (ROWB / 16), cc = c % (ROWB / 16);
+      const i32x4 d = *(const i32x4*)(slab + r * PITCH + cc * 16);
+      uint8_t* out = (uint8_t*)p.C + ((int64_t)(wrow0 + m * 16 + r) * p.ldc + wcol0) * OB + cc * 16;
+      *(i32x4*)out = d;
+    }
+  }
+}
+
 template <int DT, int OUT, int BM, int BN, int WM, int WN>
 __device__ __forceinline__ void gemm_stream_body(const GemmArgs& p) {
   constexpr int NW = WM * WN;
@@ -282,68 +353,7 @@ __device__ __forceinline__ void gemm_stream_body(const GemmArgs& p) {
   __builtin_amdgcn_sched_barrier(0);
   mfmas(S1{});
 
-  // ---- epilogue ----------------------------------------------------------------------------
-  // Scale, bias and cast in registers, then turn each 16-row slab of the wave tile
-  // around in LDS so that every lane stores 16 contiguous bytes and every store
-  // instruction covers whole 128-byte lines of C.  (A lane owns 4 consecutive
-  // columns of one row per MFMA tile; stored directly that is 8 bytes per lane and
-  // 32-byte pieces per row, which costs ~7 % of the kernel.)  The lane id is
-  // recomputed here, opaque to the optimiser, so that no lane-derived value has to
-  // stay in a VGPR across the K loop.
-  int lane_e;
-  asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lane_e));
-  const int li_e = lane_e & 15, lq_e = lane_e >> 4;
-  float scale = 1.0f;
-  if (p.scale_a) scale *= *p.scale_a;
-  if (p.scale_b) scale *= *p.scale_b;
-  constexpr int OB = (OUT == ASTERGEMM_F32) ? 4 : 2;  // bytes per output element
-  constexpr int WCOLS = TN * 16;                      // columns of the wave tile
-  constexpr int ROWB = WCOLS * OB;                    // bytes of one slab row
-  constexpr int PITCH = ROWB + 16;                    // padded LDS pitch
-  constexpr int SLAB = 16 * PITCH;
-  constexpr int CHUNKS = 16 * ROWB / 16;              // 16-byte chunks per slab
-  static_assert(CHUNKS % 64 == 0, "whole store instructions per slab");
-  static_assert(2 * SLAB * NW <= NSLOT * SLOT, "staging fits in the ring");
-  // every wave is done reading fragments before LDS is reused
-  __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
-  __builtin_amdgcn_s_barrier();
-  asm volatile("" ::: "memory");
-  uint8_t* stage = lds + wave * 2 * SLAB;
-  const int wrow0 = row0 + wm * TM * 16, wcol0 = col0 + wn * WCOLS;
-  float bias_v[TN][4];
-#pragma unroll
-  for (int n = 0; n < TN; ++n)
-#pragma unroll
-    for (int e = 0; e < 4; ++e)
-      bias_v[n][e] = p.bias ? p.bias[wcol0 + n * 16 + 4 * lq_e + e] : 0.f;
-#pragma unroll
-  for (int m = 0; m < TM; ++m) {
-    uint8_t* slab = stage + (m & 1) * SLAB;
-#pragma unroll
-    for (int n = 0; n < TN; ++n) {
-      f32x4 v = acc[m][n] * scale;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) v[e] += bias_v[n][e];
-      uint8_t* dst = slab + li_e * PITCH + (n * 16 + 4 * lq_e) * OB;
-      if constexpr (OUT == ASTERGEMM_F32) {
-        *(f32x4*)dst = v;
-      } else {
-        u16x4 h;
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-          h[e] = (OUT == ASTERGEMM_BF16) ? f32_to_bf16_rne(v[e]) : f32_to_f16_rne(v[e]);
-        *(u16x4*)dst = h;
-      }
-    }
-#pragma unroll
-    for (int t = 0; t < CHUNKS / 64; ++t) {
-      const int c = t * 64 + lane_e;
-      const int r = c / (ROWB / 16), cc = c % (ROWB / 16);
-      const i32x4 d = *(const i32x4*)(slab + r * PITCH + cc * 16);
-      uint8_t* out = (uint8_t*)p.C + ((int64_t)(wrow0 + m * 16 + r) * p.ldc + wcol0) * OB + cc * 16;
-      *(i32x4*)out = d;
-    }
-  }
+  stream_epilogue<OUT, BM, BN, WM, WN>(p, acc, lds, wave, row0, col0);
 }
 
 template <int DT, int OUT, int BM, int BN, int WM, int WN>

@@ -2,6 +2,7 @@
 // (device code: gemm_tile_kernel.hpp).
 #include "gemm_pipe_kernel.hpp"
 #include "gemm_stream_kernel.hpp"
+#include "gemm_stream8_kernel.hpp"
 
 namespace astergemm {
 namespace {
@@ -114,6 +115,29 @@ const char* check_stream(const astergemm_config& c) {
         launch_stream<DT, OUT, BM, BN, WM, WN>, check_stream                     \
   }
 
+template <int DT, int OUT, int BM, int BN, int WM, int WN>
+int launch_stream8(const GemmArgs& a, int grid, hipStream_t s) {
+  constexpr int lds = 5 * BM * kRowBytes;
+  auto k = gemm_stream8_kernel<DT, OUT, BM, BN, WM, WN>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)k,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess) return (int)e;
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(k, dim3(grid), dim3(WM * WN * 64), lds, s, a);
+  return (int)hipGetLastError();
+}
+
+#define AG_STREAM8(name, DT, OUT)                                                \
+  Variant {                                                                      \
+    name, ASTERGEMM_KERNEL_TILE, DT, OUT, 256, 256, kRowBytes, 2, 4, 3, 2,       \
+        5 * 256 * kRowBytes,                                                     \
+        (const void*)gemm_stream8_kernel<DT, OUT, 256, 256, 2, 4>,               \
+        launch_stream8<DT, OUT, 256, 256, 2, 4>, check_stream                    \
+  }
+
 #define AG_STREAM_SET(prefix, DT)                                                      \
   AG_STREAM(prefix "_256x256_w2x4_bf16", DT, ASTERGEMM_BF16, 256, 256, 2, 4),          \
       AG_STREAM(prefix "_256x256_w2x4_f32", DT, ASTERGEMM_F32, 256, 256, 2, 4),        \
@@ -130,6 +154,9 @@ const Variant kTileVariants[] = {
     AG_PIPE_SET("pipe_fp8", ASTERGEMM_FP8_E4M3),
     AG_STREAM_SET("stream_bf16", ASTERGEMM_BF16),
     AG_STREAM_SET("stream_f16", ASTERGEMM_F16),
+    AG_STREAM8("stream_fp8_256x256_w2x4_bf16", ASTERGEMM_FP8_E4M3, ASTERGEMM_BF16),
+    AG_STREAM8("stream_fp8_256x256_w2x4_f32", ASTERGEMM_FP8_E4M3, ASTERGEMM_F32),
+    AG_STREAM8("stream_fp8_256x256_w2x4_f16", ASTERGEMM_FP8_E4M3, ASTERGEMM_F16),
 };
 
 }  // namespace

@@ -52,16 +52,18 @@ __device__ __forceinline__ float bf16_bits_to_f32(unsigned short b) {
 }
 
 // fp32 -> bf16 round-to-nearest-even, NaN kept quiet.
-__device__ __forceinline__ unsigned short f32_to_bf16_rne(float f) {
-  unsigned u = __builtin_bit_cast(unsigned, f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)((u >> 16) | 0x40);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (unsigned short)(u >> 16);
-}
-
-__device__ __forceinline__ unsigned short f32_to_f16_rne(float f) {
-  _Float16 h = (_Float16)f;
-  return __builtin_bit_cast(unsigned short, h);
+// Four fp32 values to four 16-bit outputs, round to nearest even, with the hardware
+// converters (v_cvt_pk_bf16_f32 / v_cvt_f16_f32): the integer bf16 rounding sequence is six
+// VALU operations per element, which made the epilogue of a 256x256 tile VALU bound.
+template <int OUT>
+__device__ __forceinline__ u16x4 cast4_16(f32x4 v) {
+  if constexpr (OUT == ASTERGEMM_BF16) {
+    typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+    return __builtin_bit_cast(u16x4, __builtin_convertvector(v, bf16x4_t));
+  } else {
+    typedef _Float16 f16x4_t __attribute__((ext_vector_type(4)));
+    return __builtin_bit_cast(u16x4, __builtin_convertvector(v, f16x4_t));
+  }
 }
 
 // Hardware hands workgroup b to XCD b % 8.  Give each XCD one contiguous run of
@@ -128,9 +130,8 @@ __device__ __forceinline__ void store4(void* C, int64_t idx, f32x4 v, bool vec_o
       for (int r = 0; r < ncols; ++r) p[r] = v[r];
     }
   } else {
-    unsigned short h[4];
-    for (int r = 0; r < 4; ++r)
-      h[r] = (OUT == ASTERGEMM_BF16) ? f32_to_bf16_rne(v[r]) : f32_to_f16_rne(v[r]);
+    const u16x4 hv4 = cast4_16<OUT>(v);
+    const unsigned short h[4] = {hv4.x, hv4.y, hv4.z, hv4.w};
     unsigned short* p = (unsigned short*)C + idx;
     if (vec_ok && ncols == 4) {
       u16x4 hv = {h[0], h[1], h[2], h[3]};

@@ -420,3 +420,34 @@ def test_stream_kernel_every_ring_phase(gpu, K):
     out, name = run_gemm(a, b, 256, 512, K, "bf16", "f32", family=_capi.KERNEL_TILE, wg_tile=(256, 256))
     assert name.startswith("stream")
     check(out, G.gemm(a, b, G.BF16, G.F32), "f32", 512, bar=1e-5)
+
+
+@pytest.mark.parametrize("ksteps", list(range(1, 16)) + [20, 21])
+def test_fp8_stream_kernel_every_ring_phase(gpu, ksteps):
+    # 128-byte K-steps 1..15, 20, 21: prologue only, every tail length of the six-trip slot
+    # period, one and two steady periods followed by every kind of tail
+    M, N, K = 256, 512, 128 * ksteps
+    a, b, ex = operands(M, N, K, "fp8_e4m3", seed=17, b_std=1.0)
+    out, name = run_gemm(a, b, M, N, K, "fp8_e4m3", "f32", family=_capi.KERNEL_TILE,
+                         wg_tile=(256, 256), **ex)
+    assert name.startswith("stream_fp8")
+    check(out, G.gemm(a, b, G.FP8_E4M3, G.F32, **ex), "f32", N, bar=1e-4)
+
+
+def test_fp8_stream_and_tile_kernels_pair_granules_consistently(gpu):
+    # the stream kernel visits the 128 K positions of a step in a different order than the
+    # general tile kernel; both must agree with the oracle on data where a wrong pairing of
+    # granules between A and B cannot cancel (distinct magnitude per 16-byte granule)
+    M, N, K = 256, 256, 512
+    rng = np.random.default_rng(23)
+    gran = 2.0 ** rng.integers(-3, 4, size=(K // 16)).astype(np.float32)
+    xa = (rng.standard_normal((M, K)).astype(np.float32)) * np.repeat(gran, 16)[None, :]
+    xb = rng.standard_normal((N, K)).astype(np.float32)
+    a, sa = F.quantize_fp8_tensor(xa)
+    b, sb = F.quantize_fp8_tensor(xb)
+    want = G.gemm(a, b, G.FP8_E4M3, G.F32, scale_a=sa, scale_b=sb)
+    for tile, prefix in ((256, "stream_fp8"), (128, "tile_fp8")):
+        out, name = run_gemm(a, b, M, N, K, "fp8_e4m3", "f32", scale_a=sa, scale_b=sb,
+                             family=_capi.KERNEL_TILE, wg_tile=(tile, tile))
+        assert name.startswith(prefix)
+        check(out, want, "f32", N, bar=1e-4)
