@@ -446,6 +446,19 @@ const char* check_skinny(const astergemm_config& c) {
       AG_SKINNY(prefix "_m32_" OUTN, DT, OUT, 2, 1, 4, 8),                        \
       AG_SKINNY(prefix "_m64_" OUTN, DT, OUT, 4, 1, 4, 4)
 
+// Wider variants for M = 17..64: a workgroup covers 64 weight rows, so the activations
+// are re-read from L2 once per 64 rows instead of once per 16 (at M = 64 the activation
+// traffic of the narrow variant is four times the weight traffic).  rank 1: preferred.
+#define AG_SKINNY_WIDE(name, DT, OUT, MT, NB, KW, U)                                      \
+  Variant {                                                                               \
+    name, ASTERGEMM_KERNEL_SKINNY, DT, OUT, 16 * MT, 16 * NB, 64 * U, 1, KW, 1, 1,        \
+        KW * MT * NB * 1024, (const void*)gemm_skinny_kernel<DT, OUT, MT, NB, KW, U>,      \
+        launch_skinny<DT, OUT, MT, NB, KW, U>, check_skinny                               \
+  }
+#define AG_SKINNY_WIDE_SET(prefix, DT, OUTN, OUT)                                 \
+  AG_SKINNY_WIDE(prefix "_m32n64_" OUTN, DT, OUT, 2, 4, 4, 2),                    \
+      AG_SKINNY_WIDE(prefix "_m64n64_" OUTN, DT, OUT, 4, 4, 4, 1)
+
 const Variant kSkinnyVariants[] = {
     AG_SKINNY_SET("skinny_bf16", ASTERGEMM_BF16, "bf16", ASTERGEMM_BF16),
     AG_SKINNY_SET("skinny_bf16", ASTERGEMM_BF16, "f32", ASTERGEMM_F32),
@@ -453,6 +466,12 @@ const Variant kSkinnyVariants[] = {
     AG_SKINNY_SET("skinny_f16", ASTERGEMM_F16, "bf16", ASTERGEMM_BF16),
     AG_SKINNY_SET("skinny_f16", ASTERGEMM_F16, "f32", ASTERGEMM_F32),
     AG_SKINNY_SET("skinny_f16", ASTERGEMM_F16, "f16", ASTERGEMM_F16),
+    AG_SKINNY_WIDE_SET("skinny_bf16", ASTERGEMM_BF16, "bf16", ASTERGEMM_BF16),
+    AG_SKINNY_WIDE_SET("skinny_bf16", ASTERGEMM_BF16, "f32", ASTERGEMM_F32),
+    AG_SKINNY_WIDE_SET("skinny_bf16", ASTERGEMM_BF16, "f16", ASTERGEMM_F16),
+    AG_SKINNY_WIDE_SET("skinny_f16", ASTERGEMM_F16, "bf16", ASTERGEMM_BF16),
+    AG_SKINNY_WIDE_SET("skinny_f16", ASTERGEMM_F16, "f32", ASTERGEMM_F32),
+    AG_SKINNY_WIDE_SET("skinny_f16", ASTERGEMM_F16, "f16", ASTERGEMM_F16),
     AG_SKINNY_LDS("skinnyx_bf16_m16_bf16", ASTERGEMM_BF16, ASTERGEMM_BF16),
     AG_SKINNY_LDS("skinnyx_bf16_m16_f32", ASTERGEMM_BF16, ASTERGEMM_F32),
     AG_SKINNY_LDS("skinnyx_bf16_m16_f16", ASTERGEMM_BF16, ASTERGEMM_F16),

@@ -177,13 +177,9 @@ __device__ __forceinline__ void gemm_stream8_body(const GemmArgs& p) {
       // cbsz = blgp = 0: both operands OCP e4m3; zero scale operands select the unscaled form
       acc[m][n] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fbr[n & 1], fa[m], acc[m][n], 0,
                                                                    0, 0, 0, 0, 0);
-#ifndef AG8_NO_READ
       if constexpr (m == 0 && n + 1 < TN) read_b(b_cur, std::integral_constant<int, n + 1>{});
-#endif
       if constexpr (I >= 2 && I < 2 + LH) {
-#ifndef AG8_NO_LOAD
         if (do_ld) issue_a1(k + 2, a_ld, I - 2);
-#endif
       }
       if constexpr (I == BAR - 1) {
         __builtin_amdgcn_sched_barrier(0);
@@ -195,9 +191,7 @@ __device__ __forceinline__ void gemm_stream8_body(const GemmArgs& p) {
         }
       }
       if constexpr (I >= BAR && I < BAR + LH) {
-#ifndef AG8_NO_LOAD
         if (do_ld) issue_b1(k + 2, b_cur, I - BAR);
-#endif
       }
       if constexpr (I == (TN - 1) * TM) {
         const uint8_t* sa = lds + ((unsigned)(a_next * SLOT) + a_rd);
@@ -205,12 +199,10 @@ __device__ __forceinline__ void gemm_stream8_body(const GemmArgs& p) {
         ra1 = sa + rd1;
       }
       if constexpr (I >= (TN - 1) * TM) {
-#ifndef AG8_NO_READ
         if (do_rd) {
           if constexpr (m == 0) read_b(b_next, std::integral_constant<int, 0>{});
           read_a(std::integral_constant<int, m>{}, ra0, ra1);
         }
-#endif
       }
       __builtin_amdgcn_sched_barrier(0);
     });
@@ -236,11 +228,7 @@ __device__ __forceinline__ void gemm_stream8_body(const GemmArgs& p) {
   }
   __builtin_amdgcn_sched_barrier(0);
 
-#ifndef AG8_NO_STORE
   stream_epilogue<OUT, BM, BN, WM, WN>(p, acc, lds, wave, row0, col0);
-#else
-  if (p.M == 12345) stream_epilogue<OUT, BM, BN, WM, WN>(p, acc, lds, wave, row0, col0);
-#endif
 }
 
 template <int DT, int OUT, int BM, int BN, int WM, int WN>
