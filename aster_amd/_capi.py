@@ -90,6 +90,8 @@ SIGNATURES = {
     "astergemm_variant_count": (C.c_int, []),
     "astergemm_variant_info": (C.c_int, [C.c_int, C.POINTER(Config), C.POINTER(KernelInfo)]),
     "astergemm_run": (C.c_int, [C.POINTER(Config), C.POINTER(Operands), _P]),
+    "astergemm_bench_rotate": (C.c_int, [C.POINTER(Config), C.POINTER(Operands), C.c_int, C.c_int,
+                                         C.POINTER(C.c_int64), C.c_void_p]),
     "astergemm_bench": (C.c_int, [C.POINTER(Config), C.POINTER(Operands), C.c_int,
                                   C.POINTER(C.c_int64), C.c_int64, _P]),
     "astergemm_shuffle_weight_16": (C.c_int, [_P, _P, C.c_int64, C.c_int64]),

@@ -324,6 +324,38 @@ int astergemm_run(const astergemm_config* cfg, const astergemm_operands* ops, vo
   return 0;
 }
 
+int astergemm_bench_rotate(const astergemm_config* cfg, const astergemm_operands* ops, int n_ops,
+                           int iters, int64_t* total_ns, void* stream) {
+  if (!cfg || !ops || !total_ns || iters <= 0 || n_ops <= 0) {
+    set_error("astergemm_bench_rotate: bad argument");
+    return ASTERGEMM_EINVAL;
+  }
+  int index = -1;
+  const Variant* v = choose(*cfg, &index);
+  if (!v) return g_choose_rc;
+  *total_ns = 0;
+  if (cfg->M == 0 || cfg->N == 0) return 0;
+  std::vector<GemmArgs> args((size_t)n_ops);
+  for (int i = 0; i < n_ops; ++i)
+    if (int rc = build_args(*v, *cfg, ops[i], &args[(size_t)i])) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  const int grid = grid_of(*v, *cfg);
+  hipEvent_t e0, e1;
+  AG_HIP(hipEventCreate(&e0));
+  AG_HIP(hipEventCreate(&e1));
+  int le = (int)hipEventRecord(e0, s);
+  for (int i = 0; i < iters && le == 0; ++i) le = v->launch(args[(size_t)(i % n_ops)], grid, s);
+  if (le == 0) le = (int)hipEventRecord(e1, s);
+  if (le == 0) le = (int)hipEventSynchronize(e1);
+  float ms = 0.f;
+  if (le == 0) le = (int)hipEventElapsedTime(&ms, e0, e1);
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  if (le != 0) return hip_fail((hipError_t)le, v->name, __FILE__, __LINE__);
+  *total_ns = (int64_t)((double)ms * 1e6);
+  return 0;
+}
+
 int astergemm_bench(const astergemm_config* cfg, const astergemm_operands* ops, int iters,
                     int64_t* times_ns, int64_t flush_bytes, void* stream) {
   if (!cfg || !ops || !times_ns || iters <= 0) {

@@ -271,6 +271,20 @@ __device__ __forceinline__ void gemm_tile_body(const GemmArgs& p) {
 #pragma unroll
     for (int n = 0; n < TN; ++n) acc[m][n] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+  // MX scales of a K-step are fetched one step ahead and ahead of that step's tile
+  // transfers in issue order, so that waiting for them (loads return in order) neither
+  // exposes their latency nor drains the transfers of the next stage.
+  i32x2 sa[DT == ASTERGEMM_MXFP4 ? TM : 1], sb[DT == ASTERGEMM_MXFP4 ? TN : 1];
+  i32x2 sa_nx[DT == ASTERGEMM_MXFP4 ? TM : 1], sb_nx[DT == ASTERGEMM_MXFP4 ? TN : 1];
+  auto load_scales = [&](int kt) {
+    if constexpr (DT == ASTERGEMM_MXFP4) {
+#pragma unroll
+      for (int m = 0; m < TM; ++m) sa_nx[m] = *(const i32x2*)(mxa_row[m] + kt * 8);
+#pragma unroll
+      for (int n = 0; n < TN; ++n) sb_nx[n] = *(const i32x2*)(mxb_row[n] + kt * 8);
+    }
+  };
+  load_scales(0);
   stage_step(0, 0);
 
   for (int kt = 0; kt < p.ksteps; ++kt) {
@@ -278,16 +292,18 @@ __device__ __forceinline__ void gemm_tile_body(const GemmArgs& p) {
     // everybody's have, and everybody is done reading the other stage.
     __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
     __syncthreads();
-    if (kt + 1 < p.ksteps) stage_step(kt + 1, (kt + 1) & 1);
-
-    const uint8_t* st = lds + (kt & 1) * STAGE;
-    i32x2 sa[DT == ASTERGEMM_MXFP4 ? TM : 1], sb[DT == ASTERGEMM_MXFP4 ? TN : 1];
     if constexpr (DT == ASTERGEMM_MXFP4) {
 #pragma unroll
-      for (int m = 0; m < TM; ++m) sa[m] = *(const i32x2*)(mxa_row[m] + kt * 8);
+      for (int m = 0; m < TM; ++m) sa[m] = sa_nx[m];
 #pragma unroll
-      for (int n = 0; n < TN; ++n) sb[n] = *(const i32x2*)(mxb_row[n] + kt * 8);
+      for (int n = 0; n < TN; ++n) sb[n] = sb_nx[n];
     }
+    if (kt + 1 < p.ksteps) {
+      load_scales(kt + 1);
+      stage_step(kt + 1, (kt + 1) & 1);
+    }
+
+    const uint8_t* st = lds + (kt & 1) * STAGE;
 #pragma unroll
     for (int s = 0; s < KSUB; ++s) {
       i32x4 af[TM][KGRAN], bf[TN][KGRAN];

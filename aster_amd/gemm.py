@@ -164,6 +164,21 @@ class GemmPlan:
         return list(times)
 
 
+    def bench_rotate(self, operand_sets, iters: int, stream: int = None) -> int:
+        """`iters` back-to-back launches between one event pair, launch i on operand set
+        i % len(operand_sets); each set is a dict with dA, dB, dC and optional scale_a,
+        scale_b, mx_a, mx_b, bias device pointers.  Returns the total time in ns."""
+        arr = (_capi.Operands * len(operand_sets))()
+        for i, o in enumerate(operand_sets):
+            arr[i] = self._operands(o["dA"], o["dB"], o["dC"], o.get("scale_a"), o.get("scale_b"),
+                                    o.get("mx_a"), o.get("mx_b"), o.get("bias"))
+        total = ctypes.c_int64()
+        _capi.check(_capi.load().astergemm_bench_rotate(
+            ctypes.byref(self.config), arr, len(operand_sets), iters, ctypes.byref(total),
+            ctypes.c_void_p(stream) if stream else None))
+        return total.value
+
+
 def gemm_device(dA: int, dB: int, dC: int, M: int, N: int, K: int, dtype_ab: str = "bf16",
                 dtype_c: str = "bf16", **kw) -> None:
     """One launch on caller-owned device pointers (integers)."""

@@ -163,6 +163,17 @@ int astergemm_bench(const astergemm_config* cfg, const astergemm_operands* ops,
                     int iters, int64_t* times_ns, int64_t flush_bytes,
                     void* stream);
 
+/* Steady-state timing for launches too short for an event pair each (an event
+ * pair around an empty kernel reads ~6 us on MI355X): `iters` launches go out
+ * back to back between ONE event pair, launch i using operand set
+ * ops[i % n_ops]; *total_ns = int(ms * 1e6) for all of them.  With enough
+ * distinct weight buffers (n_ops * bytes of B well above the 256 MiB last-level
+ * cache) every launch streams its weights from HBM, which is what the
+ * reference's FlushLLC hook is for (python/aster/execution/flush_llc.py:25-60).
+ * No counterpart in the reference: its harness times every launch separately. */
+int astergemm_bench_rotate(const astergemm_config* cfg, const astergemm_operands* ops,
+                           int n_ops, int iters, int64_t* total_ns, void* stream);
+
 /* Host pre-shuffle of B[N,K] 2-byte elements into per-lane MFMA order
  * (reference: shuffle_weight, contrib/kittens/test/kittens_helpers.py:90-119). */
 int astergemm_shuffle_weight_16(const uint16_t* src, uint16_t* dst, int64_t N,

@@ -451,3 +451,31 @@ def test_fp8_stream_and_tile_kernels_pair_granules_consistently(gpu):
                              family=_capi.KERNEL_TILE, wg_tile=(tile, tile))
         assert name.startswith(prefix)
         check(out, want, "f32", N, bar=1e-4)
+
+
+def test_bench_rotate_uses_every_operand_set(gpu):
+    # three weight matrices and three outputs in turn: afterwards every output holds the
+    # product with its own weights, and the total time is positive
+    M, N, K = 16, 512, 2048
+    a, _, _ = operands(M, N, K, "bf16", seed=31)
+    plan = AG.GemmPlan.create(M, N, K, "bf16", "f32")
+    bufs, sets, weights = [], [], []
+    da = GpuBuffer(a.nbytes)
+    da.copy_from_host(a)
+    for i in range(3):
+        _, b, _ = operands(M, N, K, "bf16", seed=40 + i, b_std=0.05)
+        weights.append(b)
+        db, dc = GpuBuffer(b.nbytes), GpuBuffer(M * N * 4)
+        db.copy_from_host(b)
+        bufs += [db, dc]
+        sets.append({"dA": da.ptr_value, "dB": db.ptr_value, "dC": dc.ptr_value})
+    total = plan.bench_rotate(sets, 7)
+    assert total > 0
+    for i in range(3):
+        out = np.zeros((M, N), np.float32)
+        bufs[2 * i + 1].copy_to_host(out)
+        check(out, G.gemm(a, weights[i], G.BF16, G.F32), "f32", N, bar=1e-5)
+    for bf in bufs + [da]:
+        bf.free()
+    with pytest.raises(_capi.AsterGemmError):
+        plan.bench_rotate([], 3)
