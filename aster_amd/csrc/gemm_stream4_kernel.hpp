@@ -1,0 +1,353 @@
+// Stream kernel for MXFP4 operands (e2m1 nibbles, one e8m0 scale per 32 K-elements of a
+// row, both operands): the staging, swizzle, tile map and epilogue of the fp8 stream kernel
+// with v_mfma_scale_f32_16x16x128_f8f6f4 (cbsz = blgp = 4) as the inner instruction.
+//
+// A K-step is a 128-byte row slice = 256 fp4 elements = two MFMAs per 16x16 tile.  The
+// operand of one MFMA is 16 bytes per lane = one 32-element scale block; lane (i, q) takes
+// granule q of its row for the first MFMA and granule 4+q for the second (the same two
+// reads as the fp8 kernel), with the scales of blocks q and 4+q.
+//
+// Scales travel through LDS as well: the 8 e8m0 bytes of a row and K-step are half a
+// 16-byte granule, so one transfer instruction per wave brings the scales of 64 rows for
+// TWO K-steps (a chunk), two K-steps ahead of their first use.  The wave that fetched a
+// granule re-packs it in place, one trip after it landed, into byte pairs {block q,
+// block 4+q}: a reading lane then needs one 16-bit LDS read per 16-row tile and K-step,
+// and the two MFMAs pick bytes 0 and 1 of that register with op_sel, with no per-lane
+// shifts.  (Fetching the scale bytes from global memory in the loop costs one vector
+// memory instruction per tile and K-step, which the address unit cannot absorb next to the
+// tile transfers, and their latency sits in front of the MFMAs.)
+//
+// LDS: two A slots and two B slots of 32 KiB (K-step k in slot k mod 2), 8 KiB of A scales
+// and 8 KiB of B scales (chunk c in buffer c mod 2).  The barrier of a trip sits behind
+// the last read of B(k): it certifies everything transferred for K-step k+1 and frees the
+// slots of K-step k, whose refills (K-step k+2) are issued right behind it.
+//
+// The kernel runs four waves per workgroup (one per SIMD, 128x128 of C each): two MFMAs per
+// accumulator and trip plus the scale registers do not fit next to 128 accumulators in the
+// 256 registers a wave gets at two waves per SIMD, while one wave per SIMD has 256
+// accumulation registers for the 64 accumulators and 256 architectural ones for the rest.
+#pragma once
+#include "gemm_stream_kernel.hpp"
+
+// Register file half of the accumulators: accumulation registers.
+#define ACC_CONSTRAINT(x) "+a"(x)
+
+namespace astergemm {
+namespace {
+
+template <int DT, int OUT, int BM, int BN, int WM, int WN>
+__device__ __forceinline__ void gemm_stream4_body(const GemmArgs& p) {
+  constexpr int NW = WM * WN;
+  constexpr int TM = BM / WM / 16;
+  constexpr int TN = BN / WN / 16;
+  constexpr int SLOT = BM * kRowBytes;  // 32 KiB: one operand half of one K-step
+  constexpr int LH = BM / 8 / NW;       // 1 KiB transfers per wave and slot
+  constexpr int NMF = TM * TN;          // slots per trip (two MFMAs each)
+  constexpr int BAR = (TN - 2) * TM + 4;  // slots of a trip issued ahead of its barrier
+  constexpr int NSC = 8 / NW;           // scale transfers per wave and chunk
+  constexpr int SC_A = 4 * SLOT;        // A scales: [2 buffers][256 rows][16 bytes]
+  constexpr int SC_B = SC_A + 2 * BM * 16;
+  static_assert(BM == BN, "the ring holds equal A and B halves");
+  static_assert(DT == ASTERGEMM_MXFP4, "fp4 operands");
+  static_assert(BM % (8 * NW) == 0 && (8 * NW) % 16 == 0, "tile rows per wave");
+  static_assert(TM % 2 == 0 && TM >= 4 && TN >= 2 && 8 % NW == 0, "side-instruction schedule below");
+  static_assert(BM == 4 * 64, "eight scale transfers per chunk: four cover A, four cover B");
+
+  extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wm = wave / WN, wn = wave % WN;
+
+  int tile_m, tile_n;
+  map_tile(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m, tile_m, tile_n);
+  const int row0 = tile_m * BM, col0 = tile_n * BN;
+
+  // ---- global -> LDS, tiles: identical to the other stream kernels ---------------------------
+  const int lane = threadIdx.x & 63;
+  const int lrow = lane >> 3;
+  const int g_lane = (lane & 7) ^ (((wave * 8 + lrow) >> 1) & 7);
+  const unsigned a_off = (unsigned)(lrow * (int)p.lda_bytes + g_lane * 16);
+  const unsigned b_off = (unsigned)(lrow * (int)p.ldb_bytes + g_lane * 16);
+  const uint8_t* a_base = p.A + ((int64_t)row0 + wave * 8) * p.lda_bytes;
+  const uint8_t* b_base = p.B + ((int64_t)col0 + wave * 8) * p.ldb_bytes;
+  const int64_t a_jstride = (int64_t)8 * NW * p.lda_bytes;
+  const int64_t b_jstride = (int64_t)8 * NW * p.ldb_bytes;
+  const int nk = p.ksteps;
+
+  auto g2s = [&](const uint8_t* base, unsigned voff, uint8_t* dst) {
+    const unsigned m0v = (unsigned)(size_t)AG_LDS(dst);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(m0v), "v"(voff), "s"(base)
+                 : "memory", "m0");
+  };
+  auto issue_a1 = [&](int k, int slot, int j) {  // slot: 0..1
+    g2s(a_base + (int64_t)k * kRowBytes + j * a_jstride, a_off,
+        lds + slot * SLOT + (j * NW + wave) * 8 * kRowBytes);
+  };
+  auto issue_b1 = [&](int k, int slot, int j) {  // slot: 2..3
+    g2s(b_base + (int64_t)k * kRowBytes + j * b_jstride, b_off,
+        lds + slot * SLOT + (j * NW + wave) * 8 * kRowBytes);
+  };
+
+  // ---- global -> LDS, scales: wave w < 4 brings A rows [64w, 64w+64), wave w >= 4 brings B
+  // rows [64(w-4), +64); lane L brings the 16 scale bytes of row L for chunk c (K-steps 2c
+  // and 2c+1) to [buffer c mod 2][row][16] ----------------------------------------------------
+  // transfer t = wave + i * NW (0..7): t < 4 covers A rows [64t, +64), else B rows [64(t-4), +64)
+  const uint8_t* sc_base[NSC];
+  uint8_t* sc_lds[NSC];
+  unsigned sc_off[NSC];
+#pragma unroll
+  for (int i = 0; i < NSC; ++i) {
+    const int t = wave + i * NW;
+    const bool is_a = t < 4;
+    sc_base[i] = is_a ? p.mx_a + (int64_t)row0 * p.mx_ld : p.mx_b + (int64_t)col0 * p.mx_ld;
+    sc_off[i] = (unsigned)(((t & 3) * 64 + lane) * p.mx_ld);
+    sc_lds[i] = lds + (is_a ? SC_A : SC_B) + (t & 3) * 64 * 16;
+  }
+  auto issue_scales = [&](int c) {
+#pragma unroll
+    for (int i = 0; i < NSC; ++i) g2s(sc_base[i] + c * 16, sc_off[i], sc_lds[i] + (c & 1) * BM * 16);
+  };
+  // in place: bytes b[0..15] of this lane's row -> pairs {b[8h+q], b[8h+4+q]}, h = K-step
+  // parity, q = 0..3
+  auto repack_scales = [&](int c) {
+#pragma unroll
+    for (int i = 0; i < NSC; ++i) {
+      i32x4* cell = (i32x4*)(sc_lds[i] + (c & 1) * BM * 16 + lane * 16);
+      const i32x4 v = *cell;
+      i32x4 r;
+      // v_perm_b32(hi, lo, sel): selector bytes 0-3 index lo, 4-7 index hi
+      r.x = (int)__builtin_amdgcn_perm((unsigned)v.y, (unsigned)v.x, 0x05010400u);  // q = 0, 1
+      r.y = (int)__builtin_amdgcn_perm((unsigned)v.y, (unsigned)v.x, 0x07030602u);  // q = 2, 3
+      r.z = (int)__builtin_amdgcn_perm((unsigned)v.w, (unsigned)v.z, 0x05010400u);
+      r.w = (int)__builtin_amdgcn_perm((unsigned)v.w, (unsigned)v.z, 0x07030602u);
+      *cell = r;
+    }
+  };
+
+  // ---- LDS -> fragments ---------------------------------------------------------------------
+  const int li = lane & 15, lq = lane >> 4;
+  const unsigned rd0 = (unsigned)(li * kRowBytes + ((lq ^ (li >> 1)) << 4));
+  const unsigned rd1 = (unsigned)(li * kRowBytes + (((4 + lq) ^ (li >> 1)) << 4));
+  const unsigned a_rd = (unsigned)(wm * TM * 16 * kRowBytes);
+  const unsigned b_rd = (unsigned)(wn * TN * 16 * kRowBytes);
+  // scale pair of lane (i, q) inside a 16-row tile: row i, byte 2q (+ 8 for odd K-steps)
+  const unsigned sc_rd = (unsigned)(li * 16 + lq * 2);
+  const unsigned sa_rd = (unsigned)(SC_A + wm * TM * 16 * 16);
+  const unsigned sb_rd = (unsigned)(SC_B + wn * TN * 16 * 16);
+
+  i32x4 fa_lo[TM], fa_hi[TM], fb_lo[2], fb_hi[2];
+  int sa[TM], sb[2];
+  // K-step k: tiles in slot k mod 2 (+2 for B), scales in buffer (k/2) mod 2 at byte 8*(k mod 2)
+  auto read_b = [&](int k, auto nn) {
+    constexpr int N = decltype(nn)::value;
+    const uint8_t* s = lds + ((unsigned)((2 + (k & 1)) * SLOT) + b_rd);
+    fb_lo[N & 1] = *(const i32x4*)(s + rd0 + N * 16 * kRowBytes);
+    fb_hi[N & 1] = *(const i32x4*)(s + rd1 + N * 16 * kRowBytes);
+  };
+  auto read_sb = [&](int k, auto nn) {
+    constexpr int N = decltype(nn)::value;
+    const uint8_t* s = lds + ((unsigned)(((k >> 1) & 1) * BM * 16 + (k & 1) * 8) + sb_rd);
+    sb[N & 1] = *(const unsigned short*)(s + sc_rd + N * 16 * 16);
+  };
+  auto read_a = [&](auto mm, const uint8_t* p0, const uint8_t* p1, const uint8_t* ps) {
+    constexpr int M = decltype(mm)::value;
+    fa_lo[M] = *(const i32x4*)(p0 + M * 16 * kRowBytes);
+    fa_hi[M] = *(const i32x4*)(p1 + M * 16 * kRowBytes);
+    sa[M] = *(const unsigned short*)(ps + M * 16 * 16);
+  };
+
+  f32x4 acc[TM][TN];
+#pragma unroll
+  for (int m = 0; m < TM; ++m)
+#pragma unroll
+    for (int n = 0; n < TN; ++n) {
+      acc[m][n] = f32x4{0.f, 0.f, 0.f, 0.f};
+      // Accumulators live in the accumulation half of the register file (the "a"
+      // constraint makes the compiler use that form of the MFMAs), which leaves the 128
+      // architectural registers to fragments, scales and addresses; one pool of 256 does
+      // not allocate without spilling here.  Opaque to the optimiser as well: otherwise the
+      // first MFMA of every tile reads one shared zero tuple and writes a fresh one.
+      asm volatile("" : ACC_CONSTRAINT(acc[m][n]));
+    }
+
+  // ---- prologue: scales of chunks 0 and 1 and tiles of K-steps 0 and 1 issued; chunk 0
+  // re-packed; A-row fragments and the first B-row fragment of K-step 0 read --------------------
+  issue_scales(0);
+#pragma unroll
+  for (int j = 0; j < LH; ++j) issue_a1(0, 0, j);
+#pragma unroll
+  for (int j = 0; j < LH; ++j) issue_b1(0, 2, j);
+  if (nk > 2) issue_scales(1);
+  if (nk > 1) {
+#pragma unroll
+    for (int j = 0; j < LH; ++j) issue_a1(1, 1, j);
+#pragma unroll
+    for (int j = 0; j < LH; ++j) issue_b1(1, 3, j);
+  }
+  // the first transfer (scales of chunk 0) has landed for this wave: re-pack it
+  if (nk > 2) __builtin_amdgcn_s_waitcnt(waitcnt_imm(4 * LH + NSC, 15));
+  else if (nk > 1) __builtin_amdgcn_s_waitcnt(waitcnt_imm(4 * LH, 15));
+  else __builtin_amdgcn_s_waitcnt(waitcnt_imm(2 * LH, 15));
+  asm volatile("" ::: "memory");
+  repack_scales(0);
+  // tiles of K-step 0 landed, everybody's scales re-packed
+  if (nk > 1) __builtin_amdgcn_s_waitcnt(waitcnt_imm(2 * LH, 0));
+  else __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+  using K0 = std::integral_constant<int, 0>;
+  read_b(0, K0{});
+  read_sb(0, K0{});
+  {
+    const uint8_t* s = lds + a_rd;
+    const uint8_t* ps = lds + sa_rd + sc_rd;
+    static_for<0, TM>([&](auto m) { read_a(m, s + rd0, s + rd1, ps); });
+  }
+  __builtin_amdgcn_sched_barrier(0);
+
+  // ---- K loop: trip k multiplies K-step k; pair i = (n, m) is the two MFMAs of tile (m, n) ----
+  // (slot numbers for TM = 8; group n is slots 8n .. 8n+7)
+  //   slot 8n, 8n+1      + B-row fragment n+1 of K-step k and its scales (n < TN-1)
+  //   slot 4             (odd k) re-pack the scale granules of chunk (k+1)/2 that this wave
+  //                      brought in and that the previous barrier certified
+  //   after slot BAR-1   wait for every transfer and every LDS access of this wave; barrier:
+  //                      certifies tiles of K-step k+1 (and re-packed scales), frees K-step k
+  //   slot BAR..BAR+LH-1 + transfers of B(k+2) and A(k+2) into the slots of K-step k
+  //   slot BAR+LH-1      (odd k) + scale transfers of chunk (k+3)/2 (K-steps k+3, k+4)
+  //   last group         + B-row fragment 0 of K-step k+1 and its scales, and A-row
+  //                      fragment m of K-step k+1 and its scales behind the MFMAs of tile m
+  // FIRST: pairs 0..BAR-1 and the barrier; else pairs BAR..31 (the loop body is the second
+  // part of trip k followed by the first part of trip k+1, so that the loop header follows
+  // the full wait and the compiler's own wait counts inside the body stay exact).
+  // Every condition of a part is a compile-time flag, so that each part is straight-line
+  // code: ODD = k is odd; LD = K-step k+2 exists (tile transfers); RD = K-step k+1 exists
+  // (reads, re-pack, barrier); SC = K-step k+3 exists (scale transfer, odd trips only).
+  auto part = [&](int k, auto first, auto odd_c, auto ld_c, auto rd_c, auto sc_c) {
+    constexpr bool FIRST = decltype(first)::value;
+    constexpr bool odd = decltype(odd_c)::value;
+    constexpr bool do_ld = decltype(ld_c)::value;
+    constexpr bool do_rd = decltype(rd_c)::value;
+    constexpr bool do_sc = decltype(sc_c)::value;
+    const uint8_t *ra0 = nullptr, *ra1 = nullptr, *ras = nullptr;  // set right before first use
+    static_for<(FIRST ? 0 : BAR), (FIRST ? BAR : NMF)>([&](auto ic) {
+      constexpr int I = decltype(ic)::value;
+      constexpr int n = I / TM;
+      // Slots come in couples over two A-row tiles: the even slot issues the first MFMA
+      // (granule q) of tiles m0 and m0+1, the odd slot their second MFMA (granule 4+q), so
+      // that the two MFMAs on one accumulator are never back to back.
+      constexpr int m0 = (I % TM) & ~1;
+      constexpr bool HI = (I & 1) != 0;
+      static_for<0, 2>([&](auto jc) {
+        constexpr int m = m0 + decltype(jc)::value;
+        const i32x4 b4 = HI ? fb_hi[n & 1] : fb_lo[n & 1];
+        const i32x4 a4 = HI ? fa_hi[m] : fa_lo[m];
+        // cbsz = blgp = 4: both operands e2m1 (four registers each); op_sel picks byte 0
+        // (blocks q) or byte 1 (blocks 4+q) of the scale registers.  Written as asm to tie
+        // the destination to the accumulator: the compiler otherwise lets the two MFMAs of
+        // a trip rotate an accumulator through fresh registers, which costs copies at the
+        // loop edge and more registers than there are.  Same destination and addend is also
+        // the form the hardware chains without software wait states.
+        if constexpr (!HI)
+          asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 "
+                       "op_sel_hi:[0,0,0] cbsz:4 blgp:4"
+                       : ACC_CONSTRAINT(acc[m][n])
+                       : "v"(b4), "v"(a4), "v"(sb[n & 1]), "v"(sa[m]));
+        else
+          asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 "
+                       "op_sel:[1,1,0] op_sel_hi:[0,0,0] cbsz:4 blgp:4"
+                       : ACC_CONSTRAINT(acc[m][n])
+                       : "v"(b4), "v"(a4), "v"(sb[n & 1]), "v"(sa[m]));
+        // ---- one or two side instructions behind every MFMA --------------------------------
+        if constexpr (decltype(jc)::value == 0) {
+          if constexpr (I % TM == 0 && n + 1 < TN) read_b(k, std::integral_constant<int, n + 1>{});
+          if constexpr (I % TM == 1 && n + 1 < TN) read_sb(k, std::integral_constant<int, n + 1>{});
+          if constexpr (I == 4) {
+            if (odd && do_rd) repack_scales((k + 1) >> 1);
+          }
+          if constexpr (I >= BAR && I < BAR + LH) {
+            if (do_ld) issue_b1(k + 2, 2 + (k & 1), I - BAR);
+          }
+          if constexpr (I == (TN - 1) * TM) {
+            const int kn = k + 1;
+            const uint8_t* s = lds + ((unsigned)((kn & 1) * SLOT) + a_rd);
+            ra0 = s + rd0;
+            ra1 = s + rd1;
+            ras = lds + ((unsigned)(((kn >> 1) & 1) * BM * 16 + (kn & 1) * 8) + sa_rd) + sc_rd;
+            if (do_rd) read_b(k + 1, std::integral_constant<int, 0>{});
+          }
+          if constexpr (I == (TN - 1) * TM + 1) {
+            if (do_rd) read_sb(k + 1, std::integral_constant<int, 0>{});
+          }
+        } else {
+          if constexpr (I >= BAR && I < BAR + LH) {
+            if (do_ld) issue_a1(k + 2, k & 1, I - BAR);
+          }
+          if constexpr (I == BAR + LH - 1) {
+            // chunk (k+3)/2 covers K-steps k+3 and k+4; its buffer held chunk (k-1)/2
+            // (K-steps k-1 and k), last read before this trip's barrier
+            if (odd && do_sc) issue_scales((k + 3) >> 1);
+          }
+        }
+        // refill in place for K-step k+1: the first-MFMA operands of a couple are dead after
+        // its even slot, the second-MFMA operands and the scales after its odd slot
+        if constexpr (I >= (TN - 1) * TM) {
+          if (do_rd) {
+            if constexpr (!HI) {
+              fa_lo[m] = *(const i32x4*)(ra0 + m * 16 * kRowBytes);
+            } else {
+              fa_hi[m] = *(const i32x4*)(ra1 + m * 16 * kRowBytes);
+              sa[m] = *(const unsigned short*)(ras + m * 16 * 16);
+            }
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      });
+      if constexpr (I == BAR - 1) {
+        if (do_rd) {
+          __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
+          __builtin_amdgcn_s_barrier();
+          asm volatile("" ::: "memory");
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    });
+  };
+  static_assert(BAR > (TN - 2) * TM + 1 && BAR + LH <= NMF, "schedule positions");
+  using T = std::true_type;
+  using F = std::false_type;
+  // nk is even.  part(k, first-half?, odd, LD, RD, SC)
+  int k = 0;
+  part(0, T{}, F{}, F{}, T{}, F{});
+#pragma unroll 1
+  for (; k + 4 < nk; k += 2) {
+    part(k, F{}, F{}, T{}, T{}, F{});
+    part(k + 1, T{}, T{}, F{}, T{}, F{});
+    part(k + 1, F{}, T{}, T{}, T{}, T{});
+    part(k + 2, T{}, F{}, F{}, T{}, F{});
+  }
+  if (nk >= 4) {  // k = nk - 4: the last scale chunk is already on its way
+    part(k, F{}, F{}, T{}, T{}, F{});
+    part(k + 1, T{}, T{}, F{}, T{}, F{});
+    part(k + 1, F{}, T{}, T{}, T{}, F{});
+    part(k + 2, T{}, F{}, F{}, T{}, F{});
+    k += 2;
+  }
+  // k = nk - 2: nothing left to transfer; the last trip has nothing left to read
+  part(k, F{}, F{}, F{}, T{}, F{});
+  part(k + 1, T{}, T{}, F{}, F{}, F{});
+  part(k + 1, F{}, T{}, F{}, F{}, F{});
+  __builtin_amdgcn_sched_barrier(0);
+
+  stream_epilogue<OUT, BM, BN, WM, WN>(p, acc, lds, wave, row0, col0);
+}
+
+template <int DT, int OUT, int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(WM* WN * 64) void gemm_stream4_kernel(const GemmArgs p) {
+  gemm_stream4_body<DT, OUT, BM, BN, WM, WN>(p);
+}
+
+}  // namespace
+}  // namespace astergemm
+#undef ACC_CONSTRAINT

@@ -3,6 +3,7 @@
 #include "gemm_pipe_kernel.hpp"
 #include "gemm_stream_kernel.hpp"
 #include "gemm_stream8_kernel.hpp"
+#include "gemm_stream4_kernel.hpp"
 
 namespace astergemm {
 namespace {
@@ -138,6 +139,40 @@ int launch_stream8(const GemmArgs& a, int grid, hipStream_t s) {
         launch_stream8<DT, OUT, 256, 256, 2, 4>, check_stream                    \
   }
 
+template <int DT, int OUT, int BM, int BN, int WM, int WN>
+int launch_stream4(const GemmArgs& a, int grid, hipStream_t s) {
+  constexpr int lds = 4 * BM * kRowBytes + 4 * BM * 16;
+  // the scale planes are fetched in 16-byte granules
+  if ((((uintptr_t)a.mx_a | (uintptr_t)a.mx_b) & 15) != 0 || a.mx_ld % 16 != 0)
+    return (int)hipErrorInvalidValue;
+  auto k = gemm_stream4_kernel<DT, OUT, BM, BN, WM, WN>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)k,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess) return (int)e;
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(k, dim3(grid), dim3(WM * WN * 64), lds, s, a);
+  return (int)hipGetLastError();
+}
+
+// Whole 256x256 tiles and an even number of 256-element K-steps (scales move in 16-byte
+// granules = two K-steps of a row).
+const char* check_stream4(const astergemm_config& c) {
+  if (const char* why = check_stream(c)) return why;
+  if (c.K % 512 != 0) return "K must be a multiple of 512";
+  return nullptr;
+}
+
+#define AG_STREAM4(name, DT, OUT)                                                \
+  Variant {                                                                      \
+    name, ASTERGEMM_KERNEL_TILE, DT, OUT, 256, 256, kRowBytes, 2, 2, 2, 2,       \
+        4 * 256 * kRowBytes + 4 * 256 * 16,                                      \
+        (const void*)gemm_stream4_kernel<DT, OUT, 256, 256, 2, 2>,               \
+        launch_stream4<DT, OUT, 256, 256, 2, 2>, check_stream4                   \
+  }
+
 #define AG_STREAM_SET(prefix, DT)                                                      \
   AG_STREAM(prefix "_256x256_w2x4_bf16", DT, ASTERGEMM_BF16, 256, 256, 2, 4),          \
       AG_STREAM(prefix "_256x256_w2x4_f32", DT, ASTERGEMM_F32, 256, 256, 2, 4),        \
@@ -157,6 +192,9 @@ const Variant kTileVariants[] = {
     AG_STREAM8("stream_fp8_256x256_w2x4_bf16", ASTERGEMM_FP8_E4M3, ASTERGEMM_BF16),
     AG_STREAM8("stream_fp8_256x256_w2x4_f32", ASTERGEMM_FP8_E4M3, ASTERGEMM_F32),
     AG_STREAM8("stream_fp8_256x256_w2x4_f16", ASTERGEMM_FP8_E4M3, ASTERGEMM_F16),
+    AG_STREAM4("stream_mxfp4_256x256_w2x2_bf16", ASTERGEMM_MXFP4, ASTERGEMM_BF16),
+    AG_STREAM4("stream_mxfp4_256x256_w2x2_f32", ASTERGEMM_MXFP4, ASTERGEMM_F32),
+    AG_STREAM4("stream_mxfp4_256x256_w2x2_f16", ASTERGEMM_MXFP4, ASTERGEMM_F16),
 };
 
 }  // namespace

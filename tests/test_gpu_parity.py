@@ -383,7 +383,7 @@ def _tile_variants():
 
 @pytest.mark.parametrize("vid,name,dtype_ab,dtype_c", _tile_variants(), ids=lambda v: str(v))
 def test_every_tile_variant(gpu, vid, name, dtype_ab, dtype_c):
-    M, N, K = 512, 768, 1280  # whole 256-tiles, ten 128-byte K-steps (two trips of the ring of five)
+    M, N, K = 512, 768, 1536  # whole 256-tiles; 24 / 12 / 6 K-steps of 128 bytes (16-bit / fp8 / fp4)
     a, b, ex = operands(M, N, K, dtype_ab, seed=11, a_std=1.0, b_std=1.0 if dtype_ab != "bf16" else 0.05)
     bias = np.random.default_rng(12).standard_normal(N).astype(np.float32)
     plan = AG.GemmPlan.create(M, N, K, dtype_ab, dtype_c, has_bias=True, variant=vid)
@@ -479,3 +479,27 @@ def test_bench_rotate_uses_every_operand_set(gpu):
         bf.free()
     with pytest.raises(_capi.AsterGemmError):
         plan.bench_rotate([], 3)
+
+
+@pytest.mark.parametrize("ksteps", [2, 4, 6, 8, 10, 12, 14])
+def test_mxfp4_stream_kernel_every_loop_phase(gpu, ksteps):
+    # 256-element K-steps in pairs (scales travel two K-steps at a time): final parts only,
+    # the block before them, and one to five steady iterations; random nibbles and random
+    # per-block scales, so a wrong block <-> scale byte pairing cannot cancel
+    M, N, K = 256, 512, 256 * ksteps
+    rng = np.random.default_rng(29 + ksteps)
+    a = rng.integers(0, 256, (M, K // 2)).astype(np.uint8)
+    b = rng.integers(0, 256, (N, K // 2)).astype(np.uint8)
+    mxa = rng.integers(118, 134, (M, K // 32)).astype(np.uint8)
+    mxb = rng.integers(118, 134, (N, K // 32)).astype(np.uint8)
+    out, name = run_gemm(a, b, M, N, K, "mxfp4", "f32", mx_a=mxa, mx_b=mxb,
+                         family=_capi.KERNEL_TILE, wg_tile=(256, 256))
+    assert name.startswith("stream_mxfp4")
+    check(out, G.gemm_mxfp4(a, mxa, b, mxb, out_dtype=G.F32), "f32", N, bar=1e-5)
+
+
+def test_mxfp4_stream_kernel_falls_back_for_odd_kstep_counts(gpu):
+    assert AG.GemmPlan.create(512, 512, 768, "mxfp4", "bf16", wg_tile=(256, 256)).info.name.decode() \
+        .startswith("tile_mxfp4")
+    assert AG.GemmPlan.create(4096, 14336, 4096, "mxfp4", "bf16").info.name.decode() \
+        .startswith("stream_mxfp4")
