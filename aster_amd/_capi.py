@@ -21,6 +21,7 @@ F16, BF16, FP8_E4M3, MXFP4, F32 = 0, 1, 2, 3, 4
 SCALE_NONE, SCALE_TENSOR, SCALE_MX32 = 0, 1, 2
 # astergemm_kernel_family
 KERNEL_AUTO, KERNEL_TILE, KERNEL_SKINNY = 0, 1, 2
+OPERAND_LDS, OPERAND_DIRECT_B = 0, 1
 
 DTYPE_NAMES = {"f16": F16, "bf16": BF16, "fp8_e4m3": FP8_E4M3, "mxfp4": MXFP4, "f32": F32}
 
@@ -43,7 +44,8 @@ class Config(C.Structure):
         ("wg_tile_m", C.c_int32), ("wg_tile_n", C.c_int32),
         ("waves_m", C.c_int32), ("waves_n", C.c_int32),
         ("variant", C.c_int32),
-        ("reserved", C.c_int32 * 6),
+        ("operand_path", C.c_int32),
+        ("reserved", C.c_int32 * 5),
     ]
 
 

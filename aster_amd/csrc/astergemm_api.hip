@@ -41,7 +41,7 @@ const Variant* variant_at(int index) {
 }
 
 bool variant_matches_types(const Variant& v, const astergemm_config& c) {
-  return v.dtype_ab == c.dtype_ab && v.dtype_c == c.dtype_c;
+  return v.dtype_ab == c.dtype_ab && v.dtype_c == c.dtype_c && v.operand_path == c.operand_path;
 }
 
 const char* validate_problem(const astergemm_config& c) {
@@ -52,6 +52,8 @@ const char* validate_problem(const astergemm_config& c) {
     return "dtype_c must be F32, BF16 or F16";
   if (c.scale_mode < ASTERGEMM_SCALE_NONE || c.scale_mode > ASTERGEMM_SCALE_MX32)
     return "bad scale_mode";
+  if (c.operand_path != ASTERGEMM_OPERAND_LDS && c.operand_path != ASTERGEMM_OPERAND_DIRECT_B)
+    return "bad operand_path";
   if ((c.dtype_ab == ASTERGEMM_MXFP4) != (c.scale_mode == ASTERGEMM_SCALE_MX32))
     return "MXFP4 operands and SCALE_MX32 go together";
   if (c.dtype_ab == ASTERGEMM_MXFP4 && c.K % 32 != 0) return "MXFP4 needs K % 32 == 0";
@@ -90,6 +92,7 @@ const Variant* choose(const astergemm_config& c, int* index_out) {
   int family = c.family;
   if (family == ASTERGEMM_KERNEL_AUTO)
     family = (is16 && c.M <= 64 && c.K % 32 == 0) ? ASTERGEMM_KERNEL_SKINNY : ASTERGEMM_KERNEL_TILE;
+  if (c.operand_path == ASTERGEMM_OPERAND_DIRECT_B) family = ASTERGEMM_KERNEL_SKINNY;
 
   const Variant* best = nullptr;
   int best_index = -1;

@@ -58,6 +58,8 @@ struct Variant {
   int (*launch)(const GemmArgs& a, int grid, hipStream_t s);
   // Host-side shape check: nullptr when ok, else a reason.
   const char* (*check)(const astergemm_config& c);
+  // B operand form this variant reads (astergemm_operand_path); plain row-major by default.
+  int operand_path = 0;
 };
 
 int num_tile_variants();

@@ -10,6 +10,7 @@
 //   astergemm_replay --m 8192 --n 8192 --k 8192 --ab bf16 --c bf16 --iters 100
 //                    [--warmup 20] [--tile 256] [--family tile|skinny|auto]
 //                    [--variant ID] [--flush BYTES] [--bias] [--json] [--calib BYTES]
+//                    [--direct-b]   (B taken as pre-shuffled; timing only, the fill is random)
 //
 // --calib BYTES first copies BYTES device-to-device three times: a copy kernel that
 // reads and writes a known number of bytes, against which the counters of a
@@ -107,6 +108,7 @@ int main(int argc, char** argv) {
     else if (a == "--variant") cfg.variant = atoi(val());
     else if (a == "--flush") flush = atoll(val());
     else if (a == "--calib") calib = atoll(val());
+    else if (a == "--direct-b") cfg.operand_path = ASTERGEMM_OPERAND_DIRECT_B;
     else if (a == "--bias") cfg.has_bias = 1;
     else if (a == "--json") json = 1;
     else if (a == "--family") {

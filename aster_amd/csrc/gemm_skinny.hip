@@ -21,6 +21,7 @@ namespace {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef unsigned short u16x4 __attribute__((ext_vector_type(4)));
@@ -420,6 +421,229 @@ const char* check_skinny_reg(const astergemm_config& c) {
         check_skinny_reg                                                                   \
   }
 
+// ---- M <= 16, B pre-shuffled (operand path "direct B") ---------------------------------
+//
+// B arrives in the order of the reference's shuffle_weight
+// (contrib/kittens/test/kittens_helpers.py:90-119): 1 KiB chunks (16 weight rows x 32 K
+// elements), chunk (nb, kb) at ((nb * K/32 + kb) * 1024), inside it lane d = 16*g + n holds
+// B[16 nb + n][32 kb + 4g .. 4g+3] and B[16 nb + n][32 kb + 16 + 4g .. +3].  A wave's 16-byte
+// load per lane of one chunk therefore IS its MFMA operand and is 1 KiB contiguous; the
+// eight waves take the chunks of a row block round robin, so a workgroup sweeps its part of B
+// front to back.  No LDS transposition; x is gathered once
+// into registers in the same K order.  Everything else (persistent grid, N split in
+// multiples of 8 rows, two units in flight, reduction through LDS every four row blocks) is
+// as in the kernel above.
+// CPW = chunks per wave and row block = K / 256.
+template <int DT, int OUT, int CPW>
+__global__ __launch_bounds__(512) void gemm_skinny_direct_kernel(const GemmArgs p) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t slds[];
+  constexpr int KW = 8;
+  constexpr int UPB = CPW / 8;                   // units (8 chunks) per wave and row block
+  constexpr int NBS = 4;                         // row blocks between workgroup barriers
+  static_assert(CPW % 8 == 0, "whole units");
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int li = lane & 15, lq = lane >> 4;
+  f32x4* red = (f32x4*)slds;                     // [2][NBS][KW][64]
+
+  // rows [r0, r1) of the weight matrix belong to this workgroup (multiples of 8: a row
+  // block at either end may be half of a 16-row chunk)
+  const int g = gridDim.x;
+  const int per = (((p.N + g - 1) / g) + 7) & ~7;
+  const int r0 = blockIdx.x * per;
+  const int r1 = (r0 + per) < p.N ? (r0 + per) : p.N;
+  if (r0 >= p.N) return;
+  const int nb0 = r0 >> 4;
+  const int nblk = ((r1 - 1) >> 4) - nb0 + 1;
+  const int total = nblk * UPB;
+  const int64_t blk_bytes = (int64_t)(p.K >> 5) * 1024;   // all chunks of one row block
+
+  const uint8_t* wbase = p.B + (int64_t)nb0 * blk_bytes + (int64_t)wave * CPW * 1024 + lane * 16;
+  const uint8_t* idle = p.A + lane * 16;  // nothing to fetch: lines that stay in L2
+  auto issue = [&](int j, i32x4(&dst)[8]) {      // flat index j = block * UPB + t
+    int blk = j / UPB;
+    const int t = j % UPB;
+    blk = blk < nblk ? blk : nblk - 1;
+    const int n = (nb0 + blk) * 16 + li;
+    const bool dead = j >= total || n < r0 || n >= r1;
+    const uint8_t* src = dead ? idle : wbase + (int64_t)blk * blk_bytes + t * 8192;
+    const int step = dead ? 0 : 1024;            // idle lanes re-read one line of x
+#pragma unroll
+    for (int u = 0; u < 8; ++u) dst[u] = __builtin_nontemporal_load((const i32x4*)(src + u * step));
+  };
+
+  // x operands in the K order of the shuffle: row li, elements 4q..4q+3 and 16+4q..16+4q+3 of
+  // every 32-element block of this wave's slice.  Fetched as whole lines (8 rows x 128 bytes
+  // per instruction; 8-byte gathers straight from global memory are four times the requests
+  // and cost ~4 us at the start of the kernel) and turned around in a wave-private LDS
+  // buffer: 128-byte rows, 16-byte granule index XOR (row & 7).
+  i32x4 x[CPW];
+  {
+    uint8_t* tbuf = slds + 2 * NBS * KW * 1024 + wave * 8192;
+    const int lrow = lane >> 3, lpiece = lane & 7;
+    const int wr_off = lrow * 128 + ((lpiece ^ lrow) << 4);
+    static_for<0, UPB>([&](auto T) {
+      constexpr int t = decltype(T)::value;
+      i32x4 xw[8];
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        int m = h * 8 + lrow;
+        m = m < p.M ? m : p.M - 1;
+        const uint8_t* src =
+            p.A + (int64_t)m * p.lda_bytes + (int64_t)wave * CPW * 64 + t * 512 + lpiece * 16;
+#pragma unroll
+        for (int s2 = 0; s2 < 4; ++s2) xw[s2 * 2 + h] = *(const i32x4*)(src + s2 * 128);
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        *(i32x4*)(tbuf + (i >> 1) * 2048 + (i & 1) * 1024 + wr_off) = xw[i];
+#pragma unroll
+      for (int c = 0; c < 8; ++c) {               // chunk c of this unit: line c/2, half c&1
+        const uint8_t* row = tbuf + (c >> 1) * 2048 + li * 128 + (lq & 1) * 8;
+        const int g_lo = (c & 1) * 4 + (lq >> 1), g_hi = g_lo + 2;
+        const i32x2 lo = *(const i32x2*)(row + ((g_lo ^ (li & 7)) << 4));
+        const i32x2 hi = *(const i32x2*)(row + ((g_hi ^ (li & 7)) << 4));
+        x[t * 8 + c] = i32x4{lo.x, lo.y, hi.x, hi.y};
+      }
+    });
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  // three register sets: the loaded registers are the MFMA operands themselves, so a set is
+  // busy until its MFMAs have issued; with three, two units stay in flight behind the one
+  // being multiplied
+  i32x4 w0[8], w1[8], w2[8];
+  issue(0, w0);
+  issue(1, w1);
+  issue(2, w2);
+  __builtin_amdgcn_sched_barrier(0);
+
+  float scale = 1.0f;
+  if (p.scale_a) scale *= *p.scale_a;
+  if (p.scale_b) scale *= *p.scale_b;
+
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  int parity = 0;
+  auto block_end = [&](int blk) {
+    const int slot = blk & (NBS - 1);
+    red[((parity * NBS + slot) * KW + wave) * 64 + lane] = acc;
+    acc = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (slot != NBS - 1 && blk != nblk - 1) return;
+    __syncthreads();
+    if (wave <= slot) {
+      const f32x4* src = red + ((parity * NBS + wave) * KW) * 64 + lane;
+      f32x4 v = src[0];
+#pragma unroll
+      for (int k = 1; k < KW; ++k) v += src[k * 64];
+      const int m = li, n = (nb0 + blk - slot + wave) * 16 + 4 * lq;
+      if (m < p.M && n >= r0 && n < r1) {
+        v *= scale;
+        if (p.bias)
+          for (int r = 0; r < 4; ++r) v[r] += p.bias[n + r];
+        const int64_t idx = (int64_t)m * p.ldc + n;
+        const bool vec_ok = (p.ldc & 3) == 0;
+        if constexpr (OUT == ASTERGEMM_F32) {
+          float* o = (float*)p.C + idx;
+          if (vec_ok) *(f32x4*)o = v;
+          else
+            for (int r = 0; r < 4; ++r) o[r] = v[r];
+        } else {
+          unsigned short h[4];
+          for (int r = 0; r < 4; ++r) {
+            if constexpr (OUT == ASTERGEMM_BF16) h[r] = sk_f32_to_bf16(v[r]);
+            else {
+              _Float16 hh = (_Float16)v[r];
+              h[r] = __builtin_bit_cast(unsigned short, hh);
+            }
+          }
+          unsigned short* o = (unsigned short*)p.C + idx;
+          if (vec_ok) *(u16x4*)o = u16x4{h[0], h[1], h[2], h[3]};
+          else
+            for (int r = 0; r < 4; ++r) o[r] = h[r];
+        }
+      }
+    }
+    parity ^= 1;
+  };
+  // T = unit index inside the row block (compile time: selects the x registers)
+  auto mma = [&](int blk, auto T, const i32x4(&src)[8]) {
+    constexpr int t = decltype(T)::value;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) acc = sk_mfma<DT>(src[u], x[t * 8 + u], acc);
+    if (t == UPB - 1) block_end(blk);
+  };
+
+  // flat steps in groups of lcm(3, UPB) so that register set and x indices are static
+  constexpr int TRIP = (UPB % 3 == 0) ? UPB : 3 * UPB;
+  auto step = [&](int j, auto IC) {
+    constexpr int i = decltype(IC)::value;
+    auto body = [&](i32x4(&w)[8]) {
+      mma((j + i) / UPB, std::integral_constant<int, i % UPB>{}, w);
+      __builtin_amdgcn_sched_barrier(0);
+      issue(j + i + 3, w);
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    if constexpr (i % 3 == 0) body(w0);
+    else if constexpr (i % 3 == 1) body(w1);
+    else body(w2);
+  };
+  int j = 0;
+  for (; j + TRIP <= total; j += TRIP) static_for<0, TRIP>([&](auto IC) { step(j, IC); });
+  // remainder: fewer than TRIP steps, j is a multiple of TRIP (so of 3 and of UPB)
+  static_for<0, TRIP>([&](auto IC) {
+    if (j + decltype(IC)::value < total) step(j, IC);
+  });
+}
+
+template <int DT, int OUT, int CPW>
+int launch_skinny_direct_t(const GemmArgs& a, hipStream_t s) {
+  auto k = gemm_skinny_direct_kernel<DT, OUT, CPW>;
+  constexpr int lds = 2 * 4 * 8 * 64 * 16 + 8 * 8192;
+  static bool attr_set = false;
+  static int cus = 0;
+  if (!attr_set) {
+    hipError_t e =
+        hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess) return (int)e;
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess)
+      return (int)hipGetLastError();
+    cus = prop.multiProcessorCount;
+    attr_set = true;
+  }
+  const int nblocks = (int)((a.N + 15) / 16);
+  const int g = nblocks < cus ? nblocks : cus;
+  hipLaunchKernelGGL(k, dim3(g), dim3(512), lds, s, a);
+  return (int)hipGetLastError();
+}
+
+template <int DT, int OUT>
+int launch_skinny_direct(const GemmArgs& a, int grid, hipStream_t s) {
+  (void)grid;
+  switch (a.K) {
+    case 2048: return launch_skinny_direct_t<DT, OUT, 8>(a, s);
+    case 4096: return launch_skinny_direct_t<DT, OUT, 16>(a, s);
+    case 8192: return launch_skinny_direct_t<DT, OUT, 32>(a, s);
+  }
+  return (int)hipErrorInvalidValue;
+}
+
+const char* check_skinny_direct(const astergemm_config& c) {
+  if (c.M > 16) return "pre-shuffled B is supported for M <= 16";
+  if (c.K != 2048 && c.K != 4096 && c.K != 8192)
+    return "pre-shuffled B is supported for K = 2048, 4096 or 8192";
+  if (c.N % 16 != 0) return "pre-shuffled B needs N % 16 == 0";
+  if (c.ldb != 0 && c.ldb != c.K) return "pre-shuffled B is packed (ldb = K)";
+  return nullptr;
+}
+
+#define AG_SKINNY_DIRECT(name, DT, OUT)                                                     \
+  Variant {                                                                                 \
+    name, ASTERGEMM_KERNEL_SKINNY, DT, OUT, 16, 16, 512, 1, 8, 1, 1, 131072,                \
+        (const void*)gemm_skinny_direct_kernel<DT, OUT, 16>, launch_skinny_direct<DT, OUT>, \
+        check_skinny_direct, ASTERGEMM_OPERAND_DIRECT_B                                     \
+  }
+
 template <int DT, int OUT, int MT, int NB, int KW, int U>
 int launch_skinny(const GemmArgs& a, int grid, hipStream_t s) {
   hipLaunchKernelGGL((gemm_skinny_kernel<DT, OUT, MT, NB, KW, U>), dim3(grid), dim3(KW * 64), 0,
@@ -478,6 +702,12 @@ const Variant kSkinnyVariants[] = {
     AG_SKINNY_LDS("skinnyx_f16_m16_bf16", ASTERGEMM_F16, ASTERGEMM_BF16),
     AG_SKINNY_LDS("skinnyx_f16_m16_f32", ASTERGEMM_F16, ASTERGEMM_F32),
     AG_SKINNY_LDS("skinnyx_f16_m16_f16", ASTERGEMM_F16, ASTERGEMM_F16),
+    AG_SKINNY_DIRECT("skinnyd_bf16_m16_bf16", ASTERGEMM_BF16, ASTERGEMM_BF16),
+    AG_SKINNY_DIRECT("skinnyd_bf16_m16_f32", ASTERGEMM_BF16, ASTERGEMM_F32),
+    AG_SKINNY_DIRECT("skinnyd_bf16_m16_f16", ASTERGEMM_BF16, ASTERGEMM_F16),
+    AG_SKINNY_DIRECT("skinnyd_f16_m16_bf16", ASTERGEMM_F16, ASTERGEMM_BF16),
+    AG_SKINNY_DIRECT("skinnyd_f16_m16_f32", ASTERGEMM_F16, ASTERGEMM_F32),
+    AG_SKINNY_DIRECT("skinnyd_f16_m16_f16", ASTERGEMM_F16, ASTERGEMM_F16),
 };
 
 }  // namespace

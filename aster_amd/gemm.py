@@ -125,8 +125,11 @@ class GemmPlan:
     def create(cls, M: int, N: int, K: int, dtype_ab: str = "bf16", dtype_c: str = "bf16", *,
                scale_mode: Optional[str] = None, has_bias: bool = False, lda: int = 0,
                ldb: int = 0, ldc: int = 0, family: int = _capi.KERNEL_AUTO, wg_tile=(0, 0),
-               variant: int = 0) -> "GemmPlan":
+               variant: int = 0, operand_path: str = "lds") -> "GemmPlan":
+        """`operand_path` follows GemmMappingSpec.operand_path of the reference: "lds" = B is
+        plain row-major [N, ldb]; "direct_b" = B was pre-shuffled with `shuffle_weight`."""
         c = _capi.Config()
+        c.operand_path = {"lds": _capi.OPERAND_LDS, "direct_b": _capi.OPERAND_DIRECT_B}[operand_path]
         c.M, c.N, c.K = M, N, K
         c.lda, c.ldb, c.ldc = lda, ldb, ldc
         c.dtype_ab, c.dtype_c = _DTYPE_ID[dtype_ab], _DTYPE_ID[dtype_c]

@@ -217,6 +217,26 @@ def main() -> int:
                            "us_back_to_back_8_weight_sets": round(rot_ns / 1e3, 2),
                            "gbps_back_to_back": round(p.info.bytes / rot_ns, 1),
                            "frac_back_to_back": round(p.info.bytes / rot_ns / PEAK_HBM_GBPS, 4)})
+        # the same M = 16 shape with the weights pre-shuffled into MFMA operand order
+        # (the reference's operand_path = direct_b); values do not matter for the timing
+        del a, b, c
+        a, b, keep = make_operands(torch, 16, 14336, 4096, "bf16", dev)
+        c = torch.empty(16, 14336, device=dev, dtype=torch.bfloat16)
+        p = AG.GemmPlan.create(16, 14336, 4096, "bf16", "bf16", operand_path="direct_b")
+        p50, _, _ = event_timed_p50(p, a, b, c, keep, 100, 20, flush_bytes=512 << 20)
+        wts = [b] + [torch.empty_like(b).copy_(b) for _ in range(7)]
+        sets = [{"dA": a.data_ptr(), "dB": w.data_ptr(), "dC": c.data_ptr()} for w in wts]
+        p.bench_rotate(sets, 40)
+        rot_ns = p.bench_rotate(sets, 200) / 200.0
+        del wts, sets
+        others.append({"workload": "bf16 skinny GEMM M=16 N=14336 K=4096 -> bf16, weights pre-shuffled "
+                                   "(operand_path direct_b), LLC flushed before every launch",
+                       "kernel": p.info.name.decode(), "p50_us": round(p50 / 1e3, 2),
+                       "gbps": round(p.info.bytes / p50, 1), "bound": "hbm",
+                       "frac": round(p.info.bytes / p50 / PEAK_HBM_GBPS, 4),
+                       "us_back_to_back_8_weight_sets": round(rot_ns / 1e3, 2),
+                       "gbps_back_to_back": round(p.info.bytes / rot_ns, 1),
+                       "frac_back_to_back": round(p.info.bytes / rot_ns / PEAK_HBM_GBPS, 4)})
         out["others"] = others
 
     if not args.no_cpu:

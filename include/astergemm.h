@@ -67,6 +67,17 @@ typedef enum astergemm_kernel_family {
   ASTERGEMM_KERNEL_SKINNY = 2 /* weight-streaming kernel for M <= 64        */
 } astergemm_kernel_family;
 
+/* The reference's GemmMappingSpec.operand_path (gemm_config.py:213-276): with
+ * "direct_b" the host pre-shuffles B with shuffle_weight
+ * (contrib/kittens/test/kittens_helpers.py:90-119) so that a lane's 16-byte
+ * global load is its MFMA operand and B never passes through LDS.            */
+typedef enum astergemm_operand_path {
+  ASTERGEMM_OPERAND_LDS = 0,      /* B[N, ldb] row-major as described below   */
+  ASTERGEMM_OPERAND_DIRECT_B = 1  /* B packed [N, K] and pre-shuffled with
+                                     astergemm_shuffle_weight_16 (16-bit
+                                     operands; skinny kernels only)          */
+} astergemm_operand_path;
+
 /* ---- problem + mapping --------------------------------------------------
  * C[M,N] = epilogue( sum_k A[M,K] * B[N,K] )      (B is stored N x K, i.e.
  * "column-major K x N"; reference: gemm_config.py:94, 109).
@@ -88,7 +99,8 @@ typedef struct astergemm_config {
   int32_t waves_n;       /* num_waves_per_workgroup[N]                      */
   int32_t variant;       /* explicit variant id from astergemm_variant_*,
                             or 0                                             */
-  int32_t reserved[6];
+  int32_t operand_path;  /* astergemm_operand_path: how B is stored         */
+  int32_t reserved[5];
 } astergemm_config;
 
 /* What astergemm_select() reports back; the reference gets the same facts by

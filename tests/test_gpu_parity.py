@@ -27,11 +27,13 @@ _OUT_NP = {"f32": np.float32, "bf16": np.uint16, "f16": np.uint16}
 
 
 def run_gemm(a, b, M, N, K, dtype_ab, dtype_c, *, scale_a=None, scale_b=None, mx_a=None, mx_b=None,
-             bias=None, lda=0, ldb=0, ldc=0, family=_capi.KERNEL_AUTO, wg_tile=(0, 0)):
+             bias=None, lda=0, ldb=0, ldc=0, family=_capi.KERNEL_AUTO, wg_tile=(0, 0),
+             operand_path="lds"):
     """Upload, launch once through astergemm_run, download.  Returns the raw
     output storage [M, ldc or N] and the kernel name."""
     plan = AG.GemmPlan.create(M, N, K, dtype_ab, dtype_c, has_bias=bias is not None, lda=lda,
-                              ldb=ldb, ldc=ldc, family=family, wg_tile=wg_tile)
+                              ldb=ldb, ldc=ldc, family=family, wg_tile=wg_tile,
+                              operand_path=operand_path)
     ldc_eff = ldc or N
     out = np.full((M, ldc_eff), 0x7FC1 if dtype_c != "f32" else np.nan, dtype=_OUT_NP[dtype_c])
     bufs = []
@@ -503,3 +505,30 @@ def test_mxfp4_stream_kernel_falls_back_for_odd_kstep_counts(gpu):
         .startswith("tile_mxfp4")
     assert AG.GemmPlan.create(4096, 14336, 4096, "mxfp4", "bf16").info.name.decode() \
         .startswith("stream_mxfp4")
+
+
+@pytest.mark.parametrize("M,N,K", [(16, 14336, 4096), (1, 16, 2048), (5, 784, 8192), (13, 6000, 2048),
+                                   (16, 48, 4096), (9, 4112, 8192), (16, 4096 + 16 * 7, 4096)])
+@pytest.mark.parametrize("dtype_ab,dtype_c", [("bf16", "f32"), ("f16", "f16"), ("bf16", "bf16")])
+def test_skinny_direct_b_preshuffled_weights(gpu, M, N, K, dtype_ab, dtype_c):
+    """operand_path = direct_b: B is handed over in the order of the reference's
+    shuffle_weight (kittens_helpers.py:90-119); the result must equal the GEMM on the
+    unshuffled weights.  Row ranges that start or end inside a 16-row chunk, single-workgroup
+    grids, bias and a padded output pitch."""
+    from aster_amd.kittens_helpers import shuffle_weight
+    a, b, _ = operands(M, N, K, dtype_ab, seed=51, b_std=0.05)
+    bias = np.random.default_rng(52).standard_normal(N).astype(np.float32)
+    ldc = (N + 11) & ~3
+    out, name = run_gemm(a, shuffle_weight(b), M, N, K, dtype_ab, dtype_c, bias=bias, ldc=ldc,
+                         operand_path="direct_b")
+    assert name.startswith("skinnyd")
+    want = G.gemm(a, b, _DT[dtype_ab], _DT[dtype_c], bias=bias)
+    check(out, want, dtype_c, N, bar=1e-5 if dtype_c == "f32" else REL_L2_BAR)
+    pad = out[:, N:]
+    assert np.isnan(pad).all() if dtype_c == "f32" else (pad == 0x7FC1).all()
+
+
+def test_direct_b_is_refused_where_it_is_not_implemented(gpu):
+    for kw in (dict(M=128, N=256, K=4096), dict(M=16, N=256, K=1024), dict(M=16, N=24, K=4096)):
+        with pytest.raises(_capi.AsterGemmError):
+            AG.GemmPlan.create(kw["M"], kw["N"], kw["K"], "bf16", "bf16", operand_path="direct_b")
