@@ -121,6 +121,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--no-others", action="store_true", help="skip the secondary shapes")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--results-jsonl", default=None,
+                    help="also append one BENCH_RESULT_JSON line per MFMA-bound workload to this "
+                         "file (input of `python -m aster_amd.perf_registry`)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on ONE GPU; --gpus N with N > 1 is not supported "
@@ -244,6 +247,20 @@ def main() -> int:
     else:
         out["cpu_baseline"] = None
 
+    if args.results_jsonl:
+        from aster_amd.perf_registry import RESULT_SENTINEL
+        recs = [("astergemm_bf16", 8192, 8192, 8192, plan.info.name.decode(), achieved)]
+        for o in out.get("others", []):
+            if o.get("bound") != "mfma":
+                continue
+            dt = o["workload"].split()[0]
+            m, n, k = (int(x) for x in o["workload"].split()[2].split("x"))
+            recs.append((f"astergemm_{dt}", m, n, k, o["kernel"], o["tflops"]))
+        with open(args.results_jsonl, "a") as f:
+            for bench, m, n, k, label, tf in recs:
+                f.write(RESULT_SENTINEL + json.dumps({"mcpu": "gfx950", "bench": bench, "M": m, "N": n,
+                                                       "K": k, "label": label, "tflops_median": tf,
+                                                       "sample_n": 1}) + "\n")
     print(json.dumps(out), flush=True)
     return 0
 
