@@ -151,13 +151,6 @@ __device__ __forceinline__ void gemm_stream4_body(const GemmArgs& p) {
     const uint8_t* s = lds + ((unsigned)(((k >> 1) & 1) * BM * 16 + (k & 1) * 8) + sb_rd);
     sb[N & 1] = *(const unsigned short*)(s + sc_rd + N * 16 * 16);
   };
-  auto read_a = [&](auto mm, const uint8_t* p0, const uint8_t* p1, const uint8_t* ps) {
-    constexpr int M = decltype(mm)::value;
-    fa_lo[M] = *(const i32x4*)(p0 + M * 16 * kRowBytes);
-    fa_hi[M] = *(const i32x4*)(p1 + M * 16 * kRowBytes);
-    sa[M] = *(const unsigned short*)(ps + M * 16 * 16);
-  };
-
   f32x4 acc[TM][TN];
 #pragma unroll
   for (int m = 0; m < TM; ++m)
@@ -203,7 +196,12 @@ __device__ __forceinline__ void gemm_stream4_body(const GemmArgs& p) {
   {
     const uint8_t* s = lds + a_rd;
     const uint8_t* ps = lds + sa_rd + sc_rd;
-    static_for<0, TM>([&](auto m) { read_a(m, s + rd0, s + rd1, ps); });
+    static_for<0, TM>([&](auto mc) {
+      constexpr int m = decltype(mc)::value;
+      fa_lo[m] = *(const i32x4*)(s + rd0 + m * 16 * kRowBytes);
+      fa_hi[m] = *(const i32x4*)(s + rd1 + m * 16 * kRowBytes);
+      sa[m] = *(const unsigned short*)(ps + m * 16 * 16);
+    });
   }
   __builtin_amdgcn_sched_barrier(0);
 

@@ -155,10 +155,6 @@ __device__ __forceinline__ void gemm_stream_body(const GemmArgs& p) {
   // 64 lanes x 16 bytes from (scalar base + per-lane offset) to LDS at M0 + lane*16.
   // Written as asm to keep the scalar-base form; vmcnt is tracked by hand.
   auto g2s = [&](const uint8_t* base, unsigned voff, uint8_t* dst) {
-#ifdef AG_DBG_BUILTIN_G2S
-    __builtin_amdgcn_global_load_lds(AG_GLOBAL(base + voff), AG_LDS(dst), 16, 0, 0);
-    return;
-#endif
     const unsigned m0v = (unsigned)(size_t)AG_LDS(dst);
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :
@@ -232,24 +228,11 @@ __device__ __forceinline__ void gemm_stream_body(const GemmArgs& p) {
   // C[m = lane % 16][4 consecutive n].
   auto mfmas = [&](auto sub) {
     constexpr int S = decltype(sub)::value;
-#ifdef AG_DBG_NO_MFMA
-#pragma unroll
-    for (int n = 0; n < TN; ++n) {
-      i32x4 t = fb[S][n];
-      asm volatile("" ::"v"(t));
-    }
-#pragma unroll
-    for (int m = 0; m < TM; ++m) {
-      i32x4 t = fa[S][m];
-      asm volatile("" ::"v"(t));
-    }
-#else
 #pragma unroll
     for (int n = 0; n < TN; ++n)
 #pragma unroll
       for (int m = 0; m < TM; ++m)
         acc[m][n] = mfma_step<DT>(&fb[S][n], &fa[S][m], acc[m][n], 0, 0);
-#endif
   };
   using S0 = std::integral_constant<int, 0>;
   using S1 = std::integral_constant<int, 1>;
@@ -302,33 +285,21 @@ __device__ __forceinline__ void gemm_stream_body(const GemmArgs& p) {
     static_for<0, NMF>([&](auto ic) {
       constexpr int I = decltype(ic)::value;
       constexpr int n = I / TM, m = I % TM;
-#ifndef AG_DBG_NO_MFMA
       acc[m][n] = mfma_step<DT>(&fb[1][n], &fa[1][m], acc[m][n], 0, 0);
-#endif
-#ifndef AG_DBG_NO_LOAD
       if constexpr (I < LH) {
         if (do_b) issue_b1(k + 2, (2 * KM) % NSLOT, I);
       }
-#endif
-#ifndef AG_DBG_NO_READ
       if constexpr (I >= LH && I < LH + NF) read_one(KN{}, S0{}, std::integral_constant<int, I - LH>{});
-#endif
       __builtin_amdgcn_sched_barrier(0);
     });
     static_for<0, NMF>([&](auto ic) {
       constexpr int I = decltype(ic)::value;
       constexpr int n = I / TM, m = I % TM;
-#ifndef AG_DBG_NO_MFMA
       acc[m][n] = mfma_step<DT>(&fb[0][n], &fa[0][m], acc[m][n], 0, 0);
-#endif
-#ifndef AG_DBG_NO_READ
       if constexpr (I < NF) read_one(KN{}, S1{}, std::integral_constant<int, I>{});
-#endif
-#ifndef AG_DBG_NO_LOAD
       if constexpr (I >= NF && I < NF + LH) {
         if (do_a) issue_a1(k + 3, (2 * KM + 1) % NSLOT, I - NF);
       }
-#endif
       __builtin_amdgcn_sched_barrier(0);
     });
   };

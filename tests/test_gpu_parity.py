@@ -532,3 +532,23 @@ def test_direct_b_is_refused_where_it_is_not_implemented(gpu):
     for kw in (dict(M=128, N=256, K=4096), dict(M=16, N=256, K=1024), dict(M=16, N=24, K=4096)):
         with pytest.raises(_capi.AsterGemmError):
             AG.GemmPlan.create(kw["M"], kw["N"], kw["K"], "bf16", "bf16", operand_path="direct_b")
+
+
+# ---- linalg.matmul-shaped caller (B given K x N) ------------------------------------------
+
+@pytest.mark.parametrize("M,N,K", [(32, 32, 32), (48, 200, 72), (512, 768, 256), (16, 1024, 2048)])
+def test_linalg_matmul_kxn(gpu, M, N, K):
+    # contrib/mlir-air/test/integration/test_linalg_matmul_e2e.py:52-75: seed 42, randn * 0.1,
+    # B given K x N, rtol = atol = 1e-2
+    from aster_amd.linalg import matmul
+    np.random.seed(42)
+    a = (np.random.randn(M, K) * 0.1).astype(np.float16)
+    b_kxn = (np.random.randn(K, N) * 0.1).astype(np.float16)
+    c = matmul(a, b_kxn)
+    expected = a.astype(np.float32) @ b_kxn.astype(np.float32)
+    np.testing.assert_allclose(c, expected, rtol=1e-2, atol=1e-2)
+    assert G.rel_l2(c, expected) <= 1e-5
+    with pytest.raises(ValueError):
+        matmul(a, b_kxn[:-1])
+    with pytest.raises(ValueError):
+        matmul(a.astype(np.float32), b_kxn)
