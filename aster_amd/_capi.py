@@ -97,6 +97,9 @@ SIGNATURES = {
     "astergemm_bench": (C.c_int, [C.POINTER(Config), C.POINTER(Operands), C.c_int,
                                   C.POINTER(C.c_int64), C.c_int64, _P]),
     "astergemm_shuffle_weight_16": (C.c_int, [_P, _P, C.c_int64, C.c_int64]),
+    "astergemm_absmax_f32": (C.c_int, [_P, C.c_int64, _P, _P]),
+    "astergemm_quantize_fp8_tensor": (C.c_int, [_P, C.c_int64, _P, _P, _P]),
+    "astergemm_quantize_mxfp4": (C.c_int, [_P, C.c_int64, C.c_int64, C.c_int64, _P, _P, _P]),
     "aster_rt_init": (C.c_int, []),
     "aster_rt_peek_at_last_error": (C.c_int, []),
     "aster_rt_clear_last_error": (C.c_int, []),

@@ -11,6 +11,8 @@
 //                    [--warmup 20] [--tile 256] [--family tile|skinny|auto]
 //                    [--variant ID] [--flush BYTES] [--bias] [--json] [--calib BYTES]
 //                    [--direct-b]   (B taken as pre-shuffled; timing only, the fill is random)
+//   astergemm_replay --quantize fp8|mxfp4 --m ROWS --k K --iters 100
+//                    (operand quantiser on a ROWS x K fp32 source instead of a GEMM)
 //
 // --calib BYTES first copies BYTES device-to-device three times: a copy kernel that
 // reads and writes a known number of bytes, against which the counters of a
@@ -80,6 +82,47 @@ static void fill(std::vector<uint8_t>& buf, int dtype, uint64_t seed) {
   }
 }
 
+
+// --quantize: time astergemm_quantize_fp8_tensor / astergemm_quantize_mxfp4 on a rows x K
+// fp32 source, one event pair per call on the null stream.
+static int run_quantize(const char* kind, long long rows, long long K, int iters, int warmup) {
+  CHECK(aster_rt_init());
+  const size_t n = (size_t)rows * (size_t)K;
+  std::vector<float> h(n);
+  uint64_t x = 88172645463325252ull;
+  for (size_t i = 0; i < n; ++i) {
+    x ^= x << 13, x ^= x >> 7, x ^= x << 17;
+    h[i] = (float)((double)(int64_t)x * (1.0 / 9223372036854775808.0));  // (-1, 1)
+  }
+  void *src, *dst, *sc, *e0, *e1;
+  CHECK(aster_rt_malloc(&src, n * 4));
+  CHECK(aster_rt_malloc(&dst, n));
+  CHECK(aster_rt_malloc(&sc, n / 32 + 256));
+  CHECK(aster_rt_memcpy_h2d(src, h.data(), n * 4));
+  CHECK(aster_rt_event_create(&e0));
+  CHECK(aster_rt_event_create(&e1));
+  const bool fp8 = !strcmp(kind, "fp8");
+  std::vector<double> us;
+  for (int i = 0; i < iters; ++i) {
+    CHECK(aster_rt_event_record(e0, nullptr));
+    if (fp8) CHECK(astergemm_quantize_fp8_tensor((const float*)src, (int64_t)n, (uint8_t*)dst, (float*)sc, nullptr));
+    else CHECK(astergemm_quantize_mxfp4((const float*)src, rows, K, 0, (uint8_t*)dst, (uint8_t*)sc, nullptr));
+    CHECK(aster_rt_event_record(e1, nullptr));
+    CHECK(aster_rt_event_synchronize(e1));
+    float ms = 0;
+    CHECK(aster_rt_event_elapsed_ms(e0, e1, &ms));
+    if (i >= warmup) us.push_back(ms * 1e3);
+  }
+  std::sort(us.begin(), us.end());
+  const double p50 = us[us.size() / 2];
+  // algorithmic bytes: fp8 reads the source twice (absmax, encode) and writes n bytes;
+  // mxfp4 reads it once and writes n/2 + n/32 bytes
+  const double bytes = fp8 ? (double)n * 9.0 : (double)n * (4.0 + 0.5 + 1.0 / 32.0);
+  printf("quantize_%s rows=%lld K=%lld  p50 %.2f us  %.1f GB/s (algorithmic bytes %.0f)\n", kind,
+         rows, K, p50, bytes / p50 * 1e-3, bytes);
+  return 0;
+}
+
 int main(int argc, char** argv) {
   astergemm_config cfg;
   memset(&cfg, 0, sizeof(cfg));
@@ -88,6 +131,7 @@ int main(int argc, char** argv) {
   cfg.dtype_c = ASTERGEMM_BF16;
   int iters = 100, warmup = 20, json = 0;
   long long flush = 0, calib = 0;
+  const char* quantize = nullptr;
   for (int i = 1; i < argc; ++i) {
     std::string a = argv[i];
     auto val = [&]() -> const char* {
@@ -111,6 +155,7 @@ int main(int argc, char** argv) {
     else if (a == "--direct-b") cfg.operand_path = ASTERGEMM_OPERAND_DIRECT_B;
     else if (a == "--bias") cfg.has_bias = 1;
     else if (a == "--json") json = 1;
+    else if (a == "--quantize") quantize = val();
     else if (a == "--family") {
       const char* f = val();
       cfg.family = !strcmp(f, "tile") ? ASTERGEMM_KERNEL_TILE
@@ -125,6 +170,13 @@ int main(int argc, char** argv) {
   if (iters <= warmup) {
     fprintf(stderr, "--iters must exceed --warmup\n");
     return 2;
+  }
+  if (quantize) {
+    if (strcmp(quantize, "fp8") && strcmp(quantize, "mxfp4")) {
+      fprintf(stderr, "--quantize fp8|mxfp4\n");
+      return 2;
+    }
+    return run_quantize(quantize, cfg.M, cfg.K, iters, warmup);
   }
 
   CHECK(aster_rt_init());

@@ -1,0 +1,267 @@
+// Operand quantisers for the fp8 and MXFP4 GEMM paths: fp32 -> OCP e4m3 with a per-tensor
+// absmax scale, and fp32 -> MXFP4 (e2m1 nibbles + one e8m0 byte per 32 elements).
+//
+// These produce, on the device, exactly the bytes the GEMM kernels consume (operand
+// layouts of astergemm_config: row-major, e2m1 low nibble first, scales [rows, K/32]).
+// The e4m3 rounding follows the converter the reference's tests hold
+// (f32_to_fp8_e4m3(val, fnuz=False), test/integration/test_conversion_pack_e2e.py:91-167:
+// bias 7, round to nearest even with carry into the exponent, saturation to 0x7E = 448,
+// NaN and infinities to S|0x7F, signed zero), with the subnormal range rounded to nearest
+// even as the hardware converter does.  The MX block format is the one the scaled MFMA
+// expects (v_mfma_scale_f32_16x16x128_f8f6f4, e8m0 scale per 32 K-elements).
+// Both are HBM-bound byte work: one pass over the source (two for the per-tensor scale).
+#include "astergemm_internal.h"
+
+namespace astergemm {
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+// Vector elements are passed by value (__float_as_uint) before their bits are taken: a bit
+// cast applied to the element expression itself read element 0 for every index.
+
+// fp32 -> e4m3 code, round to nearest even, saturating: |x| > 448 -> 0x7E, NaN / inf -> 0x7F.
+// Normal range (|x| >= 2^-6): round the fp32 bit pattern to 3 fraction bits in integer
+// arithmetic (a carry out of the fraction flows into the exponent) and re-bias 127 -> 7.
+// Below that the codes are multiples of 2^-9: adding 2^14 makes the fp32 adder round |x| to
+// that grid, ties to even, and leaves the code in the low bits of the sum.
+__device__ __forceinline__ unsigned e4m3_rne_sat(float x) {
+  const unsigned b = __float_as_uint(x);
+  const unsigned s = (b >> 24) & 0x80u;
+  const unsigned m = b & 0x7FFFFFFFu;
+  unsigned code;
+  if (m >= 0x3C800000u) {  // 2^-6
+    code = ((m + 0x7FFFFu + ((m >> 20) & 1u)) >> 20) - ((127u - 7u) << 3);
+    code = code > 0x7Eu ? 0x7Eu : code;
+    code = m >= 0x7F800000u ? 0x7Fu : code;
+  } else {
+    code = __float_as_uint(__uint_as_float(m) + 16384.0f) & 0xFu;
+  }
+  return s | code;
+}
+
+// fp32 -> e2m1 code (0..15): nearest value of {0, .5, 1, 1.5, 2, 3, 4, 6}, ties to the code
+// with an even index, saturation to 6, NaN -> S|7.  Same two tricks: one fraction bit kept
+// for |x| >= 1, the grid of 0.5 below (2^22 has an ulp of 0.5).
+__device__ __forceinline__ unsigned e2m1_rne_sat(float x) {
+  const unsigned b = __float_as_uint(x);
+  const unsigned s = (b >> 28) & 0x8u;
+  const unsigned m = b & 0x7FFFFFFFu;
+  unsigned code;
+  if (m >= 0x3F800000u) {  // 1.0
+    code = ((m + 0x1FFFFFu + ((m >> 22) & 1u)) >> 22) - ((127u - 1u) << 1);
+    code = code > 7u ? 7u : code;
+  } else {
+    code = __float_as_uint(__uint_as_float(m) + 4194304.0f) & 0x3u;
+  }
+  return s | code;
+}
+
+__global__ void zero_u32_kernel(unsigned* p) { *p = 0u; }
+
+// max over |x| as unsigned bits (non-negative floats order like their bit patterns; NaNs
+// compare above infinity and so survive the maximum, as they do in numpy's max).  Four
+// independent loads per trip; one atomic per workgroup.
+__global__ __launch_bounds__(256) void absmax_kernel(const float* __restrict__ src, int64_t n,
+                                                     unsigned* __restrict__ out) {
+  __shared__ unsigned wave_max[4];
+  unsigned m = 0;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  const int64_t n4 = n >> 2;
+  const f32x4* p = (const f32x4*)src;
+  int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+  auto fold = [&](const f32x4 v) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const unsigned b = __float_as_uint(v[e]) & 0x7FFFFFFFu;
+      m = b > m ? b : m;
+    }
+  };
+  for (; i + 3 * stride < n4; i += 4 * stride) {
+    const f32x4 v0 = __builtin_nontemporal_load(p + i);
+    const f32x4 v1 = __builtin_nontemporal_load(p + i + stride);
+    const f32x4 v2 = __builtin_nontemporal_load(p + i + 2 * stride);
+    const f32x4 v3 = __builtin_nontemporal_load(p + i + 3 * stride);
+    fold(v0), fold(v1), fold(v2), fold(v3);
+  }
+  for (; i < n4; i += stride) fold(__builtin_nontemporal_load(p + i));
+  for (int64_t j = (n4 << 2) + blockIdx.x * (int64_t)blockDim.x + threadIdx.x; j < n; j += stride) {
+    const unsigned b = __float_as_uint(src[j]) & 0x7FFFFFFFu;
+    m = b > m ? b : m;
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const unsigned o = (unsigned)__shfl_xor((int)m, off, 64);
+    m = o > m ? o : m;
+  }
+  if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = m;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < 4; ++w) m = wave_max[w] > m ? wave_max[w] : m;
+    if (m != 0) atomicMax(out, m);
+  }
+}
+
+// scale = absmax / 448 in fp32, 1.0 when absmax is zero (or NaN)
+__global__ void fp8_scale_kernel(const unsigned* amax_bits, float* scale) {
+  const float a = __builtin_bit_cast(float, *amax_bits);
+  *scale = (a > 0.0f) ? a / 448.0f : 1.0f;
+}
+
+__global__ __launch_bounds__(256) void quantize_fp8_kernel(const float* __restrict__ src, int64_t n,
+                                                           const float* __restrict__ scale,
+                                                           uint8_t* __restrict__ dst) {
+  const float s = *scale;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  const int64_t n4 = n >> 2;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n4; i += stride) {
+    const f32x4 v = __builtin_nontemporal_load((const f32x4*)src + i);
+    unsigned w = 0;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) w |= e4m3_rne_sat(v[e] / s) << (8 * e);
+    ((unsigned*)dst)[i] = w;
+  }
+  for (int64_t i = (n4 << 2) + blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += stride)
+    dst[i] = (uint8_t)e4m3_rne_sat(src[i] / s);
+}
+
+// Eight lanes per 32-element block: a lane loads 16 bytes (4 elements), so one wave-wide load
+// covers 1 KB of contiguous source (8 blocks); four such loads are in flight per trip.  The
+// block maximum goes round the 8 lanes with three exchanges; every lane then encodes its 4
+// elements (2 bytes out) and lane 0 of the group writes the scale byte.  CONTIG: ld == K, so
+// block t sits at element 32 t and no (row, column) split is needed.
+template <bool CONTIG>
+__global__ __launch_bounds__(256) void quantize_mxfp4_kernel(const float* __restrict__ src,
+                                                             int64_t nblocks, unsigned bpr,
+                                                             int64_t ld,
+                                                             uint8_t* __restrict__ packed,
+                                                             uint8_t* __restrict__ scales) {
+  constexpr int U = 4;
+  const int lane = threadIdx.x & 63, g = lane >> 3, l8 = lane & 7;
+  const int64_t nwaves = (int64_t)gridDim.x * 4;
+  for (int64_t base = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * (8 * U); base < nblocks;
+       base += nwaves * (8 * U)) {
+    f32x4 v[U];
+    int64_t t[U];
+    bool live[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      t[u] = base + u * 8 + g;
+      live[u] = t[u] < nblocks;
+      if (!live[u]) t[u] = nblocks - 1;  // stay inside the source; nothing is stored
+      int64_t off;
+      if (CONTIG) {
+        off = t[u] * 32;
+      } else {
+        const unsigned r = (unsigned)t[u] / bpr, c = (unsigned)t[u] - r * bpr;
+        off = (int64_t)r * ld + (int64_t)c * 32;
+      }
+      v[u] = __builtin_nontemporal_load((const f32x4*)(src + off) + l8);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      unsigned mb = 0;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const unsigned b = __float_as_uint(v[u][e]) & 0x7FFFFFFFu;
+        mb = b > mb ? b : mb;
+      }
+#pragma unroll
+      for (int off = 1; off < 8; off <<= 1) {
+        const unsigned o = (unsigned)__shfl_xor((int)mb, off, 64);
+        mb = o > mb ? o : mb;
+      }
+      // shared exponent = floor(log2(absmax)) - 2; an all-zero block gets exponent 0, a block
+      // holding NaN / inf gets scale byte 0xFF and its elements are scaled by 2^2
+      const bool bad = mb >= 0x7F800000u;
+      int fl;
+      if (mb == 0 || bad) fl = bad ? 0 : 2;                    // -> shared 0 (zero) / -2 (bad)
+      else if (mb >= 0x00800000u) fl = (int)(mb >> 23) - 127;  // normal
+      else fl = -149 + (31 - __builtin_clz(mb));               // fp32 subnormal
+      int sbyte = (fl - 2) + 127;
+      sbyte = sbyte < 0 ? 0 : (sbyte > 254 ? 254 : sbyte);
+      const int shift = -(sbyte - 127);
+      unsigned w = 0;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        // exact scaling by a power of two in two steps (|shift| can exceed the fp32 exponent
+        // range of a single factor)
+        const float q = ldexpf(ldexpf(v[u][e], shift / 2), shift - shift / 2);
+        w |= e2m1_rne_sat(q) << (4 * e);
+      }
+      if (live[u]) {
+        *(unsigned short*)(packed + t[u] * 16 + l8 * 2) = (unsigned short)w;
+        if (l8 == 0) scales[t[u]] = bad ? (uint8_t)0xFF : (uint8_t)sbyte;
+      }
+    }
+  }
+}
+
+// workgroups of 256 threads for `work_items` thread-items, at most 8 per compute unit
+int blocks_for(int64_t work_items) {
+  const int64_t b = (work_items + 255) / 256, cap = 256 * 8;
+  return (int)(b < 1 ? 1 : (b > cap ? cap : b));
+}
+
+}  // namespace
+}  // namespace astergemm
+
+using namespace astergemm;
+
+extern "C" int astergemm_absmax_f32(const float* dSrc, int64_t n, float* dAbsmax, void* stream) {
+  if ((!dSrc && n > 0) || !dAbsmax || n < 0 || (((uintptr_t)dSrc) & 15)) {
+    set_error("astergemm_absmax_f32: bad argument (dSrc must be 16-byte aligned)");
+    return ASTERGEMM_EINVAL;
+  }
+  hipStream_t s = (hipStream_t)stream;
+  hipLaunchKernelGGL(zero_u32_kernel, dim3(1), dim3(1), 0, s, (unsigned*)dAbsmax);
+  if (n > 0)
+    hipLaunchKernelGGL(absmax_kernel, dim3(blocks_for(n / 4 + 1)), dim3(256), 0, s, dSrc, n,
+                       (unsigned*)dAbsmax);
+  AG_HIP(hipGetLastError());
+  return 0;
+}
+
+extern "C" int astergemm_quantize_fp8_tensor(const float* dSrc, int64_t n, uint8_t* dDst,
+                                             float* dScale, void* stream) {
+  if ((!dSrc && n > 0) || (!dDst && n > 0) || !dScale || n < 0 || (((uintptr_t)dSrc) & 15) ||
+      (((uintptr_t)dDst) & 3)) {
+    set_error("astergemm_quantize_fp8_tensor: bad argument (dSrc 16-byte, dDst 4-byte aligned)");
+    return ASTERGEMM_EINVAL;
+  }
+  hipStream_t s = (hipStream_t)stream;
+  // dScale doubles as the absmax accumulator: bits of a non-negative float
+  if (int rc = astergemm_absmax_f32(dSrc, n, dScale, stream)) return rc;
+  hipLaunchKernelGGL(fp8_scale_kernel, dim3(1), dim3(1), 0, s, (const unsigned*)dScale, dScale);
+  if (n > 0)
+    hipLaunchKernelGGL(quantize_fp8_kernel, dim3(blocks_for(n / 4 + 1)), dim3(256), 0, s, dSrc, n,
+                       dScale, dDst);
+  AG_HIP(hipGetLastError());
+  return 0;
+}
+
+extern "C" int astergemm_quantize_mxfp4(const float* dSrc, int64_t rows, int64_t K, int64_t ld_src,
+                                        uint8_t* dPacked, uint8_t* dScales, void* stream) {
+  if (ld_src == 0) ld_src = K;
+  if (rows < 0 || K < 0 || K % 32 != 0 || ld_src < K || ld_src % 4 != 0 ||
+      ((rows > 0 && K > 0) && (!dSrc || !dPacked || !dScales)) || (((uintptr_t)dSrc) & 15) ||
+      (((uintptr_t)dPacked) & 15)) {
+    set_error("astergemm_quantize_mxfp4: need K %% 32 == 0, ld_src >= K, ld_src %% 4 == 0, "
+              "dSrc and dPacked 16-byte aligned");
+    return ASTERGEMM_EINVAL;
+  }
+  if (rows == 0 || K == 0) return 0;
+  const int64_t nblocks = rows * (K / 32);
+  if (nblocks >= (int64_t)1 << 31) {
+    set_error("astergemm_quantize_mxfp4: more than 2^31 blocks");
+    return ASTERGEMM_EINVAL;
+  }
+  const dim3 grid(blocks_for(nblocks * 2));  // a workgroup takes 128 blocks per trip
+  if (ld_src == K)
+    hipLaunchKernelGGL(quantize_mxfp4_kernel<true>, grid, dim3(256), 0, (hipStream_t)stream, dSrc,
+                       nblocks, (unsigned)(K / 32), ld_src, dPacked, dScales);
+  else
+    hipLaunchKernelGGL(quantize_mxfp4_kernel<false>, grid, dim3(256), 0, (hipStream_t)stream, dSrc,
+                       nblocks, (unsigned)(K / 32), ld_src, dPacked, dScales);
+  AG_HIP(hipGetLastError());
+  return 0;
+}

@@ -1,0 +1,71 @@
+"""Operand quantisers on the device: fp32 -> e4m3 with a per-tensor scale, fp32 -> MXFP4.
+
+They write the bytes the fp8 and MXFP4 GEMM kernels read.  The e4m3 rounding is the one of
+the converter the reference's tests hold (f32_to_fp8_e4m3(val, fnuz=False),
+test/integration/test_conversion_pack_e2e.py:91-167); the MXFP4 block layout is the operand
+layout of v_mfma_scale_f32_16x16x128_f8f6f4 (include/aster/Dialect/AMDGCN/IR/Instructions/
+MMA.td:792).  `*_device` functions work on device pointers the caller owns; the array
+functions upload, quantise on the GPU and download with synchronous copies (tests, one-off
+conversions).  There is no
+CPU path.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional, Tuple
+
+import numpy as np
+
+from . import _capi
+from .execution import GpuBuffer
+
+
+def _s(stream):
+    return ctypes.c_void_p(stream) if stream else None
+
+
+def absmax_f32_device(d_src: int, n: int, d_absmax: int, stream: Optional[int] = None) -> None:
+    _capi.check(_capi.load().astergemm_absmax_f32(ctypes.c_void_p(d_src), n,
+                                                  ctypes.c_void_p(d_absmax), _s(stream)))
+
+
+def quantize_fp8_tensor_device(d_src: int, n: int, d_dst: int, d_scale: int,
+                               stream: Optional[int] = None) -> None:
+    """d_dst[i] = e4m3(d_src[i] / scale), *d_scale = scale = absmax / 448 (1.0 for absmax 0)."""
+    _capi.check(_capi.load().astergemm_quantize_fp8_tensor(
+        ctypes.c_void_p(d_src), n, ctypes.c_void_p(d_dst), ctypes.c_void_p(d_scale), _s(stream)))
+
+
+def quantize_mxfp4_device(d_src: int, rows: int, K: int, d_packed: int, d_scales: int, *,
+                          ld_src: int = 0, stream: Optional[int] = None) -> None:
+    """rows x K fp32 -> packed e2m1 [rows, K/2] and e8m0 scale bytes [rows, K/32]."""
+    _capi.check(_capi.load().astergemm_quantize_mxfp4(
+        ctypes.c_void_p(d_src), rows, K, ld_src, ctypes.c_void_p(d_packed),
+        ctypes.c_void_p(d_scales), _s(stream)))
+
+
+def quantize_fp8_tensor(x: np.ndarray) -> Tuple[np.ndarray, np.float32]:
+    """Array version: (e4m3 bytes of x's shape, fp32 scale)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    src, dst, sc = GpuBuffer(x.nbytes), GpuBuffer(x.size), GpuBuffer(4)
+    src.copy_from_host(x)
+    quantize_fp8_tensor_device(src.ptr_value, x.size, dst.ptr_value, sc.ptr_value)
+    q, s = np.empty(x.shape, np.uint8), np.empty(1, np.float32)
+    dst.copy_to_host(q)
+    sc.copy_to_host(s)
+    return q, s[0]
+
+
+def quantize_mxfp4(x: np.ndarray) -> Tuple[np.ndarray, np.ndarray]:
+    """Array version: x[rows, K] -> (packed [rows, K/2] uint8, scales [rows, K/32] uint8)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    if x.ndim != 2 or x.shape[1] % 32:
+        raise ValueError("quantize_mxfp4 needs a [rows, K] array with K % 32 == 0")
+    rows, K = x.shape
+    src, pk, sc = GpuBuffer(x.nbytes), GpuBuffer(rows * K // 2), GpuBuffer(rows * K // 32)
+    src.copy_from_host(x)
+    quantize_mxfp4_device(src.ptr_value, rows, K, pk.ptr_value, sc.ptr_value)
+    packed, scales = np.empty((rows, K // 2), np.uint8), np.empty((rows, K // 32), np.uint8)
+    pk.copy_to_host(packed)
+    sc.copy_to_host(scales)
+    return packed, scales

@@ -191,6 +191,38 @@ int astergemm_bench_rotate(const astergemm_config* cfg, const astergemm_operands
 int astergemm_shuffle_weight_16(const uint16_t* src, uint16_t* dst, int64_t N,
                                 int64_t K);
 
+/* ---- operand quantisers (device to device, on `stream`) -------------------
+ * They write the bytes the fp8 / MXFP4 GEMM paths read (dtype_ab
+ * ASTERGEMM_FP8_E4M3 / ASTERGEMM_MXFP4), so that a caller holding fp32
+ * activations or weights in HBM needs no host round trip.
+ *
+ * astergemm_absmax_f32: *dAbsmax = max |dSrc[i]| (0 for n == 0; NaN if any
+ * element is NaN).  dSrc 16-byte aligned.
+ *
+ * astergemm_quantize_fp8_tensor: *dScale = absmax / 448 (1.0 when absmax is
+ * zero), dDst[i] = e4m3(dSrc[i] / *dScale) with the rounding of the converter
+ * the reference's tests hold (f32_to_fp8_e4m3, fnuz=False:
+ * test/integration/test_conversion_pack_e2e.py:91-167): nearest even, carry
+ * into the exponent, saturation to 448 = 0x7E, NaN / inf -> S|0x7F, signed
+ * zero; the subnormal range rounds to nearest even.  *dScale is what
+ * astergemm_operands.dScaleA / dScaleB take.  dDst 4-byte aligned.
+ *
+ * astergemm_quantize_mxfp4: rows x K fp32 (row stride ld_src elements, 0 =
+ * K) -> dPacked[rows, K/2] (element 2j in the low nibble of byte j) and
+ * dScales[rows, K/32] e8m0 bytes, the operand layout of the scaled MFMA
+ * (v_mfma_scale_f32_16x16x128_f8f6f4; reference instruction definition
+ * include/aster/Dialect/AMDGCN/IR/Instructions/MMA.td:792).  Per 32-element block: scale
+ * exponent floor(log2(absmax)) - 2 clamped to [-127, 127] (0 for an all-zero
+ * block), elements e2m1 round-to-nearest-even of x / 2^exponent saturated to
+ * +-6; a block holding NaN or inf gets scale byte 0xFF.  K % 32 == 0,
+ * ld_src % 4 == 0, dSrc and dPacked 16-byte aligned.                        */
+int astergemm_absmax_f32(const float* dSrc, int64_t n, float* dAbsmax, void* stream);
+int astergemm_quantize_fp8_tensor(const float* dSrc, int64_t n, uint8_t* dDst,
+                                  float* dScale, void* stream);
+int astergemm_quantize_mxfp4(const float* dSrc, int64_t rows, int64_t K,
+                             int64_t ld_src, uint8_t* dPacked, uint8_t* dScales,
+                             void* stream);
+
 /* ---- runtime seam: 1:1 with RuntimeModule.cpp:140-418 -------------------- */
 int aster_rt_init(void);
 int aster_rt_peek_at_last_error(void);
