@@ -22,6 +22,7 @@ namespace {
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 typedef int i32x2 __attribute__((ext_vector_type(2)));
+typedef int i32x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef unsigned short u16x4 __attribute__((ext_vector_type(4)));
@@ -337,9 +338,22 @@ __global__ __launch_bounds__(512) void gemm_skinny_reg_kernel(const GemmArgs p) 
   // T = unit index inside the block (compile time: selects the x registers)
   auto mma = [&](int blk, auto T) {
     constexpr int t = decltype(T)::value;
+    if constexpr (DT == ASTERGEMM_FP8_E4M3) {
+      // one 16x16x128 MFMA per 128-byte step: a lane's 32 operand bytes are pieces lq and
+      // 4 + lq of the row, for the weights and the activations alike
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      acc = sk_mfma<DT>(operand(i >> 1, i & 1), x[t * 8 + i], acc);
+      for (int s = 0; s < 4; ++s) {
+        const i32x4 lo = operand(s, 0), hi = operand(s, 1);
+        const i32x4 xl = x[t * 8 + 2 * s], xh = x[t * 8 + 2 * s + 1];
+        acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+            i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]},
+            i32x8{xl[0], xl[1], xl[2], xl[3], xh[0], xh[1], xh[2], xh[3]}, acc, 0, 0, 0, 0, 0, 0);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        acc = sk_mfma<DT>(operand(i >> 1, i & 1), x[t * 8 + i], acc);
+      }
     }
     if (t == UPB - 1) block_end(blk);
   };
@@ -399,18 +413,21 @@ int launch_skinny_reg_t(const GemmArgs& a, hipStream_t s) {
 template <int DT, int OUT>
 int launch_skinny_reg(const GemmArgs& a, int grid, hipStream_t s) {
   (void)grid;
-  switch (a.K) {
-    case 2048: return launch_skinny_reg_t<DT, OUT, 4>(a, s);
-    case 4096: return launch_skinny_reg_t<DT, OUT, 8>(a, s);
-    case 8192: return launch_skinny_reg_t<DT, OUT, 16>(a, s);
+  switch (row_bytes(DT, a.K)) {  // eight waves x SPB steps of 128 bytes
+    case 4096: return launch_skinny_reg_t<DT, OUT, 4>(a, s);
+    case 8192: return launch_skinny_reg_t<DT, OUT, 8>(a, s);
+    case 16384: return launch_skinny_reg_t<DT, OUT, 16>(a, s);
   }
   return (int)hipErrorInvalidValue;
 }
 
 const char* check_skinny_reg(const astergemm_config& c) {
   if (c.M > 16) return "resident-activation path needs M <= 16";
-  if (c.K != 2048 && c.K != 4096 && c.K != 8192)
-    return "resident-activation path needs K = 2048, 4096 or 8192";
+  const int64_t rb = row_bytes(c.dtype_ab, c.K);
+  if (rb != 4096 && rb != 8192 && rb != 16384)
+    return c.dtype_ab == ASTERGEMM_FP8_E4M3
+               ? "resident-activation path needs K = 4096, 8192 or 16384 for fp8"
+               : "resident-activation path needs K = 2048, 4096 or 8192";
   return nullptr;
 }
 
@@ -702,6 +719,9 @@ const Variant kSkinnyVariants[] = {
     AG_SKINNY_LDS("skinnyx_f16_m16_bf16", ASTERGEMM_F16, ASTERGEMM_BF16),
     AG_SKINNY_LDS("skinnyx_f16_m16_f32", ASTERGEMM_F16, ASTERGEMM_F32),
     AG_SKINNY_LDS("skinnyx_f16_m16_f16", ASTERGEMM_F16, ASTERGEMM_F16),
+    AG_SKINNY_LDS("skinnyx_fp8_m16_bf16", ASTERGEMM_FP8_E4M3, ASTERGEMM_BF16),
+    AG_SKINNY_LDS("skinnyx_fp8_m16_f32", ASTERGEMM_FP8_E4M3, ASTERGEMM_F32),
+    AG_SKINNY_LDS("skinnyx_fp8_m16_f16", ASTERGEMM_FP8_E4M3, ASTERGEMM_F16),
     AG_SKINNY_DIRECT("skinnyd_bf16_m16_bf16", ASTERGEMM_BF16, ASTERGEMM_BF16),
     AG_SKINNY_DIRECT("skinnyd_bf16_m16_f32", ASTERGEMM_BF16, ASTERGEMM_F32),
     AG_SKINNY_DIRECT("skinnyd_bf16_m16_f16", ASTERGEMM_BF16, ASTERGEMM_F16),

@@ -114,6 +114,53 @@ def cpu_baseline(M, N, K, budget_s=12.0):
                       f"B ({N}x{K}), {t:.2f} s, BLAS threads={cores}"}
 
 
+def vendor_library(torch, dev, iters=100, drop=20):
+    """The vendor's GEMM (torch.matmul / torch._scaled_mm, which call hipBLASLt) on the headline
+    shapes with the same timing protocol (one event pair per launch, p50 after dropping the
+    first launches).  Reported beside the build's own numbers as the practical ceiling of the
+    box; nothing in the product path uses it."""
+    rows = []
+
+    def timed(fn):
+        for _ in range(drop):
+            fn()
+        torch.cuda.synchronize()
+        ts = []
+        for _ in range(iters - drop):
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s.record()
+            fn()
+            e.record()
+            e.synchronize()
+            ts.append(s.elapsed_time(e) * 1e3)
+        ts.sort()
+        return _percentile(ts, 50)
+
+    g = torch.Generator(device=dev).manual_seed(42)
+    for (m, n, k, dt) in ((8192, 8192, 8192, "bf16"), (8192, 8192, 8192, "fp8_e4m3"),
+                          (16, 14336, 4096, "bf16")):
+        try:
+            a = torch.randn(m, k, device=dev, generator=g)
+            b = torch.randn(n, k, device=dev, generator=g) * 0.02
+            if dt == "bf16":
+                a, b = a.bfloat16(), b.bfloat16()
+                us = timed(lambda: torch.matmul(a, b.t()))
+            else:
+                one = torch.ones((), device=dev)
+                a, b = a.to(torch.float8_e4m3fn), b.to(torch.float8_e4m3fn)
+                us = timed(lambda: torch._scaled_mm(a, b.t(), scale_a=one, scale_b=one,
+                                                    out_dtype=torch.bfloat16))
+            row = {"workload": f"{dt} GEMM {m}x{n}x{k} -> bf16", "library": "hipBLASLt via torch",
+                   "p50_us": round(us, 2), "tflops": round(2.0 * m * n * k / us * 1e-6, 1)}
+            if m <= 64:
+                row["gbps"] = round((n * k * 2 + m * k * 2 + m * n * 2) / us * 1e-3, 1)
+            rows.append(row)
+            del a, b
+        except Exception as exc:  # a missing library kernel is not this build's failure
+            rows.append({"workload": f"{dt} GEMM {m}x{n}x{k} -> bf16", "error": repr(exc)[:200]})
+    return rows
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -121,6 +168,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--no-others", action="store_true", help="skip the secondary shapes")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-vendor", action="store_true",
+                    help="skip timing the vendor library (hipBLASLt through torch) on the same shapes")
     ap.add_argument("--results-jsonl", default=None,
                     help="also append one BENCH_RESULT_JSON line per MFMA-bound workload to this "
                          "file (input of `python -m aster_amd.perf_registry`)")
@@ -241,6 +290,10 @@ def main() -> int:
                        "gbps_back_to_back": round(p.info.bytes / rot_ns, 1),
                        "frac_back_to_back": round(p.info.bytes / rot_ns / PEAK_HBM_GBPS, 4)})
         out["others"] = others
+
+    if not args.no_vendor:
+        del a, b, c
+        out["vendor_library"] = vendor_library(torch, dev)
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(M, N, K)

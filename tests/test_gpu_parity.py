@@ -239,6 +239,48 @@ def test_skinny_resident_activations(gpu, M, N, K, dtype_ab, dtype_c):
     assert np.isnan(pad).all() if dtype_c == "f32" else (pad == 0x7FC1).all()
 
 
+@pytest.mark.parametrize("M,N,K", [(16, 14336, 4096), (1, 8, 4096), (5, 777, 8192), (16, 24, 16384),
+                                   (13, 6000, 4096), (16, 14337, 8192)])
+@pytest.mark.parametrize("dtype_c", ["bf16", "f32", "f16"])
+def test_skinny_fp8_resident_activations(gpu, M, N, K, dtype_c):
+    """fp8 weights through the same persistent kernel (one 16x16x128 MFMA per 128-byte step);
+    the result equals the tile kernel's up to fp32 summation order."""
+    a, b, extra = operands(M, N, K, "fp8_e4m3", seed=31, b_std=0.05)
+    bias = np.random.default_rng(32).standard_normal(N).astype(np.float32)
+    ldc = (N + 11) & ~3
+    out, name = run_gemm(a, b, M, N, K, "fp8_e4m3", dtype_c, bias=bias, ldc=ldc, **extra)
+    assert name.startswith("skinnyx_fp8")
+    want = G.gemm_fp8(a, b, extra["scale_a"], extra["scale_b"], out_dtype=_DT[dtype_c], bias=bias)
+    if dtype_c == "f32" or M * N >= 4096:
+        check(out, want, dtype_c, N, bar=1e-4 if dtype_c == "f32" else REL_L2_BAR)
+    else:
+        # few outputs: a handful of flipped roundings decide rel-L2, so bound every element by
+        # two units in the last place of the 16-bit output (under 1 % above one unit) plus the
+        # summation noise of the fp8 MFMA, which matters where the bias cancels the sum
+        got, ref = G.output_to_f32(out[:, :N], _DT[dtype_c]), G.output_to_f32(want, _DT[dtype_c])
+        ulp = 2.0 ** -7 if dtype_c == "bf16" else 2.0 ** -10
+        err = np.abs(got - ref)
+        assert np.all(err <= 2 * ulp * np.abs(ref) + 1e-4 * np.abs(ref).max())
+        assert np.mean(err > ulp * np.abs(ref) + 1e-4 * np.abs(ref).max()) < 0.01
+    pad = out[:, N:]
+    assert np.isnan(pad).all() if dtype_c == "f32" else (pad == 0x7FC1).all()
+    if dtype_c == "f32":
+        tile, tname = run_gemm(a, b, M, N, K, "fp8_e4m3", "f32", bias=bias, family=_capi.KERNEL_TILE,
+                               **extra)
+        assert tname.startswith("tile")
+        assert G.rel_l2(out[:, :N], tile) <= 1e-5
+
+
+def test_skinny_fp8_falls_back_to_tile_kernels(gpu):
+    # K outside the resident kernel's set, or M > 16: AUTO keeps the tile family
+    for (M, N, K) in ((16, 256, 1024), (17, 256, 4096)):
+        a, b, extra = operands(M, N, K, "fp8_e4m3", seed=33)
+        out, name = run_gemm(a, b, M, N, K, "fp8_e4m3", "f32", **extra)
+        assert name.startswith("tile")
+        check(out, G.gemm_fp8(a, b, extra["scale_a"], extra["scale_b"], out_dtype=G.F32), "f32", N,
+              bar=1e-4)
+
+
 # ---- edge cases: ragged M / N, K tails, leading dimensions, epilogue -----------------
 
 @pytest.mark.parametrize("M,N,K", [(1, 1, 8), (65, 16, 8), (130, 257, 72), (300, 520, 776), (129, 1, 64)])
