@@ -83,6 +83,21 @@ class DeviceProps(C.Structure):
     ]
 
 
+class WeightHeader(C.Structure):
+    """astergemm_weight_header: the 128-byte header of a weight artefact file."""
+    _fields_ = [
+        ("magic", C.c_char * 8),
+        ("version", C.c_uint32), ("header_bytes", C.c_uint32),
+        ("dtype", C.c_uint32), ("layout", C.c_uint32), ("scale_mode", C.c_uint32),
+        ("tensor_scale", C.c_float),
+        ("N", C.c_int64), ("K", C.c_int64),
+        ("payload_offset", C.c_int64), ("payload_bytes", C.c_int64),
+        ("scales_offset", C.c_int64), ("scales_bytes", C.c_int64),
+        ("payload_crc32", C.c_uint32), ("scales_crc32", C.c_uint32),
+        ("reserved", C.c_uint8 * 40),
+    ]
+
+
 # name -> (restype, argtypes); every symbol include/astergemm.h declares.
 _P = C.c_void_p
 SIGNATURES = {
@@ -97,6 +112,13 @@ SIGNATURES = {
     "astergemm_bench": (C.c_int, [C.POINTER(Config), C.POINTER(Operands), C.c_int,
                                   C.POINTER(C.c_int64), C.c_int64, _P]),
     "astergemm_shuffle_weight_16": (C.c_int, [_P, _P, C.c_int64, C.c_int64]),
+    "astergemm_weight_crc32": (C.c_uint32, [_P, C.c_size_t]),
+    "astergemm_weight_header_init": (C.c_int, [C.POINTER(WeightHeader), C.c_int, C.c_int, C.c_int64,
+                                               C.c_int64, C.c_float]),
+    "astergemm_weight_header_check": (C.c_int, [_P, C.c_size_t, C.POINTER(WeightHeader)]),
+    "astergemm_weight_verify": (C.c_int, [_P, C.c_size_t]),
+    "astergemm_weight_config": (C.c_int, [C.POINTER(WeightHeader), C.c_int64, C.c_int,
+                                          C.POINTER(Config)]),
     "astergemm_absmax_f32": (C.c_int, [_P, C.c_int64, _P, _P]),
     "astergemm_quantize_fp8_tensor": (C.c_int, [_P, C.c_int64, _P, _P, _P]),
     "astergemm_quantize_mxfp4": (C.c_int, [_P, C.c_int64, C.c_int64, C.c_int64, _P, _P, _P]),

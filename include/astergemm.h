@@ -223,6 +223,52 @@ int astergemm_quantize_mxfp4(const float* dSrc, int64_t rows, int64_t K,
                              int64_t ld_src, uint8_t* dPacked, uint8_t* dScales,
                              void* stream);
 
+/* ---- weight artefact files (host side) -------------------------------------
+ * A weight matrix B[N, K] on disk in the bytes the kernels stream, so that
+ * loading is one read + one upload: no conversion, no permutation.  The
+ * reference has no file format for this: its execute_fn pre-shuffles B with
+ * shuffle_weight on every call
+ * (contrib/kittens/test/test_102_gemm_python_multitile_g2s_directb_cdna4.py:440-467,
+ * contrib/kittens/test/kittens_helpers.py:90-119) and its fp8 tests convert on
+ * the host each time (test/integration/test_conversion_pack_e2e.py:91-167).
+ *
+ * File = this 128-byte little-endian header, then the payload at
+ * payload_offset (N rows; layout ASTERGEMM_OPERAND_LDS = row-major,
+ * ASTERGEMM_OPERAND_DIRECT_B = astergemm_shuffle_weight_16 order, 16-bit
+ * dtypes only), then for MXFP4 the e8m0 plane [N, K/32] at scales_offset.
+ * Sections start on 256-byte boundaries.  FP8 carries its tensor scale in the
+ * header.  Checksums are CRC-32 (the zlib polynomial) of each section.       */
+#define ASTERGEMM_WEIGHT_VERSION 1u
+typedef struct astergemm_weight_header {
+  char magic[8];           /* "ASTGEMW\0"                                   */
+  uint32_t version;        /* ASTERGEMM_WEIGHT_VERSION                      */
+  uint32_t header_bytes;   /* 128                                           */
+  uint32_t dtype;          /* astergemm_dtype of the stored elements        */
+  uint32_t layout;         /* astergemm_operand_path                        */
+  uint32_t scale_mode;     /* astergemm_scale_mode implied by dtype         */
+  float tensor_scale;      /* FP8: the per-tensor scale; else 1.0           */
+  int64_t N, K;
+  int64_t payload_offset, payload_bytes;
+  int64_t scales_offset, scales_bytes; /* 0, 0 unless MXFP4                 */
+  uint32_t payload_crc32, scales_crc32;
+  uint8_t reserved[40];
+} astergemm_weight_header;
+
+uint32_t astergemm_weight_crc32(const void* data, size_t bytes);
+/* Fills a header (offsets, sizes, scale mode) for the given matrix; the
+ * caller writes the sections and their checksums. */
+int astergemm_weight_header_init(astergemm_weight_header* h, int dtype, int layout,
+                                 int64_t N, int64_t K, float tensor_scale);
+/* Validates the header of a file image (magic, version, sizes against N, K
+ * and dtype, sections inside the file) and copies it to *out. */
+int astergemm_weight_header_check(const void* file, size_t file_bytes,
+                                  astergemm_weight_header* out);
+/* header_check + both checksums over the whole file image. */
+int astergemm_weight_verify(const void* file, size_t file_bytes);
+/* The astergemm_config for C[M, N] = A[M, K] * B^T with this weight. */
+int astergemm_weight_config(const astergemm_weight_header* h, int64_t M, int dtype_c,
+                            astergemm_config* cfg);
+
 /* ---- runtime seam: 1:1 with RuntimeModule.cpp:140-418 -------------------- */
 int aster_rt_init(void);
 int aster_rt_peek_at_last_error(void);
