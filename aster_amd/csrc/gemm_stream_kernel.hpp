@@ -51,6 +51,21 @@ __device__ __forceinline__ void static_for(Fn&& f) {
 // 32-byte pieces per row, which costs ~7 % of the kernel.)  The lane id is
 // recomputed here, opaque to the optimiser, so that no lane-derived value has to
 // stay in a VGPR across the K loop.
+// Scalar bases of a wave's LH row groups (8 rows each, 8 * NW rows apart) for the global->LDS
+// transfers.  Operand heights are multiples of 8, so a group lies either inside the matrix or
+// wholly past its end; the latter re-read the last 8 rows (their products land in output rows
+// or columns the epilogue does not store).
+template <int LH, int NW>
+__device__ __forceinline__ void group_bases(const uint8_t* mat, int64_t ld_bytes, int first_row,
+                                            int rows, const uint8_t* (&out)[LH]) {
+#pragma unroll
+  for (int j = 0; j < LH; ++j) {
+    int r = first_row + j * 8 * NW;
+    r = r < rows - 8 ? r : rows - 8;
+    out[j] = mat + (int64_t)r * ld_bytes;
+  }
+}
+
 template <int OUT, int BM, int BN, int WM, int WN>
 __device__ __forceinline__ void stream_epilogue(const GemmArgs& p,
                                                 f32x4 (&acc)[BM / WM / 16][BN / WN / 16],
@@ -86,7 +101,11 @@ __device__ __forceinline__ void stream_epilogue(const GemmArgs& p,
   for (int n = 0; n < TN; ++n)
 #pragma unroll
     for (int e = 0; e < 4; ++e)
-      bias_v[n][e] = p.bias ? p.bias[wcol0 + n * 16 + 4 * lq_e + e] : 0.f;
+    {
+      int col = wcol0 + n * 16 + 4 * lq_e + e;
+      col = col < p.N ? col : p.N - 1;
+      bias_v[n][e] = p.bias ? p.bias[col] : 0.f;
+    }
 #pragma unroll
   for (int m = 0; m < TM; ++m) {
     uint8_t* slab = stage + (m & 1) * SLAB;
@@ -109,7 +128,8 @@ __device__ __forceinline__ void stream_epilogue(const GemmArgs& p,
       const int r = c / (ROWB / 16), cc = c % (ROWB / 16);
       const i32x4 d = *(const i32x4*)(slab + r * PITCH + cc * 16);
       uint8_t* out = (uint8_t*)p.C + ((int64_t)(wrow0 + m * 16 + r) * p.ldc + wcol0) * OB + cc * 16;
-      *(i32x4*)out = d;
+      // edge tiles: N is a multiple of 8, so a 16-byte chunk is inside a row or past its end
+      if (wrow0 + m * 16 + r < p.M && wcol0 + cc * (16 / OB) < p.N) *(i32x4*)out = d;
     }
   }
 }
@@ -146,10 +166,10 @@ __device__ __forceinline__ void gemm_stream_body(const GemmArgs& p) {
   const int g_lane = (lane & 7) ^ (((wave * 8 + lrow) >> 1) & 7);
   const unsigned a_off = (unsigned)(lrow * (int)p.lda_bytes + g_lane * 16);
   const unsigned b_off = (unsigned)(lrow * (int)p.ldb_bytes + g_lane * 16);
-  const uint8_t* a_base = p.A + ((int64_t)row0 + wave * 8) * p.lda_bytes;
-  const uint8_t* b_base = p.B + ((int64_t)col0 + wave * 8) * p.ldb_bytes;
-  const int64_t a_jstride = (int64_t)8 * NW * p.lda_bytes;
-  const int64_t b_jstride = (int64_t)8 * NW * p.ldb_bytes;
+  const uint8_t* a_base[LH];
+  const uint8_t* b_base[LH];
+  group_bases<LH, NW>(p.A, p.lda_bytes, row0 + wave * 8, p.M, a_base);
+  group_bases<LH, NW>(p.B, p.ldb_bytes, col0 + wave * 8, p.N, b_base);
   const int nk = p.ksteps;
 
   // 64 lanes x 16 bytes from (scalar base + per-lane offset) to LDS at M0 + lane*16.
@@ -163,11 +183,11 @@ __device__ __forceinline__ void gemm_stream_body(const GemmArgs& p) {
   };
   // transfer j (0..LH-1) of this wave for the A / B half of K-step k
   auto issue_a1 = [&](int k, int slot, int j) {
-    g2s(a_base + (int64_t)k * kRowBytes + j * a_jstride, a_off,
+    g2s(a_base[j] + (int64_t)k * kRowBytes, a_off,
         lds + slot * SLOT + (j * NW + wave) * 8 * kRowBytes);
   };
   auto issue_b1 = [&](int k, int slot, int j) {
-    g2s(b_base + (int64_t)k * kRowBytes + j * b_jstride, b_off,
+    g2s(b_base[j] + (int64_t)k * kRowBytes, b_off,
         lds + slot * SLOT + (j * NW + wave) * 8 * kRowBytes);
   };
   auto issue_a = [&](int k, int slot) {

@@ -102,7 +102,8 @@ int launch_stream(const GemmArgs& a, int grid, hipStream_t s) {
 // Whole 256x256 tiles and whole 128-byte K-steps only; other shapes go to the
 // general tile kernel.
 const char* check_stream(const astergemm_config& c) {
-  if (c.M % 256 != 0 || c.N % 256 != 0) return "M and N must be multiples of 256";
+  // edge tiles are handled in units of 8 operand rows and 16-byte output chunks
+  if (c.M % 8 != 0 || c.N % 8 != 0 || c.M < 8 || c.N < 8) return "M and N must be multiples of 8";
   if (row_bytes(c.dtype_ab, c.K) % kRowBytes != 0) return "K must fill whole 128-byte row chunks";
   if (c.ldc % 8 != 0) return "ldc must be a multiple of 8 elements";
   return nullptr;
@@ -161,6 +162,7 @@ int launch_stream4(const GemmArgs& a, int grid, hipStream_t s) {
 // granules = two K-steps of a row).
 const char* check_stream4(const astergemm_config& c) {
   if (const char* why = check_stream(c)) return why;
+  if (c.M % 256 != 0 || c.N % 256 != 0) return "M and N must be multiples of 256";
   if (c.K % 512 != 0) return "K must be a multiple of 512";
   return nullptr;
 }

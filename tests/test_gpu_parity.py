@@ -281,6 +281,35 @@ def test_skinny_fp8_falls_back_to_tile_kernels(gpu):
               bar=1e-4)
 
 
+@pytest.mark.parametrize("M,N,K", [(8, 8, 64), (264, 520, 128), (504, 1000, 192), (1000, 264, 1024),
+                                   (2056, 1800, 256), (256, 776, 320)])
+@pytest.mark.parametrize("dtype_ab,dtype_c", [("bf16", "bf16"), ("f16", "f32"), ("fp8_e4m3", "bf16"),
+                                              ("fp8_e4m3", "f32")])
+def test_stream_kernels_edge_tiles(gpu, M, N, K, dtype_ab, dtype_c):
+    """M and N multiples of 8 but not of the 256 x 256 tile: row groups past the end re-read
+    valid rows, the epilogue stores only what is inside, pad columns stay untouched."""
+    if dtype_ab == "fp8_e4m3" and K % 128:
+        pytest.skip("fp8 stream kernel takes whole 128-byte K steps")
+    a, b, extra = operands(M, N, K, dtype_ab, seed=51, b_std=0.05)
+    bias = np.random.default_rng(52).standard_normal(N).astype(np.float32)
+    ldc = N + 16
+    out, name = run_gemm(a, b, M, N, K, dtype_ab, dtype_c, bias=bias, ldc=ldc,
+                         family=_capi.KERNEL_TILE, wg_tile=(256, 256), **extra)
+    assert name.startswith("stream_")
+    if dtype_ab == "fp8_e4m3":
+        want = G.gemm_fp8(a, b, extra["scale_a"], extra["scale_b"], out_dtype=_DT[dtype_c], bias=bias)
+    else:
+        want = G.gemm(a, b, _DT[dtype_ab], _DT[dtype_c], bias=bias)
+    bar = REL_L2_BAR if dtype_c != "f32" else (1e-4 if dtype_ab == "fp8_e4m3" else 1e-5)
+    if M * N >= 4096:
+        check(out, want, dtype_c, N, bar=bar)
+    else:
+        got, ref = G.output_to_f32(out[:, :N], _DT[dtype_c]), G.output_to_f32(want, _DT[dtype_c])
+        assert np.all(np.abs(got - ref) <= 2.0 ** -6 * np.abs(ref) + 1e-4 * np.abs(ref).max())
+    pad = out[:, N:]
+    assert np.isnan(pad).all() if dtype_c == "f32" else (pad == 0x7FC1).all()
+
+
 # ---- edge cases: ragged M / N, K tails, leading dimensions, epilogue -----------------
 
 @pytest.mark.parametrize("M,N,K", [(1, 1, 8), (65, 16, 8), (130, 257, 72), (300, 520, 776), (129, 1, 64)])
