@@ -161,6 +161,68 @@ def vendor_library(torch, dev, iters=100, drop=20):
     return rows
 
 
+SWEEP_SHAPES = [(1024, 1024, 1024), (2048, 2048, 2048), (4096, 4096, 4096), (8192, 8192, 1024),
+                (4096, 14336, 4096), (8000, 8000, 8000), (512, 8192, 8192), (128, 14336, 4096),
+                (256, 14336, 4096), (8192, 1024, 8192), (3000, 5000, 7008), (16384, 16384, 4096)]
+
+
+def shape_sweep(torch, dev):
+    """`--sweep`: this build next to the vendor library over square, skinny, fat and ragged
+    shapes, bf16 and fp8, p50 of event-timed launches.  Prints one line per shape."""
+    from aster_amd import gemm as AG
+
+    def vendor(m, n, k, dt):
+        a, b = torch.randn(m, k, device=dev), torch.randn(n, k, device=dev) * 0.02
+        if dt == "bf16":
+            a, b = a.bfloat16(), b.bfloat16()
+            fn = lambda: torch.matmul(a, b.t())
+        else:
+            a, b = a.to(torch.float8_e4m3fn), b.to(torch.float8_e4m3fn)
+            one = torch.ones((), device=dev)
+            fn = lambda: torch._scaled_mm(a, b.t(), scale_a=one, scale_b=one,
+                                          out_dtype=torch.bfloat16)
+        for _ in range(15):
+            fn()
+        torch.cuda.synchronize()
+        ts = []
+        for _ in range(45):
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s.record()
+            fn()
+            e.record()
+            e.synchronize()
+            ts.append(s.elapsed_time(e) * 1e3)
+        ts.sort()
+        return _percentile(ts, 50)
+
+    rows = []
+    for dt in ("bf16", "fp8_e4m3"):
+        for (m, n, k) in SWEEP_SHAPES:
+            a, b, keep = make_operands(torch, m, n, k, dt, dev)
+            c = torch.empty(m, n, device=dev, dtype=torch.bfloat16)
+            p = AG.GemmPlan.create(m, n, k, dt, "bf16")
+            ours, _, _ = event_timed_p50(p, a, b, c, keep, 60, 15)
+            ours /= 1e3
+            del a, b, c, keep
+            try:
+                ven = vendor(m, n, k, dt)
+            except Exception as exc:  # shapes the vendor entry point refuses
+                ven = None
+                note = repr(exc)[:60]
+            fl = 2.0 * m * n * k
+            row = {"dtype": dt, "M": m, "N": n, "K": k, "kernel": p.info.name.decode(),
+                   "us": round(ours, 1), "tflops": round(fl / ours * 1e-6, 1),
+                   "vendor_us": None if ven is None else round(ven, 1),
+                   "vendor_tflops": None if ven is None else round(fl / ven * 1e-6, 1),
+                   "vendor_over_ours": None if ven is None else round(ven / ours, 2)}
+            rows.append(row)
+            print(f"{dt:9s} {m:6d}x{n:6d}x{k:6d}  {row['us']:9.1f} us {row['tflops']:7.1f} TF   vendor "
+                  + (f"{row['vendor_us']:9.1f} us {row['vendor_tflops']:7.1f} TF  x{row['vendor_over_ours']:.2f}"
+                     if ven is not None else f"refused ({note})")
+                  + f"   {row['kernel']}", flush=True)
+    return rows
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -170,6 +232,9 @@ def main() -> int:
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-vendor", action="store_true",
                     help="skip timing the vendor library (hipBLASLt through torch) on the same shapes")
+    ap.add_argument("--sweep", action="store_true",
+                    help="instead of the bench line: time a list of shapes here and in the vendor "
+                         "library, one text line per shape and one JSON line at the end")
     ap.add_argument("--results-jsonl", default=None,
                     help="also append one BENCH_RESULT_JSON line per MFMA-bound workload to this "
                          "file (input of `python -m aster_amd.perf_registry`)")
@@ -189,6 +254,9 @@ def main() -> int:
         return 3
     dev = torch.device("cuda:0")
     lib = _capi.load()
+    if args.sweep:
+        print(json.dumps({"sweep": shape_sweep(torch, dev)}), flush=True)
+        return 0
 
     M = N = K = 8192
     a, b, keep = make_operands(torch, M, N, K, "bf16", dev)
