@@ -116,11 +116,13 @@ const Variant* choose(const astergemm_config& c, int* index_out) {
     if (!best) {
       better = true;
     } else if (family == ASTERGEMM_KERNEL_SKINNY) {
-      // smallest activation tile that still covers M
+      // among the variants that cover M: the resident-activation kernels (rank >= 2) by
+      // rank, otherwise the smallest activation tile, rank breaking ties
       const bool fits = v->tile_m >= c.M, best_fits = best->tile_m >= c.M;
-      better = (fits && !best_fits) || (fits == best_fits && fits && v->tile_m < best->tile_m) ||
-               (!fits && !best_fits && v->tile_m > best->tile_m) ||
-               (v->tile_m == best->tile_m && v->rank > best->rank);
+      if (fits != best_fits) better = fits;
+      else if (!fits) better = v->tile_m > best->tile_m;
+      else if (v->rank >= 2 || best->rank >= 2) better = v->rank > best->rank;
+      else better = v->tile_m < best->tile_m || (v->tile_m == best->tile_m && v->rank > best->rank);
     } else {
       // largest tile that still yields at least one workgroup per CU (256)
       auto wgs = [&](const Variant* x) {
@@ -168,6 +170,13 @@ int grid_of(const Variant& v, const astergemm_config& c) {
   if (v.family == ASTERGEMM_KERNEL_SKINNY) {
     const int blocks = (int)((c.N + v.tile_n - 1) / v.tile_n);
     // the resident-activation kernels (8 waves) are persistent: one workgroup per CU
+    if (v.waves_n == 8 && v.tile_m == 64 && device_cus() > 0) {
+      // 32 < M <= 64: pairs of workgroups per row range, whole pairs on each of the 8 XCDs
+      const int mh = c.M > 32 ? 2 : 1;
+      int g = blocks * mh < device_cus() ? blocks * mh : device_cus();
+      if (mh == 2) g = g < 16 ? 16 : (g & ~15);
+      return g;
+    }
     if (v.waves_n == 8 && device_cus() > 0 && blocks > device_cus()) return device_cus();
     return blocks;
   }

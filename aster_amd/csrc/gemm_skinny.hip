@@ -410,6 +410,260 @@ int launch_skinny_reg_t(const GemmArgs& a, hipStream_t s) {
   return (int)hipGetLastError();
 }
 
+// ---- 16 < M <= 64: the same persistent kernel with two activation tiles per wave --------
+//
+// A wave still owns a K slice of every row, now for 32 activation rows: MT * SPB * 2 = 128
+// operand registers at K = 4096, half of what a wave of an eight-wave workgroup can hold,
+// so 32 rows is the limit (64 rows x 8 KB would be the whole register file of the CU).
+// Every weight operand read back from the wave's LDS buffer feeds MT MFMAs; the partial
+// tiles of a row block are reduced after every block, tile mt by wave mt.
+// M > 32 (MH = 2): two workgroups on the same XCD (block ids 8 apart) take the same weight
+// rows and one half of the activation rows each.  They run side by side, so the second
+// read of a weight line is served by that XCD's L2 and HBM still sees every line once.
+template <int DT, int OUT, int SPB, int MT, int MH>
+__global__ __launch_bounds__(512) void gemm_skinny_regm_kernel(const GemmArgs p) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t slds[];
+  constexpr int KW = 8;
+  constexpr int UPB = SPB / 4;                   // units per block
+  constexpr int slice = SPB * 128;               // bytes of every row owned by one wave
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int li = lane & 15, lq = lane >> 4;
+  uint8_t* tbuf = slds + wave * 8192;            // 4 steps x 2 KiB, private to the wave
+  constexpr int NBS = 2;                         // blocks between workgroup barriers
+  f32x4* red = (f32x4*)(slds + KW * 8192);       // [2][NBS][MT][KW][64]
+
+  // block b runs on XCD b % 8; with MH = 2 blocks b and b + 8 share a row range
+  const int q = blockIdx.x >> 3;
+  const int half = MH == 2 ? (q & 1) : 0;
+  const int rid = MH == 2 ? ((q >> 1) << 3) | (blockIdx.x & 7) : (int)blockIdx.x;
+  const int g = gridDim.x / MH;
+  const int per = (((p.N + g - 1) / g) + 7) & ~7;
+  const int r0 = rid * per;
+  const int m0 = half * MT * 16;                 // first activation row of this workgroup
+  const int r1 = (r0 + per) < p.N ? (r0 + per) : p.N;
+  if (r0 >= p.N) return;
+  const int nblk = (r1 - r0 + 15) >> 4;
+  const int total = nblk * UPB;
+
+  const int lrow = lane >> 3, lpiece = lane & 7;
+  const uint8_t* wbase = p.B + wave * slice + lpiece * 16;
+  auto issue = [&](int j, i32x4(&dst)[8]) {      // flat index j = block * UPB + t
+    int blk = j / UPB;
+    const int t = j % UPB;
+    blk = blk < nblk ? blk : nblk - 1;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int nh = r0 + blk * 16 + h * 8;
+      int n = nh + lrow;
+      n = n < r1 ? n : r1 - 1;
+      const uint8_t* src = wbase + (int64_t)n * p.ldb_bytes + t * 512;
+      if (j >= total || nh >= r1) src = p.A + lpiece * 16;  // nothing to fetch: a line that stays in L2
+#pragma unroll
+      for (int s = 0; s < 4; ++s)
+        dst[s * 2 + h] = __builtin_nontemporal_load((const i32x4*)(src + s * 128));
+    }
+  };
+
+  const int wr_off = lrow * 128 + ((lpiece ^ lrow) << 4);
+  const int rd_off = li * 128;
+  auto stash = [&](const i32x4(&src)[8]) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      *(i32x4*)(tbuf + (i >> 1) * 2048 + (i & 1) * 1024 + wr_off) = src[i];
+  };
+  auto operand = [&](int s, int u) {
+    return *(const i32x4*)(tbuf + s * 2048 + rd_off + (((4 * u + lq) ^ (li & 7)) << 4));
+  };
+
+  // x: MT * UPB units, fetched like the weights (whole lines, through the LDS buffer) but
+  // cacheable; two units in flight, behind the first two weight units.
+  i32x4 x[MT][SPB * 2];
+  auto x_load = [&](int xi, i32x4(&dst)[8]) {    // xi = mt * UPB + t
+    const int mt = xi / UPB, t = xi % UPB;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      int m = m0 + mt * 16 + h * 8 + lrow;
+      m = m < p.M ? m : p.M - 1;
+      const uint8_t* src = p.A + (int64_t)m * p.lda_bytes + wave * slice + t * 512 + lpiece * 16;
+#pragma unroll
+      for (int s = 0; s < 4; ++s) dst[s * 2 + h] = *(const i32x4*)(src + s * 128);
+    }
+  };
+  i32x4 w0[8], w1[8];
+  {
+    i32x4 xa[8], xb[8];
+    issue(0, w0);
+    issue(1, w1);
+    __builtin_amdgcn_sched_barrier(0);
+    x_load(0, xa);
+    x_load(1, xb);
+    static_for<0, MT * UPB>([&](auto I) {
+      constexpr int xi = decltype(I)::value;
+      constexpr int mt = xi / UPB, t = xi % UPB;
+      if constexpr (xi % 2 == 0) stash(xa); else stash(xb);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) x[mt][t * 8 + i] = operand(i >> 1, i & 1);
+      if constexpr (xi + 2 < MT * UPB) {
+        if constexpr (xi % 2 == 0) x_load(xi + 2, xa); else x_load(xi + 2, xb);
+      }
+    });
+  }
+  __builtin_amdgcn_sched_barrier(0);
+
+  float scale = 1.0f;
+  if (p.scale_a) scale *= *p.scale_a;
+  if (p.scale_b) scale *= *p.scale_b;
+
+  f32x4 acc[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  int parity = 0;
+
+  // Partial tiles go to red[parity][block % NBS][mt][wave]; the workgroup meets once per NBS
+  // blocks, then wave w sums and stores tile w % MT of block w / MT of the group.
+  auto block_end = [&](int blk) {
+    const int slot = blk & (NBS - 1);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      red[(((parity * NBS + slot) * MT + mt) * KW + wave) * 64 + lane] = acc[mt];
+      acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    if (slot != NBS - 1 && blk != nblk - 1) return;
+    __syncthreads();
+    if (wave < (slot + 1) * MT) {
+      const int rb = wave / MT, rt = wave % MT;
+      const f32x4* src = red + (((parity * NBS + rb) * MT + rt) * KW) * 64 + lane;
+      f32x4 v = src[0];
+#pragma unroll
+      for (int k = 1; k < KW; ++k) v += src[k * 64];
+      const int m = m0 + rt * 16 + li, n = r0 + (blk - slot + rb) * 16 + 4 * lq;
+      if (m < p.M && n < r1) {
+        v *= scale;
+        const int ncols = (r1 - n) < 4 ? (r1 - n) : 4;
+        if (p.bias)
+          for (int r = 0; r < ncols; ++r) v[r] += p.bias[n + r];
+        const int64_t idx = (int64_t)m * p.ldc + n;
+        const bool vec_ok = (p.ldc & 3) == 0 && ncols == 4;
+        if constexpr (OUT == ASTERGEMM_F32) {
+          float* o = (float*)p.C + idx;
+          if (vec_ok) *(f32x4*)o = v;
+          else
+            for (int r = 0; r < ncols; ++r) o[r] = v[r];
+        } else {
+          unsigned short h[4];
+          for (int r = 0; r < 4; ++r) {
+            if constexpr (OUT == ASTERGEMM_BF16) h[r] = sk_f32_to_bf16(v[r]);
+            else {
+              _Float16 hh = (_Float16)v[r];
+              h[r] = __builtin_bit_cast(unsigned short, hh);
+            }
+          }
+          unsigned short* o = (unsigned short*)p.C + idx;
+          if (vec_ok) *(u16x4*)o = u16x4{h[0], h[1], h[2], h[3]};
+          else
+            for (int r = 0; r < ncols; ++r) o[r] = h[r];
+        }
+      }
+    }
+    parity ^= 1;
+  };
+
+  auto mma = [&](int blk, auto T) {
+    constexpr int t = decltype(T)::value;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const i32x4 w = operand(i >> 1, i & 1);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) acc[mt] = sk_mfma<DT>(w, x[mt][t * 8 + i], acc[mt]);
+    }
+    if (t == UPB - 1) block_end(blk);
+  };
+
+  constexpr int TRIP = UPB < 2 ? 2 : UPB;
+  int j = 0;
+  for (; j + TRIP <= total; j += TRIP) {
+    const int blk = j / UPB;
+    static_for<0, TRIP / 2>([&](auto I) {
+      constexpr int i = decltype(I)::value * 2;
+      stash(w0);
+      __builtin_amdgcn_sched_barrier(0);
+      issue(j + i + 2, w0);
+      __builtin_amdgcn_sched_barrier(0);
+      mma(blk + i / UPB, std::integral_constant<int, i % UPB>{});
+      __builtin_amdgcn_sched_barrier(0);
+      stash(w1);
+      __builtin_amdgcn_sched_barrier(0);
+      issue(j + i + 3, w1);
+      __builtin_amdgcn_sched_barrier(0);
+      mma(blk + (i + 1) / UPB, std::integral_constant<int, (i + 1) % UPB>{});
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  }
+  if (j < total) {  // UPB == 1, odd block count
+    stash(w0);
+    mma(j / UPB, std::integral_constant<int, 0>{});
+  }
+}
+
+template <int DT, int OUT, int SPB, int MT, int MH>
+int launch_skinny_regm_t(const GemmArgs& a, hipStream_t s) {
+  auto k = gemm_skinny_regm_kernel<DT, OUT, SPB, MT, MH>;
+  constexpr int lds = 8 * 8192 + 2 * 2 * MT * 8 * 64 * 16;
+  static bool attr_set = false;
+  static int cus = 0;
+  if (!attr_set) {
+    hipError_t e =
+        hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess) return (int)e;
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess)
+      return (int)hipGetLastError();
+    cus = prop.multiProcessorCount;
+    attr_set = true;
+  }
+  // one workgroup per CU; with MH = 2 the grid is whole pairs on each of the 8 XCDs
+  const int nblocks = (int)((a.N + 15) / 16) * MH;
+  int g = nblocks < cus ? nblocks : cus;
+  if (MH == 2) g = g < 16 ? 16 : (g & ~15);
+  hipLaunchKernelGGL(k, dim3(g), dim3(512), lds, s, a);
+  return (int)hipGetLastError();
+}
+
+template <int DT, int OUT>
+int launch_skinny_regm(const GemmArgs& a, int grid, hipStream_t s) {
+  (void)grid;
+  const int64_t rb = row_bytes(DT, a.K);
+  if (a.M <= 32) {
+    switch (rb) {
+      case 4096: return launch_skinny_regm_t<DT, OUT, 4, 2, 1>(a, s);
+      case 8192: return launch_skinny_regm_t<DT, OUT, 8, 2, 1>(a, s);
+    }
+  } else {
+    switch (rb) {
+      case 4096: return launch_skinny_regm_t<DT, OUT, 4, 2, 2>(a, s);
+      case 8192: return launch_skinny_regm_t<DT, OUT, 8, 2, 2>(a, s);
+    }
+  }
+  return (int)hipErrorInvalidValue;
+}
+
+const char* check_skinny_regm(const astergemm_config& c) {
+  if (c.M > 64) return "resident-activation path needs M <= 64";
+  const int64_t rb = row_bytes(c.dtype_ab, c.K);
+  if (rb != 4096 && rb != 8192)
+    return "resident-activation path for 16 < M <= 64 needs K = 2048 or 4096";
+  return nullptr;
+}
+
+#define AG_SKINNY_LDSM(name, DT, OUT)                                                      \
+  Variant {                                                                                \
+    name, ASTERGEMM_KERNEL_SKINNY, DT, OUT, 64, 16, 512, 1, 8, 1, 2, 8 * 8192 + 65536,      \
+        (const void*)gemm_skinny_regm_kernel<DT, OUT, 8, 2, 2>, launch_skinny_regm<DT, OUT>, \
+        check_skinny_regm                                                                  \
+  }
+
 template <int DT, int OUT>
 int launch_skinny_reg(const GemmArgs& a, int grid, hipStream_t s) {
   (void)grid;
@@ -433,7 +687,7 @@ const char* check_skinny_reg(const astergemm_config& c) {
 
 #define AG_SKINNY_LDS(name, DT, OUT)                                                       \
   Variant {                                                                                \
-    name, ASTERGEMM_KERNEL_SKINNY, DT, OUT, 16, 16, 512, 1, 8, 1, 1, 8 * 8192 + 65536,      \
+    name, ASTERGEMM_KERNEL_SKINNY, DT, OUT, 16, 16, 512, 1, 8, 1, 3, 8 * 8192 + 65536,      \
         (const void*)gemm_skinny_reg_kernel<DT, OUT, 8>, launch_skinny_reg<DT, OUT>,       \
         check_skinny_reg                                                                   \
   }
@@ -719,6 +973,12 @@ const Variant kSkinnyVariants[] = {
     AG_SKINNY_LDS("skinnyx_f16_m16_bf16", ASTERGEMM_F16, ASTERGEMM_BF16),
     AG_SKINNY_LDS("skinnyx_f16_m16_f32", ASTERGEMM_F16, ASTERGEMM_F32),
     AG_SKINNY_LDS("skinnyx_f16_m16_f16", ASTERGEMM_F16, ASTERGEMM_F16),
+    AG_SKINNY_LDSM("skinnyx_bf16_m64_bf16", ASTERGEMM_BF16, ASTERGEMM_BF16),
+    AG_SKINNY_LDSM("skinnyx_bf16_m64_f32", ASTERGEMM_BF16, ASTERGEMM_F32),
+    AG_SKINNY_LDSM("skinnyx_bf16_m64_f16", ASTERGEMM_BF16, ASTERGEMM_F16),
+    AG_SKINNY_LDSM("skinnyx_f16_m64_bf16", ASTERGEMM_F16, ASTERGEMM_BF16),
+    AG_SKINNY_LDSM("skinnyx_f16_m64_f32", ASTERGEMM_F16, ASTERGEMM_F32),
+    AG_SKINNY_LDSM("skinnyx_f16_m64_f16", ASTERGEMM_F16, ASTERGEMM_F16),
     AG_SKINNY_LDS("skinnyx_fp8_m16_bf16", ASTERGEMM_FP8_E4M3, ASTERGEMM_BF16),
     AG_SKINNY_LDS("skinnyx_fp8_m16_f32", ASTERGEMM_FP8_E4M3, ASTERGEMM_F32),
     AG_SKINNY_LDS("skinnyx_fp8_m16_f16", ASTERGEMM_FP8_E4M3, ASTERGEMM_F16),

@@ -239,6 +239,23 @@ def test_skinny_resident_activations(gpu, M, N, K, dtype_ab, dtype_c):
     assert np.isnan(pad).all() if dtype_c == "f32" else (pad == 0x7FC1).all()
 
 
+@pytest.mark.parametrize("M,N,K", [(64, 14336, 4096), (17, 8, 2048), (32, 777, 4096), (33, 6000, 2048),
+                                   (50, 24, 4096), (64, 14337, 2048), (48, 4104, 4096), (64, 136, 4096)])
+@pytest.mark.parametrize("dtype_ab,dtype_c", [("bf16", "f32"), ("f16", "f16"), ("bf16", "bf16")])
+def test_skinny_resident_activations_up_to_64_rows(gpu, M, N, K, dtype_ab, dtype_c):
+    """16 < M <= 64 with K in {2048, 4096}: two activation tiles per wave, and above 32 rows
+    two workgroups per row range (one half of the activation rows each)."""
+    a, b, _ = operands(M, N, K, dtype_ab, seed=61, b_std=0.05)
+    bias = np.random.default_rng(62).standard_normal(N).astype(np.float32)
+    ldc = (N + 11) & ~3
+    out, name = run_gemm(a, b, M, N, K, dtype_ab, dtype_c, bias=bias, ldc=ldc)
+    assert name.startswith("skinnyx") and "_m64_" in name
+    want = G.gemm(a, b, _DT[dtype_ab], _DT[dtype_c], bias=bias)
+    check(out, want, dtype_c, N, bar=1e-5 if dtype_c == "f32" else REL_L2_BAR)
+    pad = out[:, N:]
+    assert np.isnan(pad).all() if dtype_c == "f32" else (pad == 0x7FC1).all()
+
+
 @pytest.mark.parametrize("M,N,K", [(16, 14336, 4096), (1, 8, 4096), (5, 777, 8192), (16, 24, 16384),
                                    (13, 6000, 4096), (16, 14337, 8192)])
 @pytest.mark.parametrize("dtype_c", ["bf16", "f32", "f16"])
