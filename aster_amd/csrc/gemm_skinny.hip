@@ -571,11 +571,27 @@ __global__ __launch_bounds__(512) void gemm_skinny_regm_kernel(const GemmArgs p)
 
   auto mma = [&](int blk, auto T) {
     constexpr int t = decltype(T)::value;
+    if constexpr (DT == ASTERGEMM_FP8_E4M3) {
+      // one 16x16x128 MFMA per 128-byte step and activation tile (pieces lq and 4 + lq)
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const i32x4 w = operand(i >> 1, i & 1);
+      for (int s = 0; s < 4; ++s) {
+        const i32x4 lo = operand(s, 0), hi = operand(s, 1);
+        const i32x8 w = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) acc[mt] = sk_mfma<DT>(w, x[mt][t * 8 + i], acc[mt]);
+        for (int mt = 0; mt < MT; ++mt) {
+          const i32x4 xl = x[mt][t * 8 + 2 * s], xh = x[mt][t * 8 + 2 * s + 1];
+          acc[mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+              w, i32x8{xl[0], xl[1], xl[2], xl[3], xh[0], xh[1], xh[2], xh[3]}, acc[mt], 0, 0, 0,
+              0, 0, 0);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const i32x4 w = operand(i >> 1, i & 1);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[mt] = sk_mfma<DT>(w, x[mt][t * 8 + i], acc[mt]);
+      }
     }
     if (t == UPB - 1) block_end(blk);
   };
@@ -653,7 +669,9 @@ const char* check_skinny_regm(const astergemm_config& c) {
   if (c.M > 64) return "resident-activation path needs M <= 64";
   const int64_t rb = row_bytes(c.dtype_ab, c.K);
   if (rb != 4096 && rb != 8192)
-    return "resident-activation path for 16 < M <= 64 needs K = 2048 or 4096";
+    return c.dtype_ab == ASTERGEMM_FP8_E4M3
+               ? "resident-activation path for 16 < M <= 64 needs K = 4096 or 8192 for fp8"
+               : "resident-activation path for 16 < M <= 64 needs K = 2048 or 4096";
   return nullptr;
 }
 
@@ -979,6 +997,9 @@ const Variant kSkinnyVariants[] = {
     AG_SKINNY_LDSM("skinnyx_f16_m64_bf16", ASTERGEMM_F16, ASTERGEMM_BF16),
     AG_SKINNY_LDSM("skinnyx_f16_m64_f32", ASTERGEMM_F16, ASTERGEMM_F32),
     AG_SKINNY_LDSM("skinnyx_f16_m64_f16", ASTERGEMM_F16, ASTERGEMM_F16),
+    AG_SKINNY_LDSM("skinnyx_fp8_m64_bf16", ASTERGEMM_FP8_E4M3, ASTERGEMM_BF16),
+    AG_SKINNY_LDSM("skinnyx_fp8_m64_f32", ASTERGEMM_FP8_E4M3, ASTERGEMM_F32),
+    AG_SKINNY_LDSM("skinnyx_fp8_m64_f16", ASTERGEMM_FP8_E4M3, ASTERGEMM_F16),
     AG_SKINNY_LDS("skinnyx_fp8_m16_bf16", ASTERGEMM_FP8_E4M3, ASTERGEMM_BF16),
     AG_SKINNY_LDS("skinnyx_fp8_m16_f32", ASTERGEMM_FP8_E4M3, ASTERGEMM_F32),
     AG_SKINNY_LDS("skinnyx_fp8_m16_f16", ASTERGEMM_FP8_E4M3, ASTERGEMM_F16),

@@ -288,9 +288,26 @@ def test_skinny_fp8_resident_activations(gpu, M, N, K, dtype_c):
         assert G.rel_l2(out[:, :N], tile) <= 1e-5
 
 
+@pytest.mark.parametrize("M,N,K", [(64, 14336, 4096), (17, 8, 4096), (33, 777, 8192), (48, 6000, 4096)])
+@pytest.mark.parametrize("dtype_c", ["bf16", "f32"])
+def test_skinny_fp8_up_to_64_rows(gpu, M, N, K, dtype_c):
+    a, b, extra = operands(M, N, K, "fp8_e4m3", seed=35, b_std=0.05)
+    bias = np.random.default_rng(36).standard_normal(N).astype(np.float32)
+    out, name = run_gemm(a, b, M, N, K, "fp8_e4m3", dtype_c, bias=bias, ldc=N + 8, **extra)
+    assert name.startswith("skinnyx_fp8_m64")
+    want = G.gemm_fp8(a, b, extra["scale_a"], extra["scale_b"], out_dtype=_DT[dtype_c], bias=bias)
+    if dtype_c == "f32" or M * N >= 4096:
+        check(out, want, dtype_c, N, bar=1e-4 if dtype_c == "f32" else REL_L2_BAR)
+    else:
+        got, ref = G.output_to_f32(out[:, :N], _DT[dtype_c]), G.output_to_f32(want, _DT[dtype_c])
+        assert np.all(np.abs(got - ref) <= 2.0 ** -6 * np.abs(ref) + 1e-4 * np.abs(ref).max())
+    pad = out[:, N:]
+    assert np.isnan(pad).all() if dtype_c == "f32" else (pad == 0x7FC1).all()
+
+
 def test_skinny_fp8_falls_back_to_tile_kernels(gpu):
-    # K outside the resident kernel's set, or M > 16: AUTO keeps the tile family
-    for (M, N, K) in ((16, 256, 1024), (17, 256, 4096)):
+    # K outside the resident kernels' set, or M > 64: AUTO keeps the tile family
+    for (M, N, K) in ((16, 256, 1024), (65, 256, 4096), (17, 256, 16384)):
         a, b, extra = operands(M, N, K, "fp8_e4m3", seed=33)
         out, name = run_gemm(a, b, M, N, K, "fp8_e4m3", "f32", **extra)
         assert name.startswith("tile")
