@@ -124,14 +124,21 @@ const Variant* choose(const astergemm_config& c, int* index_out) {
       else if (v->rank >= 2 || best->rank >= 2) better = v->rank > best->rank;
       else better = v->tile_m < best->tile_m || (v->tile_m == best->tile_m && v->rank > best->rank);
     } else {
-      // largest tile that still yields at least one workgroup per CU (256)
+      // Measured on MI355X (256 CUs): the 256 x 256 kernels (one workgroup per CU) win once
+      // they nearly fill the chip; below that the largest smaller tile that still gives
+      // about two workgroups per CU; for tiny problems the smallest tile.
       auto wgs = [&](const Variant* x) {
         return ((c.M + x->tile_m - 1) / x->tile_m) * ((c.N + x->tile_n - 1) / x->tile_n);
       };
-      const bool big_ok = wgs(v) >= 256, best_big_ok = wgs(best) >= 256;
+      auto tier = [&](const Variant* x) {
+        const int area = x->tile_m * x->tile_n;
+        if (area >= 256 * 256) return wgs(x) >= 230 ? 2 : -1;
+        return wgs(x) >= 448 ? 1 : 0;
+      };
+      const int tv = tier(v), tb = tier(best);
       const int area = v->tile_m * v->tile_n, best_area = best->tile_m * best->tile_n;
-      if (big_ok != best_big_ok) better = big_ok;
-      else if (area != best_area) better = big_ok ? area > best_area : area < best_area;
+      if (tv != tb) better = tv > tb;
+      else if (area != best_area) better = (tv >= 1) ? area > best_area : area < best_area;
       else better = v->rank > best->rank;
     }
     if (better) {
@@ -335,6 +342,7 @@ int astergemm_run(const astergemm_config* cfg, const astergemm_operands* ops, vo
   if (cfg->M == 0 || cfg->N == 0) return 0;
   GemmArgs a;
   if (int rc = build_args(*v, *cfg, *ops, &a)) return rc;
+  (void)hipGetLastError();  // the launchers report hipGetLastError(): drop what an earlier call left
   const int e = v->launch(a, grid_of(*v, *cfg), (hipStream_t)stream);
   if (e != 0) return hip_fail((hipError_t)e, v->name, __FILE__, __LINE__);
   return 0;
@@ -360,6 +368,7 @@ int astergemm_bench_rotate(const astergemm_config* cfg, const astergemm_operands
   AG_HIP(hipEventCreate(&e0));
   AG_HIP(hipEventCreate(&e1));
   int le = (int)hipEventRecord(e0, s);
+  (void)hipGetLastError();
   for (int i = 0; i < iters && le == 0; ++i) le = v->launch(args[(size_t)(i % n_ops)], grid, s);
   if (le == 0) le = (int)hipEventRecord(e1, s);
   if (le == 0) le = (int)hipEventSynchronize(e1);
@@ -399,6 +408,7 @@ int astergemm_bench(const astergemm_config* cfg, const astergemm_operands* ops, 
   AG_HIP(hipEventCreate(&e0));
   AG_HIP(hipEventCreate(&e1));
   int rc = 0;
+  (void)hipGetLastError();  // the launchers report hipGetLastError()
   for (int i = 0; i < iters && rc == 0; ++i) {
     if (flush)
       hipLaunchKernelGGL(flush_llc_kernel, dim3(2048), dim3(256), 0, s, flush,

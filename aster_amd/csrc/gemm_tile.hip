@@ -48,7 +48,13 @@ const char* check_tile(const astergemm_config& c) {
       AG_TILE(prefix "_256x256_w2x4_f16", DT, ASTERGEMM_F16, 256, 256, 2, 4),          \
       AG_TILE(prefix "_128x128_w2x2_bf16", DT, ASTERGEMM_BF16, 128, 128, 2, 2),        \
       AG_TILE(prefix "_128x128_w2x2_f32", DT, ASTERGEMM_F32, 128, 128, 2, 2),          \
-      AG_TILE(prefix "_128x128_w2x2_f16", DT, ASTERGEMM_F16, 128, 128, 2, 2)
+      AG_TILE(prefix "_128x128_w2x2_f16", DT, ASTERGEMM_F16, 128, 128, 2, 2),          \
+      AG_TILE(prefix "_128x64_w2x2_bf16", DT, ASTERGEMM_BF16, 128, 64, 2, 2),          \
+      AG_TILE(prefix "_128x64_w2x2_f32", DT, ASTERGEMM_F32, 128, 64, 2, 2),            \
+      AG_TILE(prefix "_128x64_w2x2_f16", DT, ASTERGEMM_F16, 128, 64, 2, 2),            \
+      AG_TILE(prefix "_64x64_w2x2_bf16", DT, ASTERGEMM_BF16, 64, 64, 2, 2),            \
+      AG_TILE(prefix "_64x64_w2x2_f32", DT, ASTERGEMM_F32, 64, 64, 2, 2),              \
+      AG_TILE(prefix "_64x64_w2x2_f16", DT, ASTERGEMM_F16, 64, 64, 2, 2)
 
 template <int DT, int OUT, int BM, int BN, int WM, int WN>
 int launch_pipe(const GemmArgs& a0, int grid, hipStream_t s) {

@@ -213,6 +213,7 @@ extern "C" int astergemm_absmax_f32(const float* dSrc, int64_t n, float* dAbsmax
     return ASTERGEMM_EINVAL;
   }
   hipStream_t s = (hipStream_t)stream;
+  (void)hipGetLastError();  // only this call's launches are reported below
   hipLaunchKernelGGL(zero_u32_kernel, dim3(1), dim3(1), 0, s, (unsigned*)dAbsmax);
   if (n > 0)
     hipLaunchKernelGGL(absmax_kernel, dim3(blocks_for(n / 4 + 1)), dim3(256), 0, s, dSrc, n,
@@ -256,6 +257,7 @@ extern "C" int astergemm_quantize_mxfp4(const float* dSrc, int64_t rows, int64_t
     return ASTERGEMM_EINVAL;
   }
   const dim3 grid(blocks_for(nblocks * 2));  // a workgroup takes 128 blocks per trip
+  (void)hipGetLastError();
   if (ld_src == K)
     hipLaunchKernelGGL(quantize_mxfp4_kernel<true>, grid, dim3(256), 0, (hipStream_t)stream, dSrc,
                        nblocks, (unsigned)(K / 32), ld_src, dPacked, dScales);

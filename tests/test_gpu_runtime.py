@@ -114,3 +114,25 @@ def test_execute_hsaco_inout_and_missing_kernel(gpu):
     assert np.all(c == 0x4300)  # 128.0 in bf16
     with pytest.raises(RuntimeError):
         execute_hsaco(B.HSACO_PATH, "no_such_kernel", [InOutArray(c)])
+
+
+def test_failed_runtime_call_does_not_poison_later_launches(gpu):
+    """A HIP call that failed (a kernel name the code object does not hold) leaves its error as
+    the thread's last error; GEMM launches and quantiser calls that follow must not report it."""
+    from aster_amd import gemm, quantize
+
+    with pytest.raises(RuntimeError):
+        execute_hsaco(B.HSACO_PATH, "no_such_kernel", [InOutArray(np.zeros(4, np.float32))])
+    M, N, K = 16, 64, 4096
+    a = np.full((M, K), 0x3F80, np.uint16)
+    bufs = [GpuBuffer(M * K * 2), GpuBuffer(N * K * 2), GpuBuffer(M * N * 4)]
+    bufs[0].copy_from_host(a)
+    bufs[1].copy_from_host(np.full((N, K), 0x3F80, np.uint16))
+    gemm.GemmPlan.create(M, N, K, "bf16", "f32").run(*(b.ptr_value for b in bufs))
+    out = np.empty((M, N), np.float32)
+    bufs[2].copy_to_host(out)
+    assert np.all(out == K)
+    with pytest.raises(RuntimeError):
+        execute_hsaco(B.HSACO_PATH, "no_such_kernel", [InOutArray(np.zeros(4, np.float32))])
+    q, s = quantize.quantize_fp8_tensor(np.linspace(-448, 448, 1024, dtype=np.float32))
+    assert s == 1.0 and q[0] == 0xFE and q[-1] == 0x7E
