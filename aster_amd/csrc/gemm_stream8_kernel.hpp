@@ -60,7 +60,7 @@ __device__ __forceinline__ void gemm_stream8_body(const GemmArgs& p) {
   const uint8_t* b_base[LH];
   group_bases<LH, NW>(p.A, p.lda_bytes, row0 + wave * 8, p.M, a_base);
   group_bases<LH, NW>(p.B, p.ldb_bytes, col0 + wave * 8, p.N, b_base);
-  const int nk = p.ksteps;
+  const int nk = p.ksteps - (p.tail_granules ? 1 : 0);  // whole 128-byte steps
 
   auto g2s = [&](const uint8_t* base, unsigned voff, uint8_t* dst) {
     const unsigned m0v = (unsigned)(size_t)AG_LDS(dst);
@@ -228,6 +228,7 @@ __device__ __forceinline__ void gemm_stream8_body(const GemmArgs& p) {
   }
   __builtin_amdgcn_sched_barrier(0);
 
+  if (p.tail_granules) stream_k_tail<DT, BM, BN, WM, WN>(p, acc, wave, row0, col0, nk);
   stream_epilogue<OUT, BM, BN, WM, WN>(p, acc, lds, wave, row0, col0);
 }
 

@@ -66,6 +66,52 @@ __device__ __forceinline__ void group_bases(const uint8_t* mat, int64_t ld_bytes
   }
 }
 
+// K tail: when a row does not end on a 128-byte step, the K loop runs over the whole steps and
+// the remaining 1..7 granules (16 bytes each) are multiplied here, once per tile, straight from
+// global memory: lane (li, lq) loads the granules it would have read from LDS (s * 4 + lq for
+// the 16-bit types, lq and 4 + lq for fp8) when they exist and takes zeros otherwise.  The lane
+// index is recomputed, opaque to the optimiser, so that nothing here lives across the K loop.
+template <int DT, int BM, int BN, int WM, int WN>
+__device__ __forceinline__ void stream_k_tail(const GemmArgs& p,
+                                              f32x4 (&acc)[BM / WM / 16][BN / WN / 16], int wave,
+                                              int row0, int col0, int nfull) {
+  constexpr int TM = BM / WM / 16;
+  constexpr int TN = BN / WN / 16;
+  constexpr int SUB = Enc<DT>::kSub, GR = Enc<DT>::kGran;
+  int lane_t;
+  asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lane_t));
+  const int li = lane_t & 15, lq = lane_t >> 4;
+  const int wm = wave / WN, wn = wave % WN;
+  const int tg = p.tail_granules;
+  const int64_t koff = (int64_t)nfull * kRowBytes;
+  const i32x4 zero = {0, 0, 0, 0};
+#pragma unroll
+  for (int s = 0; s < SUB; ++s) {
+    i32x4 fbt[TN][GR], fat[TM][GR];
+#pragma unroll
+    for (int g = 0; g < GR; ++g) {
+      const int gran = (SUB == 2 ? s : g) * 4 + lq;
+      const bool live = gran < tg;
+#pragma unroll
+      for (int n = 0; n < TN; ++n) {
+        int r = col0 + (wn * TN + n) * 16 + li;
+        r = r < p.N ? r : p.N - 1;
+        fbt[n][g] = live ? *(const i32x4*)(p.B + (int64_t)r * p.ldb_bytes + koff + gran * 16) : zero;
+      }
+#pragma unroll
+      for (int m = 0; m < TM; ++m) {
+        int r = row0 + (wm * TM + m) * 16 + li;
+        r = r < p.M ? r : p.M - 1;
+        fat[m][g] = live ? *(const i32x4*)(p.A + (int64_t)r * p.lda_bytes + koff + gran * 16) : zero;
+      }
+    }
+#pragma unroll
+    for (int m = 0; m < TM; ++m)
+#pragma unroll
+      for (int n = 0; n < TN; ++n) acc[m][n] = mfma_step<DT>(fbt[n], fat[m], acc[m][n], 0, 0);
+  }
+}
+
 template <int OUT, int BM, int BN, int WM, int WN>
 __device__ __forceinline__ void stream_epilogue(const GemmArgs& p,
                                                 f32x4 (&acc)[BM / WM / 16][BN / WN / 16],
@@ -170,7 +216,7 @@ __device__ __forceinline__ void gemm_stream_body(const GemmArgs& p) {
   const uint8_t* b_base[LH];
   group_bases<LH, NW>(p.A, p.lda_bytes, row0 + wave * 8, p.M, a_base);
   group_bases<LH, NW>(p.B, p.ldb_bytes, col0 + wave * 8, p.N, b_base);
-  const int nk = p.ksteps;
+  const int nk = p.ksteps - (p.tail_granules ? 1 : 0);  // whole 128-byte steps
 
   // 64 lanes x 16 bytes from (scalar base + per-lane offset) to LDS at M0 + lane*16.
   // Written as asm to keep the scalar-base form; vmcnt is tracked by hand.
@@ -344,6 +390,9 @@ __device__ __forceinline__ void gemm_stream_body(const GemmArgs& p) {
   __builtin_amdgcn_sched_barrier(0);
   mfmas(S1{});
 
+  if constexpr (WM * WN == 8) {  // the four-wave variant has no registers to spare for it
+    if (p.tail_granules) stream_k_tail<DT, BM, BN, WM, WN>(p, acc, wave, row0, col0, nk);
+  }
   stream_epilogue<OUT, BM, BN, WM, WN>(p, acc, lds, wave, row0, col0);
 }
 

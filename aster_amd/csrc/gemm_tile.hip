@@ -110,8 +110,16 @@ int launch_stream(const GemmArgs& a, int grid, hipStream_t s) {
 const char* check_stream(const astergemm_config& c) {
   // edge tiles are handled in units of 8 operand rows and 16-byte output chunks
   if (c.M % 8 != 0 || c.N % 8 != 0 || c.M < 8 || c.N < 8) return "M and N must be multiples of 8";
-  if (row_bytes(c.dtype_ab, c.K) % kRowBytes != 0) return "K must fill whole 128-byte row chunks";
+  // a K tail of 1..7 granules is multiplied after the loop; at least one whole step is needed
+  if (row_bytes(c.dtype_ab, c.K) % 16 != 0) return "K must cover a whole number of 16-byte granules";
+  if (row_bytes(c.dtype_ab, c.K) < kRowBytes) return "K must cover at least one 128-byte row chunk";
   if (c.ldc % 8 != 0) return "ldc must be a multiple of 8 elements";
+  return nullptr;
+}
+
+const char* check_stream_whole_k(const astergemm_config& c) {
+  if (const char* why = check_stream(c)) return why;
+  if (row_bytes(c.dtype_ab, c.K) % kRowBytes != 0) return "K must fill whole 128-byte row chunks";
   return nullptr;
 }
 
@@ -120,7 +128,8 @@ const char* check_stream(const astergemm_config& c) {
     name, ASTERGEMM_KERNEL_TILE, DT, OUT, BM, BN, kRowBytes, WM, WN, 3,          \
         (WM * WN == 8) ? 2 : 0, 5 * BM * kRowBytes,                                                      \
         (const void*)gemm_stream_kernel<DT, OUT, BM, BN, WM, WN>,                \
-        launch_stream<DT, OUT, BM, BN, WM, WN>, check_stream                     \
+        launch_stream<DT, OUT, BM, BN, WM, WN>,                                  \
+        (WM * WN == 8) ? check_stream : check_stream_whole_k                     \
   }
 
 template <int DT, int OUT, int BM, int BN, int WM, int WN>
@@ -167,7 +176,7 @@ int launch_stream4(const GemmArgs& a, int grid, hipStream_t s) {
 // Whole 256x256 tiles and an even number of 256-element K-steps (scales move in 16-byte
 // granules = two K-steps of a row).
 const char* check_stream4(const astergemm_config& c) {
-  if (const char* why = check_stream(c)) return why;
+  if (const char* why = check_stream_whole_k(c)) return why;
   if (c.M % 256 != 0 || c.N % 256 != 0) return "M and N must be multiples of 256";
   if (c.K % 512 != 0) return "K must be a multiple of 512";
   return nullptr;

@@ -315,15 +315,17 @@ def test_skinny_fp8_falls_back_to_tile_kernels(gpu):
               bar=1e-4)
 
 
-@pytest.mark.parametrize("M,N,K", [(8, 8, 64), (264, 520, 128), (504, 1000, 192), (1000, 264, 1024),
-                                   (2056, 1800, 256), (256, 776, 320)])
+@pytest.mark.parametrize("M,N,K", [(8, 8, 128), (264, 520, 128), (504, 1000, 192), (1000, 264, 1024),
+                                   (2056, 1800, 256), (256, 776, 320), (256, 256, 136), (512, 264, 1016),
+                                   (264, 256, 7008), (256, 512, 144), (256, 256, 240)])
 @pytest.mark.parametrize("dtype_ab,dtype_c", [("bf16", "bf16"), ("f16", "f32"), ("fp8_e4m3", "bf16"),
                                               ("fp8_e4m3", "f32")])
 def test_stream_kernels_edge_tiles(gpu, M, N, K, dtype_ab, dtype_c):
     """M and N multiples of 8 but not of the 256 x 256 tile: row groups past the end re-read
-    valid rows, the epilogue stores only what is inside, pad columns stay untouched."""
-    if dtype_ab == "fp8_e4m3" and K % 128:
-        pytest.skip("fp8 stream kernel takes whole 128-byte K steps")
+    valid rows, the epilogue stores only what is inside, pad columns stay untouched.  K that
+    does not end on a 128-byte step: the last 1..7 granules are multiplied after the loop."""
+    if dtype_ab == "fp8_e4m3" and K % 16:
+        pytest.skip("rows are whole 16-byte granules")
     a, b, extra = operands(M, N, K, dtype_ab, seed=51, b_std=0.05)
     bias = np.random.default_rng(52).standard_normal(N).astype(np.float32)
     ldc = N + 16
@@ -515,9 +517,13 @@ def test_stream_kernel_is_the_default_for_whole_tiles(gpu):
     p = AG.GemmPlan.create(8192, 8192, 8192, "bf16", "bf16")
     assert p.info.name.decode().startswith("stream_bf16_256x256")
     assert p.info.lds_bytes == 163840
+    # edge tiles in units of 8 rows and a K tail of whole granules are its own
+    assert AG.GemmPlan.create(8192, 8192, 8200, "bf16", "bf16").info.name.decode().startswith("stream_")
+    assert AG.GemmPlan.create(8000, 8104, 8192, "bf16", "bf16").info.name.decode().startswith("stream_")
     # shapes it does not take fall back to the general tile kernel
-    assert AG.GemmPlan.create(8192, 8192, 8200, "bf16", "bf16").info.name.decode().startswith("tile_")
     assert AG.GemmPlan.create(8192, 8100, 8192, "bf16", "bf16").info.name.decode().startswith("tile_")
+    with pytest.raises(_capi.AsterGemmError, match="16-byte granules"):
+        AG.GemmPlan.create(8192, 8192, 8196, "bf16", "bf16", lda=8200, ldb=8200)
 
 
 @pytest.mark.parametrize("K", [64, 128, 192, 256, 320, 384, 448, 512, 576, 640, 704])
