@@ -305,6 +305,36 @@ def test_skinny_fp8_up_to_64_rows(gpu, M, N, K, dtype_c):
     assert np.isnan(pad).all() if dtype_c == "f32" else (pad == 0x7FC1).all()
 
 
+@pytest.mark.parametrize("M,N,K", [(16, 14336, 4096), (1, 8, 4096), (5, 777, 8192), (16, 24, 16384),
+                                   (13, 6000, 4096), (16, 14337, 8192), (9, 1000, 16384)])
+@pytest.mark.parametrize("dtype_c", ["bf16", "f32"])
+def test_skinny_mxfp4_resident_activations(gpu, M, N, K, dtype_c):
+    """MXFP4 weights and activations through the persistent kernel: two scaled MFMAs per
+    128-byte step, every lane with its own e8m0 byte for both operands."""
+    a, b, extra = operands(M, N, K, "mxfp4", seed=41, b_std=0.05)
+    # spread the block scales so that a wrong byte cannot go unnoticed
+    rng = np.random.default_rng(43)
+    extra["mx_a"] = (extra["mx_a"].astype(np.int32) + rng.integers(-3, 4, extra["mx_a"].shape)).astype(np.uint8)
+    extra["mx_b"] = (extra["mx_b"].astype(np.int32) + rng.integers(-3, 4, extra["mx_b"].shape)).astype(np.uint8)
+    bias = np.random.default_rng(42).standard_normal(N).astype(np.float32)
+    ldc = (N + 11) & ~3
+    out, name = run_gemm(a, b, M, N, K, "mxfp4", dtype_c, bias=bias, ldc=ldc, **extra)
+    assert name.startswith("skinnyx_mxfp4")
+    want = G.gemm_mxfp4(a, extra["mx_a"], b, extra["mx_b"], out_dtype=_DT[dtype_c], bias=bias)
+    if dtype_c == "f32" or M * N >= 4096:
+        check(out, want, dtype_c, N, bar=1e-5 if dtype_c == "f32" else REL_L2_BAR)
+    else:
+        got, ref = G.output_to_f32(out[:, :N], _DT[dtype_c]), G.output_to_f32(want, _DT[dtype_c])
+        assert np.all(np.abs(got - ref) <= 2.0 ** -6 * np.abs(ref) + 1e-4 * np.abs(ref).max())
+    pad = out[:, N:]
+    assert np.isnan(pad).all() if dtype_c == "f32" else (pad == 0x7FC1).all()
+    if dtype_c == "f32":
+        tile, tname = run_gemm(a, b, M, N, K, "mxfp4", "f32", bias=bias, family=_capi.KERNEL_TILE,
+                               **extra)
+        assert tname.startswith("tile")
+        assert G.rel_l2(out[:, :N], tile) <= 1e-5
+
+
 def test_skinny_fp8_falls_back_to_tile_kernels(gpu):
     # K outside the resident kernels' set, or M > 64: AUTO keeps the tile family
     for (M, N, K) in ((16, 256, 1024), (65, 256, 4096), (17, 256, 16384)):
