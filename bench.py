@@ -138,11 +138,22 @@ def vendor_library(torch, dev, iters=100, drop=20):
 
     g = torch.Generator(device=dev).manual_seed(42)
     for (m, n, k, dt) in ((8192, 8192, 8192, "bf16"), (8192, 8192, 8192, "fp8_e4m3"),
-                          (16, 14336, 4096, "bf16")):
+                          (4096, 14336, 4096, "mxfp4"), (16, 14336, 4096, "bf16")):
         try:
             a = torch.randn(m, k, device=dev, generator=g)
             b = torch.randn(n, k, device=dev, generator=g) * 0.02
-            if dt == "bf16":
+            if dt == "mxfp4":
+                # random nibbles and scale bytes around 2^0, as in this build's own MXFP4 line
+                def rnd(shape, lo, hi, view):
+                    return torch.randint(lo, hi, shape, device=dev, dtype=torch.uint8,
+                                         generator=g).view(view)
+                a = rnd((m, k // 2), 0, 256, torch.float4_e2m1fn_x2)
+                b = rnd((n, k // 2), 0, 256, torch.float4_e2m1fn_x2)
+                sa = rnd((m, k // 32), 124, 130, torch.float8_e8m0fnu)
+                sb = rnd((n, k // 32), 124, 130, torch.float8_e8m0fnu)
+                us = timed(lambda: torch._scaled_mm(a, b.t(), scale_a=sa, scale_b=sb,
+                                                    out_dtype=torch.bfloat16))
+            elif dt == "bf16":
                 a, b = a.bfloat16(), b.bfloat16()
                 us = timed(lambda: torch.matmul(a, b.t()))
             else:
@@ -335,6 +346,28 @@ def main() -> int:
                            "frac": round(gbs / PEAK_HBM_GBPS, 4),
                            "p50_us_cache_warm": round(hot / 1e3, 2),
                            "us_back_to_back_8_weight_sets": round(rot_ns / 1e3, 2),
+                           "gbps_back_to_back": round(p.info.bytes / rot_ns, 1),
+                           "frac_back_to_back": round(p.info.bytes / rot_ns / PEAK_HBM_GBPS, 4)})
+        # the decode shape with quantised weights and activations (same kernel frame)
+        for dt in ("fp8_e4m3", "mxfp4"):
+            del a, b, c
+            a, b, keep = make_operands(torch, 16, 14336, 4096, dt, dev)
+            c = torch.empty(16, 14336, device=dev, dtype=torch.bfloat16)
+            p = AG.GemmPlan.create(16, 14336, 4096, dt, "bf16")
+            p50, _, _ = event_timed_p50(p, a, b, c, keep, 100, 20, flush_bytes=512 << 20)
+            nsets = 12 if dt == "fp8_e4m3" else 24      # > 2.5x the last-level cache in all
+            wts = [b] + [torch.empty_like(b).copy_(b) for _ in range(nsets - 1)]
+            kw = {k: v.data_ptr() for k, v in keep.items()}
+            sets = [dict(dA=a.data_ptr(), dB=w.data_ptr(), dC=c.data_ptr(), **kw) for w in wts]
+            p.bench_rotate(sets, 48)
+            rot_ns = p.bench_rotate(sets, 240) / 240.0
+            del wts, sets
+            others.append({"workload": f"{dt} skinny GEMM M=16 N=14336 K=4096 -> bf16, LLC flushed "
+                                       "before every launch",
+                           "kernel": p.info.name.decode(), "p50_us": round(p50 / 1e3, 2),
+                           "gbps": round(p.info.bytes / p50, 1), "bound": "hbm",
+                           "frac": round(p.info.bytes / p50 / PEAK_HBM_GBPS, 4),
+                           f"us_back_to_back_{nsets}_weight_sets": round(rot_ns / 1e3, 2),
                            "gbps_back_to_back": round(p.info.bytes / rot_ns, 1),
                            "frac_back_to_back": round(p.info.bytes / rot_ns / PEAK_HBM_GBPS, 4)})
         # the same M = 16 shape with the weights pre-shuffled into MFMA operand order
