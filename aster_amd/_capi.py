@@ -119,9 +119,9 @@ SIGNATURES = {
     "astergemm_weight_verify": (C.c_int, [_P, C.c_size_t]),
     "astergemm_weight_config": (C.c_int, [C.POINTER(WeightHeader), C.c_int64, C.c_int,
                                           C.POINTER(Config)]),
-    "astergemm_absmax_f32": (C.c_int, [_P, C.c_int64, _P, _P]),
-    "astergemm_quantize_fp8_tensor": (C.c_int, [_P, C.c_int64, _P, _P, _P]),
-    "astergemm_quantize_mxfp4": (C.c_int, [_P, C.c_int64, C.c_int64, C.c_int64, _P, _P, _P]),
+    "astergemm_absmax": (C.c_int, [_P, C.c_int, C.c_int64, _P, _P]),
+    "astergemm_quantize_fp8_tensor": (C.c_int, [_P, C.c_int, C.c_int64, _P, _P, _P]),
+    "astergemm_quantize_mxfp4": (C.c_int, [_P, C.c_int, C.c_int64, C.c_int64, C.c_int64, _P, _P, _P]),
     "aster_rt_init": (C.c_int, []),
     "aster_rt_peek_at_last_error": (C.c_int, []),
     "aster_rt_clear_last_error": (C.c_int, []),

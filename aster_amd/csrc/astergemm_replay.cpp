@@ -105,8 +105,8 @@ static int run_quantize(const char* kind, long long rows, long long K, int iters
   std::vector<double> us;
   for (int i = 0; i < iters; ++i) {
     CHECK(aster_rt_event_record(e0, nullptr));
-    if (fp8) CHECK(astergemm_quantize_fp8_tensor((const float*)src, (int64_t)n, (uint8_t*)dst, (float*)sc, nullptr));
-    else CHECK(astergemm_quantize_mxfp4((const float*)src, rows, K, 0, (uint8_t*)dst, (uint8_t*)sc, nullptr));
+    if (fp8) CHECK(astergemm_quantize_fp8_tensor(src, ASTERGEMM_F32, (int64_t)n, (uint8_t*)dst, (float*)sc, nullptr));
+    else CHECK(astergemm_quantize_mxfp4(src, ASTERGEMM_F32, rows, K, 0, (uint8_t*)dst, (uint8_t*)sc, nullptr));
     CHECK(aster_rt_event_record(e1, nullptr));
     CHECK(aster_rt_event_synchronize(e1));
     float ms = 0;

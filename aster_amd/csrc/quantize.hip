@@ -1,5 +1,5 @@
-// Operand quantisers for the fp8 and MXFP4 GEMM paths: fp32 -> OCP e4m3 with a per-tensor
-// absmax scale, and fp32 -> MXFP4 (e2m1 nibbles + one e8m0 byte per 32 elements).
+// Operand quantisers for the fp8 and MXFP4 GEMM paths: fp32 / bf16 / f16 -> OCP e4m3 with a
+// per-tensor absmax scale, and -> MXFP4 (e2m1 nibbles + one e8m0 byte per 32 elements).
 //
 // These produce, on the device, exactly the bytes the GEMM kernels consume (operand
 // layouts of astergemm_config: row-major, e2m1 low nibble first, scales [rows, K/32]).
@@ -10,6 +10,8 @@
 // even as the hardware converter does.  The MX block format is the one the scaled MFMA
 // expects (v_mfma_scale_f32_16x16x128_f8f6f4, e8m0 scale per 32 K-elements).
 // Both are HBM-bound byte work: one pass over the source (two for the per-tensor scale).
+#include <type_traits>
+
 #include "astergemm_internal.h"
 
 namespace astergemm {
@@ -58,16 +60,44 @@ __device__ __forceinline__ unsigned e2m1_rne_sat(float x) {
 
 __global__ void zero_u32_kernel(unsigned* p) { *p = 0u; }
 
+// Source element types: fp32, or the 16-bit types a GEMM of this library writes (both widen
+// to fp32 exactly, so quantising them equals quantising the widened values).
+template <int SRC>
+struct Src {
+  static constexpr int kBytes = SRC == ASTERGEMM_F32 ? 4 : 2;
+};
+template <int SRC>
+__device__ __forceinline__ float widen(unsigned short h) {
+  if constexpr (SRC == ASTERGEMM_BF16) return __uint_as_float((unsigned)h << 16);
+  else return (float)__builtin_bit_cast(_Float16, h);
+}
+// four consecutive elements (16 or 8 bytes, naturally aligned) as fp32
+template <int SRC>
+__device__ __forceinline__ f32x4 load4(const void* base, int64_t group) {
+  if constexpr (SRC == ASTERGEMM_F32) {
+    return __builtin_nontemporal_load((const f32x4*)base + group);
+  } else {
+    typedef unsigned short u16x4 __attribute__((ext_vector_type(4)));
+    const u16x4 h = __builtin_nontemporal_load((const u16x4*)base + group);
+    return f32x4{widen<SRC>(h[0]), widen<SRC>(h[1]), widen<SRC>(h[2]), widen<SRC>(h[3])};
+  }
+}
+template <int SRC>
+__device__ __forceinline__ float load1(const void* base, int64_t i) {
+  if constexpr (SRC == ASTERGEMM_F32) return ((const float*)base)[i];
+  else return widen<SRC>(((const unsigned short*)base)[i]);
+}
+
 // max over |x| as unsigned bits (non-negative floats order like their bit patterns; NaNs
 // compare above infinity and so survive the maximum, as they do in numpy's max).  Four
 // independent loads per trip; one atomic per workgroup.
-__global__ __launch_bounds__(256) void absmax_kernel(const float* __restrict__ src, int64_t n,
+template <int SRC>
+__global__ __launch_bounds__(256) void absmax_kernel(const void* __restrict__ src, int64_t n,
                                                      unsigned* __restrict__ out) {
   __shared__ unsigned wave_max[4];
   unsigned m = 0;
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   const int64_t n4 = n >> 2;
-  const f32x4* p = (const f32x4*)src;
   int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
   auto fold = [&](const f32x4 v) {
 #pragma unroll
@@ -77,15 +107,15 @@ __global__ __launch_bounds__(256) void absmax_kernel(const float* __restrict__ s
     }
   };
   for (; i + 3 * stride < n4; i += 4 * stride) {
-    const f32x4 v0 = __builtin_nontemporal_load(p + i);
-    const f32x4 v1 = __builtin_nontemporal_load(p + i + stride);
-    const f32x4 v2 = __builtin_nontemporal_load(p + i + 2 * stride);
-    const f32x4 v3 = __builtin_nontemporal_load(p + i + 3 * stride);
+    const f32x4 v0 = load4<SRC>(src, i);
+    const f32x4 v1 = load4<SRC>(src, i + stride);
+    const f32x4 v2 = load4<SRC>(src, i + 2 * stride);
+    const f32x4 v3 = load4<SRC>(src, i + 3 * stride);
     fold(v0), fold(v1), fold(v2), fold(v3);
   }
-  for (; i < n4; i += stride) fold(__builtin_nontemporal_load(p + i));
+  for (; i < n4; i += stride) fold(load4<SRC>(src, i));
   for (int64_t j = (n4 << 2) + blockIdx.x * (int64_t)blockDim.x + threadIdx.x; j < n; j += stride) {
-    const unsigned b = __float_as_uint(src[j]) & 0x7FFFFFFFu;
+    const unsigned b = __float_as_uint(load1<SRC>(src, j)) & 0x7FFFFFFFu;
     m = b > m ? b : m;
   }
 #pragma unroll
@@ -107,21 +137,22 @@ __global__ void fp8_scale_kernel(const unsigned* amax_bits, float* scale) {
   *scale = (a > 0.0f) ? a / 448.0f : 1.0f;
 }
 
-__global__ __launch_bounds__(256) void quantize_fp8_kernel(const float* __restrict__ src, int64_t n,
+template <int SRC>
+__global__ __launch_bounds__(256) void quantize_fp8_kernel(const void* __restrict__ src, int64_t n,
                                                            const float* __restrict__ scale,
                                                            uint8_t* __restrict__ dst) {
   const float s = *scale;
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   const int64_t n4 = n >> 2;
   for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n4; i += stride) {
-    const f32x4 v = __builtin_nontemporal_load((const f32x4*)src + i);
+    const f32x4 v = load4<SRC>(src, i);
     unsigned w = 0;
 #pragma unroll
     for (int e = 0; e < 4; ++e) w |= e4m3_rne_sat(v[e] / s) << (8 * e);
     ((unsigned*)dst)[i] = w;
   }
   for (int64_t i = (n4 << 2) + blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += stride)
-    dst[i] = (uint8_t)e4m3_rne_sat(src[i] / s);
+    dst[i] = (uint8_t)e4m3_rne_sat(load1<SRC>(src, i) / s);
 }
 
 // Eight lanes per 32-element block: a lane loads 16 bytes (4 elements), so one wave-wide load
@@ -129,8 +160,8 @@ __global__ __launch_bounds__(256) void quantize_fp8_kernel(const float* __restri
 // block maximum goes round the 8 lanes with three exchanges; every lane then encodes its 4
 // elements (2 bytes out) and lane 0 of the group writes the scale byte.  CONTIG: ld == K, so
 // block t sits at element 32 t and no (row, column) split is needed.
-template <bool CONTIG>
-__global__ __launch_bounds__(256) void quantize_mxfp4_kernel(const float* __restrict__ src,
+template <int SRC, bool CONTIG>
+__global__ __launch_bounds__(256) void quantize_mxfp4_kernel(const void* __restrict__ src,
                                                              int64_t nblocks, unsigned bpr,
                                                              int64_t ld,
                                                              uint8_t* __restrict__ packed,
@@ -155,7 +186,7 @@ __global__ __launch_bounds__(256) void quantize_mxfp4_kernel(const float* __rest
         const unsigned r = (unsigned)t[u] / bpr, c = (unsigned)t[u] - r * bpr;
         off = (int64_t)r * ld + (int64_t)c * 32;
       }
-      v[u] = __builtin_nontemporal_load((const f32x4*)(src + off) + l8);
+      v[u] = load4<SRC>((const uint8_t*)src + off * Src<SRC>::kBytes, l8);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -207,47 +238,68 @@ int blocks_for(int64_t work_items) {
 
 using namespace astergemm;
 
-extern "C" int astergemm_absmax_f32(const float* dSrc, int64_t n, float* dAbsmax, void* stream) {
-  if ((!dSrc && n > 0) || !dAbsmax || n < 0 || (((uintptr_t)dSrc) & 15)) {
-    set_error("astergemm_absmax_f32: bad argument (dSrc must be 16-byte aligned)");
+namespace {
+bool src_ok(int dt) { return dt == ASTERGEMM_F32 || dt == ASTERGEMM_BF16 || dt == ASTERGEMM_F16; }
+
+// Calls f with the source type as a compile-time constant.
+template <class F>
+void with_src(int dt, F&& f) {
+  switch (dt) {
+    case ASTERGEMM_F32: f(std::integral_constant<int, ASTERGEMM_F32>{}); break;
+    case ASTERGEMM_BF16: f(std::integral_constant<int, ASTERGEMM_BF16>{}); break;
+    default: f(std::integral_constant<int, ASTERGEMM_F16>{}); break;
+  }
+}
+}  // namespace
+
+extern "C" int astergemm_absmax(const void* dSrc, int src_dtype, int64_t n, float* dAbsmax,
+                                void* stream) {
+  if ((!dSrc && n > 0) || !dAbsmax || n < 0 || (((uintptr_t)dSrc) & 15) || !src_ok(src_dtype)) {
+    set_error("astergemm_absmax: bad argument (source F32, BF16 or F16, 16-byte aligned)");
     return ASTERGEMM_EINVAL;
   }
   hipStream_t s = (hipStream_t)stream;
   (void)hipGetLastError();  // only this call's launches are reported below
   hipLaunchKernelGGL(zero_u32_kernel, dim3(1), dim3(1), 0, s, (unsigned*)dAbsmax);
   if (n > 0)
-    hipLaunchKernelGGL(absmax_kernel, dim3(blocks_for(n / 4 + 1)), dim3(256), 0, s, dSrc, n,
-                       (unsigned*)dAbsmax);
+    with_src(src_dtype, [&](auto T) {
+      hipLaunchKernelGGL(absmax_kernel<decltype(T)::value>, dim3(blocks_for(n / 4 + 1)), dim3(256),
+                         0, s, dSrc, n, (unsigned*)dAbsmax);
+    });
   AG_HIP(hipGetLastError());
   return 0;
 }
 
-extern "C" int astergemm_quantize_fp8_tensor(const float* dSrc, int64_t n, uint8_t* dDst,
-                                             float* dScale, void* stream) {
+extern "C" int astergemm_quantize_fp8_tensor(const void* dSrc, int src_dtype, int64_t n,
+                                             uint8_t* dDst, float* dScale, void* stream) {
   if ((!dSrc && n > 0) || (!dDst && n > 0) || !dScale || n < 0 || (((uintptr_t)dSrc) & 15) ||
-      (((uintptr_t)dDst) & 3)) {
-    set_error("astergemm_quantize_fp8_tensor: bad argument (dSrc 16-byte, dDst 4-byte aligned)");
+      (((uintptr_t)dDst) & 3) || !src_ok(src_dtype)) {
+    set_error("astergemm_quantize_fp8_tensor: bad argument (source F32, BF16 or F16, 16-byte "
+              "aligned; dDst 4-byte aligned)");
     return ASTERGEMM_EINVAL;
   }
   hipStream_t s = (hipStream_t)stream;
   // dScale doubles as the absmax accumulator: bits of a non-negative float
-  if (int rc = astergemm_absmax_f32(dSrc, n, dScale, stream)) return rc;
+  if (int rc = astergemm_absmax(dSrc, src_dtype, n, dScale, stream)) return rc;
   hipLaunchKernelGGL(fp8_scale_kernel, dim3(1), dim3(1), 0, s, (const unsigned*)dScale, dScale);
   if (n > 0)
-    hipLaunchKernelGGL(quantize_fp8_kernel, dim3(blocks_for(n / 4 + 1)), dim3(256), 0, s, dSrc, n,
-                       dScale, dDst);
+    with_src(src_dtype, [&](auto T) {
+      hipLaunchKernelGGL(quantize_fp8_kernel<decltype(T)::value>, dim3(blocks_for(n / 4 + 1)),
+                         dim3(256), 0, s, dSrc, n, dScale, dDst);
+    });
   AG_HIP(hipGetLastError());
   return 0;
 }
 
-extern "C" int astergemm_quantize_mxfp4(const float* dSrc, int64_t rows, int64_t K, int64_t ld_src,
-                                        uint8_t* dPacked, uint8_t* dScales, void* stream) {
+extern "C" int astergemm_quantize_mxfp4(const void* dSrc, int src_dtype, int64_t rows, int64_t K,
+                                        int64_t ld_src, uint8_t* dPacked, uint8_t* dScales,
+                                        void* stream) {
   if (ld_src == 0) ld_src = K;
-  if (rows < 0 || K < 0 || K % 32 != 0 || ld_src < K || ld_src % 4 != 0 ||
+  if (rows < 0 || K < 0 || K % 32 != 0 || ld_src < K || ld_src % 8 != 0 || !src_ok(src_dtype) ||
       ((rows > 0 && K > 0) && (!dSrc || !dPacked || !dScales)) || (((uintptr_t)dSrc) & 15) ||
       (((uintptr_t)dPacked) & 15)) {
-    set_error("astergemm_quantize_mxfp4: need K %% 32 == 0, ld_src >= K, ld_src %% 4 == 0, "
-              "dSrc and dPacked 16-byte aligned");
+    set_error("astergemm_quantize_mxfp4: need a source of F32, BF16 or F16, K %% 32 == 0, "
+              "ld_src >= K, ld_src %% 8 == 0, dSrc and dPacked 16-byte aligned");
     return ASTERGEMM_EINVAL;
   }
   if (rows == 0 || K == 0) return 0;
@@ -258,12 +310,17 @@ extern "C" int astergemm_quantize_mxfp4(const float* dSrc, int64_t rows, int64_t
   }
   const dim3 grid(blocks_for(nblocks * 2));  // a workgroup takes 128 blocks per trip
   (void)hipGetLastError();
-  if (ld_src == K)
-    hipLaunchKernelGGL(quantize_mxfp4_kernel<true>, grid, dim3(256), 0, (hipStream_t)stream, dSrc,
-                       nblocks, (unsigned)(K / 32), ld_src, dPacked, dScales);
-  else
-    hipLaunchKernelGGL(quantize_mxfp4_kernel<false>, grid, dim3(256), 0, (hipStream_t)stream, dSrc,
-                       nblocks, (unsigned)(K / 32), ld_src, dPacked, dScales);
+  with_src(src_dtype, [&](auto T) {
+    constexpr int SRC = decltype(T)::value;
+    if (ld_src == K)
+      hipLaunchKernelGGL((quantize_mxfp4_kernel<SRC, true>), grid, dim3(256), 0,
+                         (hipStream_t)stream, dSrc, nblocks, (unsigned)(K / 32), ld_src, dPacked,
+                         dScales);
+    else
+      hipLaunchKernelGGL((quantize_mxfp4_kernel<SRC, false>), grid, dim3(256), 0,
+                         (hipStream_t)stream, dSrc, nblocks, (unsigned)(K / 32), ld_src, dPacked,
+                         dScales);
+  });
   AG_HIP(hipGetLastError());
   return 0;
 }

@@ -1,4 +1,4 @@
-"""Operand quantisers on the device: fp32 -> e4m3 with a per-tensor scale, fp32 -> MXFP4.
+"""Operand quantisers on the device: fp32 / bf16 / f16 -> e4m3 with a per-tensor scale, -> MXFP4.
 
 They write the bytes the fp8 and MXFP4 GEMM kernels read.  The e4m3 rounding is the one of
 the converter the reference's tests hold (f32_to_fp8_e4m3(val, fnuz=False),
@@ -24,47 +24,68 @@ def _s(stream):
     return ctypes.c_void_p(stream) if stream else None
 
 
-def absmax_f32_device(d_src: int, n: int, d_absmax: int, stream: Optional[int] = None) -> None:
-    _capi.check(_capi.load().astergemm_absmax_f32(ctypes.c_void_p(d_src), n,
-                                                  ctypes.c_void_p(d_absmax), _s(stream)))
+def _src(dtype: str) -> int:
+    if dtype not in ("f32", "bf16", "f16"):
+        raise ValueError(f"quantiser source must be f32, bf16 or f16, not {dtype!r}")
+    return _capi.DTYPE_NAMES[dtype]
 
 
-def quantize_fp8_tensor_device(d_src: int, n: int, d_dst: int, d_scale: int,
-                               stream: Optional[int] = None) -> None:
+def absmax_device(d_src: int, n: int, d_absmax: int, *, src_dtype: str = "f32",
+                  stream: Optional[int] = None) -> None:
+    _capi.check(_capi.load().astergemm_absmax(ctypes.c_void_p(d_src), _src(src_dtype), n,
+                                              ctypes.c_void_p(d_absmax), _s(stream)))
+
+
+def quantize_fp8_tensor_device(d_src: int, n: int, d_dst: int, d_scale: int, *,
+                               src_dtype: str = "f32", stream: Optional[int] = None) -> None:
     """d_dst[i] = e4m3(d_src[i] / scale), *d_scale = scale = absmax / 448 (1.0 for absmax 0)."""
     _capi.check(_capi.load().astergemm_quantize_fp8_tensor(
-        ctypes.c_void_p(d_src), n, ctypes.c_void_p(d_dst), ctypes.c_void_p(d_scale), _s(stream)))
+        ctypes.c_void_p(d_src), _src(src_dtype), n, ctypes.c_void_p(d_dst),
+        ctypes.c_void_p(d_scale), _s(stream)))
 
 
 def quantize_mxfp4_device(d_src: int, rows: int, K: int, d_packed: int, d_scales: int, *,
-                          ld_src: int = 0, stream: Optional[int] = None) -> None:
-    """rows x K fp32 -> packed e2m1 [rows, K/2] and e8m0 scale bytes [rows, K/32]."""
+                          src_dtype: str = "f32", ld_src: int = 0,
+                          stream: Optional[int] = None) -> None:
+    """rows x K elements -> packed e2m1 [rows, K/2] and e8m0 scale bytes [rows, K/32]."""
     _capi.check(_capi.load().astergemm_quantize_mxfp4(
-        ctypes.c_void_p(d_src), rows, K, ld_src, ctypes.c_void_p(d_packed),
+        ctypes.c_void_p(d_src), _src(src_dtype), rows, K, ld_src, ctypes.c_void_p(d_packed),
         ctypes.c_void_p(d_scales), _s(stream)))
 
 
-def quantize_fp8_tensor(x: np.ndarray) -> Tuple[np.ndarray, np.float32]:
+def _host_source(x: np.ndarray, dtype: Optional[str]):
+    """(contiguous array, source dtype name): float32 and float16 arrays are taken as they are,
+    uint16 arrays are bfloat16 bits when `dtype` says "bf16"."""
+    x = np.asarray(x)
+    if dtype is None:
+        dtype = {np.dtype(np.float16): "f16", np.dtype(np.uint16): "bf16"}.get(x.dtype, "f32")
+    want = {"f32": np.float32, "f16": np.float16, "bf16": np.uint16}[dtype]
+    if dtype == "bf16" and x.dtype != np.uint16:
+        raise ValueError("bf16 sources are passed as uint16 bit patterns")
+    return np.ascontiguousarray(x, dtype=want), dtype
+
+
+def quantize_fp8_tensor(x: np.ndarray, dtype: Optional[str] = None) -> Tuple[np.ndarray, np.float32]:
     """Array version: (e4m3 bytes of x's shape, fp32 scale)."""
-    x = np.ascontiguousarray(x, dtype=np.float32)
-    src, dst, sc = GpuBuffer(x.nbytes), GpuBuffer(x.size), GpuBuffer(4)
+    x, dtype = _host_source(x, dtype)
+    src, dst, sc = GpuBuffer(max(x.nbytes, 16)), GpuBuffer(max(x.size, 4)), GpuBuffer(4)
     src.copy_from_host(x)
-    quantize_fp8_tensor_device(src.ptr_value, x.size, dst.ptr_value, sc.ptr_value)
+    quantize_fp8_tensor_device(src.ptr_value, x.size, dst.ptr_value, sc.ptr_value, src_dtype=dtype)
     q, s = np.empty(x.shape, np.uint8), np.empty(1, np.float32)
     dst.copy_to_host(q)
     sc.copy_to_host(s)
     return q, s[0]
 
 
-def quantize_mxfp4(x: np.ndarray) -> Tuple[np.ndarray, np.ndarray]:
+def quantize_mxfp4(x: np.ndarray, dtype: Optional[str] = None) -> Tuple[np.ndarray, np.ndarray]:
     """Array version: x[rows, K] -> (packed [rows, K/2] uint8, scales [rows, K/32] uint8)."""
-    x = np.ascontiguousarray(x, dtype=np.float32)
+    x, dtype = _host_source(x, dtype)
     if x.ndim != 2 or x.shape[1] % 32:
         raise ValueError("quantize_mxfp4 needs a [rows, K] array with K % 32 == 0")
     rows, K = x.shape
     src, pk, sc = GpuBuffer(x.nbytes), GpuBuffer(rows * K // 2), GpuBuffer(rows * K // 32)
     src.copy_from_host(x)
-    quantize_mxfp4_device(src.ptr_value, rows, K, pk.ptr_value, sc.ptr_value)
+    quantize_mxfp4_device(src.ptr_value, rows, K, pk.ptr_value, sc.ptr_value, src_dtype=dtype)
     packed, scales = np.empty((rows, K // 2), np.uint8), np.empty((rows, K // 32), np.uint8)
     pk.copy_to_host(packed)
     sc.copy_to_host(scales)

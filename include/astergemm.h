@@ -193,10 +193,14 @@ int astergemm_shuffle_weight_16(const uint16_t* src, uint16_t* dst, int64_t N,
 
 /* ---- operand quantisers (device to device, on `stream`) -------------------
  * They write the bytes the fp8 / MXFP4 GEMM paths read (dtype_ab
- * ASTERGEMM_FP8_E4M3 / ASTERGEMM_MXFP4), so that a caller holding fp32
- * activations or weights in HBM needs no host round trip.
+ * ASTERGEMM_FP8_E4M3 / ASTERGEMM_MXFP4), so that a caller holding activations
+ * or weights in HBM needs no host round trip.
  *
- * astergemm_absmax_f32: *dAbsmax = max |dSrc[i]| (0 for n == 0; NaN if any
+ * The source is fp32, or the bf16 / f16 a GEMM of this library wrote
+ * (src_dtype = ASTERGEMM_F32 / _BF16 / _F16; the 16-bit types widen to fp32
+ * exactly, so the result equals quantising the widened values).
+ *
+ * astergemm_absmax: *dAbsmax = max |dSrc[i]| (0 for n == 0; NaN if any
  * element is NaN).  dSrc 16-byte aligned.
  *
  * astergemm_quantize_fp8_tensor: *dScale = absmax / 448 (1.0 when absmax is
@@ -207,19 +211,19 @@ int astergemm_shuffle_weight_16(const uint16_t* src, uint16_t* dst, int64_t N,
  * zero; the subnormal range rounds to nearest even.  *dScale is what
  * astergemm_operands.dScaleA / dScaleB take.  dDst 4-byte aligned.
  *
- * astergemm_quantize_mxfp4: rows x K fp32 (row stride ld_src elements, 0 =
- * K) -> dPacked[rows, K/2] (element 2j in the low nibble of byte j) and
+ * astergemm_quantize_mxfp4: rows x K elements (row stride ld_src elements,
+ * 0 = K) -> dPacked[rows, K/2] (element 2j in the low nibble of byte j) and
  * dScales[rows, K/32] e8m0 bytes, the operand layout of the scaled MFMA
  * (v_mfma_scale_f32_16x16x128_f8f6f4; reference instruction definition
- * include/aster/Dialect/AMDGCN/IR/Instructions/MMA.td:792).  Per 32-element block: scale
- * exponent floor(log2(absmax)) - 2 clamped to [-127, 127] (0 for an all-zero
- * block), elements e2m1 round-to-nearest-even of x / 2^exponent saturated to
- * +-6; a block holding NaN or inf gets scale byte 0xFF.  K % 32 == 0,
- * ld_src % 4 == 0, dSrc and dPacked 16-byte aligned.                        */
-int astergemm_absmax_f32(const float* dSrc, int64_t n, float* dAbsmax, void* stream);
-int astergemm_quantize_fp8_tensor(const float* dSrc, int64_t n, uint8_t* dDst,
+ * include/aster/Dialect/AMDGCN/IR/Instructions/MMA.td:792).  Per 32-element
+ * block: scale exponent floor(log2(absmax)) - 2 clamped to [-127, 127] (0 for
+ * an all-zero block), elements e2m1 round-to-nearest-even of x / 2^exponent
+ * saturated to +-6; a block holding NaN or inf gets scale byte 0xFF.
+ * K % 32 == 0, ld_src % 8 == 0, dSrc and dPacked 16-byte aligned.           */
+int astergemm_absmax(const void* dSrc, int src_dtype, int64_t n, float* dAbsmax, void* stream);
+int astergemm_quantize_fp8_tensor(const void* dSrc, int src_dtype, int64_t n, uint8_t* dDst,
                                   float* dScale, void* stream);
-int astergemm_quantize_mxfp4(const float* dSrc, int64_t rows, int64_t K,
+int astergemm_quantize_mxfp4(const void* dSrc, int src_dtype, int64_t rows, int64_t K,
                              int64_t ld_src, uint8_t* dPacked, uint8_t* dScales,
                              void* stream);
 

@@ -81,7 +81,7 @@ def test_absmax_matches_numpy():
         src, out = GpuBuffer(max(x.nbytes, 16)), GpuBuffer(4)
         src.copy_from_host(x)
         print(f"absmax n={n}", flush=True)
-        Q.absmax_f32_device(src.ptr_value, n, out.ptr_value)
+        Q.absmax_device(src.ptr_value, n, out.ptr_value)
         got = np.empty(1, np.float32)
         out.copy_to_host(got)
         assert got[0] == (np.max(np.abs(x)) if n else 0.0)
@@ -209,3 +209,60 @@ def test_quantise_then_gemm_on_device_mxfp4():
     want = G.gemm_mxfp4(a_p, a_s, b_p, b_s, out_dtype=G.F32)
     rel = G.rel_l2(out, G.output_to_f32(want, G.F32))
     assert rel <= 1e-3, rel
+
+
+@pytest.mark.parametrize("src", ["bf16", "f16"])
+def test_quantisers_take_16_bit_sources(src):
+    """bf16 / f16 sources (what a GEMM of this library writes) give the bytes of the widened
+    values, bit for bit."""
+    rng = np.random.default_rng(91)
+    x32 = (rng.standard_normal((48, 4096)) * rng.choice([1e-3, 0.1, 1.0, 30.0], (48, 1))).astype(np.float32)
+    if src == "bf16":
+        bits = F.f32_to_bf16_bits(x32)
+        wide = F.bf16_bits_to_f32(bits)
+        host = bits
+    else:
+        host = x32.astype(np.float16)
+        wide = host.astype(np.float32)
+    host[0, :40] = 0                                   # an all-zero block and signed zeros
+    wide[0, :40] = 0
+    print(f"quantisers from {src}", flush=True)
+    q, s = Q.quantize_fp8_tensor(host, src)
+    qo, so = F.quantize_fp8_tensor(wide)
+    assert np.float32(s).tobytes() == np.float32(so).tobytes() and np.array_equal(q, qo)
+    p, sc = Q.quantize_mxfp4(host, src)
+    po, sco = F.quantize_mxfp4(wide)
+    assert np.array_equal(sc, sco) and np.array_equal(p, po)
+    # odd lengths take the scalar tail
+    q, s = Q.quantize_fp8_tensor(host.reshape(-1)[:1003], src)
+    qo, so = F.quantize_fp8_tensor(wide.reshape(-1)[:1003])
+    assert np.float32(s).tobytes() == np.float32(so).tobytes() and np.array_equal(q, qo)
+
+
+def test_gemm_output_feeds_the_next_quantised_gemm():
+    """bf16 GEMM -> MXFP4 quantiser on its bf16 output -> MXFP4 decode GEMM, all on the device."""
+    M, K1, K2, N = 16, 1024, 4096, 512
+    rng = np.random.default_rng(92)
+    x = F.f32_to_bf16_bits(rng.standard_normal((M, K1)).astype(np.float32))
+    w1 = F.f32_to_bf16_bits((rng.standard_normal((K2, K1)) * 0.03).astype(np.float32))
+    w2 = (rng.standard_normal((N, K2)) * 0.05).astype(np.float32)
+    w2p, w2s = F.quantize_mxfp4(w2)
+    bufs = {k: GpuBuffer(v.nbytes) for k, v in dict(x=x, w1=w1, w2p=w2p, w2s=w2s).items()}
+    for k, v in dict(x=x, w1=w1, w2p=w2p, w2s=w2s).items():
+        bufs[k].copy_from_host(np.ascontiguousarray(v))
+    h, hp, hs, y = GpuBuffer(M * K2 * 2), GpuBuffer(M * K2 // 2), GpuBuffer(M * K2 // 32), GpuBuffer(M * N * 4)
+    print("bf16 gemm -> mxfp4 quantise -> mxfp4 gemm", flush=True)
+    AG.GemmPlan.create(M, K2, K1, "bf16", "bf16").run(bufs["x"].ptr_value, bufs["w1"].ptr_value, h.ptr_value)
+    Q.quantize_mxfp4_device(h.ptr_value, M, K2, hp.ptr_value, hs.ptr_value, src_dtype="bf16")
+    plan = AG.GemmPlan.create(M, N, K2, "mxfp4", "f32")
+    assert plan.info.name.decode().startswith("skinnyx_mxfp4")
+    plan.run(hp.ptr_value, bufs["w2p"].ptr_value, y.ptr_value, mx_a=hs.ptr_value,
+             mx_b=bufs["w2s"].ptr_value)
+    out = np.empty((M, N), np.float32)
+    y.copy_to_host(out)
+    # oracle: the device's own bf16 intermediate, quantised and multiplied on the CPU
+    hb = np.empty((M, K2), np.uint16)
+    h.copy_to_host(hb)
+    hq, hsc = F.quantize_mxfp4(F.bf16_bits_to_f32(hb))
+    want = G.gemm_mxfp4(hq, hsc, w2p, w2s, out_dtype=G.F32)
+    assert G.rel_l2(out, G.output_to_f32(want, G.F32)) <= 1e-5
