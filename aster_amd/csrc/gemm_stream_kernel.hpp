@@ -180,6 +180,21 @@ __device__ __forceinline__ void stream_epilogue(const GemmArgs& p,
   }
 }
 
+// acc += srcA * srcB for the 16-bit types.  AX: the accumulator lives in the accumulation
+// half of the register file and destination and addend are tied (a four-wave workgroup owns
+// 256 architectural + 256 accumulation registers per wave; only the constraint makes the
+// compiler use the latter, and the tie keeps it from rotating accumulators through copies).
+template <int DT, bool AX>
+__device__ __forceinline__ void stream_mma(const i32x4& a, const i32x4& b, f32x4& acc) {
+  if constexpr (!AX) {
+    acc = mfma_step<DT>(&a, &b, acc, 0, 0);
+  } else if constexpr (DT == ASTERGEMM_BF16) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+  } else {
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+  }
+}
+
 template <int DT, int OUT, int BM, int BN, int WM, int WN>
 __device__ __forceinline__ void gemm_stream_body(const GemmArgs& p) {
   constexpr int NW = WM * WN;
@@ -188,6 +203,7 @@ __device__ __forceinline__ void gemm_stream_body(const GemmArgs& p) {
   constexpr int SLOT = BM * kRowBytes;  // 32 KiB: one operand half of one K-step
   constexpr int NSLOT = 5;
   constexpr int LH = BM / 8 / NW;       // 1 KiB (8 rows x 128 B) transfers per wave and slot
+  constexpr bool AX = NW == 4;          // one wave per SIMD: accumulators in accumulation registers
   static_assert(BM == BN, "the ring holds equal A and B halves");
   static_assert(DT == ASTERGEMM_BF16 || DT == ASTERGEMM_F16, "16-bit operands");
   static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "tile rows per wave");
@@ -273,7 +289,10 @@ __device__ __forceinline__ void gemm_stream_body(const GemmArgs& p) {
 #pragma unroll
   for (int m = 0; m < TM; ++m)
 #pragma unroll
-    for (int n = 0; n < TN; ++n) acc[m][n] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int n = 0; n < TN; ++n) {
+      acc[m][n] = f32x4{0.f, 0.f, 0.f, 0.f};
+      if constexpr (AX) asm volatile("" : "+a"(acc[m][n]));
+    }
 
   // fragment I of substep S of the K-step with ring position KM: I < TN is B tile I,
   // else A tile I - TN
@@ -298,7 +317,7 @@ __device__ __forceinline__ void gemm_stream_body(const GemmArgs& p) {
     for (int n = 0; n < TN; ++n)
 #pragma unroll
       for (int m = 0; m < TM; ++m)
-        acc[m][n] = mfma_step<DT>(&fb[S][n], &fa[S][m], acc[m][n], 0, 0);
+        stream_mma<DT, AX>(fb[S][n], fa[S][m], acc[m][n]);
   };
   using S0 = std::integral_constant<int, 0>;
   using S1 = std::integral_constant<int, 1>;
@@ -351,7 +370,7 @@ __device__ __forceinline__ void gemm_stream_body(const GemmArgs& p) {
     static_for<0, NMF>([&](auto ic) {
       constexpr int I = decltype(ic)::value;
       constexpr int n = I / TM, m = I % TM;
-      acc[m][n] = mfma_step<DT>(&fb[1][n], &fa[1][m], acc[m][n], 0, 0);
+      stream_mma<DT, AX>(fb[1][n], fa[1][m], acc[m][n]);
       if constexpr (I < LH) {
         if (do_b) issue_b1(k + 2, (2 * KM) % NSLOT, I);
       }
@@ -361,7 +380,7 @@ __device__ __forceinline__ void gemm_stream_body(const GemmArgs& p) {
     static_for<0, NMF>([&](auto ic) {
       constexpr int I = decltype(ic)::value;
       constexpr int n = I / TM, m = I % TM;
-      acc[m][n] = mfma_step<DT>(&fb[0][n], &fa[0][m], acc[m][n], 0, 0);
+      stream_mma<DT, AX>(fb[0][n], fa[0][m], acc[m][n]);
       if constexpr (I < NF) read_one(KN{}, S1{}, std::integral_constant<int, I>{});
       if constexpr (I >= NF && I < NF + LH) {
         if (do_a) issue_a1(k + 3, (2 * KM + 1) % NSLOT, I - NF);
