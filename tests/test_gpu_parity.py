@@ -693,3 +693,63 @@ def test_linalg_matmul_kxn(gpu, M, N, K):
         matmul(a, b_kxn[:-1])
     with pytest.raises(ValueError):
         matmul(a.astype(np.float32), b_kxn)
+
+
+# ---- seeded random shapes through AUTO selection ------------------------------------------------
+
+def _random_cases(n_cases=96, seed=2024):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for i in range(n_cases):
+        dt = ("bf16", "f16", "fp8_e4m3", "mxfp4")[i % 4]
+        kind = rng.integers(0, 4)
+        if kind == 0:      # decode shapes
+            M = int(rng.choice([1, 7, 16, 16, 17, 32, 33, 64]))
+            N = int(rng.integers(1, 400)) * 8
+            K = int(rng.choice([2048, 4096, 8192]))
+        elif kind == 1:    # big enough for the 256 x 256 kernels, edges and K tails
+            M = int(rng.integers(490, 540)) * 8
+            N = int(rng.integers(490, 540)) * 8
+            K = int(rng.integers(8, 40)) * 16
+        elif kind == 2:    # mid-sized, any M and N
+            M = int(rng.integers(65, 900))
+            N = int(rng.integers(1, 900))
+            K = int(rng.integers(4, 64)) * 16
+        else:              # tiny
+            M = int(rng.integers(1, 64))
+            N = int(rng.integers(1, 64))
+            K = int(rng.integers(1, 16)) * 16
+        if dt == "mxfp4":
+            K = max(256, (K + 255) // 256 * 256)
+        if dt in ("bf16", "f16"):
+            K = max(8, K // 8 * 8)
+        out = ("f32", "bf16", "f16")[int(rng.integers(0, 3))]
+        cases.append((dt, out, M, N, K, bool(rng.integers(0, 2)), int(rng.integers(0, 3)) * 8))
+    return cases
+
+
+@pytest.mark.parametrize("dt,out_dt,M,N,K,with_bias,pad", _random_cases())
+def test_random_shapes_through_auto_selection(gpu, dt, out_dt, M, N, K, with_bias, pad):
+    """Whatever kernel AUTO picks for a shape (stream with edge tiles and K tails, the four tile
+    sizes, the skinny kernels), the result equals the oracle's; pad columns stay untouched."""
+    a, b, extra = operands(M, N, K, dt, seed=1000 + M + N + K, b_std=0.05)
+    bias = np.random.default_rng(5).standard_normal(N).astype(np.float32) if with_bias else None
+    ldc = N + pad if pad else 0
+    out, name = run_gemm(a, b, M, N, K, dt, out_dt, bias=bias, ldc=ldc, **extra)
+    if dt == "fp8_e4m3":
+        want = G.gemm_fp8(a, b, extra["scale_a"], extra["scale_b"], out_dtype=_DT[out_dt], bias=bias)
+    elif dt == "mxfp4":
+        want = G.gemm_mxfp4(a, extra["mx_a"], b, extra["mx_b"], out_dtype=_DT[out_dt], bias=bias)
+    else:
+        want = G.gemm(a, b, _DT[dt], _DT[out_dt], bias=bias)
+    got, ref = G.output_to_f32(out[:, :N], _DT[out_dt]), G.output_to_f32(want, _DT[out_dt])
+    assert not np.isnan(got).any(), name
+    ulp = {"f32": 2.0 ** -20, "bf16": 2.0 ** -7, "f16": 2.0 ** -10}[out_dt]
+    tol = 2 * ulp * np.abs(ref) + 2e-4 * np.abs(ref).max()
+    assert np.all(np.abs(got - ref) <= tol), (name, float(np.abs(got - ref).max()))
+    if M * N >= 4096:
+        bar = REL_L2_BAR if out_dt != "f32" else (1e-4 if dt == "fp8_e4m3" else 1e-5)
+        assert G.rel_l2(got, ref) <= bar, name
+    if pad:
+        tail = out[:, N:]
+        assert np.isnan(tail).all() if out_dt == "f32" else (tail == 0x7FC1).all()
