@@ -68,10 +68,10 @@ __device__ __forceinline__ void gemm_stream4_body(const GemmArgs& p) {
   const int g_lane = (lane & 7) ^ (((wave * 8 + lrow) >> 1) & 7);
   const unsigned a_off = (unsigned)(lrow * (int)p.lda_bytes + g_lane * 16);
   const unsigned b_off = (unsigned)(lrow * (int)p.ldb_bytes + g_lane * 16);
-  const uint8_t* a_base = p.A + ((int64_t)row0 + wave * 8) * p.lda_bytes;
-  const uint8_t* b_base = p.B + ((int64_t)col0 + wave * 8) * p.ldb_bytes;
-  const int64_t a_jstride = (int64_t)8 * NW * p.lda_bytes;
-  const int64_t b_jstride = (int64_t)8 * NW * p.ldb_bytes;
+  const uint8_t* a_base[LH];
+  const uint8_t* b_base[LH];
+  group_bases<LH, NW>(p.A, p.lda_bytes, row0 + wave * 8, p.M, a_base);
+  group_bases<LH, NW>(p.B, p.ldb_bytes, col0 + wave * 8, p.N, b_base);
   const int nk = p.ksteps;
 
   auto g2s = [&](const uint8_t* base, unsigned voff, uint8_t* dst) {
@@ -82,11 +82,11 @@ __device__ __forceinline__ void gemm_stream4_body(const GemmArgs& p) {
                  : "memory", "m0");
   };
   auto issue_a1 = [&](int k, int slot, int j) {  // slot: 0..1
-    g2s(a_base + (int64_t)k * kRowBytes + j * a_jstride, a_off,
+    g2s(a_base[j] + (int64_t)k * kRowBytes, a_off,
         lds + slot * SLOT + (j * NW + wave) * 8 * kRowBytes);
   };
   auto issue_b1 = [&](int k, int slot, int j) {  // slot: 2..3
-    g2s(b_base + (int64_t)k * kRowBytes + j * b_jstride, b_off,
+    g2s(b_base[j] + (int64_t)k * kRowBytes, b_off,
         lds + slot * SLOT + (j * NW + wave) * 8 * kRowBytes);
   };
 
@@ -102,7 +102,11 @@ __device__ __forceinline__ void gemm_stream4_body(const GemmArgs& p) {
     const int t = wave + i * NW;
     const bool is_a = t < 4;
     sc_base[i] = is_a ? p.mx_a + (int64_t)row0 * p.mx_ld : p.mx_b + (int64_t)col0 * p.mx_ld;
-    sc_off[i] = (unsigned)(((t & 3) * 64 + lane) * p.mx_ld);
+    // rows past the end of an edge tile re-read the operand's last row
+    const int first = is_a ? row0 : col0, rows = is_a ? p.M : p.N;
+    int r = (t & 3) * 64 + lane;
+    r = first + r < rows ? r : rows - 1 - first;
+    sc_off[i] = (unsigned)(r * p.mx_ld);
     sc_lds[i] = lds + (is_a ? SC_A : SC_B) + (t & 3) * 64 * 16;
   }
   auto issue_scales = [&](int c) {

@@ -177,7 +177,6 @@ int launch_stream4(const GemmArgs& a, int grid, hipStream_t s) {
 // granules = two K-steps of a row).
 const char* check_stream4(const astergemm_config& c) {
   if (const char* why = check_stream_whole_k(c)) return why;
-  if (c.M % 256 != 0 || c.N % 256 != 0) return "M and N must be multiples of 256";
   if (c.K % 512 != 0) return "K must be a multiple of 512";
   return nullptr;
 }

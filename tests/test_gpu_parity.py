@@ -695,6 +695,27 @@ def test_linalg_matmul_kxn(gpu, M, N, K):
         matmul(a.astype(np.float32), b_kxn)
 
 
+@pytest.mark.parametrize("M,N,K", [(264, 520, 512), (504, 1000, 1024), (1000, 264, 1536), (8, 8, 512)])
+@pytest.mark.parametrize("dtype_c", ["bf16", "f32"])
+def test_mxfp4_stream_kernel_edge_tiles(gpu, M, N, K, dtype_c):
+    a, b, extra = operands(M, N, K, "mxfp4", seed=71, b_std=0.05)
+    rng = np.random.default_rng(72)
+    extra["mx_a"] = (extra["mx_a"].astype(np.int32) + rng.integers(-3, 4, extra["mx_a"].shape)).astype(np.uint8)
+    extra["mx_b"] = (extra["mx_b"].astype(np.int32) + rng.integers(-3, 4, extra["mx_b"].shape)).astype(np.uint8)
+    bias = rng.standard_normal(N).astype(np.float32)
+    out, name = run_gemm(a, b, M, N, K, "mxfp4", dtype_c, bias=bias, ldc=N + 16,
+                         family=_capi.KERNEL_TILE, wg_tile=(256, 256), **extra)
+    assert name.startswith("stream_mxfp4")
+    want = G.gemm_mxfp4(a, extra["mx_a"], b, extra["mx_b"], out_dtype=_DT[dtype_c], bias=bias)
+    if M * N >= 4096:
+        check(out, want, dtype_c, N, bar=1e-5 if dtype_c == "f32" else REL_L2_BAR)
+    else:
+        got, ref = G.output_to_f32(out[:, :N], _DT[dtype_c]), G.output_to_f32(want, _DT[dtype_c])
+        assert np.all(np.abs(got - ref) <= 2.0 ** -6 * np.abs(ref) + 1e-4 * np.abs(ref).max())
+    pad = out[:, N:]
+    assert np.isnan(pad).all() if dtype_c == "f32" else (pad == 0x7FC1).all()
+
+
 # ---- seeded random shapes through AUTO selection ------------------------------------------------
 
 def _random_cases(n_cases=96, seed=2024):
