@@ -664,6 +664,277 @@ const char* check_skinny_fp4(const astergemm_config& c) {
         launch_skinny_fp4<OUT>, check_skinny_fp4                                           \
   }
 
+// The MXFP4 kernel above with two activation tiles per wave and, for M > 32, two workgroups
+// per weight row range (see gemm_skinny_regm_kernel).
+template <int OUT, int SPB, int SU, int MT, int MH>
+__global__ __launch_bounds__(512) void gemm_skinny_fp4m_kernel(const GemmArgs p) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t slds[];
+  constexpr int KW = 8;
+  constexpr int UPB = SPB / SU;                  // units per block
+  constexpr int NL = 2 * SU;                     // loads per unit
+  constexpr int slice = SPB * 128;               // bytes of every row owned by one wave
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int li = lane & 15, lq = lane >> 4;
+  uint8_t* tbuf = slds + wave * 8192;            // SU steps x 2 KiB, private to the wave
+  constexpr int NBS = 2;                         // blocks between workgroup barriers
+  f32x4* red = (f32x4*)(slds + KW * 8192);       // [2][NBS][MT][KW][64]
+
+  // block b runs on XCD b % 8; with MH = 2 blocks b and b + 8 share a row range
+  const int q = blockIdx.x >> 3;
+  const int half = MH == 2 ? (q & 1) : 0;
+  const int rid = MH == 2 ? ((q >> 1) << 3) | (blockIdx.x & 7) : (int)blockIdx.x;
+  const int g = gridDim.x / MH;
+  const int per = (((p.N + g - 1) / g) + 7) & ~7;
+  const int r0 = rid * per;
+  const int m0 = half * MT * 16;                 // first activation row of this workgroup
+  const int r1 = (r0 + per) < p.N ? (r0 + per) : p.N;
+  if (r0 >= p.N) return;
+  const int nblk = (r1 - r0 + 15) >> 4;
+  const int total = nblk * UPB;
+
+  const int lrow = lane >> 3, lpiece = lane & 7;
+  const uint8_t* wbase = p.B + wave * slice + lpiece * 16;
+  const uint8_t* sbase = p.mx_b + wave * (SPB * 8);       // this wave's scale bytes of a row
+  auto issue = [&](int j, i32x4(&dst)[NL], i32x2(&sc)[SU]) {  // flat index j = block * UPB + t
+    int blk = j / UPB;
+    const int t = j % UPB;
+    blk = blk < nblk ? blk : nblk - 1;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int nh = r0 + blk * 16 + h * 8;
+      int n = nh + lrow;
+      n = n < r1 ? n : r1 - 1;
+      const uint8_t* src = wbase + (int64_t)n * p.ldb_bytes + t * (SU * 128);
+      if (j >= total || nh >= r1) src = p.A + lpiece * 16;  // nothing to fetch: a line that stays in L2
+#pragma unroll
+      for (int s = 0; s < SU; ++s)
+        dst[s * 2 + h] = __builtin_nontemporal_load((const i32x4*)(src + s * 128));
+    }
+    int n = r0 + blk * 16 + li;                  // the row this lane multiplies
+    n = n < r1 ? n : r1 - 1;
+    const uint8_t* ssrc = sbase + (int64_t)n * p.mx_ld + t * (SU * 8);
+#pragma unroll
+    for (int s = 0; s < SU; ++s) sc[s] = *(const i32x2*)(ssrc + s * 8);
+  };
+
+  const int wr_off = lrow * 128 + ((lpiece ^ lrow) << 4);
+  const int rd_off = li * 128;
+  auto stash = [&](const i32x4(&src)[NL]) {
+#pragma unroll
+    for (int i = 0; i < NL; ++i)
+      *(i32x4*)(tbuf + (i >> 1) * 2048 + (i & 1) * 1024 + wr_off) = src[i];
+  };
+  auto operand = [&](int s, int u) {             // piece 4u + lq of step s, row li
+    return *(const i32x4*)(tbuf + s * 2048 + rd_off + (((4 * u + lq) ^ (li & 7)) << 4));
+  };
+
+  // x and its scales: operand registers for the SPB * 2 MFMAs of a block
+  i32x4 x[MT][SPB * 2];
+  int xs[MT][SPB * 2];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    int m = m0 + mt * 16 + li;
+    m = m < p.M ? m : p.M - 1;
+    const uint8_t* xsrc = p.mx_a + (int64_t)m * p.mx_ld + wave * (SPB * 8);
+#pragma unroll
+    for (int s = 0; s < SPB; ++s) {
+      const i32x2 v = *(const i32x2*)(xsrc + s * 8);
+      xs[mt][s * 2] = (int)((unsigned)v[0] >> (8 * lq));
+      xs[mt][s * 2 + 1] = (int)((unsigned)v[1] >> (8 * lq));
+    }
+  }
+  auto x_load = [&](int mt, int t, i32x4(&dst)[NL]) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      int m = m0 + mt * 16 + h * 8 + lrow;
+      m = m < p.M ? m : p.M - 1;
+      const uint8_t* src = p.A + (int64_t)m * p.lda_bytes + wave * slice + t * (SU * 128) + lpiece * 16;
+#pragma unroll
+      for (int s = 0; s < SU; ++s) dst[s * 2 + h] = *(const i32x4*)(src + s * 128);
+    }
+  };
+  i32x4 w0[NL], w1[NL];
+  i32x2 s0[SU], s1[SU];
+  {
+    i32x4 xa[NL];
+    issue(0, w0, s0);
+    issue(1, w1, s1);
+    __builtin_amdgcn_sched_barrier(0);
+    static_for<0, MT * UPB>([&](auto T) {
+      constexpr int mt = decltype(T)::value / UPB, t = decltype(T)::value % UPB;
+      x_load(mt, t, xa);
+      stash(xa);
+#pragma unroll
+      for (int i = 0; i < NL; ++i) x[mt][t * NL + i] = operand(i >> 1, i & 1);
+    });
+  }
+  __builtin_amdgcn_sched_barrier(0);
+
+  f32x4 acc[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  int parity = 0;
+
+  // wave w sums and stores tile w % MT of block w / MT of the group
+  auto block_end = [&](int blk) {
+    const int slot = blk & (NBS - 1);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      red[(((parity * NBS + slot) * MT + mt) * KW + wave) * 64 + lane] = acc[mt];
+      acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    if (slot != NBS - 1 && blk != nblk - 1) return;
+    __syncthreads();
+    if (wave < (slot + 1) * MT) {
+      const int rb = wave / MT, rt = wave % MT;
+      const f32x4* src = red + (((parity * NBS + rb) * MT + rt) * KW) * 64 + lane;
+      f32x4 v = src[0];
+#pragma unroll
+      for (int k = 1; k < KW; ++k) v += src[k * 64];
+      const int m = m0 + rt * 16 + li, n = r0 + (blk - slot + rb) * 16 + 4 * lq;
+      if (m < p.M && n < r1) {
+        const int ncols = (r1 - n) < 4 ? (r1 - n) : 4;
+        if (p.bias)
+          for (int r = 0; r < ncols; ++r) v[r] += p.bias[n + r];
+        const int64_t idx = (int64_t)m * p.ldc + n;
+        const bool vec_ok = (p.ldc & 3) == 0 && ncols == 4;
+        if constexpr (OUT == ASTERGEMM_F32) {
+          float* o = (float*)p.C + idx;
+          if (vec_ok) *(f32x4*)o = v;
+          else
+            for (int r = 0; r < ncols; ++r) o[r] = v[r];
+        } else {
+          unsigned short h[4];
+          for (int r = 0; r < 4; ++r) {
+            if constexpr (OUT == ASTERGEMM_BF16) h[r] = sk_f32_to_bf16(v[r]);
+            else {
+              _Float16 hh = (_Float16)v[r];
+              h[r] = __builtin_bit_cast(unsigned short, hh);
+            }
+          }
+          unsigned short* o = (unsigned short*)p.C + idx;
+          if (vec_ok) *(u16x4*)o = u16x4{h[0], h[1], h[2], h[3]};
+          else
+            for (int r = 0; r < ncols; ++r) o[r] = h[r];
+        }
+      }
+    }
+    parity ^= 1;
+  };
+
+  // T = unit index inside the block (compile time: selects the x registers); sc = the unit's
+  // weight scale dwords, this lane's byte already in byte 0
+  auto mma = [&](int blk, auto T, const int (&sc)[NL]) {
+    constexpr int t = decltype(T)::value;
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+      const i32x4 w = operand(i >> 1, i & 1);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const i32x4 xv = x[mt][t * NL + i];
+        acc[mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+            i32x8{w[0], w[1], w[2], w[3], 0, 0, 0, 0},
+            i32x8{xv[0], xv[1], xv[2], xv[3], 0, 0, 0, 0}, acc[mt], 4, 4, 0, sc[i], 0,
+            xs[mt][t * NL + i]);
+      }
+    }
+    if (t == UPB - 1) block_end(blk);
+  };
+  auto take_scales = [&](const i32x2(&src)[SU], int (&dst)[NL]) {
+#pragma unroll
+    for (int s = 0; s < SU; ++s) {
+      dst[s * 2] = (int)((unsigned)src[s][0] >> (8 * lq));
+      dst[s * 2 + 1] = (int)((unsigned)src[s][1] >> (8 * lq));
+    }
+  };
+
+  constexpr int TRIP = UPB < 2 ? 2 : UPB;
+  int j = 0;
+  int sc[NL];
+  for (; j + TRIP <= total; j += TRIP) {
+    const int blk = j / UPB;
+    static_for<0, TRIP / 2>([&](auto I) {
+      constexpr int i = decltype(I)::value * 2;
+      stash(w0);
+      take_scales(s0, sc);
+      __builtin_amdgcn_sched_barrier(0);
+      issue(j + i + 2, w0, s0);
+      __builtin_amdgcn_sched_barrier(0);
+      mma(blk + i / UPB, std::integral_constant<int, i % UPB>{}, sc);
+      __builtin_amdgcn_sched_barrier(0);
+      stash(w1);
+      take_scales(s1, sc);
+      __builtin_amdgcn_sched_barrier(0);
+      issue(j + i + 3, w1, s1);
+      __builtin_amdgcn_sched_barrier(0);
+      mma(blk + (i + 1) / UPB, std::integral_constant<int, (i + 1) % UPB>{}, sc);
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  }
+  if (j < total) {  // UPB == 1, odd block count
+    stash(w0);
+    take_scales(s0, sc);
+    mma(j / UPB, std::integral_constant<int, 0>{}, sc);
+  }
+}
+
+template <int OUT, int SPB, int SU, int MH>
+int launch_skinny_fp4m_t(const GemmArgs& a, hipStream_t s) {
+  constexpr int MT = 2;
+  auto k = gemm_skinny_fp4m_kernel<OUT, SPB, SU, MT, MH>;
+  constexpr int lds = 8 * 8192 + 2 * 2 * MT * 8 * 64 * 16;
+  static bool attr_set = false;
+  static int cus = 0;
+  if (!attr_set) {
+    hipError_t e =
+        hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess) return (int)e;
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess)
+      return (int)hipGetLastError();
+    cus = prop.multiProcessorCount;
+    attr_set = true;
+  }
+  const int nblocks = (int)((a.N + 15) / 16) * MH;
+  int g = nblocks < cus ? nblocks : cus;
+  if (MH == 2) g = g < 16 ? 16 : (g & ~15);
+  hipLaunchKernelGGL(k, dim3(g), dim3(512), lds, s, a);
+  return (int)hipGetLastError();
+}
+
+template <int OUT>
+int launch_skinny_fp4m(const GemmArgs& a, int grid, hipStream_t s) {
+  (void)grid;
+  if (a.M <= 32) {
+    switch (a.K) {
+      case 4096: return launch_skinny_fp4m_t<OUT, 2, 2, 1>(a, s);
+      case 8192: return launch_skinny_fp4m_t<OUT, 4, 4, 1>(a, s);
+    }
+  } else {
+    switch (a.K) {
+      case 4096: return launch_skinny_fp4m_t<OUT, 2, 2, 2>(a, s);
+      case 8192: return launch_skinny_fp4m_t<OUT, 4, 4, 2>(a, s);
+    }
+  }
+  return (int)hipErrorInvalidValue;
+}
+
+const char* check_skinny_fp4m(const astergemm_config& c) {
+  if (c.M > 64) return "resident-activation MXFP4 path needs M <= 64";
+  if (c.K != 4096 && c.K != 8192)
+    return "resident-activation MXFP4 path for 16 < M <= 64 needs K = 4096 or 8192";
+  return nullptr;
+}
+
+#define AG_SKINNY_FP4M(name, OUT)                                                          \
+  Variant {                                                                                \
+    name, ASTERGEMM_KERNEL_SKINNY, ASTERGEMM_MXFP4, OUT, 64, 16, 512, 1, 8, 1, 2,           \
+        8 * 8192 + 65536, (const void*)gemm_skinny_fp4m_kernel<OUT, 2, 2, 2, 2>,           \
+        launch_skinny_fp4m<OUT>, check_skinny_fp4m                                         \
+  }
+
 // ---- 16 < M <= 64: the same persistent kernel with two activation tiles per wave --------
 //
 // A wave still owns a K slice of every row, now for 32 activation rows: MT * SPB * 2 = 128
@@ -1257,6 +1528,9 @@ const Variant kSkinnyVariants[] = {
     AG_SKINNY_LDS("skinnyx_fp8_m16_bf16", ASTERGEMM_FP8_E4M3, ASTERGEMM_BF16),
     AG_SKINNY_LDS("skinnyx_fp8_m16_f32", ASTERGEMM_FP8_E4M3, ASTERGEMM_F32),
     AG_SKINNY_LDS("skinnyx_fp8_m16_f16", ASTERGEMM_FP8_E4M3, ASTERGEMM_F16),
+    AG_SKINNY_FP4M("skinnyx_mxfp4_m64_bf16", ASTERGEMM_BF16),
+    AG_SKINNY_FP4M("skinnyx_mxfp4_m64_f32", ASTERGEMM_F32),
+    AG_SKINNY_FP4M("skinnyx_mxfp4_m64_f16", ASTERGEMM_F16),
     AG_SKINNY_FP4("skinnyx_mxfp4_m16_bf16", ASTERGEMM_BF16),
     AG_SKINNY_FP4("skinnyx_mxfp4_m16_f32", ASTERGEMM_F32),
     AG_SKINNY_FP4("skinnyx_mxfp4_m16_f16", ASTERGEMM_F16),

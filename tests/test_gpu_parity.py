@@ -335,6 +335,27 @@ def test_skinny_mxfp4_resident_activations(gpu, M, N, K, dtype_c):
         assert G.rel_l2(out[:, :N], tile) <= 1e-5
 
 
+@pytest.mark.parametrize("M,N,K", [(64, 14336, 4096), (17, 8, 4096), (33, 777, 8192), (48, 6000, 4096),
+                                   (32, 1000, 8192)])
+@pytest.mark.parametrize("dtype_c", ["bf16", "f32"])
+def test_skinny_mxfp4_up_to_64_rows(gpu, M, N, K, dtype_c):
+    a, b, extra = operands(M, N, K, "mxfp4", seed=45, b_std=0.05)
+    rng = np.random.default_rng(46)
+    extra["mx_a"] = (extra["mx_a"].astype(np.int32) + rng.integers(-3, 4, extra["mx_a"].shape)).astype(np.uint8)
+    extra["mx_b"] = (extra["mx_b"].astype(np.int32) + rng.integers(-3, 4, extra["mx_b"].shape)).astype(np.uint8)
+    bias = rng.standard_normal(N).astype(np.float32)
+    out, name = run_gemm(a, b, M, N, K, "mxfp4", dtype_c, bias=bias, ldc=N + 8, **extra)
+    assert name.startswith("skinnyx_mxfp4_m64")
+    want = G.gemm_mxfp4(a, extra["mx_a"], b, extra["mx_b"], out_dtype=_DT[dtype_c], bias=bias)
+    if dtype_c == "f32" or M * N >= 4096:
+        check(out, want, dtype_c, N, bar=1e-5 if dtype_c == "f32" else REL_L2_BAR)
+    else:
+        got, ref = G.output_to_f32(out[:, :N], _DT[dtype_c]), G.output_to_f32(want, _DT[dtype_c])
+        assert np.all(np.abs(got - ref) <= 2.0 ** -6 * np.abs(ref) + 1e-4 * np.abs(ref).max())
+    pad = out[:, N:]
+    assert np.isnan(pad).all() if dtype_c == "f32" else (pad == 0x7FC1).all()
+
+
 def test_skinny_fp8_falls_back_to_tile_kernels(gpu):
     # K outside the resident kernels' set, or M > 64: AUTO keeps the tile family
     for (M, N, K) in ((16, 256, 1024), (65, 256, 4096), (17, 256, 16384)):
