@@ -127,15 +127,16 @@ const Variant* choose(const astergemm_config& c, int* index_out) {
       else better = v->tile_m < best->tile_m || (v->tile_m == best->tile_m && v->rank > best->rank);
     } else {
       // Measured on MI355X (256 CUs): the 256 x 256 kernels (one workgroup per CU) win once
-      // they nearly fill the chip; below that the largest smaller tile that still gives
-      // about two workgroups per CU; for tiny problems the smallest tile.
+      // they nearly fill the chip; below that the 128 x 128 stream kernel (rank 2, two
+      // workgroups per CU) from about 0.8 workgroups per CU on, else the largest tile that
+      // still gives about two workgroups per CU; for tiny problems the smallest tile.
       auto wgs = [&](const Variant* x) {
         return ((c.M + x->tile_m - 1) / x->tile_m) * ((c.N + x->tile_n - 1) / x->tile_n);
       };
       auto tier = [&](const Variant* x) {
         const int area = x->tile_m * x->tile_n;
         if (area >= 256 * 256) return wgs(x) >= 230 ? 2 : -1;
-        return wgs(x) >= 448 ? 1 : 0;
+        return wgs(x) >= ((x->rank >= 2) ? 200 : 448) ? 1 : 0;
       };
       const int tv = tier(v), tb = tier(best);
       const int area = v->tile_m * v->tile_n, best_area = best->tile_m * best->tile_n;

@@ -126,7 +126,7 @@ const char* check_stream_whole_k(const astergemm_config& c) {
 #define AG_STREAM(name, DT, OUT, BM, BN, WM, WN)                                 \
   Variant {                                                                      \
     name, ASTERGEMM_KERNEL_TILE, DT, OUT, BM, BN, kRowBytes, WM, WN, 3,          \
-        (WM * WN == 8) ? 2 : 0, 5 * BM * kRowBytes,                                                      \
+        (WM * WN == 8 || BM == 128) ? 2 : 0, 5 * BM * kRowBytes,                \
         (const void*)gemm_stream_kernel<DT, OUT, BM, BN, WM, WN>,                \
         launch_stream<DT, OUT, BM, BN, WM, WN>,                                  \
         (WM * WN == 8) ? check_stream : check_stream_whole_k                     \
@@ -193,7 +193,10 @@ const char* check_stream4(const astergemm_config& c) {
   AG_STREAM(prefix "_256x256_w2x4_bf16", DT, ASTERGEMM_BF16, 256, 256, 2, 4),          \
       AG_STREAM(prefix "_256x256_w2x4_f32", DT, ASTERGEMM_F32, 256, 256, 2, 4),        \
       AG_STREAM(prefix "_256x256_w2x4_f16", DT, ASTERGEMM_F16, 256, 256, 2, 4),        \
-      AG_STREAM(prefix "_256x256_w2x2_bf16", DT, ASTERGEMM_BF16, 256, 256, 2, 2)
+      AG_STREAM(prefix "_256x256_w2x2_bf16", DT, ASTERGEMM_BF16, 256, 256, 2, 2),        \
+      AG_STREAM(prefix "_128x128_w2x2_bf16", DT, ASTERGEMM_BF16, 128, 128, 2, 2),        \
+      AG_STREAM(prefix "_128x128_w2x2_f32", DT, ASTERGEMM_F32, 128, 128, 2, 2),          \
+      AG_STREAM(prefix "_128x128_w2x2_f16", DT, ASTERGEMM_F16, 128, 128, 2, 2)
 
 const Variant kTileVariants[] = {
     AG_TILE_SET("tile_bf16", ASTERGEMM_BF16),

@@ -47,14 +47,20 @@ def test_select_headline_configs():
     for M, want in ((1, 117477376), (16, 118030336), (64, 119799808)):
         p = gemm.GemmPlan.create(M, 14336, 4096, "bf16", "bf16")
         assert p.info.family == _capi.KERNEL_SKINNY and p.info.bytes == want
-    # tile choice: 256 x 256 once it nearly fills the 256 CUs, else the largest smaller tile
-    # with about two workgroups per CU, else the smallest tile
-    for (M, N, K), want in (((256, 256, 256), (64, 64)), ((2048, 2048, 2048), (128, 64)),
-                            ((8192, 1024, 8192), (128, 128)), ((4096, 4096, 4096), (256, 256)),
-                            ((128, 14336, 4096), (64, 64)), ((3000, 5000, 7008), (256, 256))):
+    # tile choice: 256 x 256 once it nearly fills the 256 CUs, else the 128 x 128 stream kernel
+    # from 200 workgroups on, else the largest tile with about two workgroups per CU, else the
+    # smallest tile
+    for (M, N, K), want, kind in (((256, 256, 256), (64, 64), "tile"),
+                                  ((2048, 2048, 2048), (128, 128), "stream"),
+                                  ((8192, 1024, 8192), (128, 128), "stream"),
+                                  ((4096, 4096, 4096), (256, 256), "stream"),
+                                  ((128, 14336, 4096), (64, 64), "tile"),
+                                  ((3000, 5000, 7008), (256, 256), "stream"),
+                                  ((2044, 2044, 2048), (128, 64), "tile")):   # M, N not multiples of 8
         p = gemm.GemmPlan.create(M, N, K, "f16", "f32")
         assert p.info.family == _capi.KERNEL_TILE
         assert (p.info.wg_tile_m, p.info.wg_tile_n) == want, (M, N, K)
+        assert p.info.name.decode().startswith(kind), (M, N, K)
 
 
 def test_explicit_variant_and_enumeration():
