@@ -409,7 +409,7 @@ __device__ __forceinline__ void gemm_stream_body(const GemmArgs& p) {
   __builtin_amdgcn_sched_barrier(0);
   mfmas(S1{});
 
-  if constexpr (WM * WN == 8) {  // the four-wave variant has no registers to spare for it
+  if constexpr (WM * WN == 8 || BM == 128) {  // four waves on 256 x 256 have no registers to spare
     if (p.tail_granules) stream_k_tail<DT, BM, BN, WM, WN>(p, acc, wave, row0, col0, nk);
   }
   stream_epilogue<OUT, BM, BN, WM, WN>(p, acc, lds, wave, row0, col0);

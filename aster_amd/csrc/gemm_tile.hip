@@ -129,7 +129,7 @@ const char* check_stream_whole_k(const astergemm_config& c) {
         (WM * WN == 8 || BM == 128) ? 2 : 0, 5 * BM * kRowBytes,                \
         (const void*)gemm_stream_kernel<DT, OUT, BM, BN, WM, WN>,                \
         launch_stream<DT, OUT, BM, BN, WM, WN>,                                  \
-        (WM * WN == 8) ? check_stream : check_stream_whole_k                     \
+        (WM * WN == 8 || BM == 128) ? check_stream : check_stream_whole_k        \
   }
 
 template <int DT, int OUT, int BM, int BN, int WM, int WN>

@@ -737,6 +737,21 @@ def test_mxfp4_stream_kernel_edge_tiles(gpu, M, N, K, dtype_c):
     assert np.isnan(pad).all() if dtype_c == "f32" else (pad == 0x7FC1).all()
 
 
+@pytest.mark.parametrize("M,N,K", [(128, 128, 64), (264, 520, 136), (504, 1000, 1016), (1000, 264, 7008),
+                                   (2056, 1800, 256), (136, 128, 72)])
+@pytest.mark.parametrize("dtype_ab,dtype_c", [("bf16", "bf16"), ("f16", "f32")])
+def test_stream_kernel_128_tiles_edges_and_k_tails(gpu, M, N, K, dtype_ab, dtype_c):
+    a, b, _ = operands(M, N, K, dtype_ab, seed=81, b_std=0.05)
+    bias = np.random.default_rng(82).standard_normal(N).astype(np.float32)
+    out, name = run_gemm(a, b, M, N, K, dtype_ab, dtype_c, bias=bias, ldc=N + 16,
+                         family=_capi.KERNEL_TILE, wg_tile=(128, 128))
+    assert name.startswith("stream_") and "128x128" in name
+    want = G.gemm(a, b, _DT[dtype_ab], _DT[dtype_c], bias=bias)
+    check(out, want, dtype_c, N, bar=REL_L2_BAR if dtype_c != "f32" else 1e-5)
+    pad = out[:, N:]
+    assert np.isnan(pad).all() if dtype_c == "f32" else (pad == 0x7FC1).all()
+
+
 # ---- seeded random shapes through AUTO selection ------------------------------------------------
 
 def _random_cases(n_cases=96, seed=2024):
