@@ -133,10 +133,18 @@ const Variant* choose(const astergemm_config& c, int* index_out) {
       auto wgs = [&](const Variant* x) {
         return ((c.M + x->tile_m - 1) / x->tile_m) * ((c.N + x->tile_n - 1) / x->tile_n);
       };
+      // 256 x 256 from 230 workgroups on; already from 140 on when the dtype has no 128 x 128
+      // stream kernel, or when that kernel's last round (512 workgroups fill the chip) would
+      // be less than about a third full.  The 128 x 128 stream kernel from 200 workgroups on,
+      // from 128 on when rows are long (8 KiB and more: few prologues per byte streamed).
+      const int64_t g128 = ((c.M + 127) / 128) * ((c.N + 127) / 128);
+      const bool ragged_128 = g128 > 512 && g128 % 512 != 0 && g128 % 512 < 180;
+      const int thr256 = (!is16 || ragged_128) ? 140 : 230;
+      const int thr128s = row_bytes(c.dtype_ab, c.K) >= 8192 ? 128 : 200;
       auto tier = [&](const Variant* x) {
         const int area = x->tile_m * x->tile_n;
-        if (area >= 256 * 256) return wgs(x) >= 230 ? 2 : -1;
-        return wgs(x) >= ((x->rank >= 2) ? 200 : 448) ? 1 : 0;
+        if (area >= 256 * 256) return wgs(x) >= thr256 ? 2 : -1;
+        return wgs(x) >= ((x->rank >= 2) ? thr128s : 448) ? 1 : 0;
       };
       const int tv = tier(v), tb = tier(best);
       const int area = v->tile_m * v->tile_n, best_area = best->tile_m * best->tile_n;
@@ -381,6 +389,67 @@ int astergemm_bench_rotate(const astergemm_config* cfg, const astergemm_operands
   (void)hipEventDestroy(e1);
   if (le != 0) return hip_fail((hipError_t)le, v->name, __FILE__, __LINE__);
   *total_ns = (int64_t)((double)ms * 1e6);
+  return 0;
+}
+
+int astergemm_tune(const astergemm_config* cfg, const astergemm_operands* ops, int iters,
+                   int* best_variant, int64_t* best_ns, void* stream) {
+  if (!cfg || !ops || !best_variant || iters <= 0) {
+    set_error("astergemm_tune: bad argument");
+    return ASTERGEMM_EINVAL;
+  }
+  if (const char* why = validate_problem(*cfg)) {
+    set_error("astergemm: invalid config: %s", why);
+    return ASTERGEMM_EINVAL;
+  }
+  *best_variant = 0;
+  if (best_ns) *best_ns = 0;
+  hipStream_t s = (hipStream_t)stream;
+  hipEvent_t e0, e1;
+  AG_HIP(hipEventCreate(&e0));
+  AG_HIP(hipEventCreate(&e1));
+  double best = 0.0;
+  int rc = 0;
+  for (int i = 0; i < total_variants() && rc == 0; ++i) {
+    const Variant* v = variant_at(i);
+    // every variant that can run the config: right types, family if one is asked for, shape
+    // check passed, activation tile covering M on the weight-streaming path
+    if (!variant_matches_types(*v, *cfg) || v->check(*cfg)) continue;
+    if (cfg->family != ASTERGEMM_KERNEL_AUTO && cfg->family != v->family) continue;
+    if (v->family == ASTERGEMM_KERNEL_SKINNY && v->tile_m < cfg->M) continue;
+    if (cfg->M == 0 || cfg->N == 0) {
+      *best_variant = i + 1;
+      break;
+    }
+    GemmArgs a;
+    if ((rc = build_args(*v, *cfg, *ops, &a)) != 0) break;
+    const int grid = grid_of(*v, *cfg);
+    (void)hipGetLastError();
+    int le = 0;
+    for (int w = 0; w < 2 && le == 0; ++w) le = v->launch(a, grid, s);  // warm-up
+    if (le == 0) le = (int)hipEventRecord(e0, s);
+    for (int k = 0; k < iters && le == 0; ++k) le = v->launch(a, grid, s);
+    if (le == 0) le = (int)hipEventRecord(e1, s);
+    if (le == 0) le = (int)hipEventSynchronize(e1);
+    float ms = 0.f;
+    if (le == 0) le = (int)hipEventElapsedTime(&ms, e0, e1);
+    if (le != 0) {
+      rc = hip_fail((hipError_t)le, v->name, __FILE__, __LINE__);
+      break;
+    }
+    if (*best_variant == 0 || ms < best) {
+      best = ms;
+      *best_variant = i + 1;
+    }
+  }
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  if (rc != 0) return rc;
+  if (*best_variant == 0) {
+    set_error("astergemm_tune: no kernel variant can run this config");
+    return ASTERGEMM_ENOTSUP;
+  }
+  if (best_ns) *best_ns = (int64_t)(best * 1e6 / iters);
   return 0;
 }
 

@@ -167,6 +167,24 @@ class GemmPlan:
         return list(times)
 
 
+    def tune(self, dA: int, dB: int, dC: int, iters: int = 10, *, scale_a: int = None,
+             scale_b: int = None, mx_a: int = None, mx_b: int = None, bias: int = None,
+             stream: int = None) -> "GemmPlan":
+        """Times every variant that can run this plan's problem on the given operands and
+        returns a plan pinned to the fastest (`plan.tuned_ns` = its time per launch).  dC is
+        overwritten by every candidate."""
+        ops = self._operands(dA, dB, dC, scale_a, scale_b, mx_a, mx_b, bias)
+        cfg = _capi.Config.from_buffer_copy(self.config)
+        cfg.variant = 0
+        best, ns = ctypes.c_int(), ctypes.c_int64()
+        _capi.check(_capi.load().astergemm_tune(
+            ctypes.byref(cfg), ctypes.byref(ops), iters, ctypes.byref(best), ctypes.byref(ns),
+            ctypes.c_void_p(stream) if stream else None))
+        cfg.variant = best.value
+        plan = GemmPlan(cfg, select(cfg))
+        plan.tuned_ns = ns.value
+        return plan
+
     def bench_rotate(self, operand_sets, iters: int, stream: int = None) -> int:
         """`iters` back-to-back launches between one event pair, launch i on operand set
         i % len(operand_sets); each set is a dict with dA, dB, dC and optional scale_a,

@@ -186,6 +186,17 @@ int astergemm_bench(const astergemm_config* cfg, const astergemm_operands* ops,
 int astergemm_bench_rotate(const astergemm_config* cfg, const astergemm_operands* ops,
                            int n_ops, int iters, int64_t* total_ns, void* stream);
 
+/* Measures every variant that can run cfg on the given operands (`iters`
+ * back-to-back launches between one event pair each, after two warm-up
+ * launches) and returns the fastest: *best_variant is what cfg->variant takes
+ * to pin it, *best_ns (may be NULL) its time per launch.  cfg->family
+ * restricts the candidates when it is not AUTO; cfg->variant is ignored.  dC
+ * is overwritten by every candidate.  This is the reference's sweep step
+ * (run_single over a list of mappings, bench_harness.py:1738-1850, feeding
+ * tools/perf_best_known_update.py) on the prebuilt variants. */
+int astergemm_tune(const astergemm_config* cfg, const astergemm_operands* ops, int iters,
+                   int* best_variant, int64_t* best_ns, void* stream);
+
 /* Host pre-shuffle of B[N,K] 2-byte elements into per-lane MFMA order
  * (reference: shuffle_weight, contrib/kittens/test/kittens_helpers.py:90-119). */
 int astergemm_shuffle_weight_16(const uint16_t* src, uint16_t* dst, int64_t N,

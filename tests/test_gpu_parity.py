@@ -810,3 +810,32 @@ def test_random_shapes_through_auto_selection(gpu, dt, out_dt, M, N, K, with_bia
     if pad:
         tail = out[:, N:]
         assert np.isnan(tail).all() if out_dt == "f32" else (tail == 0x7FC1).all()
+
+
+@pytest.mark.parametrize("M,N,K,dt", [(512, 768, 1024, "bf16"), (16, 520, 4096, "bf16"), (300, 200, 512, "fp8_e4m3")])
+def test_tune_returns_a_runnable_variant_that_matches_the_oracle(gpu, M, N, K, dt):
+    a, b, extra = operands(M, N, K, dt, seed=91, b_std=0.05)
+    bufs = [GpuBuffer(x.nbytes) for x in (a, b)] + [GpuBuffer(M * N * 4)]
+    bufs[0].copy_from_host(np.ascontiguousarray(a))
+    bufs[1].copy_from_host(np.ascontiguousarray(b))
+    kw = {}
+    if dt == "fp8_e4m3":
+        sc = GpuBuffer(8)
+        sc.copy_from_host(np.array([extra["scale_a"], extra["scale_b"]], np.float32))
+        kw = dict(scale_a=sc.ptr_value, scale_b=sc.ptr_value + 4)
+    auto = AG.GemmPlan.create(M, N, K, dt, "f32")
+    print(f"tune {dt} M={M} N={N} K={K}", flush=True)
+    tuned = auto.tune(*(x.ptr_value for x in bufs), iters=5, **kw)
+    assert tuned.config.variant == tuned.info.variant > 0 and tuned.tuned_ns > 0
+    tuned.run(*(x.ptr_value for x in bufs), **kw)
+    out = np.empty((M, N), np.float32)
+    bufs[2].copy_to_host(out)
+    if dt == "fp8_e4m3":
+        want = G.gemm_fp8(a, b, extra["scale_a"], extra["scale_b"], out_dtype=G.F32)
+    else:
+        want = G.gemm(a, b, _DT[dt], G.F32)
+    assert G.rel_l2(out, G.output_to_f32(want, G.F32)) <= 1e-4
+    # restricting the family restricts the candidates
+    only_tile = AG.GemmPlan.create(M, N, K, dt, "f32", family=_capi.KERNEL_TILE).tune(
+        *(x.ptr_value for x in bufs), iters=3, **kw)
+    assert only_tile.info.family == _capi.KERNEL_TILE

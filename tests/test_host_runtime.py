@@ -42,6 +42,9 @@ def test_select_headline_configs():
     assert p.info.grid_x * p.info.wg_tile_m * p.info.wg_tile_n == 8192 * 8192
     p = gemm.GemmPlan.create(8192, 8192, 8192, "fp8_e4m3", "bf16")
     assert p.info.bytes == 268435464 and p.info.wg_tile_k == 128
+    # no 128 x 128 stream kernel for fp8: the 256 x 256 one from 140 workgroups on
+    assert gemm.GemmPlan.create(3072, 3072, 3072, "fp8_e4m3", "bf16").info.name.decode().startswith("stream_fp8")
+    assert gemm.GemmPlan.create(2048, 4096, 4096, "fp8_e4m3", "bf16").info.name.decode().startswith("tile_fp8_128x128")
     p = gemm.GemmPlan.create(4096, 14336, 4096, "mxfp4", "bf16")
     assert p.info.bytes == 157548544 and p.info.wg_tile_k == 256
     for M, want in ((1, 117477376), (16, 118030336), (64, 119799808)):
@@ -56,7 +59,10 @@ def test_select_headline_configs():
                                   ((4096, 4096, 4096), (256, 256), "stream"),
                                   ((128, 14336, 4096), (64, 64), "tile"),
                                   ((3000, 5000, 7008), (256, 256), "stream"),
-                                  ((2044, 2044, 2048), (128, 64), "tile")):   # M, N not multiples of 8
+                                  ((2044, 2044, 2048), (128, 64), "tile"),    # M, N not multiples of 8
+                                  ((3072, 3072, 3072), (256, 256), "stream"),  # 576 = 512 + 64 tiles of 128
+                                  ((2048, 4096, 4096), (128, 128), "stream"),
+                                  ((1536, 1536, 8192), (128, 128), "stream")):  # long rows
         p = gemm.GemmPlan.create(M, N, K, "f16", "f32")
         assert p.info.family == _capi.KERNEL_TILE
         assert (p.info.wg_tile_m, p.info.wg_tile_n) == want, (M, N, K)
