@@ -188,6 +188,14 @@ def shape_sweep(torch, dev):
         if dt == "bf16":
             a, b = a.bfloat16(), b.bfloat16()
             fn = lambda: torch.matmul(a, b.t())
+        elif dt == "mxfp4":
+            def rnd(shape, lo, hi, view):
+                return torch.randint(lo, hi, shape, device=dev, dtype=torch.uint8).view(view)
+            a = rnd((m, k // 2), 0, 256, torch.float4_e2m1fn_x2)
+            b = rnd((n, k // 2), 0, 256, torch.float4_e2m1fn_x2)
+            sa = rnd((m, k // 32), 124, 130, torch.float8_e8m0fnu)
+            sb = rnd((n, k // 32), 124, 130, torch.float8_e8m0fnu)
+            fn = lambda: torch._scaled_mm(a, b.t(), scale_a=sa, scale_b=sb, out_dtype=torch.bfloat16)
         else:
             a, b = a.to(torch.float8_e4m3fn), b.to(torch.float8_e4m3fn)
             one = torch.ones((), device=dev)
@@ -208,8 +216,10 @@ def shape_sweep(torch, dev):
         return _percentile(ts, 50)
 
     rows = []
-    for dt in ("bf16", "fp8_e4m3"):
+    for dt in ("bf16", "fp8_e4m3", "mxfp4"):
         for (m, n, k) in SWEEP_SHAPES:
+            if dt == "mxfp4" and k % 256:
+                continue                    # the MXFP4 kernels take whole 128-byte K steps
             a, b, keep = make_operands(torch, m, n, k, dt, dev)
             c = torch.empty(m, n, device=dev, dtype=torch.bfloat16)
             p = AG.GemmPlan.create(m, n, k, dt, "bf16")
