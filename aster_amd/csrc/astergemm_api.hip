@@ -172,16 +172,18 @@ const Variant* choose(const astergemm_config& c, int* index_out) {
 
 // Compute units of the current device (0 when there is none), cached.
 int device_cus() {
-  static int cus = -1;
-  if (cus < 0) {
+  static std::atomic<int> cus{-1};
+  int n = cus.load();
+  if (n < 0) {
     int dev = 0;
     hipDeviceProp_t prop;
     if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-      cus = prop.multiProcessorCount;
+      n = prop.multiProcessorCount;
     else
-      (void)hipGetLastError(), cus = 0;
+      (void)hipGetLastError(), n = 0;
+    cus.store(n);
   }
-  return cus;
+  return n;
 }
 
 int grid_of(const Variant& v, const astergemm_config& c) {

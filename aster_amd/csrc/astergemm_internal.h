@@ -1,5 +1,6 @@
 // Internal declarations shared by the HIP translation units of libastergemm.
 #pragma once
+#include <atomic>
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 

@@ -391,8 +391,8 @@ template <int DT, int OUT, int SPB>
 int launch_skinny_reg_t(const GemmArgs& a, hipStream_t s) {
   auto k = gemm_skinny_reg_kernel<DT, OUT, SPB>;
   constexpr int lds = 8 * 8192 + 2 * 4 * 8 * 64 * 16;
-  static bool attr_set = false;
-  static int cus = 0;
+  static std::atomic<bool> attr_set{false};
+  static std::atomic<int> cus{0};
   if (!attr_set) {
     hipError_t e =
         hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
@@ -405,7 +405,7 @@ int launch_skinny_reg_t(const GemmArgs& a, hipStream_t s) {
     attr_set = true;
   }
   const int nblocks = (int)((a.N + 15) / 16);
-  const int g = nblocks < cus ? nblocks : cus;
+  const int g = nblocks < cus.load() ? nblocks : cus.load();
   hipLaunchKernelGGL(k, dim3(g), dim3(512), lds, s, a);
   return (int)hipGetLastError();
 }
@@ -620,8 +620,8 @@ template <int OUT, int SPB, int SU>
 int launch_skinny_fp4_t(const GemmArgs& a, hipStream_t s) {
   auto k = gemm_skinny_fp4_kernel<OUT, SPB, SU>;
   constexpr int lds = 8 * 8192 + 2 * 4 * 8 * 64 * 16;
-  static bool attr_set = false;
-  static int cus = 0;
+  static std::atomic<bool> attr_set{false};
+  static std::atomic<int> cus{0};
   if (!attr_set) {
     hipError_t e =
         hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
@@ -634,7 +634,7 @@ int launch_skinny_fp4_t(const GemmArgs& a, hipStream_t s) {
     attr_set = true;
   }
   const int nblocks = (int)((a.N + 15) / 16);
-  const int g = nblocks < cus ? nblocks : cus;
+  const int g = nblocks < cus.load() ? nblocks : cus.load();
   hipLaunchKernelGGL(k, dim3(g), dim3(512), lds, s, a);
   return (int)hipGetLastError();
 }
@@ -884,8 +884,8 @@ int launch_skinny_fp4m_t(const GemmArgs& a, hipStream_t s) {
   constexpr int MT = 2;
   auto k = gemm_skinny_fp4m_kernel<OUT, SPB, SU, MT, MH>;
   constexpr int lds = 8 * 8192 + 2 * 2 * MT * 8 * 64 * 16;
-  static bool attr_set = false;
-  static int cus = 0;
+  static std::atomic<bool> attr_set{false};
+  static std::atomic<int> cus{0};
   if (!attr_set) {
     hipError_t e =
         hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
@@ -898,7 +898,7 @@ int launch_skinny_fp4m_t(const GemmArgs& a, hipStream_t s) {
     attr_set = true;
   }
   const int nblocks = (int)((a.N + 15) / 16) * MH;
-  int g = nblocks < cus ? nblocks : cus;
+  int g = nblocks < cus.load() ? nblocks : cus.load();
   if (MH == 2) g = g < 16 ? 16 : (g & ~15);
   hipLaunchKernelGGL(k, dim3(g), dim3(512), lds, s, a);
   return (int)hipGetLastError();
@@ -1151,8 +1151,8 @@ template <int DT, int OUT, int SPB, int MT, int MH>
 int launch_skinny_regm_t(const GemmArgs& a, hipStream_t s) {
   auto k = gemm_skinny_regm_kernel<DT, OUT, SPB, MT, MH>;
   constexpr int lds = 8 * 8192 + 2 * 2 * MT * 8 * 64 * 16;
-  static bool attr_set = false;
-  static int cus = 0;
+  static std::atomic<bool> attr_set{false};
+  static std::atomic<int> cus{0};
   if (!attr_set) {
     hipError_t e =
         hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
@@ -1166,7 +1166,7 @@ int launch_skinny_regm_t(const GemmArgs& a, hipStream_t s) {
   }
   // one workgroup per CU; with MH = 2 the grid is whole pairs on each of the 8 XCDs
   const int nblocks = (int)((a.N + 15) / 16) * MH;
-  int g = nblocks < cus ? nblocks : cus;
+  int g = nblocks < cus.load() ? nblocks : cus.load();
   if (MH == 2) g = g < 16 ? 16 : (g & ~15);
   hipLaunchKernelGGL(k, dim3(g), dim3(512), lds, s, a);
   return (int)hipGetLastError();
@@ -1412,8 +1412,8 @@ template <int DT, int OUT, int CPW>
 int launch_skinny_direct_t(const GemmArgs& a, hipStream_t s) {
   auto k = gemm_skinny_direct_kernel<DT, OUT, CPW>;
   constexpr int lds = 2 * 4 * 8 * 64 * 16 + 8 * 8192;
-  static bool attr_set = false;
-  static int cus = 0;
+  static std::atomic<bool> attr_set{false};
+  static std::atomic<int> cus{0};
   if (!attr_set) {
     hipError_t e =
         hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
@@ -1426,7 +1426,7 @@ int launch_skinny_direct_t(const GemmArgs& a, hipStream_t s) {
     attr_set = true;
   }
   const int nblocks = (int)((a.N + 15) / 16);
-  const int g = nblocks < cus ? nblocks : cus;
+  const int g = nblocks < cus.load() ? nblocks : cus.load();
   hipLaunchKernelGGL(k, dim3(g), dim3(512), lds, s, a);
   return (int)hipGetLastError();
 }

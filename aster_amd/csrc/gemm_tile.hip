@@ -13,7 +13,7 @@ template <int DT, int OUT, int BM, int BN, int WM, int WN>
 int launch_tile(const GemmArgs& a, int grid, hipStream_t s) {
   constexpr int lds = 2 * (BM + BN) * kRowBytes;
   auto k = gemm_tile_kernel<DT, OUT, BM, BN, WM, WN>;
-  static bool attr_set = false;
+  static std::atomic<bool> attr_set{false};
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute((const void*)k,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds);
@@ -60,7 +60,7 @@ template <int DT, int OUT, int BM, int BN, int WM, int WN>
 int launch_pipe(const GemmArgs& a0, int grid, hipStream_t s) {
   constexpr int lds = kStages * (BM + BN) * kSubBytes;
   auto k = gemm_pipe_kernel<DT, OUT, BM, BN, WM, WN>;
-  static bool attr_set = false;
+  static std::atomic<bool> attr_set{false};
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute((const void*)k,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds);
@@ -94,7 +94,7 @@ template <int DT, int OUT, int BM, int BN, int WM, int WN>
 int launch_stream(const GemmArgs& a, int grid, hipStream_t s) {
   constexpr int lds = 5 * BM * kRowBytes;
   auto k = gemm_stream_kernel<DT, OUT, BM, BN, WM, WN>;
-  static bool attr_set = false;
+  static std::atomic<bool> attr_set{false};
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute((const void*)k,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds);
@@ -136,7 +136,7 @@ template <int DT, int OUT, int BM, int BN, int WM, int WN>
 int launch_stream8(const GemmArgs& a, int grid, hipStream_t s) {
   constexpr int lds = 5 * BM * kRowBytes;
   auto k = gemm_stream8_kernel<DT, OUT, BM, BN, WM, WN>;
-  static bool attr_set = false;
+  static std::atomic<bool> attr_set{false};
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute((const void*)k,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds);
@@ -162,7 +162,7 @@ int launch_stream4(const GemmArgs& a, int grid, hipStream_t s) {
   if ((((uintptr_t)a.mx_a | (uintptr_t)a.mx_b) & 15) != 0 || a.mx_ld % 16 != 0)
     return (int)hipErrorInvalidValue;
   auto k = gemm_stream4_kernel<DT, OUT, BM, BN, WM, WN>;
-  static bool attr_set = false;
+  static std::atomic<bool> attr_set{false};
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute((const void*)k,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds);

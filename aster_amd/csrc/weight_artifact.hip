@@ -15,17 +15,18 @@ namespace {
 
 const char kMagic[8] = {'A', 'S', 'T', 'G', 'E', 'M', 'W', '\0'};
 
-uint32_t crc_table[256];
-bool crc_ready = false;
-
-void crc_init() {
-  for (uint32_t i = 0; i < 256; ++i) {
-    uint32_t c = i;
-    for (int k = 0; k < 8; ++k) c = (c & 1u) ? 0xEDB88320u ^ (c >> 1) : c >> 1;
-    crc_table[i] = c;
+// CRC-32 table (reflected polynomial 0xEDB88320), built at compile time
+struct CrcTable {
+  uint32_t v[256];
+  constexpr CrcTable() : v() {
+    for (uint32_t i = 0; i < 256; ++i) {
+      uint32_t c = i;
+      for (int k = 0; k < 8; ++k) c = (c & 1u) ? 0xEDB88320u ^ (c >> 1) : c >> 1;
+      v[i] = c;
+    }
   }
-  crc_ready = true;
-}
+};
+constexpr CrcTable kCrc{};
 
 int fail(const char* why) {
   astergemm::set_error("astergemm_weight: %s", why);
@@ -35,10 +36,9 @@ int fail(const char* why) {
 }  // namespace
 
 extern "C" uint32_t astergemm_weight_crc32(const void* data, size_t bytes) {
-  if (!crc_ready) crc_init();
   const uint8_t* p = (const uint8_t*)data;
   uint32_t c = 0xFFFFFFFFu;
-  for (size_t i = 0; i < bytes; ++i) c = crc_table[(c ^ p[i]) & 0xFFu] ^ (c >> 8);
+  for (size_t i = 0; i < bytes; ++i) c = kCrc.v[(c ^ p[i]) & 0xFFu] ^ (c >> 8);
   return c ^ 0xFFFFFFFFu;
 }
 
