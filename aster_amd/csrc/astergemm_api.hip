@@ -139,7 +139,8 @@ const Variant* choose(const astergemm_config& c, int* index_out) {
       // from 128 on when rows are long (8 KiB and more: few prologues per byte streamed).
       const int64_t g128 = ((c.M + 127) / 128) * ((c.N + 127) / 128);
       const bool ragged_128 = g128 > 512 && g128 % 512 != 0 && g128 % 512 < 180;
-      const int thr256 = (!is16 || ragged_128) ? 140 : 230;
+      const bool has_s128 = c.dtype_ab != ASTERGEMM_MXFP4;
+      const int thr256 = (!has_s128 || ragged_128) ? 140 : 230;
       const int thr128s = row_bytes(c.dtype_ab, c.K) >= 8192 ? 128 : 200;
       auto tier = [&](const Variant* x) {
         const int area = x->tile_m * x->tile_n;

@@ -35,11 +35,13 @@ __device__ __forceinline__ void gemm_stream8_body(const GemmArgs& p) {
   constexpr int SLOT = BM * kRowBytes;  // 32 KiB: one operand half of one K-step
   constexpr int LH = BM / 8 / NW;       // 1 KiB transfers per wave and slot
   constexpr int NMF = TM * TN;
-  constexpr int BAR = 20;               // MFMAs of a trip issued ahead of its barrier
+  // MFMAs of a trip issued ahead of its barrier: behind the last read of B(k), at MFMA
+  // (TN-2)*TM, and not behind the first read of K-step k+1, at MFMA (TN-1)*TM
+  constexpr int BAR = (TN - 2) * TM + (TM == 8 ? 4 : 1);
   static_assert(BM == BN, "the ring holds equal A and B halves");
   static_assert(DT == ASTERGEMM_FP8_E4M3, "fp8 operands");
   static_assert(BM % (8 * NW) == 0 && (8 * NW) % 16 == 0, "tile rows per wave");
-  static_assert(TM == 8 && TN == 4 && LH == 4, "side-instruction schedule below");
+  static_assert((TM == 8 || TM == 4) && TN == 4 && LH == 4, "side-instruction schedule below");
 
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
 
@@ -207,7 +209,8 @@ __device__ __forceinline__ void gemm_stream8_body(const GemmArgs& p) {
       __builtin_amdgcn_sched_barrier(0);
     });
   };
-  static_assert(BAR > 2 + LH && BAR > 16 && BAR + LH <= (TN - 1) * TM, "schedule positions");
+  static_assert(BAR > 2 + LH && BAR > (TN - 2) * TM && BAR <= (TN - 1) * TM && BAR + LH <= NMF,
+                "schedule positions");
   using T = std::true_type;
   using F = std::false_type;
   int k = 0, ia = 0, ib = 0;

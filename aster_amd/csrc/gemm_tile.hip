@@ -154,6 +154,13 @@ int launch_stream8(const GemmArgs& a, int grid, hipStream_t s) {
         (const void*)gemm_stream8_kernel<DT, OUT, 256, 256, 2, 4>,               \
         launch_stream8<DT, OUT, 256, 256, 2, 4>, check_stream                    \
   }
+#define AG_STREAM8_128(name, DT, OUT)                                            \
+  Variant {                                                                      \
+    name, ASTERGEMM_KERNEL_TILE, DT, OUT, 128, 128, kRowBytes, 2, 2, 3, 2,       \
+        5 * 128 * kRowBytes,                                                     \
+        (const void*)gemm_stream8_kernel<DT, OUT, 128, 128, 2, 2>,               \
+        launch_stream8<DT, OUT, 128, 128, 2, 2>, check_stream                    \
+  }
 
 template <int DT, int OUT, int BM, int BN, int WM, int WN>
 int launch_stream4(const GemmArgs& a, int grid, hipStream_t s) {
@@ -211,6 +218,9 @@ const Variant kTileVariants[] = {
     AG_STREAM8("stream_fp8_256x256_w2x4_bf16", ASTERGEMM_FP8_E4M3, ASTERGEMM_BF16),
     AG_STREAM8("stream_fp8_256x256_w2x4_f32", ASTERGEMM_FP8_E4M3, ASTERGEMM_F32),
     AG_STREAM8("stream_fp8_256x256_w2x4_f16", ASTERGEMM_FP8_E4M3, ASTERGEMM_F16),
+    AG_STREAM8_128("stream_fp8_128x128_w2x2_bf16", ASTERGEMM_FP8_E4M3, ASTERGEMM_BF16),
+    AG_STREAM8_128("stream_fp8_128x128_w2x2_f32", ASTERGEMM_FP8_E4M3, ASTERGEMM_F32),
+    AG_STREAM8_128("stream_fp8_128x128_w2x2_f16", ASTERGEMM_FP8_E4M3, ASTERGEMM_F16),
     AG_STREAM4("stream_mxfp4_256x256_w2x2_bf16", ASTERGEMM_MXFP4, ASTERGEMM_BF16),
     AG_STREAM4("stream_mxfp4_256x256_w2x2_f32", ASTERGEMM_MXFP4, ASTERGEMM_F32),
     AG_STREAM4("stream_mxfp4_256x256_w2x2_f16", ASTERGEMM_MXFP4, ASTERGEMM_F16),

@@ -586,6 +586,16 @@ def test_stream_kernel_every_ring_phase(gpu, K):
     check(out, G.gemm(a, b, G.BF16, G.F32), "f32", 512, bar=1e-5)
 
 
+@pytest.mark.parametrize("ksteps", list(range(1, 14)))
+def test_fp8_stream_kernel_128_every_ring_phase(gpu, ksteps):
+    M, N, K = 128, 256, 128 * ksteps
+    a, b, ex = operands(M, N, K, "fp8_e4m3", seed=19, b_std=1.0)
+    out, name = run_gemm(a, b, M, N, K, "fp8_e4m3", "f32", family=_capi.KERNEL_TILE,
+                         wg_tile=(128, 128), **ex)
+    assert name.startswith("stream_fp8_128")
+    check(out, G.gemm_fp8(a, b, ex["scale_a"], ex["scale_b"], out_dtype=G.F32), "f32", N, bar=1e-4)
+
+
 @pytest.mark.parametrize("ksteps", list(range(1, 16)) + [20, 21])
 def test_fp8_stream_kernel_every_ring_phase(gpu, ksteps):
     # 128-byte K-steps 1..15, 20, 21: prologue only, every tail length of the six-trip slot
@@ -610,7 +620,7 @@ def test_fp8_stream_and_tile_kernels_pair_granules_consistently(gpu):
     a, sa = F.quantize_fp8_tensor(xa)
     b, sb = F.quantize_fp8_tensor(xb)
     want = G.gemm(a, b, G.FP8_E4M3, G.F32, scale_a=sa, scale_b=sb)
-    for tile, prefix in ((256, "stream_fp8"), (128, "tile_fp8")):
+    for tile, prefix in ((256, "stream_fp8_256"), (128, "stream_fp8_128"), (64, "tile_fp8")):
         out, name = run_gemm(a, b, M, N, K, "fp8_e4m3", "f32", scale_a=sa, scale_b=sb,
                              family=_capi.KERNEL_TILE, wg_tile=(tile, tile))
         assert name.startswith(prefix)
@@ -739,15 +749,22 @@ def test_mxfp4_stream_kernel_edge_tiles(gpu, M, N, K, dtype_c):
 
 @pytest.mark.parametrize("M,N,K", [(128, 128, 64), (264, 520, 136), (504, 1000, 1016), (1000, 264, 7008),
                                    (2056, 1800, 256), (136, 128, 72)])
-@pytest.mark.parametrize("dtype_ab,dtype_c", [("bf16", "bf16"), ("f16", "f32")])
+@pytest.mark.parametrize("dtype_ab,dtype_c", [("bf16", "bf16"), ("f16", "f32"), ("fp8_e4m3", "bf16"),
+                                              ("fp8_e4m3", "f32")])
 def test_stream_kernel_128_tiles_edges_and_k_tails(gpu, M, N, K, dtype_ab, dtype_c):
-    a, b, _ = operands(M, N, K, dtype_ab, seed=81, b_std=0.05)
+    if dtype_ab == "fp8_e4m3":
+        K = (K + 15) // 16 * 16 * 2       # whole granules, and a few more K steps
+    a, b, extra = operands(M, N, K, dtype_ab, seed=81, b_std=0.05)
     bias = np.random.default_rng(82).standard_normal(N).astype(np.float32)
     out, name = run_gemm(a, b, M, N, K, dtype_ab, dtype_c, bias=bias, ldc=N + 16,
-                         family=_capi.KERNEL_TILE, wg_tile=(128, 128))
+                         family=_capi.KERNEL_TILE, wg_tile=(128, 128), **extra)
     assert name.startswith("stream_") and "128x128" in name
-    want = G.gemm(a, b, _DT[dtype_ab], _DT[dtype_c], bias=bias)
-    check(out, want, dtype_c, N, bar=REL_L2_BAR if dtype_c != "f32" else 1e-5)
+    if dtype_ab == "fp8_e4m3":
+        want = G.gemm_fp8(a, b, extra["scale_a"], extra["scale_b"], out_dtype=_DT[dtype_c], bias=bias)
+        check(out, want, dtype_c, N, bar=REL_L2_BAR if dtype_c != "f32" else 1e-4)
+    else:
+        want = G.gemm(a, b, _DT[dtype_ab], _DT[dtype_c], bias=bias)
+        check(out, want, dtype_c, N, bar=REL_L2_BAR if dtype_c != "f32" else 1e-5)
     pad = out[:, N:]
     assert np.isnan(pad).all() if dtype_c == "f32" else (pad == 0x7FC1).all()
 
