@@ -133,14 +133,13 @@ const Variant* choose(const astergemm_config& c, int* index_out) {
       auto wgs = [&](const Variant* x) {
         return ((c.M + x->tile_m - 1) / x->tile_m) * ((c.N + x->tile_n - 1) / x->tile_n);
       };
-      // 256 x 256 from 230 workgroups on; already from 140 on when the dtype has no 128 x 128
-      // stream kernel, or when that kernel's last round (512 workgroups fill the chip) would
-      // be less than about a third full.  The 128 x 128 stream kernel from 200 workgroups on,
+      // 256 x 256 from 230 workgroups on; already from 140 on when the last round of the
+      // 128 x 128 stream kernel (512 workgroups fill the chip) would be less than about a
+      // third full.  The 128 x 128 stream kernel from 200 workgroups on,
       // from 128 on when rows are long (8 KiB and more: few prologues per byte streamed).
       const int64_t g128 = ((c.M + 127) / 128) * ((c.N + 127) / 128);
       const bool ragged_128 = g128 > 512 && g128 % 512 != 0 && g128 % 512 < 180;
-      const bool has_s128 = c.dtype_ab != ASTERGEMM_MXFP4;
-      const int thr256 = (!has_s128 || ragged_128) ? 140 : 230;
+      const int thr256 = ragged_128 ? 140 : 230;
       const int thr128s = row_bytes(c.dtype_ab, c.K) >= 8192 ? 128 : 200;
       auto tier = [&](const Variant* x) {
         const int area = x->tile_m * x->tile_n;

@@ -44,14 +44,16 @@ __device__ __forceinline__ void gemm_stream4_body(const GemmArgs& p) {
   constexpr int LH = BM / 8 / NW;       // 1 KiB transfers per wave and slot
   constexpr int NMF = TM * TN;          // slots per trip (two MFMAs each)
   constexpr int BAR = (TN - 2) * TM + 4;  // slots of a trip issued ahead of its barrier
-  constexpr int NSC = 8 / NW;           // scale transfers per wave and chunk
+  constexpr int NSR = BM / 64;          // scale transfers per operand and chunk (64 rows each)
+  constexpr int NSC = 2 * NSR / NW;     // scale transfers per wave and chunk
   constexpr int SC_A = 4 * SLOT;        // A scales: [2 buffers][256 rows][16 bytes]
   constexpr int SC_B = SC_A + 2 * BM * 16;
   static_assert(BM == BN, "the ring holds equal A and B halves");
   static_assert(DT == ASTERGEMM_MXFP4, "fp4 operands");
   static_assert(BM % (8 * NW) == 0 && (8 * NW) % 16 == 0, "tile rows per wave");
-  static_assert(TM % 2 == 0 && TM >= 4 && TN >= 2 && 8 % NW == 0, "side-instruction schedule below");
-  static_assert(BM == 4 * 64, "eight scale transfers per chunk: four cover A, four cover B");
+  static_assert(TM % 2 == 0 && TM >= 4 && TN >= 2 && (2 * NSR) % NW == 0 && NSC >= 1,
+                "side-instruction schedule below");
+  static_assert(BM % 64 == 0, "scale transfers cover 64 rows each");
 
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
 
@@ -100,14 +102,14 @@ __device__ __forceinline__ void gemm_stream4_body(const GemmArgs& p) {
 #pragma unroll
   for (int i = 0; i < NSC; ++i) {
     const int t = wave + i * NW;
-    const bool is_a = t < 4;
+    const bool is_a = t < NSR;
     sc_base[i] = is_a ? p.mx_a + (int64_t)row0 * p.mx_ld : p.mx_b + (int64_t)col0 * p.mx_ld;
     // rows past the end of an edge tile re-read the operand's last row
     const int first = is_a ? row0 : col0, rows = is_a ? p.M : p.N;
-    int r = (t & 3) * 64 + lane;
+    int r = (t % NSR) * 64 + lane;
     r = first + r < rows ? r : rows - 1 - first;
     sc_off[i] = (unsigned)(r * p.mx_ld);
-    sc_lds[i] = lds + (is_a ? SC_A : SC_B) + (t & 3) * 64 * 16;
+    sc_lds[i] = lds + (is_a ? SC_A : SC_B) + (t % NSR) * 64 * 16;
   }
   auto issue_scales = [&](int c) {
 #pragma unroll

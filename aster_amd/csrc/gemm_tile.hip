@@ -195,6 +195,13 @@ const char* check_stream4(const astergemm_config& c) {
         (const void*)gemm_stream4_kernel<DT, OUT, 256, 256, 2, 2>,               \
         launch_stream4<DT, OUT, 256, 256, 2, 2>, check_stream4                   \
   }
+#define AG_STREAM4_128(name, DT, OUT)                                            \
+  Variant {                                                                      \
+    name, ASTERGEMM_KERNEL_TILE, DT, OUT, 128, 128, kRowBytes, 2, 2, 2, 2,       \
+        4 * 128 * kRowBytes + 4 * 128 * 16,                                      \
+        (const void*)gemm_stream4_kernel<DT, OUT, 128, 128, 2, 2>,               \
+        launch_stream4<DT, OUT, 128, 128, 2, 2>, check_stream4                   \
+  }
 
 #define AG_STREAM_SET(prefix, DT)                                                      \
   AG_STREAM(prefix "_256x256_w2x4_bf16", DT, ASTERGEMM_BF16, 256, 256, 2, 4),          \
@@ -224,6 +231,9 @@ const Variant kTileVariants[] = {
     AG_STREAM4("stream_mxfp4_256x256_w2x2_bf16", ASTERGEMM_MXFP4, ASTERGEMM_BF16),
     AG_STREAM4("stream_mxfp4_256x256_w2x2_f32", ASTERGEMM_MXFP4, ASTERGEMM_F32),
     AG_STREAM4("stream_mxfp4_256x256_w2x2_f16", ASTERGEMM_MXFP4, ASTERGEMM_F16),
+    AG_STREAM4_128("stream_mxfp4_128x128_w2x2_bf16", ASTERGEMM_MXFP4, ASTERGEMM_BF16),
+    AG_STREAM4_128("stream_mxfp4_128x128_w2x2_f32", ASTERGEMM_MXFP4, ASTERGEMM_F32),
+    AG_STREAM4_128("stream_mxfp4_128x128_w2x2_f16", ASTERGEMM_MXFP4, ASTERGEMM_F16),
 };
 
 }  // namespace

@@ -656,7 +656,8 @@ def test_bench_rotate_uses_every_operand_set(gpu):
 
 
 @pytest.mark.parametrize("ksteps", [2, 4, 6, 8, 10, 12, 14])
-def test_mxfp4_stream_kernel_every_loop_phase(gpu, ksteps):
+@pytest.mark.parametrize("tile", [256, 128])
+def test_mxfp4_stream_kernel_every_loop_phase(gpu, ksteps, tile):
     # 256-element K-steps in pairs (scales travel two K-steps at a time): final parts only,
     # the block before them, and one to five steady iterations; random nibbles and random
     # per-block scales, so a wrong block <-> scale byte pairing cannot cancel
@@ -667,8 +668,8 @@ def test_mxfp4_stream_kernel_every_loop_phase(gpu, ksteps):
     mxa = rng.integers(118, 134, (M, K // 32)).astype(np.uint8)
     mxb = rng.integers(118, 134, (N, K // 32)).astype(np.uint8)
     out, name = run_gemm(a, b, M, N, K, "mxfp4", "f32", mx_a=mxa, mx_b=mxb,
-                         family=_capi.KERNEL_TILE, wg_tile=(256, 256))
-    assert name.startswith("stream_mxfp4")
+                         family=_capi.KERNEL_TILE, wg_tile=(tile, tile))
+    assert name.startswith(f"stream_mxfp4_{tile}")
     check(out, G.gemm_mxfp4(a, mxa, b, mxb, out_dtype=G.F32), "f32", N, bar=1e-5)
 
 
@@ -728,15 +729,16 @@ def test_linalg_matmul_kxn(gpu, M, N, K):
 
 @pytest.mark.parametrize("M,N,K", [(264, 520, 512), (504, 1000, 1024), (1000, 264, 1536), (8, 8, 512)])
 @pytest.mark.parametrize("dtype_c", ["bf16", "f32"])
-def test_mxfp4_stream_kernel_edge_tiles(gpu, M, N, K, dtype_c):
+@pytest.mark.parametrize("tile", [256, 128])
+def test_mxfp4_stream_kernel_edge_tiles(gpu, M, N, K, dtype_c, tile):
     a, b, extra = operands(M, N, K, "mxfp4", seed=71, b_std=0.05)
     rng = np.random.default_rng(72)
     extra["mx_a"] = (extra["mx_a"].astype(np.int32) + rng.integers(-3, 4, extra["mx_a"].shape)).astype(np.uint8)
     extra["mx_b"] = (extra["mx_b"].astype(np.int32) + rng.integers(-3, 4, extra["mx_b"].shape)).astype(np.uint8)
     bias = rng.standard_normal(N).astype(np.float32)
     out, name = run_gemm(a, b, M, N, K, "mxfp4", dtype_c, bias=bias, ldc=N + 16,
-                         family=_capi.KERNEL_TILE, wg_tile=(256, 256), **extra)
-    assert name.startswith("stream_mxfp4")
+                         family=_capi.KERNEL_TILE, wg_tile=(tile, tile), **extra)
+    assert name.startswith(f"stream_mxfp4_{tile}")
     want = G.gemm_mxfp4(a, extra["mx_a"], b, extra["mx_b"], out_dtype=_DT[dtype_c], bias=bias)
     if M * N >= 4096:
         check(out, want, dtype_c, N, bar=1e-5 if dtype_c == "f32" else REL_L2_BAR)
