@@ -140,9 +140,15 @@ const Variant* choose(const astergemm_config& c, int* index_out) {
       const int64_t g128 = ((c.M + 127) / 128) * ((c.N + 127) / 128);
       const bool ragged_128 = g128 > 512 && g128 % 512 != 0 && g128 % 512 < 180;
       const int thr256 = ragged_128 ? 140 : 230;
-      const int thr128s = row_bytes(c.dtype_ab, c.K) >= 8192 ? 128 : 200;
+      // MXFP4: the generic tile kernels are weak next to the stream kernels, so the 128 x 128
+      // stream kernel from 16 workgroups on when K >= 4096, and instead of the 256 x 256 one
+      // (long prologue: two K-steps and their scales) when K < 4096
+      const bool fp4 = c.dtype_ab == ASTERGEMM_MXFP4;
+      const int thr128s = fp4 ? (c.K >= 4096 ? 16 : 200)
+                              : (row_bytes(c.dtype_ab, c.K) >= 8192 ? 128 : 200);
       auto tier = [&](const Variant* x) {
         const int area = x->tile_m * x->tile_n;
+        if (area >= 256 * 256 && fp4 && c.K < 4096 && c.K % 512 == 0) return -1;
         if (area >= 256 * 256) return wgs(x) >= thr256 ? 2 : -1;
         return wgs(x) >= ((x->rank >= 2) ? thr128s : 448) ? 1 : 0;
       };

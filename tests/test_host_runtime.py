@@ -44,7 +44,9 @@ def test_select_headline_configs():
     assert p.info.bytes == 268435464 and p.info.wg_tile_k == 128
     assert gemm.GemmPlan.create(3072, 3072, 3072, "fp8_e4m3", "bf16").info.name.decode().startswith("stream_fp8_256")
     assert gemm.GemmPlan.create(2048, 4096, 4096, "fp8_e4m3", "bf16").info.name.decode().startswith("stream_fp8_128")
-    assert gemm.GemmPlan.create(3072, 3072, 3072, "mxfp4", "bf16").info.name.decode().startswith("stream_mxfp4_256")
+    assert gemm.GemmPlan.create(3072, 3072, 3072, "mxfp4", "bf16").info.name.decode().startswith("stream_mxfp4_128")
+    assert gemm.GemmPlan.create(4096, 14336, 4096, "mxfp4", "bf16").info.name.decode().startswith("stream_mxfp4_256")
+    assert gemm.GemmPlan.create(96, 4096, 4096, "mxfp4", "bf16").info.name.decode().startswith("stream_mxfp4_128")
     assert gemm.GemmPlan.create(2048, 4096, 4096, "mxfp4", "bf16").info.name.decode().startswith("stream_mxfp4_128")
     p = gemm.GemmPlan.create(4096, 14336, 4096, "mxfp4", "bf16")
     assert p.info.bytes == 157548544 and p.info.wg_tile_k == 256
