@@ -21,7 +21,7 @@ LIB_DIR = os.path.join(PKG_DIR, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libastergemm.so")
 OBJ_DIR = os.path.join(ROOT, "build", "obj")
 
-SOURCES = ["gemm_tile.hip", "gemm_skinny.hip", "astergemm_api.hip", "quantize.hip",
+SOURCES = ["gemm_tile.hip", "gemm_stream.hip", "gemm_skinny.hip", "astergemm_api.hip", "quantize.hip",
            "weight_artifact.hip"]
 HSACO_SOURCE = "hsaco_kernels.hip"
 HSACO_PATH = os.path.join(LIB_DIR, "astergemm_kernels.hsaco")

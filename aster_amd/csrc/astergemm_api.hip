@@ -30,12 +30,16 @@ int hip_fail(hipError_t e, const char* what, const char* file, int line) {
 
 namespace {
 
-int total_variants() { return num_tile_variants() + num_skinny_variants(); }
+int total_variants() {
+  return num_tile_variants() + num_stream_variants() + num_skinny_variants();
+}
 
 const Variant* variant_at(int index) {
   if (index < 0) return nullptr;
   if (index < num_tile_variants()) return tile_variants() + index;
   index -= num_tile_variants();
+  if (index < num_stream_variants()) return stream_variants() + index;
+  index -= num_stream_variants();
   if (index < num_skinny_variants()) return skinny_variants() + index;
   return nullptr;
 }

@@ -65,6 +65,8 @@ struct Variant {
 
 int num_tile_variants();
 const Variant* tile_variants();
+int num_stream_variants();
+const Variant* stream_variants();
 int num_skinny_variants();
 const Variant* skinny_variants();
 

@@ -1,0 +1,155 @@
+// Stream kernels (whole-ring, hand-scheduled MFMA loops) for f16 / bf16, fp8 and MXFP4:
+// launchers, shape checks and the variant table.  Kept apart from gemm_tile.hip so that the
+// two halves of the kernel set compile side by side.
+#include "gemm_stream_kernel.hpp"
+#include "gemm_stream8_kernel.hpp"
+#include "gemm_stream4_kernel.hpp"
+
+namespace astergemm {
+namespace {
+
+template <int DT, int OUT, int BM, int BN, int WM, int WN>
+int launch_stream(const GemmArgs& a, int grid, hipStream_t s) {
+  constexpr int lds = 5 * BM * kRowBytes;
+  auto k = gemm_stream_kernel<DT, OUT, BM, BN, WM, WN>;
+  static std::atomic<bool> attr_set{false};
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)k,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess) return (int)e;
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(k, dim3(grid), dim3(WM * WN * 64), lds, s, a);
+  return (int)hipGetLastError();
+}
+
+// Whole 256x256 tiles and whole 128-byte K-steps only; other shapes go to the
+// general tile kernel.
+const char* check_stream(const astergemm_config& c) {
+  // edge tiles are handled in units of 8 operand rows and 16-byte output chunks
+  if (c.M % 8 != 0 || c.N % 8 != 0 || c.M < 8 || c.N < 8) return "M and N must be multiples of 8";
+  // a K tail of 1..7 granules is multiplied after the loop; at least one whole step is needed
+  if (row_bytes(c.dtype_ab, c.K) % 16 != 0) return "K must cover a whole number of 16-byte granules";
+  if (row_bytes(c.dtype_ab, c.K) < kRowBytes) return "K must cover at least one 128-byte row chunk";
+  if (c.ldc % 8 != 0) return "ldc must be a multiple of 8 elements";
+  return nullptr;
+}
+
+const char* check_stream_whole_k(const astergemm_config& c) {
+  if (const char* why = check_stream(c)) return why;
+  if (row_bytes(c.dtype_ab, c.K) % kRowBytes != 0) return "K must fill whole 128-byte row chunks";
+  return nullptr;
+}
+
+#define AG_STREAM(name, DT, OUT, BM, BN, WM, WN)                                 \
+  Variant {                                                                      \
+    name, ASTERGEMM_KERNEL_TILE, DT, OUT, BM, BN, kRowBytes, WM, WN, 3,          \
+        (WM * WN == 8 || BM == 128) ? 2 : 0, 5 * BM * kRowBytes,                \
+        (const void*)gemm_stream_kernel<DT, OUT, BM, BN, WM, WN>,                \
+        launch_stream<DT, OUT, BM, BN, WM, WN>,                                  \
+        (WM * WN == 8 || BM == 128) ? check_stream : check_stream_whole_k        \
+  }
+
+template <int DT, int OUT, int BM, int BN, int WM, int WN>
+int launch_stream8(const GemmArgs& a, int grid, hipStream_t s) {
+  constexpr int lds = 5 * BM * kRowBytes;
+  auto k = gemm_stream8_kernel<DT, OUT, BM, BN, WM, WN>;
+  static std::atomic<bool> attr_set{false};
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)k,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess) return (int)e;
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(k, dim3(grid), dim3(WM * WN * 64), lds, s, a);
+  return (int)hipGetLastError();
+}
+
+#define AG_STREAM8(name, DT, OUT)                                                \
+  Variant {                                                                      \
+    name, ASTERGEMM_KERNEL_TILE, DT, OUT, 256, 256, kRowBytes, 2, 4, 3, 2,       \
+        5 * 256 * kRowBytes,                                                     \
+        (const void*)gemm_stream8_kernel<DT, OUT, 256, 256, 2, 4>,               \
+        launch_stream8<DT, OUT, 256, 256, 2, 4>, check_stream                    \
+  }
+#define AG_STREAM8_128(name, DT, OUT)                                            \
+  Variant {                                                                      \
+    name, ASTERGEMM_KERNEL_TILE, DT, OUT, 128, 128, kRowBytes, 2, 2, 3, 2,       \
+        5 * 128 * kRowBytes,                                                     \
+        (const void*)gemm_stream8_kernel<DT, OUT, 128, 128, 2, 2>,               \
+        launch_stream8<DT, OUT, 128, 128, 2, 2>, check_stream                    \
+  }
+
+template <int DT, int OUT, int BM, int BN, int WM, int WN>
+int launch_stream4(const GemmArgs& a, int grid, hipStream_t s) {
+  constexpr int lds = 4 * BM * kRowBytes + 4 * BM * 16;
+  // the scale planes are fetched in 16-byte granules
+  if ((((uintptr_t)a.mx_a | (uintptr_t)a.mx_b) & 15) != 0 || a.mx_ld % 16 != 0)
+    return (int)hipErrorInvalidValue;
+  auto k = gemm_stream4_kernel<DT, OUT, BM, BN, WM, WN>;
+  static std::atomic<bool> attr_set{false};
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)k,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess) return (int)e;
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(k, dim3(grid), dim3(WM * WN * 64), lds, s, a);
+  return (int)hipGetLastError();
+}
+
+// Whole 256x256 tiles and an even number of 256-element K-steps (scales move in 16-byte
+// granules = two K-steps of a row).
+const char* check_stream4(const astergemm_config& c) {
+  if (const char* why = check_stream_whole_k(c)) return why;
+  if (c.K % 512 != 0) return "K must be a multiple of 512";
+  return nullptr;
+}
+
+#define AG_STREAM4(name, DT, OUT)                                                \
+  Variant {                                                                      \
+    name, ASTERGEMM_KERNEL_TILE, DT, OUT, 256, 256, kRowBytes, 2, 2, 2, 2,       \
+        4 * 256 * kRowBytes + 4 * 256 * 16,                                      \
+        (const void*)gemm_stream4_kernel<DT, OUT, 256, 256, 2, 2>,               \
+        launch_stream4<DT, OUT, 256, 256, 2, 2>, check_stream4                   \
+  }
+#define AG_STREAM4_128(name, DT, OUT)                                            \
+  Variant {                                                                      \
+    name, ASTERGEMM_KERNEL_TILE, DT, OUT, 128, 128, kRowBytes, 2, 2, 2, 2,       \
+        4 * 128 * kRowBytes + 4 * 128 * 16,                                      \
+        (const void*)gemm_stream4_kernel<DT, OUT, 128, 128, 2, 2>,               \
+        launch_stream4<DT, OUT, 128, 128, 2, 2>, check_stream4                   \
+  }
+
+#define AG_STREAM_SET(prefix, DT)                                                      \
+  AG_STREAM(prefix "_256x256_w2x4_bf16", DT, ASTERGEMM_BF16, 256, 256, 2, 4),          \
+      AG_STREAM(prefix "_256x256_w2x4_f32", DT, ASTERGEMM_F32, 256, 256, 2, 4),        \
+      AG_STREAM(prefix "_256x256_w2x4_f16", DT, ASTERGEMM_F16, 256, 256, 2, 4),        \
+      AG_STREAM(prefix "_256x256_w2x2_bf16", DT, ASTERGEMM_BF16, 256, 256, 2, 2),        \
+      AG_STREAM(prefix "_128x128_w2x2_bf16", DT, ASTERGEMM_BF16, 128, 128, 2, 2),        \
+      AG_STREAM(prefix "_128x128_w2x2_f32", DT, ASTERGEMM_F32, 128, 128, 2, 2),          \
+      AG_STREAM(prefix "_128x128_w2x2_f16", DT, ASTERGEMM_F16, 128, 128, 2, 2)
+
+const Variant kStreamVariants[] = {
+    AG_STREAM_SET("stream_bf16", ASTERGEMM_BF16),
+    AG_STREAM_SET("stream_f16", ASTERGEMM_F16),
+    AG_STREAM8("stream_fp8_256x256_w2x4_bf16", ASTERGEMM_FP8_E4M3, ASTERGEMM_BF16),
+    AG_STREAM8("stream_fp8_256x256_w2x4_f32", ASTERGEMM_FP8_E4M3, ASTERGEMM_F32),
+    AG_STREAM8("stream_fp8_256x256_w2x4_f16", ASTERGEMM_FP8_E4M3, ASTERGEMM_F16),
+    AG_STREAM8_128("stream_fp8_128x128_w2x2_bf16", ASTERGEMM_FP8_E4M3, ASTERGEMM_BF16),
+    AG_STREAM8_128("stream_fp8_128x128_w2x2_f32", ASTERGEMM_FP8_E4M3, ASTERGEMM_F32),
+    AG_STREAM8_128("stream_fp8_128x128_w2x2_f16", ASTERGEMM_FP8_E4M3, ASTERGEMM_F16),
+    AG_STREAM4("stream_mxfp4_256x256_w2x2_bf16", ASTERGEMM_MXFP4, ASTERGEMM_BF16),
+    AG_STREAM4("stream_mxfp4_256x256_w2x2_f32", ASTERGEMM_MXFP4, ASTERGEMM_F32),
+    AG_STREAM4("stream_mxfp4_256x256_w2x2_f16", ASTERGEMM_MXFP4, ASTERGEMM_F16),
+    AG_STREAM4_128("stream_mxfp4_128x128_w2x2_bf16", ASTERGEMM_MXFP4, ASTERGEMM_BF16),
+    AG_STREAM4_128("stream_mxfp4_128x128_w2x2_f32", ASTERGEMM_MXFP4, ASTERGEMM_F32),
+    AG_STREAM4_128("stream_mxfp4_128x128_w2x2_f16", ASTERGEMM_MXFP4, ASTERGEMM_F16),
+};
+
+}  // namespace
+
+int num_stream_variants() { return (int)(sizeof(kStreamVariants) / sizeof(kStreamVariants[0])); }
+const Variant* stream_variants() { return kStreamVariants; }
+
+}  // namespace astergemm
