@@ -263,7 +263,7 @@ def main() -> int:
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on ONE GPU; --gpus N with N > 1 is not supported "
-              "(the path shards over N by splitting B's rows, see DESIGN.md)", file=sys.stderr)
+              "(the path would shard over GPUs by splitting B's rows, one slice of C per GPU, no communication)", file=sys.stderr)
         return 2
 
     import torch
