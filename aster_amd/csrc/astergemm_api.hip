@@ -96,8 +96,8 @@ const Variant* choose(const astergemm_config& c, int* index_out) {
   int family = c.family;
   if (family == ASTERGEMM_KERNEL_AUTO)
     family = ((is16 && c.M <= 64 && c.K % 32 == 0) ||
-              (c.dtype_ab == ASTERGEMM_FP8_E4M3 &&
-               ((c.M <= 16 && c.K == 16384) || (c.M <= 64 && (c.K == 4096 || c.K == 8192)))) ||
+              (c.dtype_ab == ASTERGEMM_FP8_E4M3 && c.M <= 64 && c.K >= 4096 &&
+               ((c.K % 512 == 0 && c.K <= 16 * 4096) || (c.K % 8192 == 0 && c.K <= 16 * 8192))) ||
               (c.dtype_ab == ASTERGEMM_MXFP4 &&
                ((c.M <= 16 && c.K == 16384) || (c.M <= 64 && (c.K == 4096 || c.K == 8192)))))
                  ? ASTERGEMM_KERNEL_SKINNY
@@ -202,8 +202,11 @@ int grid_of(const Variant& v, const astergemm_config& c) {
     // the resident-activation kernels (8 waves) are persistent: one workgroup per CU
     if (v.waves_n == 8 && v.tile_m == 64 && device_cus() > 0) {
       // 32 < M <= 64: pairs of workgroups per row range, whole pairs on each of the 8 XCDs
+      // (rows longer than 8 KiB are also cut into K ranges, which fills the CUs sooner)
       const int mh = c.M > 32 ? 2 : 1;
-      int g = blocks * mh < device_cus() ? blocks * mh : device_cus();
+      const int64_t rb = row_bytes(c.dtype_ab, c.K);
+      const int64_t want = (int64_t)blocks * mh * (rb > 8192 ? (rb % 8192 ? rb / 4096 : rb / 8192) : 1);
+      int g = want < device_cus() ? (int)want : device_cus();
       if (mh == 2) g = g < 16 ? 16 : (g & ~15);
       return g;
     }

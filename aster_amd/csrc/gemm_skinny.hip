@@ -11,6 +11,7 @@
 // activations take the same K positions as srcB, so the K permutation cancels.
 // It is HBM-bound: no LDS for weights, many 16-byte loads in flight per wave,
 // K split over the waves of a workgroup and reduced through LDS.
+#include <mutex>
 #include <type_traits>
 #include <utility>
 
@@ -958,11 +959,19 @@ __global__ __launch_bounds__(512) void gemm_skinny_regm_kernel(const GemmArgs p)
   constexpr int NBS = 2;                         // blocks between workgroup barriers
   f32x4* red = (f32x4*)(slds + KW * 8192);       // [2][NBS][MT][KW][64]
 
-  // block b runs on XCD b % 8; with MH = 2 blocks b and b + 8 share a row range
+  // block b runs on XCD b % 8; with MH = 2 blocks b and b + 8 share a row range.
+  // Rows longer than the 8 waves' slices are cut into p.split_k K ranges: a workgroup takes
+  // one K range of one of p.tiles_n row ranges and leaves fp32 partial sums in the workspace.
   const int q = blockIdx.x >> 3;
   const int half = MH == 2 ? (q & 1) : 0;
-  const int rid = MH == 2 ? ((q >> 1) << 3) | (blockIdx.x & 7) : (int)blockIdx.x;
-  const int g = gridDim.x / MH;
+  const int idx = MH == 2 ? ((q >> 1) << 3) | (blockIdx.x & 7) : (int)blockIdx.x;
+  const int g = p.tiles_n;                       // row ranges
+  if (idx >= g * p.split_k) return;
+  const int ks = idx / g, rid = idx - ks * g;
+  const int64_t koff = (int64_t)ks * (KW * slice);
+  // the last K range may end inside the workgroup's span: a wave whose slice lies behind the
+  // row's end multiplies zeros (rows are whole slices long, the launcher checks)
+  const bool dead = koff + (wave + 1) * slice > (DT == ASTERGEMM_FP8_E4M3 ? p.K : 2 * p.K);
   const int per = (((p.N + g - 1) / g) + 7) & ~7;
   const int r0 = rid * per;
   const int m0 = half * MT * 16;                 // first activation row of this workgroup
@@ -972,7 +981,7 @@ __global__ __launch_bounds__(512) void gemm_skinny_regm_kernel(const GemmArgs p)
   const int total = nblk * UPB;
 
   const int lrow = lane >> 3, lpiece = lane & 7;
-  const uint8_t* wbase = p.B + wave * slice + lpiece * 16;
+  const uint8_t* wbase = p.B + koff + wave * slice + lpiece * 16;
   auto issue = [&](int j, i32x4(&dst)[8]) {      // flat index j = block * UPB + t
     int blk = j / UPB;
     const int t = j % UPB;
@@ -983,7 +992,8 @@ __global__ __launch_bounds__(512) void gemm_skinny_regm_kernel(const GemmArgs p)
       int n = nh + lrow;
       n = n < r1 ? n : r1 - 1;
       const uint8_t* src = wbase + (int64_t)n * p.ldb_bytes + t * 512;
-      if (j >= total || nh >= r1) src = p.A + lpiece * 16;  // nothing to fetch: a line that stays in L2
+      if (j >= total || nh >= r1 || dead)
+        src = p.A + lpiece * 16;                   // nothing to fetch: a line that stays in L2
 #pragma unroll
       for (int s = 0; s < 4; ++s)
         dst[s * 2 + h] = __builtin_nontemporal_load((const i32x4*)(src + s * 128));
@@ -1010,9 +1020,11 @@ __global__ __launch_bounds__(512) void gemm_skinny_regm_kernel(const GemmArgs p)
     for (int h = 0; h < 2; ++h) {
       int m = m0 + mt * 16 + h * 8 + lrow;
       m = m < p.M ? m : p.M - 1;
-      const uint8_t* src = p.A + (int64_t)m * p.lda_bytes + wave * slice + t * 512 + lpiece * 16;
+      const uint8_t* src =
+          p.A + (int64_t)m * p.lda_bytes + koff + wave * slice + t * 512 + lpiece * 16;
 #pragma unroll
-      for (int s = 0; s < 4; ++s) dst[s * 2 + h] = *(const i32x4*)(src + s * 128);
+      for (int s = 0; s < 4; ++s)
+        dst[s * 2 + h] = dead ? i32x4{0, 0, 0, 0} : *(const i32x4*)(src + s * 128);
     }
   };
   i32x4 w0[8], w1[8];
@@ -1063,7 +1075,14 @@ __global__ __launch_bounds__(512) void gemm_skinny_regm_kernel(const GemmArgs p)
 #pragma unroll
       for (int k = 1; k < KW; ++k) v += src[k * 64];
       const int m = m0 + rt * 16 + li, n = r0 + (blk - slot + rb) * 16 + 4 * lq;
-      if (m < p.M && n < r1) {
+      if (m < p.M && n < r1 && p.split_k > 1) {
+        // partial sums of this K range: [split][M][N] fp32, finished by the reduce kernel
+        const int ncols = (r1 - n) < 4 ? (r1 - n) : 4;
+        float* o = p.workspace + ((int64_t)ks * p.M + m) * p.N + n;
+        if ((p.N & 3) == 0 && ncols == 4) *(f32x4*)o = v;
+        else
+          for (int r = 0; r < ncols; ++r) o[r] = v[r];
+      } else if (m < p.M && n < r1) {
         v *= scale;
         const int ncols = (r1 - n) < 4 ? (r1 - n) : 4;
         if (p.bias)
@@ -1147,8 +1166,68 @@ __global__ __launch_bounds__(512) void gemm_skinny_regm_kernel(const GemmArgs p)
   }
 }
 
+// out[m][n] = cast(scale * sum over splits of partial[s][m][n] + bias[n]), splits in order
+template <int OUT>
+__global__ __launch_bounds__(256) void skinny_splitk_reduce_kernel(const float* ws, int S, int M,
+                                                                   int N, int64_t ldc,
+                                                                   const float* scale_a,
+                                                                   const float* scale_b,
+                                                                   const float* bias, void* C) {
+  float scale = 1.0f;
+  if (scale_a) scale *= *scale_a;
+  if (scale_b) scale *= *scale_b;
+  const int64_t total = (int64_t)M * N;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int m = (int)(i / N), n = (int)(i - (int64_t)m * N);
+    float v = ws[i];
+    for (int s = 1; s < S; ++s) v += ws[(int64_t)s * total + i];
+    v *= scale;
+    if (bias) v += bias[n];
+    const int64_t o = (int64_t)m * ldc + n;
+    if constexpr (OUT == ASTERGEMM_F32) ((float*)C)[o] = v;
+    else if constexpr (OUT == ASTERGEMM_BF16) ((unsigned short*)C)[o] = sk_f32_to_bf16(v);
+    else {
+      const _Float16 h = (_Float16)v;
+      ((unsigned short*)C)[o] = __builtin_bit_cast(unsigned short, h);
+    }
+  }
+}
+
+// fp32 scratch for the K-split partial sums, one buffer per process, grown on demand (the
+// device is synchronised before an old buffer is released: launches that still use it).
+std::mutex g_ws_mutex;
+float* g_ws = nullptr;
+size_t g_ws_bytes = 0;
+
+int splitk_workspace(size_t bytes, float** out) {
+  std::lock_guard<std::mutex> lock(g_ws_mutex);
+  if (bytes > g_ws_bytes) {
+    if (g_ws) {
+      if (hipDeviceSynchronize() != hipSuccess) return (int)hipGetLastError();
+      (void)hipFree(g_ws);
+      g_ws = nullptr, g_ws_bytes = 0;
+    }
+    const size_t want = bytes < ((size_t)8 << 20) ? ((size_t)8 << 20) : bytes;
+    if (hipMalloc((void**)&g_ws, want) != hipSuccess) return (int)hipGetLastError();
+    g_ws_bytes = want;
+  }
+  *out = g_ws;
+  return 0;
+}
+
+// K ranges for a row of `rb` bytes: rb / 8 KiB when that is whole (one range: the eight
+// waves' 1 KiB slices cover the row), else ranges of 4 KiB in 512-byte slices, the last one
+// possibly short; 0 when the row is not a whole number of slices or needs over 16 ranges.
+__host__ inline int skinny_split_of(int64_t rb, int* spb) {
+  if (rb < 4096) return 0;                       // most waves would idle: the generic kernel
+  if (rb % 8192 == 0 && rb / 8192 <= 16) return *spb = 8, (int)(rb / 8192);
+  if (rb % 512 == 0 && (rb + 4095) / 4096 <= 16) return *spb = 4, (int)((rb + 4095) / 4096);
+  return 0;
+}
+
 template <int DT, int OUT, int SPB, int MT, int MH>
-int launch_skinny_regm_t(const GemmArgs& a, hipStream_t s) {
+int launch_skinny_regm_t(const GemmArgs& a0, int S, hipStream_t s) {
   auto k = gemm_skinny_regm_kernel<DT, OUT, SPB, MT, MH>;
   constexpr int lds = 8 * 8192 + 2 * 2 * MT * 8 * 64 * 16;
   static std::atomic<bool> attr_set{false};
@@ -1164,39 +1243,55 @@ int launch_skinny_regm_t(const GemmArgs& a, hipStream_t s) {
     cus = prop.multiProcessorCount;
     attr_set = true;
   }
-  // one workgroup per CU; with MH = 2 the grid is whole pairs on each of the 8 XCDs
-  const int nblocks = (int)((a.N + 15) / 16) * MH;
-  int g = nblocks < cus.load() ? nblocks : cus.load();
-  if (MH == 2) g = g < 16 ? 16 : (g & ~15);
+  GemmArgs a = a0;
+  // one workgroup per CU: S K ranges x R row ranges (x 2 halves of the activation rows with
+  // MH = 2, whose grid is whole pairs on each of the 8 XCDs)
+  const int nblocks = (int)((a.N + 15) / 16);
+  const int slots = (MH == 2 ? (cus.load() / 16) * 8 : cus.load());
+  int R = slots / S;
+  R = R < 1 ? 1 : (R > nblocks ? nblocks : R);
+  a.tiles_n = R;
+  a.split_k = S;
+  int g = MH * S * R;
+  if (MH == 2) g = (g + 15) & ~15;
+  if (S > 1) {
+    if (int rc = splitk_workspace((size_t)S * a.M * a.N * sizeof(float), &a.workspace)) return rc;
+  }
   hipLaunchKernelGGL(k, dim3(g), dim3(512), lds, s, a);
+  if (S > 1) {
+    const int64_t total = (int64_t)a.M * a.N;
+    const int rg = (int)((total + 255) / 256 < 1024 ? (total + 255) / 256 : 1024);
+    hipLaunchKernelGGL(skinny_splitk_reduce_kernel<OUT>, dim3(rg), dim3(256), 0, s, a.workspace, S,
+                       a.M, a.N, a.ldc, a.scale_a, a.scale_b, a.bias, a.C);
+  }
   return (int)hipGetLastError();
 }
 
 template <int DT, int OUT>
 int launch_skinny_regm(const GemmArgs& a, int grid, hipStream_t s) {
   (void)grid;
-  const int64_t rb = row_bytes(DT, a.K);
-  if (a.M <= 32) {
-    switch (rb) {
-      case 4096: return launch_skinny_regm_t<DT, OUT, 4, 2, 1>(a, s);
-      case 8192: return launch_skinny_regm_t<DT, OUT, 8, 2, 1>(a, s);
-    }
-  } else {
-    switch (rb) {
-      case 4096: return launch_skinny_regm_t<DT, OUT, 4, 2, 2>(a, s);
-      case 8192: return launch_skinny_regm_t<DT, OUT, 8, 2, 2>(a, s);
-    }
-  }
-  return (int)hipErrorInvalidValue;
+  int spb = 0;
+  const int S = skinny_split_of(row_bytes(DT, a.K), &spb);
+  if (S == 0) return (int)hipErrorInvalidValue;
+  if (a.M <= 16 && S > 1)
+    return spb == 8 ? launch_skinny_regm_t<DT, OUT, 8, 1, 1>(a, S, s)
+                    : launch_skinny_regm_t<DT, OUT, 4, 1, 1>(a, S, s);
+  if (a.M <= 32)
+    return spb == 8 ? launch_skinny_regm_t<DT, OUT, 8, 2, 1>(a, S, s)
+                    : launch_skinny_regm_t<DT, OUT, 4, 2, 1>(a, S, s);
+  return spb == 8 ? launch_skinny_regm_t<DT, OUT, 8, 2, 2>(a, S, s)
+                  : launch_skinny_regm_t<DT, OUT, 4, 2, 2>(a, S, s);
 }
 
 const char* check_skinny_regm(const astergemm_config& c) {
   if (c.M > 64) return "resident-activation path needs M <= 64";
-  const int64_t rb = row_bytes(c.dtype_ab, c.K);
-  if (rb != 4096 && rb != 8192)
+  int spb = 0;
+  if (skinny_split_of(row_bytes(c.dtype_ab, c.K), &spb) == 0)
     return c.dtype_ab == ASTERGEMM_FP8_E4M3
-               ? "resident-activation path for 16 < M <= 64 needs K = 4096 or 8192 for fp8"
-               : "resident-activation path for 16 < M <= 64 needs K = 2048 or 4096";
+               ? "resident-activation path for fp8 needs K >= 4096, a multiple of 512, at most 65536 "
+                 "(131072 in multiples of 8192)"
+               : "resident-activation path needs K >= 2048, a multiple of 256, at most 32768 (65536 in "
+                 "multiples of 4096)";
   return nullptr;
 }
 

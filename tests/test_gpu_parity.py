@@ -256,6 +256,47 @@ def test_skinny_resident_activations_up_to_64_rows(gpu, M, N, K, dtype_ab, dtype
     assert np.isnan(pad).all() if dtype_c == "f32" else (pad == 0x7FC1).all()
 
 
+@pytest.mark.parametrize("M,N,K", [(16, 4096, 14336), (1, 8, 6144), (33, 777, 14336), (64, 4096, 14336),
+                                   (16, 1000, 28672), (64, 24, 10240), (7, 4104, 32768), (40, 2050, 12288),
+                                   (16, 4096, 11008), (16, 5120, 13824), (33, 100, 2304), (64, 520, 6400),
+                                   (5, 64, 3840)])
+@pytest.mark.parametrize("dtype_ab,dtype_c", [("bf16", "f32"), ("f16", "f16"), ("bf16", "bf16")])
+def test_skinny_resident_activations_long_rows(gpu, M, N, K, dtype_ab, dtype_c):
+    """Rows that are not 4 or 8 KiB (down-projections): the persistent kernel runs one K range
+    per workgroup, the last range possibly short, leaves fp32 partial sums in the library's
+    workspace and a second kernel adds them in a fixed order; run twice, the results are the
+    same bits."""
+    a, b, _ = operands(M, N, K, dtype_ab, seed=71, b_std=0.05)
+    bias = np.random.default_rng(72).standard_normal(N).astype(np.float32)
+    ldc = (N + 11) & ~3
+    out, name = run_gemm(a, b, M, N, K, dtype_ab, dtype_c, bias=bias, ldc=ldc)
+    assert name.startswith("skinnyx") and "_m64_" in name
+    want = G.gemm(a, b, _DT[dtype_ab], _DT[dtype_c], bias=bias)
+    check(out, want, dtype_c, N, bar=1e-5 if dtype_c == "f32" else REL_L2_BAR)
+    pad = out[:, N:]
+    assert np.isnan(pad).all() if dtype_c == "f32" else (pad == 0x7FC1).all()
+    again, _ = run_gemm(a, b, M, N, K, dtype_ab, dtype_c, bias=bias, ldc=ldc)
+    assert np.array_equal(out[:, :N].view(np.uint8), again[:, :N].view(np.uint8))
+
+
+@pytest.mark.parametrize("M,N,K", [(16, 4096, 14336), (3, 8, 12288), (48, 777, 28672), (64, 4104, 16384),
+                                   (16, 520, 11264), (40, 64, 4608)])
+@pytest.mark.parametrize("dtype_c", ["bf16", "f32"])
+def test_skinny_fp8_long_rows(gpu, M, N, K, dtype_c):
+    a, b, extra = operands(M, N, K, "fp8_e4m3", seed=75, b_std=0.05)
+    bias = np.random.default_rng(76).standard_normal(N).astype(np.float32)
+    out, name = run_gemm(a, b, M, N, K, "fp8_e4m3", dtype_c, bias=bias, ldc=N + 8, **extra)
+    assert name.startswith("skinnyx_fp8_m64")
+    want = G.gemm_fp8(a, b, extra["scale_a"], extra["scale_b"], out_dtype=_DT[dtype_c], bias=bias)
+    if dtype_c == "f32" or M * N >= 4096:
+        check(out, want, dtype_c, N, bar=1e-4 if dtype_c == "f32" else REL_L2_BAR)
+    else:
+        got, ref = G.output_to_f32(out[:, :N], _DT[dtype_c]), G.output_to_f32(want, _DT[dtype_c])
+        assert np.all(np.abs(got - ref) <= 2.0 ** -6 * np.abs(ref) + 1e-4 * np.abs(ref).max())
+    pad = out[:, N:]
+    assert np.isnan(pad).all() if dtype_c == "f32" else (pad == 0x7FC1).all()
+
+
 @pytest.mark.parametrize("M,N,K", [(16, 14336, 4096), (1, 8, 4096), (5, 777, 8192), (16, 24, 16384),
                                    (13, 6000, 4096), (16, 14337, 8192)])
 @pytest.mark.parametrize("dtype_c", ["bf16", "f32", "f16"])
@@ -357,8 +398,8 @@ def test_skinny_mxfp4_up_to_64_rows(gpu, M, N, K, dtype_c):
 
 
 def test_skinny_fp8_falls_back_to_tile_kernels(gpu):
-    # K outside the resident kernels' set, or M > 64: AUTO keeps the tile family
-    for (M, N, K) in ((16, 256, 1024), (65, 256, 4096), (17, 256, 16384)):
+    # rows shorter than 4 KiB or not whole 512-byte slices, or M > 64: AUTO keeps the tile family
+    for (M, N, K) in ((16, 256, 1024), (65, 256, 4096), (17, 256, 11008)):
         a, b, extra = operands(M, N, K, "fp8_e4m3", seed=33)
         out, name = run_gemm(a, b, M, N, K, "fp8_e4m3", "f32", **extra)
         assert name.startswith("tile")
