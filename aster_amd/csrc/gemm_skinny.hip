@@ -11,6 +11,7 @@
 // activations take the same K positions as srcB, so the K permutation cancels.
 // It is HBM-bound: no LDS for weights, many 16-byte loads in flight per wave,
 // K split over the waves of a workgroup and reduced through LDS.
+#include <map>
 #include <mutex>
 #include <type_traits>
 #include <utility>
@@ -1194,25 +1195,33 @@ __global__ __launch_bounds__(256) void skinny_splitk_reduce_kernel(const float* 
   }
 }
 
-// fp32 scratch for the K-split partial sums, one buffer per process, grown on demand (the
-// device is synchronised before an old buffer is released: launches that still use it).
+// fp32 scratch for the K-split partial sums: one buffer per (device, stream), so launches on
+// different streams never share one; launches on one stream are ordered and reuse it.  A
+// buffer grows on demand (the stream is drained before the old one is released) and lives
+// until the process ends.
+struct SplitWorkspace {
+  float* ptr = nullptr;
+  size_t bytes = 0;
+};
 std::mutex g_ws_mutex;
-float* g_ws = nullptr;
-size_t g_ws_bytes = 0;
+std::map<std::pair<int, hipStream_t>, SplitWorkspace> g_ws;
 
-int splitk_workspace(size_t bytes, float** out) {
+int splitk_workspace(size_t bytes, hipStream_t stream, float** out) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return (int)hipGetLastError();
   std::lock_guard<std::mutex> lock(g_ws_mutex);
-  if (bytes > g_ws_bytes) {
-    if (g_ws) {
-      if (hipDeviceSynchronize() != hipSuccess) return (int)hipGetLastError();
-      (void)hipFree(g_ws);
-      g_ws = nullptr, g_ws_bytes = 0;
+  SplitWorkspace& w = g_ws[{dev, stream}];
+  if (bytes > w.bytes) {
+    if (w.ptr) {
+      if (hipStreamSynchronize(stream) != hipSuccess) return (int)hipGetLastError();
+      (void)hipFree(w.ptr);
+      w = SplitWorkspace{};
     }
     const size_t want = bytes < ((size_t)8 << 20) ? ((size_t)8 << 20) : bytes;
-    if (hipMalloc((void**)&g_ws, want) != hipSuccess) return (int)hipGetLastError();
-    g_ws_bytes = want;
+    if (hipMalloc((void**)&w.ptr, want) != hipSuccess) return (int)hipGetLastError();
+    w.bytes = want;
   }
-  *out = g_ws;
+  *out = w.ptr;
   return 0;
 }
 
@@ -1255,7 +1264,7 @@ int launch_skinny_regm_t(const GemmArgs& a0, int S, hipStream_t s) {
   int g = MH * S * R;
   if (MH == 2) g = (g + 15) & ~15;
   if (S > 1) {
-    if (int rc = splitk_workspace((size_t)S * a.M * a.N * sizeof(float), &a.workspace)) return rc;
+    if (int rc = splitk_workspace((size_t)S * a.M * a.N * sizeof(float), s, &a.workspace)) return rc;
   }
   hipLaunchKernelGGL(k, dim3(g), dim3(512), lds, s, a);
   if (S > 1) {

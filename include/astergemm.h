@@ -19,8 +19,13 @@
  * Conventions: every function returns 0 on success and a negative
  * ASTERGEMM_E* code on failure; nothing throws; the message of the last
  * failure on the calling thread is returned by astergemm_last_error().
- * All buffers are owned by the caller.  Pointers named d* are device
- * pointers.  Launches go to the stream that is passed (NULL = the null
+ * All buffers are owned by the caller, with one exception: decode shapes
+ * (M <= 64) whose rows are not 4 or 8 KiB long are computed in K ranges, and
+ * the fp32 partial sums live in a workspace the library allocates on first
+ * use, one per (device, stream), M * N * 4 bytes per K range (at most 16),
+ * kept until the process ends.  Calls on different streams may run
+ * concurrently; calls on one stream are ordered by it.  Pointers named d*
+ * are device pointers.  Launches go to the stream that is passed (NULL = the null
  * stream, which is what the reference uses everywhere).
  */
 #ifndef ASTERGEMM_H_

@@ -279,6 +279,54 @@ def test_skinny_resident_activations_long_rows(gpu, M, N, K, dtype_ab, dtype_c):
     assert np.array_equal(out[:, :N].view(np.uint8), again[:, :N].view(np.uint8))
 
 
+def test_skinny_long_rows_on_two_streams(gpu):
+    """Launches in K ranges on two streams at once: each stream has its own partial-sum
+    workspace, so interleaved launches give the bits of launches made alone; a larger problem
+    on the same stream afterwards grows that stream's workspace."""
+    from aster_amd.execution import GpuStream
+    shapes = [(16, 4096, 14336), (48, 2048, 11008)]
+    streams = [GpuStream(), GpuStream()]
+    jobs = []
+    for (M, N, K), st in zip(shapes, streams):
+        a, b, _ = operands(M, N, K, "bf16", seed=81 + M, b_std=0.05)
+        alone, name = run_gemm(a, b, M, N, K, "bf16", "bf16")
+        assert "_m64_" in name
+        plan = AG.GemmPlan.create(M, N, K, "bf16", "bf16")
+        bufs = [GpuBuffer(x.nbytes) for x in (a, b, alone)]
+        bufs[0].copy_from_host(np.ascontiguousarray(a))
+        bufs[1].copy_from_host(np.ascontiguousarray(b))
+        jobs.append((plan, bufs, alone, st))
+    for _ in range(8):
+        for plan, bufs, _, st in jobs:
+            plan.run(bufs[0].ptr_value, bufs[1].ptr_value, bufs[2].ptr_value, stream=st.handle.value)
+    for plan, bufs, alone, st in jobs:
+        st.synchronize()
+        got = np.empty_like(alone)
+        bufs[2].copy_to_host(got)
+        assert np.array_equal(got, alone)
+    # the first stream's workspace was sized for 16 x 4096: this one needs more
+    M, N, K = 64, 20480, 10240
+    a, b, _ = operands(M, N, K, "bf16", seed=83, b_std=0.05)
+    alone, _ = run_gemm(a, b, M, N, K, "bf16", "bf16")
+    plan = AG.GemmPlan.create(M, N, K, "bf16", "bf16")
+    big = [GpuBuffer(x.nbytes) for x in (a, b, alone)]
+    big[0].copy_from_host(np.ascontiguousarray(a))
+    big[1].copy_from_host(np.ascontiguousarray(b))
+    st = streams[0]
+    plan.run(big[0].ptr_value, big[1].ptr_value, big[2].ptr_value, stream=st.handle.value)
+    st.synchronize()
+    got = np.empty_like(alone)
+    big[2].copy_to_host(got)
+    assert np.array_equal(got, alone)
+    for _, bufs, _, _ in jobs:
+        for bf in bufs:
+            bf.free()
+    for bf in big:
+        bf.free()
+    for st in streams:
+        st.destroy()
+
+
 @pytest.mark.parametrize("M,N,K", [(16, 4096, 14336), (3, 8, 12288), (48, 777, 28672), (64, 4104, 16384),
                                    (16, 520, 11264), (40, 64, 4608)])
 @pytest.mark.parametrize("dtype_c", ["bf16", "f32"])
