@@ -1167,7 +1167,8 @@ __global__ __launch_bounds__(512) void gemm_skinny_regm_kernel(const GemmArgs p)
   }
 }
 
-// out[m][n] = cast(scale * sum over splits of partial[s][m][n] + bias[n]), splits in order
+// out[m][n..n+3] = cast(scale * sum over K ranges of partial[s][m][n..] + bias), ranges added in
+// index order; a thread takes four neighbours and has all of a pass's loads in flight at once
 template <int OUT>
 __global__ __launch_bounds__(256) void skinny_splitk_reduce_kernel(const float* ws, int S, int M,
                                                                    int N, int64_t ldc,
@@ -1177,20 +1178,52 @@ __global__ __launch_bounds__(256) void skinny_splitk_reduce_kernel(const float* 
   float scale = 1.0f;
   if (scale_a) scale *= *scale_a;
   if (scale_b) scale *= *scale_b;
-  const int64_t total = (int64_t)M * N;
-  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < total;
+  const int cg = (N + 3) >> 2;                     // groups of four columns per row
+  const int64_t plane = (int64_t)M * N;
+  const bool vec = (N & 3) == 0;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < (int64_t)M * cg;
        i += (int64_t)gridDim.x * blockDim.x) {
-    const int m = (int)(i / N), n = (int)(i - (int64_t)m * N);
-    float v = ws[i];
-    for (int s = 1; s < S; ++s) v += ws[(int64_t)s * total + i];
+    const int m = (int)(i / cg), n = (int)(i - (int64_t)m * cg) * 4;
+    const int ncols = (N - n) < 4 ? (N - n) : 4;
+    const float* src = ws + (int64_t)m * N + n;
+    f32x4 v = {0.f, 0.f, 0.f, 0.f};
+    for (int s0 = 0; s0 < S; s0 += 8) {
+      f32x4 t[8];
+#pragma unroll
+      for (int s = 0; s < 8; ++s) {
+        const int sc = (s0 + s) < S ? (s0 + s) : S - 1;
+        const float* q = src + sc * plane;
+        if (vec) t[s] = *(const f32x4*)q;
+        else
+          for (int r = 0; r < 4; ++r) t[s][r] = r < ncols ? q[r] : 0.f;
+      }
+#pragma unroll
+      for (int s = 0; s < 8; ++s)
+        if (s0 + s < S) v += t[s];
+    }
     v *= scale;
-    if (bias) v += bias[n];
+    if (bias)
+      for (int r = 0; r < ncols; ++r) v[r] += bias[n + r];
     const int64_t o = (int64_t)m * ldc + n;
-    if constexpr (OUT == ASTERGEMM_F32) ((float*)C)[o] = v;
-    else if constexpr (OUT == ASTERGEMM_BF16) ((unsigned short*)C)[o] = sk_f32_to_bf16(v);
-    else {
-      const _Float16 h = (_Float16)v;
-      ((unsigned short*)C)[o] = __builtin_bit_cast(unsigned short, h);
+    const bool vec_ok = (ldc & 3) == 0 && ncols == 4;
+    if constexpr (OUT == ASTERGEMM_F32) {
+      float* out = (float*)C + o;
+      if (vec_ok) *(f32x4*)out = v;
+      else
+        for (int r = 0; r < ncols; ++r) out[r] = v[r];
+    } else {
+      unsigned short h[4];
+      for (int r = 0; r < 4; ++r) {
+        if constexpr (OUT == ASTERGEMM_BF16) h[r] = sk_f32_to_bf16(v[r]);
+        else {
+          const _Float16 hh = (_Float16)v[r];
+          h[r] = __builtin_bit_cast(unsigned short, hh);
+        }
+      }
+      unsigned short* out = (unsigned short*)C + o;
+      if (vec_ok) *(u16x4*)out = u16x4{h[0], h[1], h[2], h[3]};
+      else
+        for (int r = 0; r < ncols; ++r) out[r] = h[r];
     }
   }
 }
@@ -1268,8 +1301,8 @@ int launch_skinny_regm_t(const GemmArgs& a0, int S, hipStream_t s) {
   }
   hipLaunchKernelGGL(k, dim3(g), dim3(512), lds, s, a);
   if (S > 1) {
-    const int64_t total = (int64_t)a.M * a.N;
-    const int rg = (int)((total + 255) / 256 < 1024 ? (total + 255) / 256 : 1024);
+    const int64_t total = (int64_t)a.M * ((a.N + 3) / 4);
+    const int rg = (int)((total + 255) / 256 < 2048 ? (total + 255) / 256 : 2048);
     hipLaunchKernelGGL(skinny_splitk_reduce_kernel<OUT>, dim3(rg), dim3(256), 0, s, a.workspace, S,
                        a.M, a.N, a.ldc, a.scale_a, a.scale_b, a.bias, a.C);
   }

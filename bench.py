@@ -415,6 +415,35 @@ def main() -> int:
                        "us_back_to_back_8_weight_sets": round(rot_ns / 1e3, 2),
                        "gbps_back_to_back": round(p.info.bytes / rot_ns, 1),
                        "frac_back_to_back": round(p.info.bytes / rot_ns / PEAK_HBM_GBPS, 4)})
+        # the down-projection of the same layer (rows of 28 KiB: the decode kernels run it in
+        # K ranges), with the vendor library's time for the same rotation of weight sets
+        for m in (16, 64):
+            del a, b, c
+            a, b, keep = make_operands(torch, m, 4096, 14336, "bf16", dev)
+            c = torch.empty(m, 4096, device=dev, dtype=torch.bfloat16)
+            p = AG.GemmPlan.create(m, 4096, 14336, "bf16", "bf16")
+            wts = [b] + [torch.empty_like(b).copy_(b) for _ in range(7)]
+            sets = [{"dA": a.data_ptr(), "dB": w.data_ptr(), "dC": c.data_ptr()} for w in wts]
+            p.bench_rotate(sets, 40)
+            rot_ns = p.bench_rotate(sets, 200) / 200.0
+            entry = {"workload": f"bf16 skinny GEMM M={m} N=4096 K=14336 -> bf16 (down-projection), "
+                                 "8 weight sets used in turn",
+                     "kernel": p.info.name.decode(), "us_back_to_back_8_weight_sets": round(rot_ns / 1e3, 2),
+                     "gbps_back_to_back": round(p.info.bytes / rot_ns, 1), "bound": "hbm",
+                     "frac_back_to_back": round(p.info.bytes / rot_ns / PEAK_HBM_GBPS, 4)}
+            if not args.no_vendor:
+                for i in range(16):
+                    torch.matmul(a, wts[i % 8].t())
+                torch.cuda.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for i in range(200):
+                    torch.matmul(a, wts[i % 8].t())
+                e1.record()
+                e1.synchronize()
+                entry["vendor_library_us_same_rotation"] = round(e0.elapsed_time(e1) * 1e3 / 200, 2)
+            del wts, sets
+            others.append(entry)
         out["others"] = others
 
     if not args.no_vendor:
