@@ -96,10 +96,11 @@ const Variant* choose(const astergemm_config& c, int* index_out) {
   int family = c.family;
   if (family == ASTERGEMM_KERNEL_AUTO)
     family = ((is16 && c.M <= 64 && c.K % 32 == 0) ||
-              (c.dtype_ab == ASTERGEMM_FP8_E4M3 && c.M <= 64 && c.K >= 4096 &&
-               ((c.K % 512 == 0 && c.K <= 16 * 4096) || (c.K % 8192 == 0 && c.K <= 16 * 8192))) ||
-              (c.dtype_ab == ASTERGEMM_MXFP4 &&
-               ((c.M <= 16 && c.K == 16384) || (c.M <= 64 && (c.K == 4096 || c.K == 8192)))))
+              // fp8 / MXFP4: only the resident-activation kernels, whose waves take whole
+              // slices of a row in at most 16 K ranges
+              ((c.dtype_ab == ASTERGEMM_FP8_E4M3 || c.dtype_ab == ASTERGEMM_MXFP4) && c.M <= 64 &&
+               c.K >= 4096 &&
+               ((c.K % 512 == 0 && c.K <= 16 * 4096) || (c.K % 8192 == 0 && c.K <= 16 * 8192))))
                  ? ASTERGEMM_KERNEL_SKINNY
                  : ASTERGEMM_KERNEL_TILE;
   if (c.operand_path == ASTERGEMM_OPERAND_DIRECT_B) family = ASTERGEMM_KERNEL_SKINNY;

@@ -666,6 +666,107 @@ const char* check_skinny_fp4(const astergemm_config& c) {
         launch_skinny_fp4<OUT>, check_skinny_fp4                                           \
   }
 
+// ---- rows cut into K ranges: partial sums, their workspace and the kernel that adds them ---
+
+// out[m][n..n+3] = cast(scale * sum over K ranges of partial[s][m][n..] + bias), ranges added in
+// index order; a thread takes four neighbours and has all of a pass's loads in flight at once
+template <int OUT>
+__global__ __launch_bounds__(256) void skinny_splitk_reduce_kernel(const float* ws, int S, int M,
+                                                                   int N, int64_t ldc,
+                                                                   const float* scale_a,
+                                                                   const float* scale_b,
+                                                                   const float* bias, void* C) {
+  float scale = 1.0f;
+  if (scale_a) scale *= *scale_a;
+  if (scale_b) scale *= *scale_b;
+  const int cg = (N + 3) >> 2;                     // groups of four columns per row
+  const int64_t plane = (int64_t)M * N;
+  const bool vec = (N & 3) == 0;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < (int64_t)M * cg;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int m = (int)(i / cg), n = (int)(i - (int64_t)m * cg) * 4;
+    const int ncols = (N - n) < 4 ? (N - n) : 4;
+    const float* src = ws + (int64_t)m * N + n;
+    f32x4 v = {0.f, 0.f, 0.f, 0.f};
+    for (int s0 = 0; s0 < S; s0 += 8) {
+      f32x4 t[8];
+#pragma unroll
+      for (int s = 0; s < 8; ++s) {
+        const int sc = (s0 + s) < S ? (s0 + s) : S - 1;
+        const float* q = src + sc * plane;
+        if (vec) t[s] = *(const f32x4*)q;
+        else
+          for (int r = 0; r < 4; ++r) t[s][r] = r < ncols ? q[r] : 0.f;
+      }
+#pragma unroll
+      for (int s = 0; s < 8; ++s)
+        if (s0 + s < S) v += t[s];
+    }
+    v *= scale;
+    if (bias)
+      for (int r = 0; r < ncols; ++r) v[r] += bias[n + r];
+    const int64_t o = (int64_t)m * ldc + n;
+    const bool vec_ok = (ldc & 3) == 0 && ncols == 4;
+    if constexpr (OUT == ASTERGEMM_F32) {
+      float* out = (float*)C + o;
+      if (vec_ok) *(f32x4*)out = v;
+      else
+        for (int r = 0; r < ncols; ++r) out[r] = v[r];
+    } else {
+      unsigned short h[4];
+      for (int r = 0; r < 4; ++r) {
+        if constexpr (OUT == ASTERGEMM_BF16) h[r] = sk_f32_to_bf16(v[r]);
+        else {
+          const _Float16 hh = (_Float16)v[r];
+          h[r] = __builtin_bit_cast(unsigned short, hh);
+        }
+      }
+      unsigned short* out = (unsigned short*)C + o;
+      if (vec_ok) *(u16x4*)out = u16x4{h[0], h[1], h[2], h[3]};
+      else
+        for (int r = 0; r < ncols; ++r) out[r] = h[r];
+    }
+  }
+}
+
+template <int OUT>
+void launch_splitk_reduce(const GemmArgs& a, int S, hipStream_t s) {
+  const int64_t total = (int64_t)a.M * ((a.N + 3) / 4);
+  const int rg = (int)((total + 255) / 256 < 2048 ? (total + 255) / 256 : 2048);
+  hipLaunchKernelGGL(skinny_splitk_reduce_kernel<OUT>, dim3(rg), dim3(256), 0, s, a.workspace, S,
+                     a.M, a.N, a.ldc, a.scale_a, a.scale_b, a.bias, a.C);
+}
+
+// fp32 scratch for the K-split partial sums: one buffer per (device, stream), so launches on
+// different streams never share one; launches on one stream are ordered and reuse it.  A
+// buffer grows on demand (the stream is drained before the old one is released) and lives
+// until the process ends.
+struct SplitWorkspace {
+  float* ptr = nullptr;
+  size_t bytes = 0;
+};
+std::mutex g_ws_mutex;
+std::map<std::pair<int, hipStream_t>, SplitWorkspace> g_ws;
+
+int splitk_workspace(size_t bytes, hipStream_t stream, float** out) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return (int)hipGetLastError();
+  std::lock_guard<std::mutex> lock(g_ws_mutex);
+  SplitWorkspace& w = g_ws[{dev, stream}];
+  if (bytes > w.bytes) {
+    if (w.ptr) {
+      if (hipStreamSynchronize(stream) != hipSuccess) return (int)hipGetLastError();
+      (void)hipFree(w.ptr);
+      w = SplitWorkspace{};
+    }
+    const size_t want = bytes < ((size_t)8 << 20) ? ((size_t)8 << 20) : bytes;
+    if (hipMalloc((void**)&w.ptr, want) != hipSuccess) return (int)hipGetLastError();
+    w.bytes = want;
+  }
+  *out = w.ptr;
+  return 0;
+}
+
 // The MXFP4 kernel above with two activation tiles per wave and, for M > 32, two workgroups
 // per weight row range (see gemm_skinny_regm_kernel).
 template <int OUT, int SPB, int SU, int MT, int MH>
@@ -682,11 +783,18 @@ __global__ __launch_bounds__(512) void gemm_skinny_fp4m_kernel(const GemmArgs p)
   constexpr int NBS = 2;                         // blocks between workgroup barriers
   f32x4* red = (f32x4*)(slds + KW * 8192);       // [2][NBS][MT][KW][64]
 
-  // block b runs on XCD b % 8; with MH = 2 blocks b and b + 8 share a row range
+  // block b runs on XCD b % 8; with MH = 2 blocks b and b + 8 share a row range.  Rows longer
+  // than the 8 waves' slices are cut into p.split_k K ranges (see gemm_skinny_regm_kernel): a
+  // workgroup takes one K range of one of p.tiles_n row ranges; a wave whose slice lies
+  // behind the row's end multiplies zeros with unit scales.
   const int q = blockIdx.x >> 3;
   const int half = MH == 2 ? (q & 1) : 0;
-  const int rid = MH == 2 ? ((q >> 1) << 3) | (blockIdx.x & 7) : (int)blockIdx.x;
-  const int g = gridDim.x / MH;
+  const int idx = MH == 2 ? ((q >> 1) << 3) | (blockIdx.x & 7) : (int)blockIdx.x;
+  const int g = p.tiles_n;                       // row ranges
+  if (idx >= g * p.split_k) return;
+  const int ks = idx / g, rid = idx - ks * g;
+  const int64_t koff = (int64_t)ks * (KW * slice);
+  const bool dead = koff + (wave + 1) * slice > p.K / 2;
   const int per = (((p.N + g - 1) / g) + 7) & ~7;
   const int r0 = rid * per;
   const int m0 = half * MT * 16;                 // first activation row of this workgroup
@@ -696,12 +804,19 @@ __global__ __launch_bounds__(512) void gemm_skinny_fp4m_kernel(const GemmArgs p)
   const int total = nblk * UPB;
 
   const int lrow = lane >> 3, lpiece = lane & 7;
-  const uint8_t* wbase = p.B + wave * slice + lpiece * 16;
-  const uint8_t* sbase = p.mx_b + wave * (SPB * 8);       // this wave's scale bytes of a row
+  const uint8_t* wbase = p.B + koff + wave * slice + lpiece * 16;
+  const uint8_t* sbase = p.mx_b + koff / 16 + wave * (SPB * 8);  // this wave's scale bytes of a row
   auto issue = [&](int j, i32x4(&dst)[NL], i32x2(&sc)[SU]) {  // flat index j = block * UPB + t
     int blk = j / UPB;
     const int t = j % UPB;
     blk = blk < nblk ? blk : nblk - 1;
+    if (dead) {
+#pragma unroll
+      for (int i = 0; i < NL; ++i) dst[i] = i32x4{0, 0, 0, 0};
+#pragma unroll
+      for (int s = 0; s < SU; ++s) sc[s] = i32x2{0x7F7F7F7F, 0x7F7F7F7F};
+      return;
+    }
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       const int nh = r0 + blk * 16 + h * 8;
@@ -738,10 +853,10 @@ __global__ __launch_bounds__(512) void gemm_skinny_fp4m_kernel(const GemmArgs p)
   for (int mt = 0; mt < MT; ++mt) {
     int m = m0 + mt * 16 + li;
     m = m < p.M ? m : p.M - 1;
-    const uint8_t* xsrc = p.mx_a + (int64_t)m * p.mx_ld + wave * (SPB * 8);
+    const uint8_t* xsrc = p.mx_a + (int64_t)m * p.mx_ld + koff / 16 + wave * (SPB * 8);
 #pragma unroll
     for (int s = 0; s < SPB; ++s) {
-      const i32x2 v = *(const i32x2*)(xsrc + s * 8);
+      const i32x2 v = dead ? i32x2{0x7F7F7F7F, 0x7F7F7F7F} : *(const i32x2*)(xsrc + s * 8);
       xs[mt][s * 2] = (int)((unsigned)v[0] >> (8 * lq));
       xs[mt][s * 2 + 1] = (int)((unsigned)v[1] >> (8 * lq));
     }
@@ -751,9 +866,11 @@ __global__ __launch_bounds__(512) void gemm_skinny_fp4m_kernel(const GemmArgs p)
     for (int h = 0; h < 2; ++h) {
       int m = m0 + mt * 16 + h * 8 + lrow;
       m = m < p.M ? m : p.M - 1;
-      const uint8_t* src = p.A + (int64_t)m * p.lda_bytes + wave * slice + t * (SU * 128) + lpiece * 16;
+      const uint8_t* src =
+          p.A + (int64_t)m * p.lda_bytes + koff + wave * slice + t * (SU * 128) + lpiece * 16;
 #pragma unroll
-      for (int s = 0; s < SU; ++s) dst[s * 2 + h] = *(const i32x4*)(src + s * 128);
+      for (int s = 0; s < SU; ++s)
+        dst[s * 2 + h] = dead ? i32x4{0, 0, 0, 0} : *(const i32x4*)(src + s * 128);
     }
   };
   i32x4 w0[NL], w1[NL];
@@ -795,7 +912,14 @@ __global__ __launch_bounds__(512) void gemm_skinny_fp4m_kernel(const GemmArgs p)
 #pragma unroll
       for (int k = 1; k < KW; ++k) v += src[k * 64];
       const int m = m0 + rt * 16 + li, n = r0 + (blk - slot + rb) * 16 + 4 * lq;
-      if (m < p.M && n < r1) {
+      if (m < p.M && n < r1 && p.split_k > 1) {
+        // sums over this K range only: [range][M][N] fp32, added up by the reduce kernel
+        const int ncols = (r1 - n) < 4 ? (r1 - n) : 4;
+        float* o = p.workspace + ((int64_t)ks * p.M + m) * p.N + n;
+        if ((p.N & 3) == 0 && ncols == 4) *(f32x4*)o = v;
+        else
+          for (int r = 0; r < ncols; ++r) o[r] = v[r];
+      } else if (m < p.M && n < r1) {
         const int ncols = (r1 - n) < 4 ? (r1 - n) : 4;
         if (p.bias)
           for (int r = 0; r < ncols; ++r) v[r] += p.bias[n + r];
@@ -881,9 +1005,18 @@ __global__ __launch_bounds__(512) void gemm_skinny_fp4m_kernel(const GemmArgs p)
   }
 }
 
-template <int OUT, int SPB, int SU, int MH>
-int launch_skinny_fp4m_t(const GemmArgs& a, hipStream_t s) {
-  constexpr int MT = 2;
+// K ranges for an MXFP4 row of `rb` bytes of nibbles: ranges of 4 KiB when the row is a whole
+// number of them, else of 2 KiB in 256-byte slices, the last one possibly short; 0 when the
+// row is shorter than 2 KiB, not whole slices, or needs more than 16 ranges.
+__host__ inline int skinny_fp4_split_of(int64_t rb, int* spb) {
+  if (rb < 2048) return 0;
+  if (rb % 4096 == 0 && rb / 4096 <= 16) return *spb = 4, (int)(rb / 4096);
+  if (rb % 256 == 0 && (rb + 2047) / 2048 <= 16) return *spb = 2, (int)((rb + 2047) / 2048);
+  return 0;
+}
+
+template <int OUT, int SPB, int SU, int MT, int MH>
+int launch_skinny_fp4m_t(const GemmArgs& a0, int S, hipStream_t s) {
   auto k = gemm_skinny_fp4m_kernel<OUT, SPB, SU, MT, MH>;
   constexpr int lds = 8 * 8192 + 2 * 2 * MT * 8 * 64 * 16;
   static std::atomic<bool> attr_set{false};
@@ -899,34 +1032,45 @@ int launch_skinny_fp4m_t(const GemmArgs& a, hipStream_t s) {
     cus = prop.multiProcessorCount;
     attr_set = true;
   }
-  const int nblocks = (int)((a.N + 15) / 16) * MH;
-  int g = nblocks < cus.load() ? nblocks : cus.load();
-  if (MH == 2) g = g < 16 ? 16 : (g & ~15);
+  GemmArgs a = a0;
+  const int nblocks = (int)((a.N + 15) / 16);
+  const int slots = (MH == 2 ? (cus.load() / 16) * 8 : cus.load());
+  int R = slots / S;
+  R = R < 1 ? 1 : (R > nblocks ? nblocks : R);
+  a.tiles_n = R;
+  a.split_k = S;
+  int g = MH * S * R;
+  if (MH == 2) g = (g + 15) & ~15;
+  if (S > 1) {
+    if (int rc = splitk_workspace((size_t)S * a.M * a.N * sizeof(float), s, &a.workspace)) return rc;
+  }
   hipLaunchKernelGGL(k, dim3(g), dim3(512), lds, s, a);
+  if (S > 1) launch_splitk_reduce<OUT>(a, S, s);
   return (int)hipGetLastError();
 }
 
 template <int OUT>
 int launch_skinny_fp4m(const GemmArgs& a, int grid, hipStream_t s) {
   (void)grid;
-  if (a.M <= 32) {
-    switch (a.K) {
-      case 4096: return launch_skinny_fp4m_t<OUT, 2, 2, 1>(a, s);
-      case 8192: return launch_skinny_fp4m_t<OUT, 4, 4, 1>(a, s);
-    }
-  } else {
-    switch (a.K) {
-      case 4096: return launch_skinny_fp4m_t<OUT, 2, 2, 2>(a, s);
-      case 8192: return launch_skinny_fp4m_t<OUT, 4, 4, 2>(a, s);
-    }
-  }
-  return (int)hipErrorInvalidValue;
+  int spb = 0;
+  const int S = skinny_fp4_split_of(a.K / 2, &spb);
+  if (S == 0) return (int)hipErrorInvalidValue;
+  if (a.M <= 16)
+    return spb == 4 ? launch_skinny_fp4m_t<OUT, 4, 4, 1, 1>(a, S, s)
+                    : launch_skinny_fp4m_t<OUT, 2, 2, 1, 1>(a, S, s);
+  if (a.M <= 32)
+    return spb == 4 ? launch_skinny_fp4m_t<OUT, 4, 4, 2, 1>(a, S, s)
+                    : launch_skinny_fp4m_t<OUT, 2, 2, 2, 1>(a, S, s);
+  return spb == 4 ? launch_skinny_fp4m_t<OUT, 4, 4, 2, 2>(a, S, s)
+                  : launch_skinny_fp4m_t<OUT, 2, 2, 2, 2>(a, S, s);
 }
 
 const char* check_skinny_fp4m(const astergemm_config& c) {
   if (c.M > 64) return "resident-activation MXFP4 path needs M <= 64";
-  if (c.K != 4096 && c.K != 8192)
-    return "resident-activation MXFP4 path for 16 < M <= 64 needs K = 4096 or 8192";
+  int spb = 0;
+  if (skinny_fp4_split_of(c.K / 2, &spb) == 0)
+    return "resident-activation MXFP4 path needs K >= 4096, a multiple of 512, at most 65536 "
+           "(131072 in multiples of 8192)";
   return nullptr;
 }
 
@@ -987,14 +1131,18 @@ __global__ __launch_bounds__(512) void gemm_skinny_regm_kernel(const GemmArgs p)
     int blk = j / UPB;
     const int t = j % UPB;
     blk = blk < nblk ? blk : nblk - 1;
+    if (dead) {                                    // zeros, so that nothing non-finite gets in
+#pragma unroll
+      for (int i = 0; i < 8; ++i) dst[i] = i32x4{0, 0, 0, 0};
+      return;
+    }
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       const int nh = r0 + blk * 16 + h * 8;
       int n = nh + lrow;
       n = n < r1 ? n : r1 - 1;
       const uint8_t* src = wbase + (int64_t)n * p.ldb_bytes + t * 512;
-      if (j >= total || nh >= r1 || dead)
-        src = p.A + lpiece * 16;                   // nothing to fetch: a line that stays in L2
+      if (j >= total || nh >= r1) src = p.A + lpiece * 16;  // nothing to fetch: a line that stays in L2
 #pragma unroll
       for (int s = 0; s < 4; ++s)
         dst[s * 2 + h] = __builtin_nontemporal_load((const i32x4*)(src + s * 128));
@@ -1167,97 +1315,6 @@ __global__ __launch_bounds__(512) void gemm_skinny_regm_kernel(const GemmArgs p)
   }
 }
 
-// out[m][n..n+3] = cast(scale * sum over K ranges of partial[s][m][n..] + bias), ranges added in
-// index order; a thread takes four neighbours and has all of a pass's loads in flight at once
-template <int OUT>
-__global__ __launch_bounds__(256) void skinny_splitk_reduce_kernel(const float* ws, int S, int M,
-                                                                   int N, int64_t ldc,
-                                                                   const float* scale_a,
-                                                                   const float* scale_b,
-                                                                   const float* bias, void* C) {
-  float scale = 1.0f;
-  if (scale_a) scale *= *scale_a;
-  if (scale_b) scale *= *scale_b;
-  const int cg = (N + 3) >> 2;                     // groups of four columns per row
-  const int64_t plane = (int64_t)M * N;
-  const bool vec = (N & 3) == 0;
-  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < (int64_t)M * cg;
-       i += (int64_t)gridDim.x * blockDim.x) {
-    const int m = (int)(i / cg), n = (int)(i - (int64_t)m * cg) * 4;
-    const int ncols = (N - n) < 4 ? (N - n) : 4;
-    const float* src = ws + (int64_t)m * N + n;
-    f32x4 v = {0.f, 0.f, 0.f, 0.f};
-    for (int s0 = 0; s0 < S; s0 += 8) {
-      f32x4 t[8];
-#pragma unroll
-      for (int s = 0; s < 8; ++s) {
-        const int sc = (s0 + s) < S ? (s0 + s) : S - 1;
-        const float* q = src + sc * plane;
-        if (vec) t[s] = *(const f32x4*)q;
-        else
-          for (int r = 0; r < 4; ++r) t[s][r] = r < ncols ? q[r] : 0.f;
-      }
-#pragma unroll
-      for (int s = 0; s < 8; ++s)
-        if (s0 + s < S) v += t[s];
-    }
-    v *= scale;
-    if (bias)
-      for (int r = 0; r < ncols; ++r) v[r] += bias[n + r];
-    const int64_t o = (int64_t)m * ldc + n;
-    const bool vec_ok = (ldc & 3) == 0 && ncols == 4;
-    if constexpr (OUT == ASTERGEMM_F32) {
-      float* out = (float*)C + o;
-      if (vec_ok) *(f32x4*)out = v;
-      else
-        for (int r = 0; r < ncols; ++r) out[r] = v[r];
-    } else {
-      unsigned short h[4];
-      for (int r = 0; r < 4; ++r) {
-        if constexpr (OUT == ASTERGEMM_BF16) h[r] = sk_f32_to_bf16(v[r]);
-        else {
-          const _Float16 hh = (_Float16)v[r];
-          h[r] = __builtin_bit_cast(unsigned short, hh);
-        }
-      }
-      unsigned short* out = (unsigned short*)C + o;
-      if (vec_ok) *(u16x4*)out = u16x4{h[0], h[1], h[2], h[3]};
-      else
-        for (int r = 0; r < ncols; ++r) out[r] = h[r];
-    }
-  }
-}
-
-// fp32 scratch for the K-split partial sums: one buffer per (device, stream), so launches on
-// different streams never share one; launches on one stream are ordered and reuse it.  A
-// buffer grows on demand (the stream is drained before the old one is released) and lives
-// until the process ends.
-struct SplitWorkspace {
-  float* ptr = nullptr;
-  size_t bytes = 0;
-};
-std::mutex g_ws_mutex;
-std::map<std::pair<int, hipStream_t>, SplitWorkspace> g_ws;
-
-int splitk_workspace(size_t bytes, hipStream_t stream, float** out) {
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess) return (int)hipGetLastError();
-  std::lock_guard<std::mutex> lock(g_ws_mutex);
-  SplitWorkspace& w = g_ws[{dev, stream}];
-  if (bytes > w.bytes) {
-    if (w.ptr) {
-      if (hipStreamSynchronize(stream) != hipSuccess) return (int)hipGetLastError();
-      (void)hipFree(w.ptr);
-      w = SplitWorkspace{};
-    }
-    const size_t want = bytes < ((size_t)8 << 20) ? ((size_t)8 << 20) : bytes;
-    if (hipMalloc((void**)&w.ptr, want) != hipSuccess) return (int)hipGetLastError();
-    w.bytes = want;
-  }
-  *out = w.ptr;
-  return 0;
-}
-
 // K ranges for a row of `rb` bytes: rb / 8 KiB when that is whole (one range: the eight
 // waves' 1 KiB slices cover the row), else ranges of 4 KiB in 512-byte slices, the last one
 // possibly short; 0 when the row is not a whole number of slices or needs over 16 ranges.
@@ -1300,12 +1357,7 @@ int launch_skinny_regm_t(const GemmArgs& a0, int S, hipStream_t s) {
     if (int rc = splitk_workspace((size_t)S * a.M * a.N * sizeof(float), s, &a.workspace)) return rc;
   }
   hipLaunchKernelGGL(k, dim3(g), dim3(512), lds, s, a);
-  if (S > 1) {
-    const int64_t total = (int64_t)a.M * ((a.N + 3) / 4);
-    const int rg = (int)((total + 255) / 256 < 2048 ? (total + 255) / 256 : 2048);
-    hipLaunchKernelGGL(skinny_splitk_reduce_kernel<OUT>, dim3(rg), dim3(256), 0, s, a.workspace, S,
-                       a.M, a.N, a.ldc, a.scale_a, a.scale_b, a.bias, a.C);
-  }
+  if (S > 1) launch_splitk_reduce<OUT>(a, S, s);
   return (int)hipGetLastError();
 }
 

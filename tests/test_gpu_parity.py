@@ -445,6 +445,42 @@ def test_skinny_mxfp4_up_to_64_rows(gpu, M, N, K, dtype_c):
     assert np.isnan(pad).all() if dtype_c == "f32" else (pad == 0x7FC1).all()
 
 
+@pytest.mark.parametrize("M,N,K", [(16, 4096, 14336), (3, 8, 12288), (48, 777, 28672), (64, 4104, 16384),
+                                   (16, 520, 11264), (40, 64, 4608), (1, 1000, 32768), (33, 136, 6144)])
+@pytest.mark.parametrize("dtype_c", ["bf16", "f32"])
+def test_skinny_mxfp4_long_rows(gpu, M, N, K, dtype_c):
+    """MXFP4 rows that are not 2 or 4 KiB of nibbles: K ranges, the last one possibly short
+    (a wave behind the row's end multiplies zeros under unit scales)."""
+    a, b, extra = operands(M, N, K, "mxfp4", seed=77, b_std=0.05)
+    rng = np.random.default_rng(80)   # spread the block scales: a wrong byte must not go unnoticed
+    extra["mx_a"] = (extra["mx_a"].astype(np.int32) + rng.integers(-3, 4, extra["mx_a"].shape)).astype(np.uint8)
+    extra["mx_b"] = (extra["mx_b"].astype(np.int32) + rng.integers(-3, 4, extra["mx_b"].shape)).astype(np.uint8)
+    bias = np.random.default_rng(78).standard_normal(N).astype(np.float32)
+    out, name = run_gemm(a, b, M, N, K, "mxfp4", dtype_c, bias=bias, ldc=N + 8, **extra)
+    assert name.startswith("skinnyx_mxfp4_m64")
+    want = G.gemm_mxfp4(a, extra["mx_a"], b, extra["mx_b"], out_dtype=_DT[dtype_c], bias=bias)
+    if dtype_c == "f32" or M * N >= 4096:
+        check(out, want, dtype_c, N, bar=1e-5 if dtype_c == "f32" else REL_L2_BAR)
+    else:
+        got, ref = G.output_to_f32(out[:, :N], _DT[dtype_c]), G.output_to_f32(want, _DT[dtype_c])
+        assert np.all(np.abs(got - ref) <= 2.0 ** -6 * np.abs(ref) + 1e-4 * np.abs(ref).max())
+    pad = out[:, N:]
+    assert np.isnan(pad).all() if dtype_c == "f32" else (pad == 0x7FC1).all()
+
+
+def test_skinny_long_rows_keep_non_finite_inputs_in_their_row(gpu):
+    """A NaN in one activation row reaches that output row only, also where the last K range is
+    short and some waves multiply nothing."""
+    M, N, K = 16, 256, 2304
+    a, b, _ = operands(M, N, K, "bf16", seed=79, b_std=0.05)
+    a = np.array(a, copy=True)
+    a[0, 0] = 0x7FC0          # bf16 NaN in the first line of the activations
+    out, name = run_gemm(a, b, M, N, K, "bf16", "f32")
+    assert "_m64_" in name
+    assert np.isnan(out[0]).all()
+    assert np.isfinite(out[1:]).all()
+
+
 def test_skinny_fp8_falls_back_to_tile_kernels(gpu):
     # rows shorter than 4 KiB or not whole 512-byte slices, or M > 64: AUTO keeps the tile family
     for (M, N, K) in ((16, 256, 1024), (65, 256, 4096), (17, 256, 11008)):
