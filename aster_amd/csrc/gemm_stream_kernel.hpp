@@ -175,7 +175,8 @@ __device__ __forceinline__ void stream_epilogue(const GemmArgs& p,
       const i32x4 d = *(const i32x4*)(slab + r * PITCH + cc * 16);
       uint8_t* out = (uint8_t*)p.C + ((int64_t)(wrow0 + m * 16 + r) * p.ldc + wcol0) * OB + cc * 16;
       // edge tiles: N is a multiple of 8, so a 16-byte chunk is inside a row or past its end
-      if (wrow0 + m * 16 + r < p.M && wcol0 + cc * (16 / OB) < p.N) *(i32x4*)out = d;
+      if (wrow0 + m * 16 + r < p.M && wcol0 + cc * (16 / OB) < p.N)
+        __builtin_nontemporal_store(d, (i32x4*)out);
     }
   }
 }
