@@ -306,7 +306,6 @@ int build_args(const Variant& v, const astergemm_config& c, const astergemm_oper
   a->tiles_m = (int32_t)((c.M + v.tile_m - 1) / v.tile_m);
   a->tiles_n = (int32_t)((c.N + v.tile_n - 1) / v.tile_n);
   a->group_m = 8;
-  if (const char* e = getenv("ASTERGEMM_GROUP_M")) a->group_m = atoi(e) > 0 ? atoi(e) : 8;
   a->split_k = 1;
   return 0;
 }
