@@ -327,6 +327,46 @@ def test_skinny_long_rows_on_two_streams(gpu):
         st.destroy()
 
 
+def test_skinny_long_rows_from_two_host_threads(gpu):
+    """Two host threads, a stream each, launching K-range GEMMs at the same time (ctypes drops
+    the interpreter lock during the call): the library's per-stream workspaces are handed out
+    under a lock, results equal those of launches made alone."""
+    import threading
+    from aster_amd.execution import GpuStream
+    shapes = [(16, 2048, 14336), (33, 1024, 11008)]
+    jobs, errors = [], []
+    for (M, N, K) in shapes:
+        a, b, _ = operands(M, N, K, "bf16", seed=91 + M, b_std=0.05)
+        alone, _ = run_gemm(a, b, M, N, K, "bf16", "bf16")
+        bufs = [GpuBuffer(x.nbytes) for x in (a, b, alone)]
+        bufs[0].copy_from_host(np.ascontiguousarray(a))
+        bufs[1].copy_from_host(np.ascontiguousarray(b))
+        jobs.append((AG.GemmPlan.create(M, N, K, "bf16", "bf16"), bufs, alone))
+
+    def work(plan, bufs):
+        try:
+            st = GpuStream()
+            for _ in range(50):
+                plan.run(bufs[0].ptr_value, bufs[1].ptr_value, bufs[2].ptr_value, stream=st.handle.value)
+            st.synchronize()
+            st.destroy()
+        except Exception as e:  # surfaced below: an assert in a thread is not seen by pytest
+            errors.append(e)
+
+    threads = [threading.Thread(target=work, args=(plan, bufs)) for plan, bufs, _ in jobs]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for _, bufs, alone in jobs:
+        got = np.empty_like(alone)
+        bufs[2].copy_to_host(got)
+        assert np.array_equal(got, alone)
+        for bf in bufs:
+            bf.free()
+
+
 @pytest.mark.parametrize("M,N,K", [(16, 4096, 14336), (3, 8, 12288), (48, 777, 28672), (64, 4104, 16384),
                                    (16, 520, 11264), (40, 64, 4608)])
 @pytest.mark.parametrize("dtype_c", ["bf16", "f32"])
