@@ -113,6 +113,7 @@ SIGNATURES = {
                                   C.POINTER(C.c_int64), C.c_int64, _P]),
     "astergemm_tune": (C.c_int, [C.POINTER(Config), C.POINTER(Operands), C.c_int, C.POINTER(C.c_int),
                                  C.POINTER(C.c_int64), _P]),
+    "astergemm_mfma_ceiling": (C.c_int, [C.c_int, _P, C.c_int64, C.c_int, C.POINTER(C.c_double), _P]),
     "astergemm_shuffle_weight_16": (C.c_int, [_P, _P, C.c_int64, C.c_int64]),
     "astergemm_weight_crc32": (C.c_uint32, [_P, C.c_size_t]),
     "astergemm_weight_header_init": (C.c_int, [C.POINTER(WeightHeader), C.c_int, C.c_int, C.c_int64,

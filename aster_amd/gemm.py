@@ -269,3 +269,16 @@ def execute_gemm_hsaco(cfg: WeakScaledMappedGemmInstance, hsaco_path: str, num_i
             if b is not None:
                 b.free()
     return C_host, times
+
+
+def mfma_ceiling(d_sample: int, sample_bytes: int, dtype_ab: str, *, target_ms: int = 50,
+                 stream: int = None) -> float:
+    """TFLOP/s the device sustains on `dtype_ab` MFMAs alone, operand registers filled from the
+    sample bytes at `d_sample` (device pointer): the rate no GEMM on such values can exceed
+    under the power limit.  The reference reads utilisation against the published peak only
+    (peak_tflops_f16, contrib/kittens/test/bench/bench_harness.py:31-41)."""
+    out = ctypes.c_double()
+    _capi.check(_capi.load().astergemm_mfma_ceiling(
+        _capi.DTYPE_NAMES[dtype_ab], ctypes.c_void_p(d_sample), sample_bytes, target_ms,
+        ctypes.byref(out), ctypes.c_void_p(stream) if stream else None))
+    return out.value

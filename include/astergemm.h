@@ -202,6 +202,19 @@ int astergemm_bench_rotate(const astergemm_config* cfg, const astergemm_operands
 int astergemm_tune(const astergemm_config* cfg, const astergemm_operands* ops, int iters,
                    int* best_variant, int64_t* best_ns, void* stream);
 
+/* The MFMA rate (TFLOP/s) the device sustains on given operand values with
+ * nothing else going on: independent MFMAs of dtype_ab's instruction over
+ * registers filled once from dSample (operand bytes as a GEMM would read
+ * them: at least 4096, a multiple of 16), for about target_ms milliseconds.
+ * Under the board's power limit the rate depends on the values (zeros run near
+ * the published peak, random data well below), so this is the ceiling to
+ * read a measured GEMM against next to the published one.  Synchronises the
+ * stream.  The reference takes its peak from a table
+ * (_PEAK_TFLOPS_F16_BY_MCPU, contrib/kittens/test/bench/bench_harness.py:31-41);
+ * it has no measured counterpart. */
+int astergemm_mfma_ceiling(int dtype_ab, const void* dSample, int64_t sample_bytes,
+                           int target_ms, double* tflops, void* stream);
+
 /* Host pre-shuffle of B[N,K] 2-byte elements into per-lane MFMA order
  * (reference: shuffle_weight, contrib/kittens/test/kittens_helpers.py:90-119). */
 int astergemm_shuffle_weight_16(const uint16_t* src, uint16_t* dst, int64_t N,
