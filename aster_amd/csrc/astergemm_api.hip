@@ -153,6 +153,9 @@ const Variant* choose(const astergemm_config& c, int* index_out) {
                               : (row_bytes(c.dtype_ab, c.K) >= 8192 ? 128 : 200);
       auto tier = [&](const Variant* x) {
         const int area = x->tile_m * x->tile_n;
+        // split K (rank 4) only passes its check where it was measured ahead of every
+        // unsplit kernel: few output tiles, long rows
+        if (x->rank == 4) return 3;
         if (area >= 256 * 256 && fp4 && c.K < 4096 && c.K % 512 == 0) return -1;
         if (area >= 256 * 256) return wgs(x) >= thr256 ? 2 : -1;
         return wgs(x) >= ((x->rank >= 2) ? thr128s : 448) ? 1 : 0;

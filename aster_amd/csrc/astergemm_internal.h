@@ -70,6 +70,12 @@ const Variant* stream_variants();
 int num_skinny_variants();
 const Variant* skinny_variants();
 
+// Split-K support shared by the decode and the tile kernels (gemm_skinny.hip): the fp32
+// workspace of a (device, stream), and the kernel that adds `splits` planes [M][N] of
+// a.workspace in index order, applies a's scales and bias and stores a.C in `out_dtype`.
+int splitk_workspace_for(size_t bytes, hipStream_t stream, float** out);
+int splitk_reduce(int out_dtype, const GemmArgs& a, int splits, hipStream_t stream);
+
 void set_error(const char* fmt, ...);
 int hip_fail(hipError_t e, const char* what, const char* file, int line);
 

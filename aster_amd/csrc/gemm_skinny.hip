@@ -1738,4 +1738,18 @@ int num_skinny_variants() {
 }
 const Variant* skinny_variants() { return kSkinnyVariants; }
 
+int splitk_workspace_for(size_t bytes, hipStream_t stream, float** out) {
+  return splitk_workspace(bytes, stream, out);
+}
+
+int splitk_reduce(int out_dtype, const GemmArgs& a, int splits, hipStream_t stream) {
+  switch (out_dtype) {
+    case ASTERGEMM_F32: launch_splitk_reduce<ASTERGEMM_F32>(a, splits, stream); break;
+    case ASTERGEMM_BF16: launch_splitk_reduce<ASTERGEMM_BF16>(a, splits, stream); break;
+    case ASTERGEMM_F16: launch_splitk_reduce<ASTERGEMM_F16>(a, splits, stream); break;
+    default: return (int)hipErrorInvalidValue;
+  }
+  return (int)hipGetLastError();
+}
+
 }  // namespace astergemm

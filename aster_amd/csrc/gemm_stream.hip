@@ -50,6 +50,67 @@ const char* check_stream_whole_k(const astergemm_config& c) {
         (WM * WN == 8 || BM == 128) ? check_stream : check_stream_whole_k        \
   }
 
+// ---- split K on the 128x128 kernel --------------------------------------------------------
+//
+// K ranges for `tiles` output tiles and rows of `ksteps` 128-byte steps: the largest divisor
+// S of ksteps (4..16, ranges of at least 8 steps) with tiles * S <= 512, two workgroups per
+// CU of a 256-CU part (a 128x128 workgroup holds half a CU's LDS); 0 if there is none.
+// Measured on MI355X against the best unsplit kernel: 3.1x at 32 tiles x 224 steps, 1.5x at
+// 128 x 224, 1.06-1.25x at 128 tiles x 64-128 steps; with S = 2 (more than 128 tiles) it loses.
+inline int stream_split_of(int64_t tiles, int64_t ksteps) {
+  int best = 0;
+  for (int S = 4; S <= 16; ++S) {
+    if (ksteps % S != 0 || ksteps / S < 8 || tiles * S > 512) continue;
+    best = S;
+  }
+  return best;
+}
+
+template <int DT, int OUT>
+int launch_stream_splitk(const GemmArgs& a0, int grid, hipStream_t s) {
+  (void)grid;
+  constexpr int lds = 5 * 128 * kRowBytes;
+  auto k = gemm_stream_splitk_kernel<DT, 128, 128, 2, 2>;
+  static std::atomic<bool> attr_set{false};
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)k,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess) return (int)e;
+    attr_set = true;
+  }
+  const int tiles = a0.tiles_m * a0.tiles_n;
+  const int S = stream_split_of(tiles, a0.ksteps);
+  if (S == 0) return (int)hipErrorInvalidValue;
+  GemmArgs a = a0;
+  if (int rc = splitk_workspace_for((size_t)S * a.M * a.N * sizeof(float), s, &a.workspace))
+    return rc;
+  GemmArgs part = a;           // what the K-range workgroups see: fp32 planes, no epilogue terms
+  part.split_k = S;
+  part.ksteps = a.ksteps / S;
+  part.ldc = a.N;
+  part.scale_a = part.scale_b = part.bias = nullptr;
+  hipLaunchKernelGGL(k, dim3(tiles * S), dim3(256), lds, s, part);
+  return splitk_reduce(OUT, a, S, s);
+}
+
+const char* check_stream_splitk(const astergemm_config& c) {
+  if (const char* why = check_stream_whole_k(c)) return why;
+  const int64_t tiles = ((c.M + 127) / 128) * ((c.N + 127) / 128);
+  if (stream_split_of(tiles, row_bytes(c.dtype_ab, c.K) / kRowBytes) == 0)
+    return "split K needs at most 128 output tiles of 128 x 128 and a K that divides into 4..16 "
+           "ranges of 8 or more 128-byte steps";
+  if (c.M * c.N > ((int64_t)1 << 26)) return "split K workspace would pass 4 GiB";
+  return nullptr;
+}
+
+#define AG_STREAM_SPLITK(name, DT, OUT)                                          \
+  Variant {                                                                      \
+    name, ASTERGEMM_KERNEL_TILE, DT, OUT, 128, 128, kRowBytes, 2, 2, 3, 4,       \
+        5 * 128 * kRowBytes,                                                     \
+        (const void*)gemm_stream_splitk_kernel<DT, 128, 128, 2, 2>,              \
+        launch_stream_splitk<DT, OUT>, check_stream_splitk                       \
+  }
+
 template <int DT, int OUT, int BM, int BN, int WM, int WN>
 int launch_stream8(const GemmArgs& a, int grid, hipStream_t s) {
   constexpr int lds = 5 * BM * kRowBytes;
@@ -132,6 +193,12 @@ const char* check_stream4(const astergemm_config& c) {
 
 const Variant kStreamVariants[] = {
     AG_STREAM_SET("stream_bf16", ASTERGEMM_BF16),
+    AG_STREAM_SPLITK("splitk_bf16_128x128_w2x2_bf16", ASTERGEMM_BF16, ASTERGEMM_BF16),
+    AG_STREAM_SPLITK("splitk_bf16_128x128_w2x2_f32", ASTERGEMM_BF16, ASTERGEMM_F32),
+    AG_STREAM_SPLITK("splitk_bf16_128x128_w2x2_f16", ASTERGEMM_BF16, ASTERGEMM_F16),
+    AG_STREAM_SPLITK("splitk_f16_128x128_w2x2_bf16", ASTERGEMM_F16, ASTERGEMM_BF16),
+    AG_STREAM_SPLITK("splitk_f16_128x128_w2x2_f32", ASTERGEMM_F16, ASTERGEMM_F32),
+    AG_STREAM_SPLITK("splitk_f16_128x128_w2x2_f16", ASTERGEMM_F16, ASTERGEMM_F16),
     AG_STREAM_SET("stream_f16", ASTERGEMM_F16),
     AG_STREAM8("stream_fp8_256x256_w2x4_bf16", ASTERGEMM_FP8_E4M3, ASTERGEMM_BF16),
     AG_STREAM8("stream_fp8_256x256_w2x4_f32", ASTERGEMM_FP8_E4M3, ASTERGEMM_F32),

@@ -197,7 +197,7 @@ __device__ __forceinline__ void stream_mma(const i32x4& a, const i32x4& b, f32x4
 }
 
 template <int DT, int OUT, int BM, int BN, int WM, int WN>
-__device__ __forceinline__ void gemm_stream_body(const GemmArgs& p) {
+__device__ __forceinline__ void gemm_stream_body(const GemmArgs& p, int bid) {
   constexpr int NW = WM * WN;
   constexpr int TM = BM / WM / 16;
   constexpr int TN = BN / WN / 16;
@@ -218,7 +218,7 @@ __device__ __forceinline__ void gemm_stream_body(const GemmArgs& p) {
   const int wm = wave / WN, wn = wave % WN;
 
   int tile_m, tile_n;
-  map_tile(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m, tile_m, tile_n);
+  map_tile(bid, p.tiles_m, p.tiles_n, p.group_m, tile_m, tile_n);
   const int row0 = tile_m * BM, col0 = tile_n * BN;
 
   // ---- global -> LDS (same layout as gemm_tile_body: 128-byte rows, granule
@@ -418,7 +418,22 @@ __device__ __forceinline__ void gemm_stream_body(const GemmArgs& p) {
 
 template <int DT, int OUT, int BM, int BN, int WM, int WN>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_stream_kernel(const GemmArgs p) {
-  gemm_stream_body<DT, OUT, BM, BN, WM, WN>(p);
+  gemm_stream_body<DT, OUT, BM, BN, WM, WN>(p, blockIdx.x);
+}
+
+// Split K: the grid is p.split_k copies of the tile grid; copy s multiplies K steps
+// [s * p.ksteps, (s + 1) * p.ksteps) of every row and leaves its fp32 sums in plane s of the
+// workspace [split_k][M][N] (no scale, no bias: the kernel that adds the planes applies them).
+// For few output tiles and long rows, where the tile grid alone leaves most CUs idle.
+template <int DT, int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(WM* WN * 64) void gemm_stream_splitk_kernel(const GemmArgs p) {
+  const int tiles = p.tiles_m * p.tiles_n;
+  const int ks = blockIdx.x / tiles;
+  GemmArgs q = p;
+  q.A = p.A + (int64_t)ks * p.ksteps * kRowBytes;
+  q.B = p.B + (int64_t)ks * p.ksteps * kRowBytes;
+  q.C = p.workspace + (int64_t)ks * p.M * p.N;
+  gemm_stream_body<DT, ASTERGEMM_F32, BM, BN, WM, WN>(q, blockIdx.x - ks * tiles);
 }
 
 }  // namespace

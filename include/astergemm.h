@@ -20,7 +20,8 @@
  * ASTERGEMM_E* code on failure; nothing throws; the message of the last
  * failure on the calling thread is returned by astergemm_last_error().
  * All buffers are owned by the caller, with one exception: decode shapes
- * (M <= 64) whose rows are not 4 or 8 KiB long are computed in K ranges, and
+ * (M <= 64) whose rows are not 4 or 8 KiB long, and shapes with at most 128
+ * output tiles of 128 x 128 and long rows, are computed in K ranges, and
  * the fp32 partial sums live in a workspace the library allocates on first
  * use, one per (device, stream), M * N * 4 bytes per K range (at most 16),
  * kept until the process ends.  Calls on different streams may run

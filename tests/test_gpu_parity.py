@@ -521,6 +521,32 @@ def test_skinny_long_rows_keep_non_finite_inputs_in_their_row(gpu):
     assert np.isfinite(out[1:]).all()
 
 
+@pytest.mark.parametrize("M,N,K", [(128, 4096, 14336), (96, 4096, 4096), (264, 520, 4096), (1000, 1000, 8192),
+                                   (512, 4096, 2048), (72, 8, 2048), (128, 14336, 4096)])
+@pytest.mark.parametrize("dtype_ab,dtype_c", [("bf16", "bf16"), ("f16", "f32"), ("bf16", "f16")])
+def test_split_k_on_few_output_tiles(gpu, M, N, K, dtype_ab, dtype_c):
+    """At most 128 output tiles of 128 x 128 and long rows: AUTO cuts K into 4..16 ranges, one
+    copy of the tile grid per range, fp32 planes in the library's workspace, summed in range
+    order by a second kernel that applies bias and cast.  Edge tiles, a padded output pitch,
+    and the same bits on a second run."""
+    a, b, _ = operands(M, N, K, dtype_ab, seed=95, b_std=0.05)
+    bias = np.random.default_rng(96).standard_normal(N).astype(np.float32)
+    ldc = N + 8
+    out, name = run_gemm(a, b, M, N, K, dtype_ab, dtype_c, bias=bias, ldc=ldc)
+    assert name.startswith("splitk_")
+    want = G.gemm(a, b, _DT[dtype_ab], _DT[dtype_c], bias=bias)
+    check(out, want, dtype_c, N, bar=1e-5 if dtype_c == "f32" else REL_L2_BAR)
+    pad = out[:, N:]
+    assert np.isnan(pad).all() if dtype_c == "f32" else (pad == 0x7FC1).all()
+    again, _ = run_gemm(a, b, M, N, K, dtype_ab, dtype_c, bias=bias, ldc=ldc)
+    assert np.array_equal(out[:, :N].view(np.uint8), again[:, :N].view(np.uint8))
+    # the unsplit kernels give the same result up to fp32 summation order
+    if dtype_c == "f32":
+        whole, wname = run_gemm(a, b, M, N, K, dtype_ab, dtype_c, bias=bias, wg_tile=(64, 64))
+        assert wname.startswith("tile")
+        assert G.rel_l2(out[:, :N], whole) <= 1e-5
+
+
 def test_skinny_fp8_falls_back_to_tile_kernels(gpu):
     # rows shorter than 4 KiB or not whole 512-byte slices, or M > 64: AUTO keeps the tile family
     for (M, N, K) in ((16, 256, 1024), (65, 256, 4096), (17, 256, 11008)):
@@ -709,6 +735,8 @@ def _tile_variants():
 @pytest.mark.parametrize("vid,name,dtype_ab,dtype_c", _tile_variants(), ids=lambda v: str(v))
 def test_every_tile_variant(gpu, vid, name, dtype_ab, dtype_c):
     M, N, K = 512, 768, 1536  # whole 256-tiles; 24 / 12 / 6 K-steps of 128 bytes (16-bit / fp8 / fp4)
+    if name.startswith("splitk"):
+        K = 2048              # 32 steps: four K ranges of eight
     a, b, ex = operands(M, N, K, dtype_ab, seed=11, a_std=1.0, b_std=1.0 if dtype_ab != "bf16" else 0.05)
     bias = np.random.default_rng(12).standard_normal(N).astype(np.float32)
     plan = AG.GemmPlan.create(M, N, K, dtype_ab, dtype_c, has_bias=True, variant=vid)

@@ -60,7 +60,10 @@ def test_select_headline_configs():
                                   ((2048, 2048, 2048), (128, 128), "stream"),
                                   ((8192, 1024, 8192), (128, 128), "stream"),
                                   ((4096, 4096, 4096), (256, 256), "stream"),
-                                  ((128, 14336, 4096), (64, 64), "tile"),
+                                  ((128, 14336, 4096), (128, 128), "splitk"),  # 112 tiles, 64 steps
+                                  ((128, 4096, 14336), (128, 128), "splitk"),
+                                  ((128, 4096, 14344), (64, 64), "tile"),      # K tail: no split
+                                  ((640, 4096, 4096), (128, 128), "stream"),   # 160 tiles: no split
                                   ((3000, 5000, 7008), (256, 256), "stream"),
                                   ((2044, 2044, 2048), (128, 64), "tile"),    # M, N not multiples of 8
                                   ((3072, 3072, 3072), (256, 256), "stream"),  # 576 = 512 + 64 tiles of 128
