@@ -57,20 +57,25 @@ const char* check_stream_whole_k(const astergemm_config& c) {
 // CU of a 256-CU part (a 128x128 workgroup holds half a CU's LDS); 0 if there is none.
 // Measured on MI355X against the best unsplit kernel: 3.1x at 32 tiles x 224 steps, 1.5x at
 // 128 x 224, 1.06-1.25x at 128 tiles x 64-128 steps; with S = 2 (more than 128 tiles) it loses.
-inline int stream_split_of(int64_t tiles, int64_t ksteps) {
+inline int stream_split_of(int64_t tiles, int64_t ksteps, bool even_ranges = false) {
   int best = 0;
   for (int S = 4; S <= 16; ++S) {
     if (ksteps % S != 0 || ksteps / S < 8 || tiles * S > 512) continue;
+    if (even_ranges && (ksteps / S) % 2 != 0) continue;
     best = S;
   }
   return best;
 }
 
-template <int DT, int OUT>
+// KIND 0: 16-bit operands, 1: fp8, 2: MXFP4 (ranges of an even number of steps)
+template <int KIND, int DT, int OUT>
 int launch_stream_splitk(const GemmArgs& a0, int grid, hipStream_t s) {
   (void)grid;
-  constexpr int lds = 5 * 128 * kRowBytes;
-  auto k = gemm_stream_splitk_kernel<DT, 128, 128, 2, 2>;
+  constexpr int lds = KIND == 2 ? 4 * 128 * kRowBytes + 4 * 128 * 16 : 5 * 128 * kRowBytes;
+  void (*k)(const GemmArgs);
+  if constexpr (KIND == 0) k = gemm_stream_splitk_kernel<DT, 128, 128, 2, 2>;
+  else if constexpr (KIND == 1) k = gemm_stream8_splitk_kernel<DT, 128, 128, 2, 2>;
+  else k = gemm_stream4_splitk_kernel<DT, 128, 128, 2, 2>;
   static std::atomic<bool> attr_set{false};
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute((const void*)k,
@@ -78,8 +83,12 @@ int launch_stream_splitk(const GemmArgs& a0, int grid, hipStream_t s) {
     if (e != hipSuccess) return (int)e;
     attr_set = true;
   }
+  if constexpr (KIND == 2) {
+    if ((((uintptr_t)a0.mx_a | (uintptr_t)a0.mx_b) & 15) != 0 || a0.mx_ld % 16 != 0)
+      return (int)hipErrorInvalidValue;
+  }
   const int tiles = a0.tiles_m * a0.tiles_n;
-  const int S = stream_split_of(tiles, a0.ksteps);
+  const int S = stream_split_of(tiles, a0.ksteps, KIND == 2);
   if (S == 0) return (int)hipErrorInvalidValue;
   GemmArgs a = a0;
   if (int rc = splitk_workspace_for((size_t)S * a.M * a.N * sizeof(float), s, &a.workspace))
@@ -95,21 +104,30 @@ int launch_stream_splitk(const GemmArgs& a0, int grid, hipStream_t s) {
 
 const char* check_stream_splitk(const astergemm_config& c) {
   if (const char* why = check_stream_whole_k(c)) return why;
+  if (c.dtype_ab == ASTERGEMM_MXFP4 && c.K % 512 != 0) return "K must be a multiple of 512";
   const int64_t tiles = ((c.M + 127) / 128) * ((c.N + 127) / 128);
-  if (stream_split_of(tiles, row_bytes(c.dtype_ab, c.K) / kRowBytes) == 0)
+  // shorter rows: the unsplit 64 x 64 kernels are ahead (fp8 256x4096x4096: 15.2 against 19.8 us)
+  const int64_t min_steps = c.dtype_ab == ASTERGEMM_MXFP4 ? 32 : 64;
+  if (row_bytes(c.dtype_ab, c.K) / kRowBytes < min_steps)
+    return "split K needs rows of at least 8 KiB (4 KiB for MXFP4)";
+  if (stream_split_of(tiles, row_bytes(c.dtype_ab, c.K) / kRowBytes,
+                      c.dtype_ab == ASTERGEMM_MXFP4) == 0)
     return "split K needs at most 128 output tiles of 128 x 128 and a K that divides into 4..16 "
-           "ranges of 8 or more 128-byte steps";
+           "ranges of 8 or more 128-byte steps (an even number of steps for MXFP4)";
   if (c.M * c.N > ((int64_t)1 << 26)) return "split K workspace would pass 4 GiB";
   return nullptr;
 }
 
-#define AG_STREAM_SPLITK(name, DT, OUT)                                          \
+#define AG_STREAM_SPLITK(name, KIND, DT, OUT, LDS, FUNC)                         \
   Variant {                                                                      \
-    name, ASTERGEMM_KERNEL_TILE, DT, OUT, 128, 128, kRowBytes, 2, 2, 3, 4,       \
-        5 * 128 * kRowBytes,                                                     \
-        (const void*)gemm_stream_splitk_kernel<DT, 128, 128, 2, 2>,              \
-        launch_stream_splitk<DT, OUT>, check_stream_splitk                       \
+    name, ASTERGEMM_KERNEL_TILE, DT, OUT, 128, 128, kRowBytes, 2, 2, 3, 4, LDS,  \
+        (const void*)FUNC<DT, 128, 128, 2, 2>, launch_stream_splitk<KIND, DT, OUT>, \
+        check_stream_splitk                                                      \
   }
+#define AG_STREAM_SPLITK_SET(prefix, KIND, DT, LDS, FUNC)                        \
+  AG_STREAM_SPLITK(prefix "_128x128_w2x2_bf16", KIND, DT, ASTERGEMM_BF16, LDS, FUNC),   \
+      AG_STREAM_SPLITK(prefix "_128x128_w2x2_f32", KIND, DT, ASTERGEMM_F32, LDS, FUNC), \
+      AG_STREAM_SPLITK(prefix "_128x128_w2x2_f16", KIND, DT, ASTERGEMM_F16, LDS, FUNC)
 
 template <int DT, int OUT, int BM, int BN, int WM, int WN>
 int launch_stream8(const GemmArgs& a, int grid, hipStream_t s) {
@@ -193,12 +211,12 @@ const char* check_stream4(const astergemm_config& c) {
 
 const Variant kStreamVariants[] = {
     AG_STREAM_SET("stream_bf16", ASTERGEMM_BF16),
-    AG_STREAM_SPLITK("splitk_bf16_128x128_w2x2_bf16", ASTERGEMM_BF16, ASTERGEMM_BF16),
-    AG_STREAM_SPLITK("splitk_bf16_128x128_w2x2_f32", ASTERGEMM_BF16, ASTERGEMM_F32),
-    AG_STREAM_SPLITK("splitk_bf16_128x128_w2x2_f16", ASTERGEMM_BF16, ASTERGEMM_F16),
-    AG_STREAM_SPLITK("splitk_f16_128x128_w2x2_bf16", ASTERGEMM_F16, ASTERGEMM_BF16),
-    AG_STREAM_SPLITK("splitk_f16_128x128_w2x2_f32", ASTERGEMM_F16, ASTERGEMM_F32),
-    AG_STREAM_SPLITK("splitk_f16_128x128_w2x2_f16", ASTERGEMM_F16, ASTERGEMM_F16),
+    AG_STREAM_SPLITK_SET("splitk_bf16", 0, ASTERGEMM_BF16, 5 * 128 * kRowBytes, gemm_stream_splitk_kernel),
+    AG_STREAM_SPLITK_SET("splitk_f16", 0, ASTERGEMM_F16, 5 * 128 * kRowBytes, gemm_stream_splitk_kernel),
+    AG_STREAM_SPLITK_SET("splitk_fp8", 1, ASTERGEMM_FP8_E4M3, 5 * 128 * kRowBytes,
+                         gemm_stream8_splitk_kernel),
+    AG_STREAM_SPLITK_SET("splitk_mxfp4", 2, ASTERGEMM_MXFP4, 4 * 128 * kRowBytes + 4 * 128 * 16,
+                         gemm_stream4_splitk_kernel),
     AG_STREAM_SET("stream_f16", ASTERGEMM_F16),
     AG_STREAM8("stream_fp8_256x256_w2x4_bf16", ASTERGEMM_FP8_E4M3, ASTERGEMM_BF16),
     AG_STREAM8("stream_fp8_256x256_w2x4_f32", ASTERGEMM_FP8_E4M3, ASTERGEMM_F32),

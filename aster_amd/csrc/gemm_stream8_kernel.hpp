@@ -28,7 +28,7 @@ namespace astergemm {
 namespace {
 
 template <int DT, int OUT, int BM, int BN, int WM, int WN>
-__device__ __forceinline__ void gemm_stream8_body(const GemmArgs& p) {
+__device__ __forceinline__ void gemm_stream8_body(const GemmArgs& p, int bid) {
   constexpr int NW = WM * WN;
   constexpr int TM = BM / WM / 16;
   constexpr int TN = BN / WN / 16;
@@ -49,7 +49,7 @@ __device__ __forceinline__ void gemm_stream8_body(const GemmArgs& p) {
   const int wm = wave / WN, wn = wave % WN;
 
   int tile_m, tile_n;
-  map_tile(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m, tile_m, tile_n);
+  map_tile(bid, p.tiles_m, p.tiles_n, p.group_m, tile_m, tile_n);
   const int row0 = tile_m * BM, col0 = tile_n * BN;
 
   // ---- global -> LDS: identical to the 16-bit stream kernel --------------------------------
@@ -237,7 +237,21 @@ __device__ __forceinline__ void gemm_stream8_body(const GemmArgs& p) {
 
 template <int DT, int OUT, int BM, int BN, int WM, int WN>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_stream8_kernel(const GemmArgs p) {
-  gemm_stream8_body<DT, OUT, BM, BN, WM, WN>(p);
+  gemm_stream8_body<DT, OUT, BM, BN, WM, WN>(p, blockIdx.x);
+}
+
+// Split K (see gemm_stream_splitk_kernel): copy s of the tile grid multiplies K steps
+// [s * p.ksteps, (s + 1) * p.ksteps) into plane s of the fp32 workspace; the tensor scales are
+// applied by the kernel that adds the planes.
+template <int DT, int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(WM* WN * 64) void gemm_stream8_splitk_kernel(const GemmArgs p) {
+  const int tiles = p.tiles_m * p.tiles_n;
+  const int ks = blockIdx.x / tiles;
+  GemmArgs q = p;
+  q.A = p.A + (int64_t)ks * p.ksteps * kRowBytes;
+  q.B = p.B + (int64_t)ks * p.ksteps * kRowBytes;
+  q.C = p.workspace + (int64_t)ks * p.M * p.N;
+  gemm_stream8_body<DT, ASTERGEMM_F32, BM, BN, WM, WN>(q, blockIdx.x - ks * tiles);
 }
 
 }  // namespace

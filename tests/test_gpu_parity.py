@@ -522,7 +522,7 @@ def test_skinny_long_rows_keep_non_finite_inputs_in_their_row(gpu):
 
 
 @pytest.mark.parametrize("M,N,K", [(128, 4096, 14336), (96, 4096, 4096), (264, 520, 4096), (1000, 1000, 8192),
-                                   (512, 4096, 2048), (72, 8, 2048), (128, 14336, 4096)])
+                                   (512, 4096, 4096), (72, 8, 4096), (128, 14336, 4096)])
 @pytest.mark.parametrize("dtype_ab,dtype_c", [("bf16", "bf16"), ("f16", "f32"), ("bf16", "f16")])
 def test_split_k_on_few_output_tiles(gpu, M, N, K, dtype_ab, dtype_c):
     """At most 128 output tiles of 128 x 128 and long rows: AUTO cuts K into 4..16 ranges, one
@@ -545,6 +545,31 @@ def test_split_k_on_few_output_tiles(gpu, M, N, K, dtype_ab, dtype_c):
         whole, wname = run_gemm(a, b, M, N, K, dtype_ab, dtype_c, bias=bias, wg_tile=(64, 64))
         assert wname.startswith("tile")
         assert G.rel_l2(out[:, :N], whole) <= 1e-5
+
+
+@pytest.mark.parametrize("M,N,K", [(128, 4096, 14336), (264, 520, 8192), (96, 1000, 16384), (512, 2048, 16384)])
+@pytest.mark.parametrize("dtype_ab", ["fp8_e4m3", "mxfp4"])
+@pytest.mark.parametrize("dtype_c", ["bf16", "f32"])
+def test_split_k_fp8_and_mxfp4(gpu, M, N, K, dtype_ab, dtype_c):
+    """Split K on the fp8 and MXFP4 128 x 128 kernels: the tensor scales are applied after the
+    planes are added; MXFP4 ranges start on whole 16-byte granules of the scale planes."""
+    a, b, extra = operands(M, N, K, dtype_ab, seed=97, b_std=0.05)
+    if dtype_ab == "mxfp4":
+        rng = np.random.default_rng(98)
+        extra["mx_a"] = (extra["mx_a"].astype(np.int32) + rng.integers(-3, 4, extra["mx_a"].shape)).astype(np.uint8)
+        extra["mx_b"] = (extra["mx_b"].astype(np.int32) + rng.integers(-3, 4, extra["mx_b"].shape)).astype(np.uint8)
+    bias = np.random.default_rng(99).standard_normal(N).astype(np.float32)
+    out, name = run_gemm(a, b, M, N, K, dtype_ab, dtype_c, bias=bias, ldc=N + 8, **extra)
+    assert name.startswith("splitk_")
+    if dtype_ab == "mxfp4":
+        want = G.gemm_mxfp4(a, extra["mx_a"], b, extra["mx_b"], out_dtype=_DT[dtype_c], bias=bias)
+        bar = 1e-5
+    else:
+        want = G.gemm_fp8(a, b, extra["scale_a"], extra["scale_b"], out_dtype=_DT[dtype_c], bias=bias)
+        bar = 1e-4
+    check(out, want, dtype_c, N, bar=bar if dtype_c == "f32" else REL_L2_BAR)
+    pad = out[:, N:]
+    assert np.isnan(pad).all() if dtype_c == "f32" else (pad == 0x7FC1).all()
 
 
 def test_skinny_fp8_falls_back_to_tile_kernels(gpu):
@@ -736,7 +761,7 @@ def _tile_variants():
 def test_every_tile_variant(gpu, vid, name, dtype_ab, dtype_c):
     M, N, K = 512, 768, 1536  # whole 256-tiles; 24 / 12 / 6 K-steps of 128 bytes (16-bit / fp8 / fp4)
     if name.startswith("splitk"):
-        K = 2048              # 32 steps: four K ranges of eight
+        K = {"fp8_e4m3": 8192, "mxfp4": 8192}.get(dtype_ab, 4096)  # 64 (MXFP4: 32) steps of 128 bytes
     a, b, ex = operands(M, N, K, dtype_ab, seed=11, a_std=1.0, b_std=1.0 if dtype_ab != "bf16" else 0.05)
     bias = np.random.default_rng(12).standard_normal(N).astype(np.float32)
     plan = AG.GemmPlan.create(M, N, K, dtype_ab, dtype_c, has_bias=True, variant=vid)
