@@ -175,7 +175,10 @@ def vendor_library(torch, dev, iters=100, drop=20):
 
 SWEEP_SHAPES = [(1024, 1024, 1024), (2048, 2048, 2048), (4096, 4096, 4096), (8192, 8192, 1024),
                 (4096, 14336, 4096), (8000, 8000, 8000), (512, 8192, 8192), (128, 14336, 4096),
-                (256, 14336, 4096), (8192, 1024, 8192), (3000, 5000, 7008), (16384, 16384, 4096)]
+                (256, 14336, 4096), (8192, 1024, 8192), (3000, 5000, 7008), (16384, 16384, 4096),
+                # down-projections: decode (K ranges in the resident kernels) and short prefill (split K)
+                (16, 4096, 14336), (64, 4096, 14336), (128, 4096, 14336), (512, 4096, 14336),
+                (16, 8192, 28672)]
 
 
 def shape_sweep(torch, dev):
