@@ -217,7 +217,13 @@ int grid_of(const Variant& v, const astergemm_config& c) {
     if (v.waves_n == 8 && device_cus() > 0 && blocks > device_cus()) return device_cus();
     return blocks;
   }
-  return (int)(((c.M + v.tile_m - 1) / v.tile_m) * ((c.N + v.tile_n - 1) / v.tile_n));
+  const int64_t tiles = ((c.M + v.tile_m - 1) / v.tile_m) * ((c.N + v.tile_n - 1) / v.tile_n);
+  if (v.rank == 4) {  // split K: one copy of the tile grid per K range
+    const int S = stream_split_of(tiles, row_bytes(c.dtype_ab, c.K) / 128,
+                                  c.dtype_ab == ASTERGEMM_MXFP4);
+    return (int)(tiles * (S > 0 ? S : 1));
+  }
+  return (int)tiles;
 }
 
 int64_t algorithmic_bytes(const astergemm_config& c) {

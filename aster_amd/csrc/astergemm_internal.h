@@ -70,6 +70,21 @@ const Variant* stream_variants();
 int num_skinny_variants();
 const Variant* skinny_variants();
 
+// K ranges for `tiles` output tiles and rows of `ksteps` 128-byte steps: the largest divisor
+// S of ksteps (4..16, ranges of at least 8 steps) with tiles * S <= 512, two workgroups per
+// CU of a 256-CU part (a 128x128 workgroup holds half a CU's LDS); 0 if there is none.
+// Measured on MI355X against the best unsplit kernel: 3.1x at 32 tiles x 224 steps, 1.5x at
+// 128 x 224, 1.06-1.25x at 128 tiles x 64-128 steps; with S = 2 (more than 128 tiles) it loses.
+inline int stream_split_of(int64_t tiles, int64_t ksteps, bool even_ranges = false) {
+  int best = 0;
+  for (int S = 4; S <= 16; ++S) {
+    if (ksteps % S != 0 || ksteps / S < 8 || tiles * S > 512) continue;
+    if (even_ranges && (ksteps / S) % 2 != 0) continue;
+    best = S;
+  }
+  return best;
+}
+
 // Split-K support shared by the decode and the tile kernels (gemm_skinny.hip): the fp32
 // workspace of a (device, stream), and the kernel that adds `splits` planes [M][N] of
 // a.workspace in index order, applies a's scales and bias and stores a.C in `out_dtype`.

@@ -52,21 +52,6 @@ const char* check_stream_whole_k(const astergemm_config& c) {
 
 // ---- split K on the 128x128 kernel --------------------------------------------------------
 //
-// K ranges for `tiles` output tiles and rows of `ksteps` 128-byte steps: the largest divisor
-// S of ksteps (4..16, ranges of at least 8 steps) with tiles * S <= 512, two workgroups per
-// CU of a 256-CU part (a 128x128 workgroup holds half a CU's LDS); 0 if there is none.
-// Measured on MI355X against the best unsplit kernel: 3.1x at 32 tiles x 224 steps, 1.5x at
-// 128 x 224, 1.06-1.25x at 128 tiles x 64-128 steps; with S = 2 (more than 128 tiles) it loses.
-inline int stream_split_of(int64_t tiles, int64_t ksteps, bool even_ranges = false) {
-  int best = 0;
-  for (int S = 4; S <= 16; ++S) {
-    if (ksteps % S != 0 || ksteps / S < 8 || tiles * S > 512) continue;
-    if (even_ranges && (ksteps / S) % 2 != 0) continue;
-    best = S;
-  }
-  return best;
-}
-
 // KIND 0: 16-bit operands, 1: fp8, 2: MXFP4 (ranges of an even number of steps)
 template <int KIND, int DT, int OUT>
 int launch_stream_splitk(const GemmArgs& a0, int grid, hipStream_t s) {
