@@ -71,14 +71,15 @@ int num_skinny_variants();
 const Variant* skinny_variants();
 
 // K ranges for `tiles` output tiles and rows of `ksteps` 128-byte steps: the largest divisor
-// S of ksteps (4..16, ranges of at least 8 steps) with tiles * S <= 512, two workgroups per
-// CU of a 256-CU part (a 128x128 workgroup holds half a CU's LDS); 0 if there is none.
-// Measured on MI355X against the best unsplit kernel: 3.1x at 32 tiles x 224 steps, 1.5x at
-// 128 x 224, 1.06-1.25x at 128 tiles x 64-128 steps; with S = 2 (more than 128 tiles) it loses.
+// S of ksteps (2..16, ranges of at least 8 steps) with tiles * S <= 256, one workgroup per CU
+// of a 256-CU part; 0 if there is none.  Measured on MI355X (bf16 and fp8, 32 to 128 tiles,
+// 64 to 224 steps): filling the CUs once beats filling them twice by 5-15 % (32 tiles x 224
+// steps: 32.3 us with 8 ranges, 37.4 with 16, 61.3 with 2; unsplit 103), and split K is ahead
+// of the best unsplit kernel wherever this returns a value and rows are 8 KiB or longer.
 inline int stream_split_of(int64_t tiles, int64_t ksteps, bool even_ranges = false) {
   int best = 0;
-  for (int S = 4; S <= 16; ++S) {
-    if (ksteps % S != 0 || ksteps / S < 8 || tiles * S > 512) continue;
+  for (int S = 2; S <= 16; ++S) {
+    if (ksteps % S != 0 || ksteps / S < 8 || tiles * S > 256) continue;
     if (even_ranges && (ksteps / S) % 2 != 0) continue;
     best = S;
   }

@@ -97,7 +97,7 @@ const char* check_stream_splitk(const astergemm_config& c) {
     return "split K needs rows of at least 8 KiB (4 KiB for MXFP4)";
   if (stream_split_of(tiles, row_bytes(c.dtype_ab, c.K) / kRowBytes,
                       c.dtype_ab == ASTERGEMM_MXFP4) == 0)
-    return "split K needs at most 128 output tiles of 128 x 128 and a K that divides into 4..16 "
+    return "split K needs at most 128 output tiles of 128 x 128 and a K that divides into 2..16 "
            "ranges of 8 or more 128-byte steps (an even number of steps for MXFP4)";
   if (c.M * c.N > ((int64_t)1 << 26)) return "split K workspace would pass 4 GiB";
   return nullptr;

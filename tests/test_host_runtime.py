@@ -73,8 +73,8 @@ def test_select_headline_configs():
         assert p.info.family == _capi.KERNEL_TILE
         assert (p.info.wg_tile_m, p.info.wg_tile_n) == want, (M, N, K)
         assert p.info.name.decode().startswith(kind), (M, N, K)
-    # split K: the grid is one copy of the 32 tiles per K range (224 steps in 16 ranges of 14)
-    assert gemm.GemmPlan.create(128, 4096, 14336, "bf16", "bf16").info.grid_x == 32 * 16
+    # split K: the grid is one copy of the 32 tiles per K range (224 steps in 8 ranges of 28)
+    assert gemm.GemmPlan.create(128, 4096, 14336, "bf16", "bf16").info.grid_x == 32 * 8
     assert gemm.GemmPlan.create(128, 4096, 14336, "mxfp4", "bf16").info.grid_x == 32 * 7
 
 
