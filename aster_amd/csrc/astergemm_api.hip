@@ -103,6 +103,22 @@ const Variant* choose(const astergemm_config& c, int* index_out) {
                ((c.K % 512 == 0 && c.K <= 16 * 4096) || (c.K % 8192 == 0 && c.K <= 16 * 8192))))
                  ? ASTERGEMM_KERNEL_SKINNY
                  : ASTERGEMM_KERNEL_TILE;
+  // 32 < M <= 64 on rows the decode kernels cut into K ranges: their paired workgroups are
+  // behind split K on the 128 x 128 kernel where that is available (cold weights, bf16
+  // 64x4096x14336: 39.0 against 34.1 us, 64x8192x28672: 131 against 93; fp8 only from 28 KiB
+  // rows on: 71 against 60 us, level below that); for M <= 32 they stay ahead (28.7 against 32.3)
+  if (c.family == ASTERGEMM_KERNEL_AUTO && family == ASTERGEMM_KERNEL_SKINNY && c.M > 32 &&
+      ((is16 && row_bytes(c.dtype_ab, c.K) > 8192) ||
+       (c.dtype_ab == ASTERGEMM_FP8_E4M3 && row_bytes(c.dtype_ab, c.K) >= 28672))) {
+    for (int i = 0; i < total_variants(); ++i) {
+      const Variant* v = variant_at(i);
+      if (v->family == ASTERGEMM_KERNEL_TILE && v->rank == 4 && variant_matches_types(*v, c) &&
+          v->check(c) == nullptr) {
+        family = ASTERGEMM_KERNEL_TILE;
+        break;
+      }
+    }
+  }
   if (c.operand_path == ASTERGEMM_OPERAND_DIRECT_B) family = ASTERGEMM_KERNEL_SKINNY;
 
   const Variant* best = nullptr;

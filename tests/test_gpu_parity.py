@@ -269,13 +269,13 @@ def test_skinny_resident_activations_long_rows(gpu, M, N, K, dtype_ab, dtype_c):
     a, b, _ = operands(M, N, K, dtype_ab, seed=71, b_std=0.05)
     bias = np.random.default_rng(72).standard_normal(N).astype(np.float32)
     ldc = (N + 11) & ~3
-    out, name = run_gemm(a, b, M, N, K, dtype_ab, dtype_c, bias=bias, ldc=ldc)
+    out, name = run_gemm(a, b, M, N, K, dtype_ab, dtype_c, bias=bias, ldc=ldc, family=_capi.KERNEL_SKINNY)
     assert name.startswith("skinnyx") and "_m64_" in name
     want = G.gemm(a, b, _DT[dtype_ab], _DT[dtype_c], bias=bias)
     check(out, want, dtype_c, N, bar=1e-5 if dtype_c == "f32" else REL_L2_BAR)
     pad = out[:, N:]
     assert np.isnan(pad).all() if dtype_c == "f32" else (pad == 0x7FC1).all()
-    again, _ = run_gemm(a, b, M, N, K, dtype_ab, dtype_c, bias=bias, ldc=ldc)
+    again, _ = run_gemm(a, b, M, N, K, dtype_ab, dtype_c, bias=bias, ldc=ldc, family=_capi.KERNEL_SKINNY)
     assert np.array_equal(out[:, :N].view(np.uint8), again[:, :N].view(np.uint8))
 
 
@@ -289,9 +289,9 @@ def test_skinny_long_rows_on_two_streams(gpu):
     jobs = []
     for (M, N, K), st in zip(shapes, streams):
         a, b, _ = operands(M, N, K, "bf16", seed=81 + M, b_std=0.05)
-        alone, name = run_gemm(a, b, M, N, K, "bf16", "bf16")
+        alone, name = run_gemm(a, b, M, N, K, "bf16", "bf16", family=_capi.KERNEL_SKINNY)
         assert "_m64_" in name
-        plan = AG.GemmPlan.create(M, N, K, "bf16", "bf16")
+        plan = AG.GemmPlan.create(M, N, K, "bf16", "bf16", family=_capi.KERNEL_SKINNY)
         bufs = [GpuBuffer(x.nbytes) for x in (a, b, alone)]
         bufs[0].copy_from_host(np.ascontiguousarray(a))
         bufs[1].copy_from_host(np.ascontiguousarray(b))
@@ -307,8 +307,8 @@ def test_skinny_long_rows_on_two_streams(gpu):
     # the first stream's workspace was sized for 16 x 4096: this one needs more
     M, N, K = 64, 20480, 10240
     a, b, _ = operands(M, N, K, "bf16", seed=83, b_std=0.05)
-    alone, _ = run_gemm(a, b, M, N, K, "bf16", "bf16")
-    plan = AG.GemmPlan.create(M, N, K, "bf16", "bf16")
+    alone, _ = run_gemm(a, b, M, N, K, "bf16", "bf16", family=_capi.KERNEL_SKINNY)
+    plan = AG.GemmPlan.create(M, N, K, "bf16", "bf16", family=_capi.KERNEL_SKINNY)
     big = [GpuBuffer(x.nbytes) for x in (a, b, alone)]
     big[0].copy_from_host(np.ascontiguousarray(a))
     big[1].copy_from_host(np.ascontiguousarray(b))
@@ -337,11 +337,11 @@ def test_skinny_long_rows_from_two_host_threads(gpu):
     jobs, errors = [], []
     for (M, N, K) in shapes:
         a, b, _ = operands(M, N, K, "bf16", seed=91 + M, b_std=0.05)
-        alone, _ = run_gemm(a, b, M, N, K, "bf16", "bf16")
+        alone, _ = run_gemm(a, b, M, N, K, "bf16", "bf16", family=_capi.KERNEL_SKINNY)
         bufs = [GpuBuffer(x.nbytes) for x in (a, b, alone)]
         bufs[0].copy_from_host(np.ascontiguousarray(a))
         bufs[1].copy_from_host(np.ascontiguousarray(b))
-        jobs.append((AG.GemmPlan.create(M, N, K, "bf16", "bf16"), bufs, alone))
+        jobs.append((AG.GemmPlan.create(M, N, K, "bf16", "bf16", family=_capi.KERNEL_SKINNY), bufs, alone))
 
     def work(plan, bufs):
         try:
@@ -373,7 +373,7 @@ def test_skinny_long_rows_from_two_host_threads(gpu):
 def test_skinny_fp8_long_rows(gpu, M, N, K, dtype_c):
     a, b, extra = operands(M, N, K, "fp8_e4m3", seed=75, b_std=0.05)
     bias = np.random.default_rng(76).standard_normal(N).astype(np.float32)
-    out, name = run_gemm(a, b, M, N, K, "fp8_e4m3", dtype_c, bias=bias, ldc=N + 8, **extra)
+    out, name = run_gemm(a, b, M, N, K, "fp8_e4m3", dtype_c, bias=bias, ldc=N + 8, family=_capi.KERNEL_SKINNY, **extra)
     assert name.startswith("skinnyx_fp8_m64")
     want = G.gemm_fp8(a, b, extra["scale_a"], extra["scale_b"], out_dtype=_DT[dtype_c], bias=bias)
     if dtype_c == "f32" or M * N >= 4096:
@@ -515,7 +515,7 @@ def test_skinny_long_rows_keep_non_finite_inputs_in_their_row(gpu):
     a, b, _ = operands(M, N, K, "bf16", seed=79, b_std=0.05)
     a = np.array(a, copy=True)
     a[0, 0] = 0x7FC0          # bf16 NaN in the first line of the activations
-    out, name = run_gemm(a, b, M, N, K, "bf16", "f32")
+    out, name = run_gemm(a, b, M, N, K, "bf16", "f32", family=_capi.KERNEL_SKINNY)
     assert "_m64_" in name
     assert np.isnan(out[0]).all()
     assert np.isfinite(out[1:]).all()
@@ -570,6 +570,26 @@ def test_split_k_fp8_and_mxfp4(gpu, M, N, K, dtype_ab, dtype_c):
     check(out, want, dtype_c, N, bar=bar if dtype_c == "f32" else REL_L2_BAR)
     pad = out[:, N:]
     assert np.isnan(pad).all() if dtype_c == "f32" else (pad == 0x7FC1).all()
+
+
+def test_long_rows_above_32_activation_rows_take_split_k(gpu):
+    """AUTO on rows the decode kernels cut into K ranges: M <= 32 stays with them, 32 < M <= 64
+    goes to split K on the 128 x 128 kernel where the shape allows it (N % 8 == 0)."""
+    for (M, N, K, dt, want) in ((32, 4096, 14336, "bf16", "skinnyx_bf16_m64"),
+                                (48, 4096, 14336, "bf16", "splitk_bf16"),
+                                (64, 4096, 14336, "f16", "splitk_f16"),
+                                (64, 4100, 14336, "bf16", "skinnyx_bf16_m64"),
+                                (64, 14336, 4096, "bf16", "skinnyx_bf16_m64"),
+                                (64, 4096, 14336, "fp8_e4m3", "skinnyx_fp8_m64"),
+                                (64, 4096, 28672, "fp8_e4m3", "splitk_fp8")):
+        a, b, extra = operands(M, N, K, dt, seed=93, b_std=0.05)
+        out, name = run_gemm(a, b, M, N, K, dt, "f32", **extra)
+        assert name.startswith(want), (M, N, K, dt, name)
+        if dt == "fp8_e4m3":
+            ref = G.gemm_fp8(a, b, extra["scale_a"], extra["scale_b"], out_dtype=G.F32)
+        else:
+            ref = G.gemm(a, b, _DT[dt], G.F32)
+        check(out, ref, "f32", N, bar=1e-4 if dt == "fp8_e4m3" else 1e-5)
 
 
 def test_skinny_fp8_falls_back_to_tile_kernels(gpu):
