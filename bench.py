@@ -456,6 +456,19 @@ def main() -> int:
                 entry["vendor_library_us_same_rotation"] = round(e0.elapsed_time(e1) * 1e3 / 200, 2)
             del wts, sets
             others.append(entry)
+        # a short prefill through the same down-projection: few output tiles, long rows (split K)
+        for dt in ("bf16", "fp8_e4m3"):
+            del a, b, c
+            a, b, keep = make_operands(torch, 128, 4096, 14336, dt, dev)
+            c = torch.empty(128, 4096, device=dev, dtype=torch.bfloat16)
+            p = AG.GemmPlan.create(128, 4096, 14336, dt, "bf16")
+            p50, _, _ = event_timed_p50(p, a, b, c, keep, 100, 20)
+            tf = p.info.flops / p50 * 1e-3
+            others.append({"workload": f"{dt} GEMM 128x4096x14336 -> bf16 (32 output tiles of 128x128)",
+                           "kernel": p.info.name.decode(), "grid": p.info.grid_x,
+                           "p50_us": round(p50 / 1e3, 2), "tflops": round(tf, 1),
+                           "gbps": round(p.info.bytes / p50, 1), "bound": "hbm",
+                           "frac": round(p.info.bytes / p50 / PEAK_HBM_GBPS, 4)})
         out["others"] = others
 
     if not args.no_vendor:
