@@ -22,6 +22,7 @@ SCALE_NONE, SCALE_TENSOR, SCALE_MX32 = 0, 1, 2
 # astergemm_kernel_family
 KERNEL_AUTO, KERNEL_TILE, KERNEL_SKINNY = 0, 1, 2
 OPERAND_LDS, OPERAND_DIRECT_B = 0, 1
+ABI_VERSION = 2
 
 DTYPE_NAMES = {"f16": F16, "bf16": BF16, "fp8_e4m3": FP8_E4M3, "mxfp4": MXFP4, "f32": F32}
 
@@ -68,6 +69,7 @@ class Operands(C.Structure):
         ("dScaleA", C.c_void_p), ("dScaleB", C.c_void_p),
         ("dMxA", C.c_void_p), ("dMxB", C.c_void_p),
         ("dBias", C.c_void_p),
+        ("dWorkspace", C.c_void_p), ("workspace_bytes", C.c_size_t),
     ]
 
 
@@ -107,13 +109,14 @@ SIGNATURES = {
     "astergemm_variant_count": (C.c_int, []),
     "astergemm_variant_info": (C.c_int, [C.c_int, C.POINTER(Config), C.POINTER(KernelInfo)]),
     "astergemm_run": (C.c_int, [C.POINTER(Config), C.POINTER(Operands), _P]),
+    "astergemm_workspace_bytes": (C.c_int, [C.POINTER(Config), C.POINTER(C.c_size_t)]),
     "astergemm_bench_rotate": (C.c_int, [C.POINTER(Config), C.POINTER(Operands), C.c_int, C.c_int,
                                          C.POINTER(C.c_int64), C.c_void_p]),
     "astergemm_bench": (C.c_int, [C.POINTER(Config), C.POINTER(Operands), C.c_int,
                                   C.POINTER(C.c_int64), C.c_int64, _P]),
     "astergemm_tune": (C.c_int, [C.POINTER(Config), C.POINTER(Operands), C.c_int, C.POINTER(C.c_int),
                                  C.POINTER(C.c_int64), _P]),
-    "astergemm_mfma_ceiling": (C.c_int, [C.c_int, _P, C.c_int64, C.c_int, C.POINTER(C.c_double), _P]),
+    "astergemm_diag_mfma_rate": (C.c_int, [C.c_int, _P, C.c_int64, C.c_int, C.POINTER(C.c_double), _P]),
     "astergemm_shuffle_weight_16": (C.c_int, [_P, _P, C.c_int64, C.c_int64]),
     "astergemm_weight_crc32": (C.c_uint32, [_P, C.c_size_t]),
     "astergemm_weight_header_init": (C.c_int, [C.POINTER(WeightHeader), C.c_int, C.c_int, C.c_int64,
@@ -144,6 +147,8 @@ SIGNATURES = {
     "aster_rt_module_get_function": (C.c_int, [_P, C.c_char_p, C.POINTER(_P)]),
     "aster_rt_module_unload": (C.c_int, [_P]),
     "aster_rt_module_launch_kernel": (C.c_int, [_P] + [C.c_uint] * 7 + [_P, C.POINTER(_P)]),
+    "aster_rt_function_free": (C.c_int, [_P]),
+    "aster_rt_module_launch_kernel_ex": (C.c_int, [_P] + [C.c_uint] * 10 + [_P, C.POINTER(_P)]),
     "aster_rt_event_create": (C.c_int, [C.POINTER(_P)]),
     "aster_rt_event_destroy": (C.c_int, [_P]),
     "aster_rt_event_record": (C.c_int, [_P, _P]),

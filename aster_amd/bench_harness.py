@@ -145,12 +145,16 @@ def _compute_stats(post_warmup: Sequence[float], total_flops: int,
 RESULT_SENTINEL = "BENCH_RESULT_JSON:"
 
 
-def emit_one_result(stream, bench: str, cfg, stats: PerfStats) -> None:
-    """One `BENCH_RESULT_JSON:{...}` line; `stream=None` discards."""
+def emit_one_result(stream, bench: str, cfg, stats: PerfStats, *, label: str = None) -> None:
+    """One `BENCH_RESULT_JSON:{...}` line; `stream=None` discards.  `label` replaces the
+    config's own label (run_single passes the name of the kernel that actually ran when the
+    mapping was not honoured, so that mappings which ran the same pre-built kernel do not
+    become separate registry entries)."""
     if stream is None:
         return
     m, n, k = cfg.spec.gemm_size
-    rec = {"mcpu": cfg.mapping.mcpu, "bench": bench, "M": m, "N": n, "K": k, "label": cfg.label,
+    rec = {"mcpu": cfg.mapping.mcpu, "bench": bench, "M": m, "N": n, "K": k,
+           "label": label or cfg.label,
            "tflops_median": stats.p50_tf, "tflops_p10": stats.p10_tf, "tflops_p90": stats.p90_tf,
            "tflops_mean": stats.mean_tf, "tflops_p0": stats.p0_tf, "tflops_p25": stats.p25_tf,
            "tflops_stddev": stats.stddev_tf, "pct_peak_p50": stats.p50_pct, "sample_n": 1}
@@ -215,6 +219,18 @@ def run_single(cfg, compile_fn, args, execute_fn, *, bench: str = "unknown", out
         _, asm = compile_fn(cfg, hsaco)
         print(f"Config: {cfg.label}", file=out)
         print(asm, file=out)
+        # what the descriptor says was selected: a mapping the pre-built kernels do not have is
+        # recorded under the name of the kernel that runs instead
+        result_label = None
+        try:
+            with open(hsaco) as f:
+                desc = json.load(f)
+            if desc.get("mapping_honoured") is False:
+                result_label = desc["kernel"]
+                print(f"Mapping not honoured ({', '.join(desc['mapping_not_honoured'])}): "
+                      f"results are recorded as {result_label}", file=out)
+        except (OSError, ValueError, KeyError):
+            pass  # a compile_fn that writes a real code object
         if getattr(args, "compile_only", False):
             return None
         if not system_has_gpu("gfx950"):
@@ -236,7 +252,7 @@ def run_single(cfg, compile_fn, args, execute_fn, *, bench: str = "unknown", out
         results_path = getattr(args, "results_file", None)
         if results_path:
             with open(results_path, "a") as rs:
-                emit_one_result(rs, bench, cfg, s)
+                emit_one_result(rs, bench, cfg, s, label=result_label)
         print("\n--- Summary ---", file=out)
         print(f"  {'metric':<8s}  {'ms':>10s}  {'TFLOPS':>10s}  {'% peak':>8s}", file=out)
         for name, ms, tf, pct in (("p0", s.p0_ms, s.p0_tf, s.p0_pct), ("p10", s.p10_ms, s.p10_tf, None),

@@ -22,7 +22,7 @@ LIB_PATH = os.path.join(LIB_DIR, "libastergemm.so")
 OBJ_DIR = os.path.join(ROOT, "build", "obj")
 
 SOURCES = ["gemm_tile.hip", "gemm_stream.hip", "gemm_skinny.hip", "astergemm_api.hip", "quantize.hip",
-           "weight_artifact.hip", "mfma_ceiling.hip"]
+           "weight_artifact.hip", "diag_mfma_rate.hip"]
 HSACO_SOURCE = "hsaco_kernels.hip"
 HSACO_PATH = os.path.join(LIB_DIR, "astergemm_kernels.hsaco")
 REPLAY_PATH = os.path.join(LIB_DIR, "astergemm_replay")

@@ -5,6 +5,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <mutex>
 #include <vector>
 
 #include "astergemm_internal.h"
@@ -26,6 +27,36 @@ void set_error(const char* fmt, ...) {
 int hip_fail(hipError_t e, const char* what, const char* file, int line) {
   set_error("%s:%d - %s (%s)", file, line, hipGetErrorString(e), what);
   return ASTERGEMM_EHIP;
+}
+
+// Compute units of the current device (0 when there is none), cached per device ordinal.
+int device_cus() {
+  static std::atomic<int> cus[64];
+  static std::atomic<bool> init{false};
+  static std::mutex init_mutex;
+  if (!init.load(std::memory_order_acquire)) {
+    std::lock_guard<std::mutex> lock(init_mutex);
+    if (!init.load()) {
+      for (auto& c : cus) c.store(-1);
+      init.store(true, std::memory_order_release);
+    }
+  }
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  std::atomic<int>& slot = cus[dev & 63];
+  int n = slot.load();
+  if (n < 0) {
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, dev) == hipSuccess)
+      n = prop.multiProcessorCount;
+    else
+      (void)hipGetLastError(), n = 0;
+    slot.store(n);
+  }
+  return n;
 }
 
 namespace {
@@ -200,46 +231,23 @@ const Variant* choose(const astergemm_config& c, int* index_out) {
   return best;
 }
 
-// Compute units of the current device (0 when there is none), cached.
-int device_cus() {
-  static std::atomic<int> cus{-1};
-  int n = cus.load();
-  if (n < 0) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-      n = prop.multiProcessorCount;
-    else
-      (void)hipGetLastError(), n = 0;
-    cus.store(n);
-  }
-  return n;
+// K ranges the launcher of `v` cuts this problem into, and the fp32 workspace that takes.
+int splits_of(const Variant& v, const astergemm_config& c) { return v.splits ? v.splits(c) : 1; }
+size_t workspace_need(const Variant& v, const astergemm_config& c) {
+  const int S = splits_of(v, c);
+  return S > 1 ? (size_t)S * (size_t)c.M * (size_t)c.N * sizeof(float) : 0;
 }
 
 int grid_of(const Variant& v, const astergemm_config& c) {
+  if (v.grid) return v.grid(c, device_cus());
   if (v.family == ASTERGEMM_KERNEL_SKINNY) {
     const int blocks = (int)((c.N + v.tile_n - 1) / v.tile_n);
-    // the resident-activation kernels (8 waves) are persistent: one workgroup per CU
-    if (v.waves_n == 8 && v.tile_m == 64 && device_cus() > 0) {
-      // 32 < M <= 64: pairs of workgroups per row range, whole pairs on each of the 8 XCDs
-      // (rows longer than 8 KiB are also cut into K ranges, which fills the CUs sooner)
-      const int mh = c.M > 32 ? 2 : 1;
-      const int64_t rb = row_bytes(c.dtype_ab, c.K);
-      const int64_t want = (int64_t)blocks * mh * (rb > 8192 ? (rb % 8192 ? rb / 4096 : rb / 8192) : 1);
-      int g = want < device_cus() ? (int)want : device_cus();
-      if (mh == 2) g = g < 16 ? 16 : (g & ~15);
-      return g;
-    }
+    // the resident-activation kernels (8 waves) are persistent: at most one workgroup per CU
     if (v.waves_n == 8 && device_cus() > 0 && blocks > device_cus()) return device_cus();
     return blocks;
   }
   const int64_t tiles = ((c.M + v.tile_m - 1) / v.tile_m) * ((c.N + v.tile_n - 1) / v.tile_n);
-  if (v.rank == 4) {  // split K: one copy of the tile grid per K range
-    const int S = stream_split_of(tiles, row_bytes(c.dtype_ab, c.K) / 128,
-                                  c.dtype_ab == ASTERGEMM_MXFP4);
-    return (int)(tiles * (S > 0 ? S : 1));
-  }
-  return (int)tiles;
+  return (int)(tiles * splits_of(v, c));  // split K: one copy of the tile grid per K range
 }
 
 int64_t algorithmic_bytes(const astergemm_config& c) {
@@ -332,8 +340,42 @@ int build_args(const Variant& v, const astergemm_config& c, const astergemm_oper
   a->tiles_n = (int32_t)((c.N + v.tile_n - 1) / v.tile_n);
   a->group_m = 8;
   a->split_k = 1;
+  // rows cut into K ranges: the caller's workspace when one is given, else the library's own
+  if (ops.dWorkspace) {
+    const size_t need = workspace_need(v, c);
+    if (ops.workspace_bytes < need) {
+      set_error("astergemm: workspace of %zu bytes given, %s needs %zu for this config",
+                (size_t)ops.workspace_bytes, v.name, need);
+      return ASTERGEMM_EINVAL;
+    }
+    if (((uintptr_t)ops.dWorkspace) & 15) {
+      set_error("astergemm: dWorkspace must be 16-byte aligned");
+      return ASTERGEMM_EINVAL;
+    }
+    if (need) a->workspace = (float*)ops.dWorkspace;
+  }
   return 0;
 }
+
+// Start / stop events of a timed region; destroyed on every return path.
+struct EventPair {
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  hipError_t create() {
+    hipError_t e = hipEventCreate(&e0);
+    if (e == hipSuccess) e = hipEventCreate(&e1);
+    return e;
+  }
+  ~EventPair() {
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+  }
+};
+struct DeviceBuffer {
+  void* ptr = nullptr;
+  ~DeviceBuffer() {
+    if (ptr) (void)hipFree(ptr);
+  }
+};
 
 // Streams a scratch buffer so the next launch finds the last-level cache cold;
 // the reference's flush kernel does the same with a global_load_dword loop
@@ -399,6 +441,18 @@ int astergemm_run(const astergemm_config* cfg, const astergemm_operands* ops, vo
   return 0;
 }
 
+int astergemm_workspace_bytes(const astergemm_config* cfg, size_t* bytes) {
+  if (!cfg || !bytes) {
+    set_error("astergemm_workspace_bytes: null argument");
+    return ASTERGEMM_EINVAL;
+  }
+  int index = -1;
+  const Variant* v = choose(*cfg, &index);
+  if (!v) return g_choose_rc;
+  *bytes = (cfg->M == 0 || cfg->N == 0) ? 0 : workspace_need(*v, *cfg);
+  return 0;
+}
+
 int astergemm_bench_rotate(const astergemm_config* cfg, const astergemm_operands* ops, int n_ops,
                            int iters, int64_t* total_ns, void* stream) {
   if (!cfg || !ops || !total_ns || iters <= 0 || n_ops <= 0) {
@@ -415,18 +469,15 @@ int astergemm_bench_rotate(const astergemm_config* cfg, const astergemm_operands
     if (int rc = build_args(*v, *cfg, ops[i], &args[(size_t)i])) return rc;
   hipStream_t s = (hipStream_t)stream;
   const int grid = grid_of(*v, *cfg);
-  hipEvent_t e0, e1;
-  AG_HIP(hipEventCreate(&e0));
-  AG_HIP(hipEventCreate(&e1));
-  int le = (int)hipEventRecord(e0, s);
+  EventPair ev;
+  AG_HIP(ev.create());
+  int le = (int)hipEventRecord(ev.e0, s);
   (void)hipGetLastError();
   for (int i = 0; i < iters && le == 0; ++i) le = v->launch(args[(size_t)(i % n_ops)], grid, s);
-  if (le == 0) le = (int)hipEventRecord(e1, s);
-  if (le == 0) le = (int)hipEventSynchronize(e1);
+  if (le == 0) le = (int)hipEventRecord(ev.e1, s);
+  if (le == 0) le = (int)hipEventSynchronize(ev.e1);
   float ms = 0.f;
-  if (le == 0) le = (int)hipEventElapsedTime(&ms, e0, e1);
-  (void)hipEventDestroy(e0);
-  (void)hipEventDestroy(e1);
+  if (le == 0) le = (int)hipEventElapsedTime(&ms, ev.e0, ev.e1);
   if (le != 0) return hip_fail((hipError_t)le, v->name, __FILE__, __LINE__);
   *total_ns = (int64_t)((double)ms * 1e6);
   return 0;
@@ -445,9 +496,9 @@ int astergemm_tune(const astergemm_config* cfg, const astergemm_operands* ops, i
   *best_variant = 0;
   if (best_ns) *best_ns = 0;
   hipStream_t s = (hipStream_t)stream;
-  hipEvent_t e0, e1;
-  AG_HIP(hipEventCreate(&e0));
-  AG_HIP(hipEventCreate(&e1));
+  EventPair ev;
+  AG_HIP(ev.create());
+  hipEvent_t e0 = ev.e0, e1 = ev.e1;
   double best = 0.0;
   int rc = 0;
   for (int i = 0; i < total_variants() && rc == 0; ++i) {
@@ -482,8 +533,6 @@ int astergemm_tune(const astergemm_config* cfg, const astergemm_operands* ops, i
       *best_variant = i + 1;
     }
   }
-  (void)hipEventDestroy(e0);
-  (void)hipEventDestroy(e1);
   if (rc != 0) return rc;
   if (*best_variant == 0) {
     set_error("astergemm_tune: no kernel variant can run this config");
@@ -511,20 +560,26 @@ int astergemm_bench(const astergemm_config* cfg, const astergemm_operands* ops, 
   hipStream_t s = (hipStream_t)stream;
   const int grid = grid_of(*v, *cfg);
 
+  DeviceBuffer flush_buf;
   uint32_t* flush = nullptr;
   if (flush_bytes > 0) {
-    AG_HIP(hipMalloc((void**)&flush, (size_t)flush_bytes));
+    AG_HIP(hipMalloc(&flush_buf.ptr, (size_t)flush_bytes));
+    flush = (uint32_t*)flush_buf.ptr;
     AG_HIP(hipMemsetAsync(flush, 0, (size_t)flush_bytes, s));
   }
-  hipEvent_t e0, e1;
-  AG_HIP(hipEventCreate(&e0));
-  AG_HIP(hipEventCreate(&e1));
+  EventPair ev;
+  AG_HIP(ev.create());
+  hipEvent_t e0 = ev.e0, e1 = ev.e1;
   int rc = 0;
   (void)hipGetLastError();  // the launchers report hipGetLastError()
   for (int i = 0; i < iters && rc == 0; ++i) {
-    if (flush)
+    if (flush) {
       hipLaunchKernelGGL(flush_llc_kernel, dim3(2048), dim3(256), 0, s, flush,
                          (size_t)flush_bytes / 4);
+      // a flush that did not launch would give warm-cache times labelled as flushed
+      const hipError_t fe = hipGetLastError();
+      if (fe != hipSuccess) return hip_fail(fe, "flush_llc_kernel", __FILE__, __LINE__);
+    }
     hipError_t e = hipEventRecord(e0, s);
     int le = (e == hipSuccess) ? v->launch(a, grid, s) : (int)e;
     if (le == 0) le = (int)hipEventRecord(e1, s);
@@ -537,9 +592,6 @@ int astergemm_bench(const astergemm_config* cfg, const astergemm_operands* ops, 
     }
     times_ns[i] = (int64_t)((double)ms * 1e6);
   }
-  (void)hipEventDestroy(e0);
-  (void)hipEventDestroy(e1);
-  if (flush) (void)hipFree(flush);
   return rc;
 }
 
@@ -665,6 +717,25 @@ int aster_rt_module_launch_kernel(void* fn, unsigned gx, unsigned gy, unsigned g
   AG_HIP(hipModuleLaunchKernel((hipFunction_t)fn, gx, gy, gz, bx, by, bz, shared_bytes,
                                (hipStream_t)stream, kernel_params, nullptr));
   return 0;
+}
+int aster_rt_function_free(void* fn) {
+  // a hipFunction_t belongs to its module and goes with aster_rt_module_unload; the reference
+  // frees only the heap cell its binding wrapped the handle in (RuntimeModule.cpp:221-226)
+  (void)fn;
+  return 0;
+}
+int aster_rt_module_launch_kernel_ex(void* fn, unsigned gx, unsigned gy, unsigned gz, unsigned bx,
+                                     unsigned by, unsigned bz, unsigned cx, unsigned cy,
+                                     unsigned cz, unsigned shared_bytes, void* stream,
+                                     void** kernel_params) {
+  // cluster launches do not exist on gfx950: a cluster of (1,1,1) is a plain launch
+  if (cx > 1 || cy > 1 || cz > 1) {
+    set_error("aster_rt_module_launch_kernel_ex: cluster launch (%u,%u,%u) is not supported on "
+              "gfx950", cx, cy, cz);
+    return ASTERGEMM_ENOTSUP;
+  }
+  return aster_rt_module_launch_kernel(fn, gx, gy, gz, bx, by, bz, shared_bytes, stream,
+                                       kernel_params);
 }
 int aster_rt_event_create(void** event) {
   hipEvent_t e;

@@ -27,7 +27,8 @@ struct GemmArgs {
   int32_t tiles_m, tiles_n;
   int32_t group_m;       // tile rows per rasterisation group
   int32_t split_k;       // skinny path: K slices per output row block
-  float* workspace;      // skinny path: fp32 partials when split_k > 1
+  float* workspace;      // fp32 partials [split_k][M][N] when a row is cut into K ranges; set by
+                         // the caller of a launcher = use this buffer, null = the library's own
 };
 
 // Bytes of one operand row covering `k` elements.
@@ -61,7 +62,29 @@ struct Variant {
   const char* (*check)(const astergemm_config& c);
   // B operand form this variant reads (astergemm_operand_path); plain row-major by default.
   int operand_path = 0;
+  // K ranges the launcher cuts the rows of this problem into (1 = none): the launch then needs
+  // splits * M * N * 4 bytes of fp32 workspace.  nullptr = never splits.
+  int (*splits)(const astergemm_config& c) = nullptr;
+  // Grid the launcher uses when it is not the number of output tiles (persistent kernels);
+  // `cus` = compute units of the current device.  nullptr = tiles (times splits).
+  int (*grid)(const astergemm_config& c, int cus) = nullptr;
 };
+
+// Compute units of the current device (0 when there is none), cached per device ordinal.
+int device_cus();
+
+// Raises a kernel's dynamic-LDS limit once per device; `devs` is a static of the launcher with
+// one bit per device ordinal.  Returns 0 or a hipError_t.
+inline int lds_attr_once(std::atomic<uint64_t>& devs, const void* func, int lds_bytes) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return (int)hipGetLastError();
+  const uint64_t bit = (uint64_t)1 << (dev & 63);
+  if (devs.load(std::memory_order_acquire) & bit) return 0;
+  const hipError_t e = hipFuncSetAttribute(func, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+  if (e != hipSuccess) return (int)e;
+  devs.fetch_or(bit, std::memory_order_release);
+  return 0;
+}
 
 int num_tile_variants();
 const Variant* tile_variants();

@@ -1,12 +1,15 @@
-// The MFMA rate the chip sustains on given operand values, with nothing else going on: a loop
-// of independent MFMAs over registers that were filled once from a sample of the caller's
-// operand bytes.  No LDS, no memory traffic, no waits -- what is left is the matrix pipe under
-// the board's power limit, and that depends on the values: with zeros the loop runs close to
-// the published peak, with N(0, 0.02) bf16 data it settles near 70 % of it.  A GEMM on the same
-// values cannot be faster than this loop, so it is the ceiling to read a kernel's TFLOP/s
-// against next to the published one.  The instruction per dtype is the one the GEMM kernels
-// use: v_mfma_f32_16x16x32_{bf16,f16} and v_mfma_scale_f32_16x16x128_f8f6f4 (fp8, fp4 with
-// unit scales), the reference's (include/aster/Dialect/AMDGCN/IR/Instructions/MMA.td:792).
+// Diagnostic, not part of the GEMM path: the MFMA rate the chip reaches on given operand values
+// with nothing else going on -- a loop of independent MFMAs over registers that were filled once
+// from a sample of the caller's operand bytes.  No LDS, no memory traffic, no waits: what is left
+// is the matrix pipe under the board's power limit, and that depends on the values (with zeros
+// the loop runs close to the published peak, with N(0, 0.02) bf16 data it settles near 70 % of
+// it).  The loop is ordered like the GEMM kernels' inner loops (the first operand is held for
+// four instructions in a row, the second changes every instruction), so its rate is a measured
+// reference to read a kernel's TFLOP/s against next to the published peak; it is not a proven
+// upper bound (another operand order or register pattern may draw less power).  The instruction
+// per dtype is the one the GEMM kernels use: v_mfma_f32_16x16x32_{bf16,f16} and
+// v_mfma_scale_f32_16x16x128_f8f6f4 (fp8, fp4 with unit scales), the reference's
+// (include/aster/Dialect/AMDGCN/IR/Instructions/MMA.td:792).
 #include "astergemm_internal.h"
 
 namespace astergemm {
@@ -21,7 +24,7 @@ typedef int i32x8_t __attribute__((ext_vector_type(8)));
 constexpr int kAcc = 16;  // independent accumulators per wave: four A x four B operands
 
 template <int DT>
-__global__ __launch_bounds__(256) void mfma_ceiling_kernel(const i32x4* sample, int64_t n16,
+__global__ __launch_bounds__(256) void mfma_rate_kernel(const i32x4* sample, int64_t n16,
                                                            int iters, float* sink) {
   const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
   constexpr int R = (DT == ASTERGEMM_FP8_E4M3) ? 2 : 1;  // 16-byte registers per operand
@@ -39,7 +42,7 @@ __global__ __launch_bounds__(256) void mfma_ceiling_kernel(const i32x4* sample, 
   for (int it = 0; it < iters; ++it) {
 #pragma unroll
     for (int i = 0; i < kAcc; ++i) {
-      const int ia = i & 3, ib = i >> 2;
+      const int ia = i >> 2, ib = i & 3;  // first operand held for four instructions
       if constexpr (DT == ASTERGEMM_BF16) {
         acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a[ia][0]),
                                                           __builtin_bit_cast(bf16x8_t, b[ib][0]),
@@ -69,7 +72,7 @@ __global__ __launch_bounds__(256) void mfma_ceiling_kernel(const i32x4* sample, 
 }
 
 template <int DT>
-int run_ceiling(const void* sample, int64_t bytes, int target_ms, double* tflops, hipStream_t s) {
+int run_mfma_rate(const void* sample, int64_t bytes, int target_ms, double* tflops, hipStream_t s) {
   int dev = 0;
   hipDeviceProp_t prop;
   AG_HIP(hipGetDevice(&dev));
@@ -95,9 +98,9 @@ int run_ceiling(const void* sample, int64_t bytes, int target_ms, double* tflops
     const int launches = pass == 0 ? 1 : (target_ms + 9) / 10;
     for (int l = 0; !rc && l < launches; ++l) {
       if ((e = hipEventRecord(e0, s)) != hipSuccess) { fail(e, "hipEventRecord"); break; }
-      hipLaunchKernelGGL(mfma_ceiling_kernel<DT>, dim3(wgs), dim3(256), 0, s, (const i32x4*)sample,
+      hipLaunchKernelGGL(mfma_rate_kernel<DT>, dim3(wgs), dim3(256), 0, s, (const i32x4*)sample,
                          bytes / 16, iters, sink);
-      if ((e = hipGetLastError()) != hipSuccess) { fail(e, "mfma_ceiling_kernel"); break; }
+      if ((e = hipGetLastError()) != hipSuccess) { fail(e, "mfma_rate_kernel"); break; }
       if ((e = hipEventRecord(e1, s)) != hipSuccess) { fail(e, "hipEventRecord"); break; }
       if ((e = hipEventSynchronize(e1)) != hipSuccess) { fail(e, "hipEventSynchronize"); break; }
       if ((e = hipEventElapsedTime(&ms, e0, e1)) != hipSuccess) { fail(e, "hipEventElapsedTime"); break; }
@@ -124,23 +127,23 @@ int run_ceiling(const void* sample, int64_t bytes, int target_ms, double* tflops
 
 using namespace astergemm;
 
-extern "C" int astergemm_mfma_ceiling(int dtype_ab, const void* dSample, int64_t sample_bytes,
+extern "C" int astergemm_diag_mfma_rate(int dtype_ab, const void* dSample, int64_t sample_bytes,
                                       int target_ms, double* tflops, void* stream) {
   if (!dSample || !tflops || sample_bytes < 4096 || (sample_bytes & 15) ||
       ((uintptr_t)dSample & 15) || target_ms <= 0 || target_ms > 10000) {
-    set_error("astergemm_mfma_ceiling: need a 16-byte aligned sample of at least 4096 bytes (a "
+    set_error("astergemm_diag_mfma_rate: need a 16-byte aligned sample of at least 4096 bytes (a "
               "multiple of 16) and 0 < target_ms <= 10000");
     return ASTERGEMM_EINVAL;
   }
   (void)hipGetLastError();
   hipStream_t s = (hipStream_t)stream;
   switch (dtype_ab) {
-    case ASTERGEMM_BF16: return run_ceiling<ASTERGEMM_BF16>(dSample, sample_bytes, target_ms, tflops, s);
-    case ASTERGEMM_F16: return run_ceiling<ASTERGEMM_F16>(dSample, sample_bytes, target_ms, tflops, s);
+    case ASTERGEMM_BF16: return run_mfma_rate<ASTERGEMM_BF16>(dSample, sample_bytes, target_ms, tflops, s);
+    case ASTERGEMM_F16: return run_mfma_rate<ASTERGEMM_F16>(dSample, sample_bytes, target_ms, tflops, s);
     case ASTERGEMM_FP8_E4M3:
-      return run_ceiling<ASTERGEMM_FP8_E4M3>(dSample, sample_bytes, target_ms, tflops, s);
-    case ASTERGEMM_MXFP4: return run_ceiling<ASTERGEMM_MXFP4>(dSample, sample_bytes, target_ms, tflops, s);
+      return run_mfma_rate<ASTERGEMM_FP8_E4M3>(dSample, sample_bytes, target_ms, tflops, s);
+    case ASTERGEMM_MXFP4: return run_mfma_rate<ASTERGEMM_MXFP4>(dSample, sample_bytes, target_ms, tflops, s);
   }
-  set_error("astergemm_mfma_ceiling: dtype_ab must be F16, BF16, FP8_E4M3 or MXFP4");
+  set_error("astergemm_diag_mfma_rate: dtype_ab must be F16, BF16, FP8_E4M3 or MXFP4");
   return ASTERGEMM_EINVAL;
 }

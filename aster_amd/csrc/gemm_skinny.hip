@@ -15,6 +15,7 @@
 #include <mutex>
 #include <type_traits>
 #include <utility>
+#include <vector>
 
 #include "astergemm_internal.h"
 
@@ -393,21 +394,12 @@ template <int DT, int OUT, int SPB>
 int launch_skinny_reg_t(const GemmArgs& a, hipStream_t s) {
   auto k = gemm_skinny_reg_kernel<DT, OUT, SPB>;
   constexpr int lds = 8 * 8192 + 2 * 4 * 8 * 64 * 16;
-  static std::atomic<bool> attr_set{false};
-  static std::atomic<int> cus{0};
-  if (!attr_set) {
-    hipError_t e =
-        hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-    if (e != hipSuccess) return (int)e;
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess)
-      return (int)hipGetLastError();
-    cus = prop.multiProcessorCount;
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> attr_devs{0};
+  if (int e = lds_attr_once(attr_devs, (const void*)k, lds)) return e;
+  const int cus = device_cus();
+  if (cus <= 0) return (int)hipErrorNoDevice;
   const int nblocks = (int)((a.N + 15) / 16);
-  const int g = nblocks < cus.load() ? nblocks : cus.load();
+  const int g = nblocks < cus ? nblocks : cus;
   hipLaunchKernelGGL(k, dim3(g), dim3(512), lds, s, a);
   return (int)hipGetLastError();
 }
@@ -622,21 +614,12 @@ template <int OUT, int SPB, int SU>
 int launch_skinny_fp4_t(const GemmArgs& a, hipStream_t s) {
   auto k = gemm_skinny_fp4_kernel<OUT, SPB, SU>;
   constexpr int lds = 8 * 8192 + 2 * 4 * 8 * 64 * 16;
-  static std::atomic<bool> attr_set{false};
-  static std::atomic<int> cus{0};
-  if (!attr_set) {
-    hipError_t e =
-        hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-    if (e != hipSuccess) return (int)e;
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess)
-      return (int)hipGetLastError();
-    cus = prop.multiProcessorCount;
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> attr_devs{0};
+  if (int e = lds_attr_once(attr_devs, (const void*)k, lds)) return e;
+  const int cus = device_cus();
+  if (cus <= 0) return (int)hipErrorNoDevice;
   const int nblocks = (int)((a.N + 15) / 16);
-  const int g = nblocks < cus.load() ? nblocks : cus.load();
+  const int g = nblocks < cus ? nblocks : cus;
   hipLaunchKernelGGL(k, dim3(g), dim3(512), lds, s, a);
   return (int)hipGetLastError();
 }
@@ -737,16 +720,19 @@ void launch_splitk_reduce(const GemmArgs& a, int S, hipStream_t s) {
                      a.M, a.N, a.ldc, a.scale_a, a.scale_b, a.bias, a.C);
 }
 
-// fp32 scratch for the K-split partial sums: one buffer per (device, stream), so launches on
-// different streams never share one; launches on one stream are ordered and reuse it.  A
-// buffer grows on demand (the stream is drained before the old one is released) and lives
-// until the process ends.
+// fp32 scratch for the K-split partial sums when the caller brings none: one buffer per
+// (device, stream), so launches on different streams never share one; launches on one stream are
+// ordered and reuse it.  A buffer that is too small is replaced by one at least twice its size
+// and stays allocated (kernels already enqueued, or being enqueued by another host thread, keep a
+// valid pointer), so the retired buffers together stay below the size of the live one; nothing
+// is released before the process ends.
 struct SplitWorkspace {
   float* ptr = nullptr;
   size_t bytes = 0;
 };
 std::mutex g_ws_mutex;
 std::map<std::pair<int, hipStream_t>, SplitWorkspace> g_ws;
+std::vector<float*> g_ws_retired;
 
 int splitk_workspace(size_t bytes, hipStream_t stream, float** out) {
   int dev = 0;
@@ -754,17 +740,34 @@ int splitk_workspace(size_t bytes, hipStream_t stream, float** out) {
   std::lock_guard<std::mutex> lock(g_ws_mutex);
   SplitWorkspace& w = g_ws[{dev, stream}];
   if (bytes > w.bytes) {
-    if (w.ptr) {
-      if (hipStreamSynchronize(stream) != hipSuccess) return (int)hipGetLastError();
-      (void)hipFree(w.ptr);
-      w = SplitWorkspace{};
-    }
-    const size_t want = bytes < ((size_t)8 << 20) ? ((size_t)8 << 20) : bytes;
-    if (hipMalloc((void**)&w.ptr, want) != hipSuccess) return (int)hipGetLastError();
+    size_t want = bytes < ((size_t)8 << 20) ? ((size_t)8 << 20) : bytes;
+    if (want < 2 * w.bytes) want = 2 * w.bytes;
+    float* fresh = nullptr;
+    if (hipMalloc((void**)&fresh, want) != hipSuccess) return (int)hipGetLastError();
+    if (w.ptr) g_ws_retired.push_back(w.ptr);
+    w.ptr = fresh;
     w.bytes = want;
   }
   *out = w.ptr;
   return 0;
+}
+
+// Grid of the K-range decode kernels: S K ranges x R row ranges, one workgroup per CU; above 32
+// activation rows two workgroups (MH = 2) share a row range, in whole pairs on each of the 8
+// XCDs.  The launchers and the description of a variant both come here.
+struct KRangeGrid {
+  int mh, rows, grid;
+};
+inline KRangeGrid krange_grid(int64_t M, int64_t N, int S, int cus) {
+  KRangeGrid g;
+  g.mh = M > 32 ? 2 : 1;
+  const int nblocks = (int)((N + 15) / 16);
+  const int slots = g.mh == 2 ? (cus / 16) * 8 : cus;
+  int R = slots / S;
+  g.rows = R < 1 ? 1 : (R > nblocks ? nblocks : R);
+  g.grid = g.mh * S * g.rows;
+  if (g.mh == 2) g.grid = (g.grid + 15) & ~15;
+  return g;
 }
 
 // The MXFP4 kernel above with two activation tiles per wave and, for M > 32, two workgroups
@@ -1019,32 +1022,19 @@ template <int OUT, int SPB, int SU, int MT, int MH>
 int launch_skinny_fp4m_t(const GemmArgs& a0, int S, hipStream_t s) {
   auto k = gemm_skinny_fp4m_kernel<OUT, SPB, SU, MT, MH>;
   constexpr int lds = 8 * 8192 + 2 * 2 * MT * 8 * 64 * 16;
-  static std::atomic<bool> attr_set{false};
-  static std::atomic<int> cus{0};
-  if (!attr_set) {
-    hipError_t e =
-        hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-    if (e != hipSuccess) return (int)e;
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess)
-      return (int)hipGetLastError();
-    cus = prop.multiProcessorCount;
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> attr_devs{0};
+  if (int e = lds_attr_once(attr_devs, (const void*)k, lds)) return e;
+  const int cus = device_cus();
+  if (cus <= 0) return (int)hipErrorNoDevice;
   GemmArgs a = a0;
-  const int nblocks = (int)((a.N + 15) / 16);
-  const int slots = (MH == 2 ? (cus.load() / 16) * 8 : cus.load());
-  int R = slots / S;
-  R = R < 1 ? 1 : (R > nblocks ? nblocks : R);
-  a.tiles_n = R;
+  const KRangeGrid kg = krange_grid(a.M, a.N, S, cus);
+  if (kg.mh != MH) return (int)hipErrorInvalidValue;
+  a.tiles_n = kg.rows;
   a.split_k = S;
-  int g = MH * S * R;
-  if (MH == 2) g = (g + 15) & ~15;
-  if (S > 1) {
+  if (S > 1 && !a.workspace) {
     if (int rc = splitk_workspace((size_t)S * a.M * a.N * sizeof(float), s, &a.workspace)) return rc;
   }
-  hipLaunchKernelGGL(k, dim3(g), dim3(512), lds, s, a);
+  hipLaunchKernelGGL(k, dim3(kg.grid), dim3(512), lds, s, a);
   if (S > 1) launch_splitk_reduce<OUT>(a, S, s);
   return (int)hipGetLastError();
 }
@@ -1074,11 +1064,21 @@ const char* check_skinny_fp4m(const astergemm_config& c) {
   return nullptr;
 }
 
+int splits_skinny_fp4m(const astergemm_config& c) {
+  int spb = 0;
+  const int S = skinny_fp4_split_of(c.K / 2, &spb);
+  return S < 1 ? 1 : S;
+}
+int grid_skinny_fp4m(const astergemm_config& c, int cus) {
+  return krange_grid(c.M, c.N, splits_skinny_fp4m(c), cus).grid;
+}
+
 #define AG_SKINNY_FP4M(name, OUT)                                                          \
   Variant {                                                                                \
     name, ASTERGEMM_KERNEL_SKINNY, ASTERGEMM_MXFP4, OUT, 64, 16, 512, 1, 8, 1, 2,           \
         8 * 8192 + 65536, (const void*)gemm_skinny_fp4m_kernel<OUT, 2, 2, 2, 2>,           \
-        launch_skinny_fp4m<OUT>, check_skinny_fp4m                                         \
+        launch_skinny_fp4m<OUT>, check_skinny_fp4m, ASTERGEMM_OPERAND_LDS,                 \
+        splits_skinny_fp4m, grid_skinny_fp4m                                               \
   }
 
 // ---- 16 < M <= 64: the same persistent kernel with two activation tiles per wave --------
@@ -1329,34 +1329,19 @@ template <int DT, int OUT, int SPB, int MT, int MH>
 int launch_skinny_regm_t(const GemmArgs& a0, int S, hipStream_t s) {
   auto k = gemm_skinny_regm_kernel<DT, OUT, SPB, MT, MH>;
   constexpr int lds = 8 * 8192 + 2 * 2 * MT * 8 * 64 * 16;
-  static std::atomic<bool> attr_set{false};
-  static std::atomic<int> cus{0};
-  if (!attr_set) {
-    hipError_t e =
-        hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-    if (e != hipSuccess) return (int)e;
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess)
-      return (int)hipGetLastError();
-    cus = prop.multiProcessorCount;
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> attr_devs{0};
+  if (int e = lds_attr_once(attr_devs, (const void*)k, lds)) return e;
+  const int cus = device_cus();
+  if (cus <= 0) return (int)hipErrorNoDevice;
   GemmArgs a = a0;
-  // one workgroup per CU: S K ranges x R row ranges (x 2 halves of the activation rows with
-  // MH = 2, whose grid is whole pairs on each of the 8 XCDs)
-  const int nblocks = (int)((a.N + 15) / 16);
-  const int slots = (MH == 2 ? (cus.load() / 16) * 8 : cus.load());
-  int R = slots / S;
-  R = R < 1 ? 1 : (R > nblocks ? nblocks : R);
-  a.tiles_n = R;
+  const KRangeGrid kg = krange_grid(a.M, a.N, S, cus);
+  if (kg.mh != MH) return (int)hipErrorInvalidValue;
+  a.tiles_n = kg.rows;
   a.split_k = S;
-  int g = MH * S * R;
-  if (MH == 2) g = (g + 15) & ~15;
-  if (S > 1) {
+  if (S > 1 && !a.workspace) {
     if (int rc = splitk_workspace((size_t)S * a.M * a.N * sizeof(float), s, &a.workspace)) return rc;
   }
-  hipLaunchKernelGGL(k, dim3(g), dim3(512), lds, s, a);
+  hipLaunchKernelGGL(k, dim3(kg.grid), dim3(512), lds, s, a);
   if (S > 1) launch_splitk_reduce<OUT>(a, S, s);
   return (int)hipGetLastError();
 }
@@ -1389,11 +1374,20 @@ const char* check_skinny_regm(const astergemm_config& c) {
   return nullptr;
 }
 
+int splits_skinny_regm(const astergemm_config& c) {
+  int spb = 0;
+  const int S = skinny_split_of(row_bytes(c.dtype_ab, c.K), &spb);
+  return S < 1 ? 1 : S;
+}
+int grid_skinny_regm(const astergemm_config& c, int cus) {
+  return krange_grid(c.M, c.N, splits_skinny_regm(c), cus).grid;
+}
+
 #define AG_SKINNY_LDSM(name, DT, OUT)                                                      \
   Variant {                                                                                \
     name, ASTERGEMM_KERNEL_SKINNY, DT, OUT, 64, 16, 512, 1, 8, 1, 2, 8 * 8192 + 65536,      \
         (const void*)gemm_skinny_regm_kernel<DT, OUT, 8, 2, 2>, launch_skinny_regm<DT, OUT>, \
-        check_skinny_regm                                                                  \
+        check_skinny_regm, ASTERGEMM_OPERAND_LDS, splits_skinny_regm, grid_skinny_regm     \
   }
 
 template <int DT, int OUT>
@@ -1601,21 +1595,12 @@ template <int DT, int OUT, int CPW>
 int launch_skinny_direct_t(const GemmArgs& a, hipStream_t s) {
   auto k = gemm_skinny_direct_kernel<DT, OUT, CPW>;
   constexpr int lds = 2 * 4 * 8 * 64 * 16 + 8 * 8192;
-  static std::atomic<bool> attr_set{false};
-  static std::atomic<int> cus{0};
-  if (!attr_set) {
-    hipError_t e =
-        hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-    if (e != hipSuccess) return (int)e;
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess)
-      return (int)hipGetLastError();
-    cus = prop.multiProcessorCount;
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> attr_devs{0};
+  if (int e = lds_attr_once(attr_devs, (const void*)k, lds)) return e;
+  const int cus = device_cus();
+  if (cus <= 0) return (int)hipErrorNoDevice;
   const int nblocks = (int)((a.N + 15) / 16);
-  const int g = nblocks < cus.load() ? nblocks : cus.load();
+  const int g = nblocks < cus ? nblocks : cus;
   hipLaunchKernelGGL(k, dim3(g), dim3(512), lds, s, a);
   return (int)hipGetLastError();
 }

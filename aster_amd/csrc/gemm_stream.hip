@@ -12,13 +12,8 @@ template <int DT, int OUT, int BM, int BN, int WM, int WN>
 int launch_stream(const GemmArgs& a, int grid, hipStream_t s) {
   constexpr int lds = 5 * BM * kRowBytes;
   auto k = gemm_stream_kernel<DT, OUT, BM, BN, WM, WN>;
-  static std::atomic<bool> attr_set{false};
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)k,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-    if (e != hipSuccess) return (int)e;
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> attr_devs{0};
+  if (int e = lds_attr_once(attr_devs, (const void*)k, lds)) return e;
   hipLaunchKernelGGL(k, dim3(grid), dim3(WM * WN * 64), lds, s, a);
   return (int)hipGetLastError();
 }
@@ -61,13 +56,8 @@ int launch_stream_splitk(const GemmArgs& a0, int grid, hipStream_t s) {
   if constexpr (KIND == 0) k = gemm_stream_splitk_kernel<DT, 128, 128, 2, 2>;
   else if constexpr (KIND == 1) k = gemm_stream8_splitk_kernel<DT, 128, 128, 2, 2>;
   else k = gemm_stream4_splitk_kernel<DT, 128, 128, 2, 2>;
-  static std::atomic<bool> attr_set{false};
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)k,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-    if (e != hipSuccess) return (int)e;
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> attr_devs{0};
+  if (int e = lds_attr_once(attr_devs, (const void*)k, lds)) return e;
   if constexpr (KIND == 2) {
     if ((((uintptr_t)a0.mx_a | (uintptr_t)a0.mx_b) & 15) != 0 || a0.mx_ld % 16 != 0)
       return (int)hipErrorInvalidValue;
@@ -76,8 +66,10 @@ int launch_stream_splitk(const GemmArgs& a0, int grid, hipStream_t s) {
   const int S = stream_split_of(tiles, a0.ksteps, KIND == 2);
   if (S == 0) return (int)hipErrorInvalidValue;
   GemmArgs a = a0;
-  if (int rc = splitk_workspace_for((size_t)S * a.M * a.N * sizeof(float), s, &a.workspace))
-    return rc;
+  if (!a.workspace) {
+    if (int rc = splitk_workspace_for((size_t)S * a.M * a.N * sizeof(float), s, &a.workspace))
+      return rc;
+  }
   GemmArgs part = a;           // what the K-range workgroups see: fp32 planes, no epilogue terms
   part.split_k = S;
   part.ksteps = a.ksteps / S;
@@ -103,11 +95,18 @@ const char* check_stream_splitk(const astergemm_config& c) {
   return nullptr;
 }
 
+int splits_stream_splitk(const astergemm_config& c) {
+  const int64_t tiles = ((c.M + 127) / 128) * ((c.N + 127) / 128);
+  const int S = stream_split_of(tiles, row_bytes(c.dtype_ab, c.K) / kRowBytes,
+                                c.dtype_ab == ASTERGEMM_MXFP4);
+  return S < 1 ? 1 : S;
+}
+
 #define AG_STREAM_SPLITK(name, KIND, DT, OUT, LDS, FUNC)                         \
   Variant {                                                                      \
     name, ASTERGEMM_KERNEL_TILE, DT, OUT, 128, 128, kRowBytes, 2, 2, 3, 4, LDS,  \
         (const void*)FUNC<DT, 128, 128, 2, 2>, launch_stream_splitk<KIND, DT, OUT>, \
-        check_stream_splitk                                                      \
+        check_stream_splitk, ASTERGEMM_OPERAND_LDS, splits_stream_splitk         \
   }
 #define AG_STREAM_SPLITK_SET(prefix, KIND, DT, LDS, FUNC)                        \
   AG_STREAM_SPLITK(prefix "_128x128_w2x2_bf16", KIND, DT, ASTERGEMM_BF16, LDS, FUNC),   \
@@ -118,13 +117,8 @@ template <int DT, int OUT, int BM, int BN, int WM, int WN>
 int launch_stream8(const GemmArgs& a, int grid, hipStream_t s) {
   constexpr int lds = 5 * BM * kRowBytes;
   auto k = gemm_stream8_kernel<DT, OUT, BM, BN, WM, WN>;
-  static std::atomic<bool> attr_set{false};
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)k,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-    if (e != hipSuccess) return (int)e;
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> attr_devs{0};
+  if (int e = lds_attr_once(attr_devs, (const void*)k, lds)) return e;
   hipLaunchKernelGGL(k, dim3(grid), dim3(WM * WN * 64), lds, s, a);
   return (int)hipGetLastError();
 }
@@ -151,13 +145,8 @@ int launch_stream4(const GemmArgs& a, int grid, hipStream_t s) {
   if ((((uintptr_t)a.mx_a | (uintptr_t)a.mx_b) & 15) != 0 || a.mx_ld % 16 != 0)
     return (int)hipErrorInvalidValue;
   auto k = gemm_stream4_kernel<DT, OUT, BM, BN, WM, WN>;
-  static std::atomic<bool> attr_set{false};
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)k,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-    if (e != hipSuccess) return (int)e;
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> attr_devs{0};
+  if (int e = lds_attr_once(attr_devs, (const void*)k, lds)) return e;
   hipLaunchKernelGGL(k, dim3(grid), dim3(WM * WN * 64), lds, s, a);
   return (int)hipGetLastError();
 }

@@ -1,6 +1,6 @@
 // Variant table and launchers of the LDS-staged MFMA tile kernels
 // (device code: gemm_tile_kernel.hpp).
-#include "gemm_pipe_kernel.hpp"
+#include "gemm_tile_kernel.hpp"
 
 namespace astergemm {
 namespace {
@@ -10,13 +10,8 @@ template <int DT, int OUT, int BM, int BN, int WM, int WN>
 int launch_tile(const GemmArgs& a, int grid, hipStream_t s) {
   constexpr int lds = 2 * (BM + BN) * kRowBytes;
   auto k = gemm_tile_kernel<DT, OUT, BM, BN, WM, WN>;
-  static std::atomic<bool> attr_set{false};
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)k,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-    if (e != hipSuccess) return (int)e;
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> attr_devs{0};
+  if (int e = lds_attr_once(attr_devs, (const void*)k, lds)) return e;
   hipLaunchKernelGGL(k, dim3(grid), dim3(WM * WN * 64), lds, s, a);
   return (int)hipGetLastError();
 }
@@ -53,48 +48,11 @@ const char* check_tile(const astergemm_config& c) {
       AG_TILE(prefix "_64x64_w2x2_f32", DT, ASTERGEMM_F32, 64, 64, 2, 2),              \
       AG_TILE(prefix "_64x64_w2x2_f16", DT, ASTERGEMM_F16, 64, 64, 2, 2)
 
-template <int DT, int OUT, int BM, int BN, int WM, int WN>
-int launch_pipe(const GemmArgs& a0, int grid, hipStream_t s) {
-  constexpr int lds = kStages * (BM + BN) * kSubBytes;
-  auto k = gemm_pipe_kernel<DT, OUT, BM, BN, WM, WN>;
-  static std::atomic<bool> attr_set{false};
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)k,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-    if (e != hipSuccess) return (int)e;
-    attr_set = true;
-  }
-  // This kernel counts K in 64-byte sub-steps.
-  GemmArgs a = a0;
-  const int64_t kb = row_bytes(DT, a.K);
-  a.ksteps = (int32_t)((kb + kSubBytes - 1) / kSubBytes);
-  a.tail_granules = (int32_t)((kb % kSubBytes) / 16);
-  hipLaunchKernelGGL(k, dim3(grid), dim3(WM * WN * 64), lds, s, a);
-  return (int)hipGetLastError();
-}
-
-#define AG_PIPE(name, DT, OUT, BM, BN, WM, WN)                                   \
-  Variant {                                                                      \
-    name, ASTERGEMM_KERNEL_TILE, DT, OUT, BM, BN, kSubBytes, WM, WN, kStages, 0, \
-        kStages * (BM + BN) * kSubBytes,                                         \
-        (const void*)gemm_pipe_kernel<DT, OUT, BM, BN, WM, WN>,                  \
-        launch_pipe<DT, OUT, BM, BN, WM, WN>, check_tile                         \
-  }
-
-#define AG_PIPE_SET(prefix, DT)                                                        \
-  AG_PIPE(prefix "_256x256_w2x4_bf16", DT, ASTERGEMM_BF16, 256, 256, 2, 4),            \
-      AG_PIPE(prefix "_256x256_w2x4_f32", DT, ASTERGEMM_F32, 256, 256, 2, 4),          \
-      AG_PIPE(prefix "_256x256_w2x4_f16", DT, ASTERGEMM_F16, 256, 256, 2, 4),          \
-      AG_PIPE(prefix "_256x256_w2x2_bf16", DT, ASTERGEMM_BF16, 256, 256, 2, 2)
-
 const Variant kTileVariants[] = {
     AG_TILE_SET("tile_bf16", ASTERGEMM_BF16),
     AG_TILE_SET("tile_f16", ASTERGEMM_F16),
     AG_TILE_SET("tile_fp8", ASTERGEMM_FP8_E4M3),
     AG_TILE_SET("tile_mxfp4", ASTERGEMM_MXFP4),
-    AG_PIPE_SET("pipe_bf16", ASTERGEMM_BF16),
-    AG_PIPE_SET("pipe_f16", ASTERGEMM_F16),
-    AG_PIPE_SET("pipe_fp8", ASTERGEMM_FP8_E4M3),
 };
 
 }  // namespace

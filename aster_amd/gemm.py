@@ -36,9 +36,10 @@ _OUT_NP = {"f32": np.float32, "bf16": np.uint16, "f16": np.float16}
 
 def config_from_instance(cfg: WeakScaledMappedGemmInstance, *, use_mapping: bool = True,
                          family: int = _capi.KERNEL_AUTO) -> _capi.Config:
-    """C-ABI config for a (spec, mapping) instance.  With `use_mapping` the
-    workgroup tile and wave grid are passed as a request; the library falls back
-    to its default variant when no pre-built kernel has that geometry."""
+    """C-ABI config for a (spec, mapping) instance.  With `use_mapping` the workgroup tile, the
+    wave grid and the operand path (`direct_b`: B pre-shuffled with `shuffle_weight`) are passed
+    as a request; `select_for_instance` falls back to the library's own choice when no pre-built
+    kernel has that geometry and says so."""
     spec, mapping = cfg.spec, cfg.mapping
     M, N, K = spec.gemm_size
     c = _capi.Config()
@@ -54,6 +55,8 @@ def config_from_instance(cfg: WeakScaledMappedGemmInstance, *, use_mapping: bool
         c.wg_tile_n = twg[DIM_N] * spec.mfma_shape[DIM_N]
         c.waves_m = mapping.num_waves_per_workgroup[DIM_M]
         c.waves_n = mapping.num_waves_per_workgroup[DIM_N]
+        if mapping.direct_b and not mapping.direct_a:
+            c.operand_path = _capi.OPERAND_DIRECT_B
     return c
 
 
@@ -63,15 +66,68 @@ def select(c: _capi.Config) -> _capi.KernelInfo:
     return info
 
 
+@dataclass
+class MappingReport:
+    """How much of a GemmMappingSpec the selected pre-built kernel follows.
+
+    `honoured`: a variant with the requested workgroup tile, wave grid and operand path exists
+    for the problem and was selected.  `not_honoured`: the requested values the kernel does not
+    have, each with what runs instead.  `fixed_by_kernel`: knobs that steer the reference's
+    compiler (pipeline strategy, scheduler preset, peeling, barriers, load type ...) and have no
+    effect on a kernel that is already built."""
+
+    honoured: bool
+    not_honoured: dict
+    fixed_by_kernel: dict
+
+
+_COMPILER_KNOBS = ("pipeline_strategy", "load_type", "lcm_unroll", "unroll_factor_multiplier",
+                   "prologue_peeling", "epilogue_peeling", "ll_sched", "hoist_wait",
+                   "set_mfma_priority", "rotate_compute_stage", "use_conservative_barriers",
+                   "num_wg_per_cu")
+
+
+def mapping_report(cfg: WeakScaledMappedGemmInstance, c: _capi.Config,
+                   info: _capi.KernelInfo) -> MappingReport:
+    spec, mapping = cfg.spec, cfg.mapping
+    twg = mapping.num_tiles_per_workgroup
+    want_tile = [twg[DIM_M] * spec.mfma_shape[DIM_M], twg[DIM_N] * spec.mfma_shape[DIM_N]]
+    want_waves = [mapping.num_waves_per_workgroup[DIM_M], mapping.num_waves_per_workgroup[DIM_N]]
+    miss = {}
+    if [info.wg_tile_m, info.wg_tile_n] != want_tile:
+        miss["wg_tile"] = {"requested": want_tile, "kernel": [info.wg_tile_m, info.wg_tile_n]}
+    if [info.waves_m, info.waves_n] != want_waves:
+        miss["waves"] = {"requested": want_waves, "kernel": [info.waves_m, info.waves_n]}
+    ran_path = "direct_b" if c.operand_path == _capi.OPERAND_DIRECT_B else "lds"
+    if mapping.operand_path.value != ran_path:
+        miss["operand_path"] = {"requested": mapping.operand_path.value, "kernel": ran_path}
+    fixed = {}
+    for k in _COMPILER_KNOBS:
+        if hasattr(mapping, k):
+            v = getattr(mapping, k)
+            fixed[k] = getattr(v, "value", v)
+    return MappingReport(not miss, miss, fixed)
+
+
 def select_for_instance(cfg: WeakScaledMappedGemmInstance) -> Tuple[_capi.Config, _capi.KernelInfo]:
-    """Honour the instance's mapping when a variant with that geometry exists,
-    otherwise let the library choose."""
+    """Honour the instance's mapping when a variant with that geometry exists, otherwise let the
+    library choose (`mapping_report` tells which happened).  A `direct_b` request that no kernel
+    takes for this shape falls back to plain row-major B."""
     c = config_from_instance(cfg, use_mapping=True)
     try:
         return c, select(c)
     except _capi.AsterGemmError as e:
         if e.code != -95:
             raise
+    if c.operand_path == _capi.OPERAND_DIRECT_B:
+        # keep the operand path, drop the geometry
+        c2 = config_from_instance(cfg, use_mapping=False)
+        c2.operand_path = _capi.OPERAND_DIRECT_B
+        try:
+            return c2, select(c2)
+        except _capi.AsterGemmError as e:
+            if e.code != -95:
+                raise
     c = config_from_instance(cfg, use_mapping=False)
     return c, select(c)
 
@@ -83,8 +139,13 @@ def compile_gemm(cfg: WeakScaledMappedGemmInstance, output_hsaco_path: str, **kw
     `.amdgpu_metadata` spelling (`.vgpr_count`, `.lds_size`...), which is what
     harness code parses the reference's asm for.  Register budgets
     (`num_vgprs`, `num_agprs`) are accepted and ignored: the kernels are built.
+    The descriptor and the summary say whether the mapping was honoured
+    (`mapping_honoured`, `mapping_not_honoured`) and which of its knobs cannot
+    change a pre-built kernel (`mapping_fixed_by_kernel`), so that a sweep over
+    mappings can tell labels that ran the same kernel apart from real variants.
     """
     c, info = select_for_instance(cfg)
+    rep = mapping_report(cfg, c, info)
     desc = {
         "format": "astergemm-descriptor-v1",
         "label": cfg.label,
@@ -96,13 +157,20 @@ def compile_gemm(cfg: WeakScaledMappedGemmInstance, output_hsaco_path: str, **kw
         "vgprs": info.vgprs,
         "wg_tile": [info.wg_tile_m, info.wg_tile_n, info.wg_tile_k],
         "waves": [info.waves_m, info.waves_n],
+        "operand_path": "direct_b" if c.operand_path == _capi.OPERAND_DIRECT_B else "lds",
+        "mapping_honoured": rep.honoured,
+        "mapping_not_honoured": rep.not_honoured,
+        "mapping_fixed_by_kernel": rep.fixed_by_kernel,
     }
     with open(output_hsaco_path, "w") as f:
         json.dump(desc, f)
     asm = (f".amdhsa_kernel {cfg.kernel_name}\n  .name: {info.name.decode()}\n"
            f"  .vgpr_count: {info.vgprs}\n  .agpr_count: {info.agprs}\n"
            f"  .group_segment_fixed_size: {info.lds_bytes}\n"
-           f"  .max_flat_workgroup_size: {info.block_x}\n")
+           f"  .max_flat_workgroup_size: {info.block_x}\n"
+           f"  ; mapping_honoured: {str(rep.honoured).lower()}\n")
+    for k, v in rep.not_honoured.items():
+        asm += f"  ; {k}: requested {v['requested']}, kernel has {v['kernel']}\n"
     return output_hsaco_path, asm
 
 
@@ -142,17 +210,29 @@ class GemmPlan:
         c.variant = variant
         return cls(c, select(c))
 
-    def _operands(self, dA, dB, dC, scale_a, scale_b, mx_a, mx_b, bias) -> _capi.Operands:
+    def _operands(self, dA, dB, dC, scale_a, scale_b, mx_a, mx_b, bias, workspace=None,
+                  workspace_bytes=0) -> _capi.Operands:
         ops = _capi.Operands()
         ops.dA, ops.dB, ops.dC = dA, dB, dC
         ops.dScaleA, ops.dScaleB = scale_a, scale_b
         ops.dMxA, ops.dMxB = mx_a, mx_b
         ops.dBias = bias
+        ops.dWorkspace, ops.workspace_bytes = workspace, workspace_bytes
         return ops
 
+    def workspace_bytes(self) -> int:
+        """Bytes of fp32 workspace a launch of this plan needs (0 unless its rows are cut into
+        K ranges); pass a buffer of that size as `workspace` to `run`, or leave it to the
+        library's own buffer."""
+        n = ctypes.c_size_t()
+        _capi.check(_capi.load().astergemm_workspace_bytes(ctypes.byref(self.config), ctypes.byref(n)))
+        return n.value
+
     def run(self, dA: int, dB: int, dC: int, *, scale_a: int = None, scale_b: int = None,
-            mx_a: int = None, mx_b: int = None, bias: int = None, stream: int = None) -> None:
-        ops = self._operands(dA, dB, dC, scale_a, scale_b, mx_a, mx_b, bias)
+            mx_a: int = None, mx_b: int = None, bias: int = None, stream: int = None,
+            workspace: int = None, workspace_bytes: int = 0) -> None:
+        ops = self._operands(dA, dB, dC, scale_a, scale_b, mx_a, mx_b, bias, workspace,
+                             workspace_bytes)
         _capi.check(_capi.load().astergemm_run(ctypes.byref(self.config), ctypes.byref(ops),
                                                ctypes.c_void_p(stream) if stream else None))
 
@@ -208,6 +288,43 @@ def gemm_device(dA: int, dB: int, dC: int, M: int, N: int, K: int, dtype_ab: str
     GemmPlan.create(M, N, K, dtype_ab, dtype_c, **kw).run(dA, dB, dC, **run_kw)
 
 
+_STORAGE = {"f16": (np.dtype(np.float16), np.dtype(np.uint16)), "bf16": (np.dtype(np.uint16),),
+            "fp8_e4m3": (np.dtype(np.uint8),), "mxfp4": (np.dtype(np.uint8),)}
+
+
+def _row_bytes(dtype_ab: str, k: int) -> int:
+    return {"f16": 2 * k, "bf16": 2 * k, "fp8_e4m3": k, "mxfp4": k // 2}[dtype_ab]
+
+
+def check_host_operands(cfg: WeakScaledMappedGemmInstance, A, B, *, mx_a=None, mx_b=None,
+                        bias=None) -> None:
+    """Sizes and storage types of host operands against `cfg`, on the host: a kernel reads
+    M*K, N*K, M*K/32, N*K/32 and N elements taken from `cfg`, so an array that is too small, or
+    in another storage type, would make it read past the device allocation."""
+    M, N, K = cfg.spec.gemm_size
+    dt = cfg.spec.dtype_ab
+    for name, arr, rows in (("A", A, M), ("B", B, N)):
+        arr = np.asarray(arr)
+        if arr.dtype not in _STORAGE[dt]:
+            raise ValueError(f"{name} has storage type {arr.dtype}, {dt} operands are passed as "
+                             f"{' or '.join(str(d) for d in _STORAGE[dt])}")
+        want = rows * _row_bytes(dt, K)
+        if arr.nbytes != want:
+            raise ValueError(f"{name} holds {arr.nbytes} bytes, the config ({rows} rows of K={K} "
+                             f"{dt} elements) needs {want}")
+    if cfg.spec.scale_mode == "mx32":
+        for name, arr, rows in (("mx_a", mx_a, M), ("mx_b", mx_b, N)):
+            if arr is None:
+                raise ValueError(f"{name} is required for MXFP4 operands")
+            arr = np.asarray(arr)
+            if arr.dtype != np.uint8 or arr.size != rows * (K // 32):
+                raise ValueError(f"{name} must be {rows * (K // 32)} uint8 e8m0 bytes "
+                                 f"([{rows}, K/32]), got {arr.size} of {arr.dtype}")
+    if cfg.spec.has_bias:
+        if bias is None or np.asarray(bias).size != N:
+            raise ValueError(f"bias must hold N={N} values")
+
+
 def execute_gemm_hsaco(cfg: WeakScaledMappedGemmInstance, hsaco_path: str, num_iterations: int,
                        A: np.ndarray, B: np.ndarray, skip_gpu_check: bool = False, *,
                        scale_a: Optional[float] = None, scale_b: Optional[float] = None,
@@ -219,9 +336,13 @@ def execute_gemm_hsaco(cfg: WeakScaledMappedGemmInstance, hsaco_path: str, num_i
     (np.float16, or np.uint16 bit patterns for bf16, np.uint8 for fp8 / packed
     fp4).  Returns `(C_flat, times_ns)`: C flattened in `cfg.spec.dtype_c`
     storage (float32; uint16 bit patterns for bf16; float16), one time per
-    launch, each launch between its own pair of HIP events.  Unlike the
-    reference's direct-B kernels no host pre-shuffle of B is needed.
+    launch, each launch between its own pair of HIP events.  B is always passed
+    row-major; when the selected kernel reads pre-shuffled B (`direct_b`) the
+    shuffle is done here.  Raises ValueError, before anything touches the GPU,
+    when an array does not have the size or storage type `cfg` implies (the
+    kernels read M*K, N*K ... elements whatever was uploaded).
     """
+    check_host_operands(cfg, A, B, mx_a=mx_a, mx_b=mx_b, bias=bias)
     mcpu = getattr(cfg.mapping, "mcpu", "gfx950")
     if not skip_gpu_check and not system_has_gpu("gfx950"):
         import pytest
@@ -235,6 +356,13 @@ def execute_gemm_hsaco(cfg: WeakScaledMappedGemmInstance, hsaco_path: str, num_i
                            f"{info.name.decode()!r}")
     M, N, K = cfg.spec.gemm_size
     out_np = _OUT_NP[cfg.spec.dtype_c]
+    if c.operand_path == _capi.OPERAND_DIRECT_B:
+        # single point of truth, as in the reference's execute_fn
+        # (test_102_gemm_python_multitile_g2s_directb_cdna4.py:446-467): the caller passes B
+        # row-major and the pre-shuffle happens here, only when the kernel that runs wants it
+        from .kittens_helpers import shuffle_weight
+
+        B = shuffle_weight(np.ascontiguousarray(B).reshape(N, K))
     C_host = np.zeros(M * N, dtype=out_np)
 
     def up(arr, dtype=None):
@@ -271,14 +399,15 @@ def execute_gemm_hsaco(cfg: WeakScaledMappedGemmInstance, hsaco_path: str, num_i
     return C_host, times
 
 
-def mfma_ceiling(d_sample: int, sample_bytes: int, dtype_ab: str, *, target_ms: int = 50,
-                 stream: int = None) -> float:
-    """TFLOP/s the device sustains on `dtype_ab` MFMAs alone, operand registers filled from the
-    sample bytes at `d_sample` (device pointer): the rate no GEMM on such values can exceed
-    under the power limit.  The reference reads utilisation against the published peak only
-    (peak_tflops_f16, contrib/kittens/test/bench/bench_harness.py:31-41)."""
+def mfma_rate(d_sample: int, sample_bytes: int, dtype_ab: str, *, target_ms: int = 50,
+              stream: int = None) -> float:
+    """Diagnostic: TFLOP/s the device reaches on `dtype_ab` MFMAs alone, operand registers filled
+    from the sample bytes at `d_sample` (device pointer), first operand held four instructions in
+    a row as in the GEMM loops.  A measured reference under the power limit, not a proven bound.
+    The reference reads utilisation against the published peak only (peak_tflops_f16,
+    contrib/kittens/test/bench/bench_harness.py:31-41)."""
     out = ctypes.c_double()
-    _capi.check(_capi.load().astergemm_mfma_ceiling(
+    _capi.check(_capi.load().astergemm_diag_mfma_rate(
         _capi.DTYPE_NAMES[dtype_ab], ctypes.c_void_p(d_sample), sample_bytes, target_ms,
         ctypes.byref(out), ctypes.c_void_p(stream) if stream else None))
     return out.value

@@ -34,7 +34,11 @@ PEAK_HBM_GBPS = 8000.0
 # the same counter reads for a 1 GiB device-to-device copy: x2.0 and x1.0); the figures
 # are in profiles/stream_bf16_8192x8192x8192_counters.txt.  A kernel that has not been
 # measured reports null.
-MEASURED_TRAFFIC_BYTES = {"stream_bf16_256x256_w2x4_bf16": 1.746e9}
+MEASURED_TRAFFIC_BYTES = {
+    "stream_bf16_256x256_w2x4_bf16": 1.746e9,   # 8192^3: 1.61e9 read + 1.34e8 written
+    "stream_fp8_256x256_w2x4_bf16": 9.40e8,     # 8192^3: 8.06e8 read + 1.34e8 written
+    "stream_mxfp4_256x256_w2x2_bf16": 3.22e8,   # 4096x14336x4096: 2.05e8 read + 1.17e8 written
+}
 
 
 def _percentile(sorted_vals, pct):
@@ -65,13 +69,22 @@ def make_operands(torch, M, N, K, dtype_ab, dev, seed=42):
         keep = {"scale_a": sa, "scale_b": sb}
         return a, b, keep
     if dtype_ab == "mxfp4":
-        # random e2m1 nibbles and e8m0 bytes around 2^0: same bytes moved and the
-        # same instruction mix as quantised N(0,1) data
-        a = torch.randint(0, 256, (M, K // 2), device=dev, dtype=torch.uint8, generator=g)
-        sa = torch.randint(124, 130, (M, K // 32), device=dev, dtype=torch.uint8, generator=g)
+        # N(0,1) sources quantised on the device (astergemm_quantize_mxfp4): e8m0 from the absmax
+        # of every 32-wide K block, e2m1 elements, as the baseline's configuration 5 states
+        from aster_amd import quantize as Q
+
+        def quantised(rows):
+            x = torch.randn(rows, K, device=dev, generator=g)
+            packed = torch.empty(rows, K // 2, device=dev, dtype=torch.uint8)
+            scales = torch.empty(rows, K // 32, device=dev, dtype=torch.uint8)
+            torch.cuda.synchronize()
+            Q.quantize_mxfp4_device(x.data_ptr(), rows, K, packed.data_ptr(), scales.data_ptr())
+            torch.cuda.synchronize()
+            return packed, scales
+
+        a, sa = quantised(M)
         g.manual_seed(seed + 1)
-        b = torch.randint(0, 256, (N, K // 2), device=dev, dtype=torch.uint8, generator=g)
-        sb = torch.randint(124, 130, (N, K // 32), device=dev, dtype=torch.uint8, generator=g)
+        b, sb = quantised(N)
         keep = {"mx_a": sa, "mx_b": sb}
         return a, b, keep
     raise ValueError(dtype_ab)
@@ -86,10 +99,11 @@ def event_timed_p50(plan, a, b, c, keep, iters, drop, flush_bytes=0):
 
 def cpu_baseline(M, N, K, budget_s=12.0):
     """numpy fp32 `A @ B.T` (the reference's CPU check) on a row sample sized to
-    about `budget_s` seconds; returns the JSON object."""
+    about `budget_s` seconds; returns the JSON object.  A second leg times the oracle's plain-C
+    restatement (OpenMP, fp32 accumulate) on a smaller row sample of the same workload."""
     import numpy as np
 
-    from oracle import formats as F, gemm as G
+    from oracle import cgemm, formats as F, gemm as G
 
     cores = int(os.environ.get("OMP_NUM_THREADS") or os.cpu_count() or 1)
     rng = np.random.default_rng(43)
@@ -110,9 +124,27 @@ def cpu_baseline(M, N, K, budget_s=12.0):
     rows = max(256, rows // 256 * 256)
     t, _ = sample(rows)
     tflops = 2.0 * rows * N * K / t / 1e12
-    return {"value": round(tflops, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
-            "sample": f"numpy fp32 A@B.T + bf16 cast on {rows} of {M} rows of A against the full "
-                      f"B ({N}x{K}), {t:.2f} s, BLAS threads={cores}"}
+    out = {"value": round(tflops, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+           "sample": f"numpy fp32 A@B.T + bf16 cast on {rows} of {M} rows of A against the full "
+                     f"B ({N}x{K}), {t:.2f} s, BLAS threads={cores}"}
+    try:
+        def csample(rows):
+            a = F.f32_to_bf16_bits(rng.standard_normal((rows, K), dtype=np.float32) * 0.02)
+            t0 = time.perf_counter()
+            cgemm.gemm_raw(a, b, G.BF16, rows, N, K)
+            return time.perf_counter() - t0
+
+        t_probe = csample(32)
+        crows = int(min(M, max(32, 32 * 6.0 / max(t_probe, 1e-6)))) // 32 * 32
+        tc = csample(crows)
+        out["c_restatement"] = {"value": round(2.0 * crows * N * K / tc / 1e12, 4), "unit": "TFLOP/s",
+                                "cores": cores, "kind": "port",
+                                "sample": f"oracle/cgemm.c (OpenMP, fp32 accumulate, bf16 decode) on "
+                                          f"{crows} of {M} rows of A against the full B, {tc:.2f} s, "
+                                          f"OMP threads={cores}"}
+    except Exception as exc:  # the second leg never fails the bench line
+        out["c_restatement"] = {"error": repr(exc)[:200]}
+    return out
 
 
 def vendor_library(torch, dev, iters=100, drop=20):
@@ -253,6 +285,9 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=30)
+    ap.add_argument("--preheat-ms", type=float, default=1500.0,
+                    help="upper bound of the untimed pre-heat of the headline kernel before the "
+                         "warm-up launches (0 = none)")
     ap.add_argument("--no-others", action="store_true", help="skip the secondary shapes")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-vendor", action="store_true",
@@ -293,6 +328,26 @@ def main() -> int:
     _capi.check(lib.aster_rt_event_create(ctypes.byref(e0)))
     _capi.check(lib.aster_rt_event_create(ctypes.byref(e1)))
 
+    # what the matrix pipe alone sustains on these operand values under the power limit
+    # (independent MFMAs over registers filled from B, no memory traffic), measured first so that
+    # its 300 ms also bring the clocks to their loaded state
+    ceil_tf = AG.mfma_rate(b.data_ptr(), b.numel() * b.element_size(), "bf16", target_ms=300)
+
+    # Untimed pre-heat of the same kernel: after idling, the first launches run up to a third
+    # slower than the steady state (clock and power management settling), which a short timed
+    # region right after a short warm-up would otherwise sit in.  Launches are event-timed one by
+    # one until ten in a row agree within 1 %, for at most `--preheat-ms`.
+    preheat_launches, t_pre = 0, time.perf_counter()
+    if args.preheat_ms > 0:
+        recent = []
+        while (time.perf_counter() - t_pre) * 1e3 < args.preheat_ms:
+            recent += plan.bench(a.data_ptr(), b.data_ptr(), c.data_ptr(), 10)
+            preheat_launches += 10
+            last = recent[-10:]
+            if preheat_launches >= 30 and max(last) <= 1.01 * min(last):
+                break
+    preheat_ms = (time.perf_counter() - t_pre) * 1e3
+
     for _ in range(args.warmup):
         plan.run(a.data_ptr(), b.data_ptr(), c.data_ptr())
     torch.cuda.synchronize()
@@ -308,6 +363,9 @@ def main() -> int:
     launch_ms = ms.value / args.steps
     value = flops * args.steps / wall / 1e12
     achieved = flops / (launch_ms * 1e-3) / 1e12
+    # the reference's protocol beside it: one event pair per launch, 100 launches, first 20
+    # dropped, p50 (bench_harness.py:93-94, 181-198)
+    p50_ns, p0_ns, _ = event_timed_p50(plan, a, b, c, keep, 100, 20)
 
     traffic = MEASURED_TRAFFIC_BYTES.get(plan.info.name.decode())
 
@@ -317,6 +375,8 @@ def main() -> int:
         "warmup": args.warmup, "ms_per_step": round(wall * 1e3 / args.steps, 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
+        "preheat_ms": round(preheat_ms, 1), "preheat_launches": preheat_launches,
+        "p50_us": round(p50_ns / 1e3, 2), "p50_tflops": round(flops / p50_ns * 1e-3, 1),
         "config": {"workload": "bf16 GEMM M=N=K=8192, A row-major, B stored NxK (column-major KxN), "
                                "N(0,1)*0.02, fp32 accumulate, bf16 output",
                    "kernel": plan.info.name.decode(), "grid": plan.info.grid_x,
@@ -325,12 +385,8 @@ def main() -> int:
                      "unit": "TFLOP/s", "frac": round(achieved / PEAK_TFLOPS["bf16"], 4),
                      "traffic": traffic},
     }
-    # what the matrix pipe alone sustains on these operand values under the power limit
-    # (independent MFMAs over registers filled from B, no memory traffic): no GEMM on this
-    # data can be faster, so the kernel's rate is also given as a fraction of it
-    ceil_tf = AG.mfma_ceiling(b.data_ptr(), b.numel() * b.element_size(), "bf16", target_ms=300)
-    out["roofline"]["mfma_sustained_on_this_data"] = round(ceil_tf, 1)
-    out["roofline"]["frac_of_sustained"] = round(achieved / ceil_tf, 4)
+    out["roofline"]["mfma_rate_measured_on_this_data"] = round(ceil_tf, 1)
+    out["roofline"]["frac_of_measured_mfma_rate"] = round(achieved / ceil_tf, 4)
 
     if not args.no_others:
         others = []
@@ -341,12 +397,17 @@ def main() -> int:
             p = AG.GemmPlan.create(m, n, k, dt, "bf16")
             p50, best, _ = event_timed_p50(p, a, b, c, keep, 100, 20)
             tf = p.info.flops / p50 * 1e-3
-            ceil_tf = AG.mfma_ceiling(b.data_ptr(), b.numel() * b.element_size(), dt, target_ms=200)
-            others.append({"workload": f"{dt} GEMM {m}x{n}x{k} -> bf16", "kernel": p.info.name.decode(),
+            ceil_tf = AG.mfma_rate(b.data_ptr(), b.numel() * b.element_size(), dt, target_ms=200)
+            src = ("e4m3 of N(0,1) sources with s = absmax/448" if dt == "fp8_e4m3" else
+                   "MXFP4 of N(0,1) sources quantised on the device (e8m0 from per-block absmax)")
+            others.append({"workload": f"{dt} GEMM {m}x{n}x{k} -> bf16", "operands": src,
+                           "kernel": p.info.name.decode(),
                            "p50_us": round(p50 / 1e3, 2), "tflops": round(tf, 1), "bound": "mfma",
                            "frac": round(tf / PEAK_TFLOPS[dt], 4),
-                           "mfma_sustained_on_this_data": round(ceil_tf, 1),
-                           "frac_of_sustained": round(tf / ceil_tf, 4)})
+                           "algorithmic_bytes": int(p.info.bytes),
+                           "traffic": MEASURED_TRAFFIC_BYTES.get(p.info.name.decode()),
+                           "mfma_rate_measured_on_this_data": round(ceil_tf, 1),
+                           "frac_of_measured_mfma_rate": round(tf / ceil_tf, 4)})
         # the two gfx950 shapes the reference publishes its own kernels' numbers for (f16
         # operands, fp32 output; contrib/kittens/test/bench/best_known.json, quoted, not re-run)
         for (m, n, k, quoted) in ((4096, 4096, 4096, 1007.0), (2048, 4096, 4096, 846.3)):

@@ -19,12 +19,15 @@
  * Conventions: every function returns 0 on success and a negative
  * ASTERGEMM_E* code on failure; nothing throws; the message of the last
  * failure on the calling thread is returned by astergemm_last_error().
- * All buffers are owned by the caller, with one exception: decode shapes
- * (M <= 64) whose rows are not 4 or 8 KiB long, and shapes with at most 128
- * output tiles of 128 x 128 and long rows, are computed in K ranges, and
- * the fp32 partial sums live in a workspace the library allocates on first
- * use, one per (device, stream), M * N * 4 bytes per K range (at most 16),
- * kept until the process ends.  Calls on different streams may run
+ * All buffers are owned by the caller.  Decode shapes (M <= 64) whose rows are
+ * not 4 or 8 KiB long, and shapes with at most 128 output tiles of 128 x 128
+ * and long rows, are computed in K ranges whose fp32 partial sums need a
+ * workspace: astergemm_workspace_bytes() says how much, and
+ * astergemm_operands.dWorkspace brings it.  Without one the library falls back
+ * to a buffer of its own, one per (device, stream), allocated on the first such
+ * call (that call therefore cannot be captured into a graph), replaced by a
+ * larger one when needed and kept until the process ends.  Calls on different
+ * streams may run
  * concurrently; calls on one stream are ordered by it.  Pointers named d*
  * are device pointers.  Launches go to the stream that is passed (NULL = the null
  * stream, which is what the reference uses everywhere).
@@ -39,7 +42,7 @@
 extern "C" {
 #endif
 
-#define ASTERGEMM_ABI_VERSION 1
+#define ASTERGEMM_ABI_VERSION 2
 
 /* ---- error codes ------------------------------------------------------ */
 #define ASTERGEMM_OK 0
@@ -138,6 +141,10 @@ typedef struct astergemm_operands {
   const uint8_t* dMxA;     /* SCALE_MX32: [M, K/32] e8m0 bytes, row-major     */
   const uint8_t* dMxB;     /*             [N, K/32]                           */
   const float* dBias;      /* [N] fp32                                        */
+  void* dWorkspace;        /* fp32 partial sums of K ranges, 16-byte aligned,
+                              at least astergemm_workspace_bytes(); NULL = the
+                              library's own buffer                            */
+  size_t workspace_bytes;  /* size of dWorkspace                              */
 } astergemm_operands;
 
 /* reference: hip_get_device_props dict (RuntimeModule.cpp:166-191) */
@@ -172,6 +179,13 @@ int astergemm_variant_info(int index, const astergemm_config* cfg,
 /* One asynchronous launch on `stream` (hipStream_t, NULL = null stream).    */
 int astergemm_run(const astergemm_config* cfg, const astergemm_operands* ops,
                   void* stream);
+/* Bytes of fp32 workspace astergemm_run needs for cfg with the variant it
+ * selects (0 for most shapes: only rows cut into K ranges need one).  The
+ * reference's kernels have no workspace (every kernel takes exactly A, B, C:
+ * test_102_gemm_python_multitile_g2s_directb_cdna4.py:150-156); this is the
+ * caller-owned form of what split K adds here.                              */
+int astergemm_workspace_bytes(const astergemm_config* cfg, size_t* bytes);
+
 /* Replaces execute_fn's timed loop (execution/core.py:690-703): `iters`
  * launches, each bracketed by its own HIP event pair on `stream`;
  * times_ns[i] = int(ms * 1e6).  If flush_bytes > 0 a streaming kernel over a
@@ -202,19 +216,6 @@ int astergemm_bench_rotate(const astergemm_config* cfg, const astergemm_operands
  * tools/perf_best_known_update.py) on the prebuilt variants. */
 int astergemm_tune(const astergemm_config* cfg, const astergemm_operands* ops, int iters,
                    int* best_variant, int64_t* best_ns, void* stream);
-
-/* The MFMA rate (TFLOP/s) the device sustains on given operand values with
- * nothing else going on: independent MFMAs of dtype_ab's instruction over
- * registers filled once from dSample (operand bytes as a GEMM would read
- * them: at least 4096, a multiple of 16), for about target_ms milliseconds.
- * Under the board's power limit the rate depends on the values (zeros run near
- * the published peak, random data well below), so this is the ceiling to
- * read a measured GEMM against next to the published one.  Synchronises the
- * stream.  The reference takes its peak from a table
- * (_PEAK_TFLOPS_F16_BY_MCPU, contrib/kittens/test/bench/bench_harness.py:31-41);
- * it has no measured counterpart. */
-int astergemm_mfma_ceiling(int dtype_ab, const void* dSample, int64_t sample_bytes,
-                           int target_ms, double* tflops, void* stream);
 
 /* Host pre-shuffle of B[N,K] 2-byte elements into per-lane MFMA order
  * (reference: shuffle_weight, contrib/kittens/test/kittens_helpers.py:90-119). */
@@ -303,7 +304,27 @@ int astergemm_weight_verify(const void* file, size_t file_bytes);
 int astergemm_weight_config(const astergemm_weight_header* h, int64_t M, int dtype_c,
                             astergemm_config* cfg);
 
-/* ---- runtime seam: 1:1 with RuntimeModule.cpp:140-418 -------------------- */
+/* ---- diagnostics (not part of the GEMM path; no reference interface) -------
+ * The MFMA rate (TFLOP/s) the device reaches on given operand values with
+ * nothing else going on: independent MFMAs of dtype_ab's instruction over
+ * registers filled once from dSample (operand bytes as a GEMM would read
+ * them: at least 4096, a multiple of 16), for about target_ms milliseconds,
+ * the first operand held for four instructions in a row as in the GEMM loops.
+ * Under the board's power limit the rate depends on the values (zeros run near
+ * the published peak, random data well below), so this is a measured
+ * reference to read a GEMM's rate against next to the published peak -- not a
+ * proven upper bound.  Synchronises the stream and allocates a small buffer.
+ * The reference takes its peak from a table (_PEAK_TFLOPS_F16_BY_MCPU,
+ * contrib/kittens/test/bench/bench_harness.py:31-41) and measures nothing.   */
+int astergemm_diag_mfma_rate(int dtype_ab, const void* dSample, int64_t sample_bytes,
+                             int target_ms, double* tflops, void* stream);
+
+/* ---- runtime seam: one function per hip_* function of the reference's
+ * nanobind module (RuntimeModule.cpp:140-418).  aster_rt_function_free is a
+ * no-op here (the reference frees the heap cell of its handle, :221-226) and
+ * aster_rt_module_launch_kernel_ex (:256-300) runs clusters of (1,1,1) as a
+ * plain launch and refuses larger ones with ASTERGEMM_ENOTSUP: gfx950 has no
+ * cluster launch (the reference uses it for gfx1250 only).                   */
 int aster_rt_init(void);
 int aster_rt_peek_at_last_error(void);
 int aster_rt_clear_last_error(void);
@@ -327,6 +348,12 @@ int aster_rt_module_launch_kernel(void* fn, unsigned gx, unsigned gy,
                                   unsigned gz, unsigned bx, unsigned by,
                                   unsigned bz, unsigned shared_bytes,
                                   void* stream, void** kernel_params);
+int aster_rt_function_free(void* fn);
+int aster_rt_module_launch_kernel_ex(void* fn, unsigned gx, unsigned gy, unsigned gz,
+                                     unsigned bx, unsigned by, unsigned bz,
+                                     unsigned cluster_x, unsigned cluster_y,
+                                     unsigned cluster_z, unsigned shared_bytes,
+                                     void* stream, void** kernel_params);
 int aster_rt_event_create(void** event);
 int aster_rt_event_destroy(void* event);
 int aster_rt_event_record(void* event, void* stream);

@@ -747,6 +747,63 @@ def test_config2_full_size_row_sample_determinism_and_scaling(gpu, big):
     assert np.array_equal(F.bf16_bits_to_f32(out4), F.bf16_bits_to_f32(out) * 4.0)
 
 
+def _sampled_rows_and_cols(M, N):
+    rows = np.random.default_rng(0).choice(M, 48, replace=False)
+    rows = np.concatenate([rows, [0, 255, 256, M - 1]])
+    cols = np.random.default_rng(1).choice(N, 32, replace=False)
+    return rows, cols
+
+
+def test_config3_full_size_fp8_row_sample_determinism_and_scaling(gpu):
+    # configuration 3 at the size the bench times: 8192^3, operands e4m3 of N(0,1) sources with
+    # s = absmax / 448 (seeds 42 / 43), bf16 output with the scales applied in the epilogue
+    M = N = K = 8192
+    a, b, ex = operands(M, N, K, "fp8_e4m3", a_std=1.0, b_std=1.0)
+    out, name = run_gemm(a, b, M, N, K, "fp8_e4m3", "bf16", **ex)
+    assert name == "stream_fp8_256x256_w2x4_bf16"
+    rows, cols = _sampled_rows_and_cols(M, N)
+    check(out[rows], G.gemm_fp8(a[rows], b, ex["scale_a"], ex["scale_b"], out_dtype=G.BF16), "bf16", N)
+    check(out[:, cols], G.gemm_fp8(a, b[cols], ex["scale_a"], ex["scale_b"], out_dtype=G.BF16),
+          "bf16", len(cols))
+    # against the float64-accumulated product on the sampled rows: at most 2 bf16 ulp
+    w64 = G.gemm_fp8(a[rows], b, ex["scale_a"], ex["scale_b"], out_dtype=G.BF16, accumulate="f64")
+    w64f = F.bf16_bits_to_f32(w64)
+    solid = np.abs(w64f) > 1e-2 * np.sqrt(np.mean(w64f.astype(np.float64) ** 2))
+    ulp = np.abs(out[rows].astype(np.int32) - w64.astype(np.int32))
+    assert ulp[solid].max() <= 2 and np.mean(ulp[solid] > 1) < 1e-3
+    # run-to-run determinism
+    out2, _ = run_gemm(a, b, M, N, K, "fp8_e4m3", "bf16", **ex)
+    assert np.array_equal(out, out2)
+    # a tensor scale four times as large is exact in the fp32 epilogue and in bf16
+    out4, _ = run_gemm(a, b, M, N, K, "fp8_e4m3", "bf16", scale_a=np.float32(ex["scale_a"]) * 4,
+                       scale_b=ex["scale_b"])
+    assert np.array_equal(F.bf16_bits_to_f32(out4), F.bf16_bits_to_f32(out) * 4.0)
+
+
+def test_config5_full_size_mxfp4_row_sample_determinism_and_scaling(gpu):
+    # configuration 5 at the size the bench times: 4096 x 14336 x 4096, both operands MXFP4 from
+    # N(0,1) sources (seeds 42 / 43), e8m0 from the absmax of every 32-wide K block
+    M, N, K = 4096, 14336, 4096
+    a, b, ex = operands(M, N, K, "mxfp4", a_std=1.0, b_std=1.0)
+    out, name = run_gemm(a, b, M, N, K, "mxfp4", "bf16", **ex)
+    assert name.startswith("stream_mxfp4_")
+    rows, cols = _sampled_rows_and_cols(M, N)
+    check(out[rows], G.gemm_mxfp4(a[rows], ex["mx_a"][rows], b, ex["mx_b"], out_dtype=G.BF16),
+          "bf16", N)
+    check(out[:, cols], G.gemm_mxfp4(a, ex["mx_a"], b[cols], ex["mx_b"][cols], out_dtype=G.BF16),
+          "bf16", len(cols))
+    out32, _ = run_gemm(a[:512], b, 512, N, K, "mxfp4", "f32", mx_a=ex["mx_a"][:512], mx_b=ex["mx_b"])
+    check(out32, G.gemm_mxfp4(a[:512], ex["mx_a"][:512], b, ex["mx_b"], out_dtype=G.F32), "f32", N,
+          bar=1e-5)
+    # run-to-run determinism
+    out2, _ = run_gemm(a, b, M, N, K, "mxfp4", "bf16", **ex)
+    assert np.array_equal(out, out2)
+    # every e8m0 byte of A one higher doubles every product exactly
+    assert ex["mx_a"].max() < 254
+    outx2, _ = run_gemm(a, b, M, N, K, "mxfp4", "bf16", mx_a=ex["mx_a"] + np.uint8(1), mx_b=ex["mx_b"])
+    assert np.array_equal(F.bf16_bits_to_f32(outx2), F.bf16_bits_to_f32(out) * 2.0)
+
+
 def test_identity_operand_is_exact_at_full_width(gpu):
     # B = I: every output is one product plus zeros, so C == A bit for bit.
     M, N = 512, 8192

@@ -138,7 +138,7 @@ def test_failed_runtime_call_does_not_poison_later_launches(gpu):
     assert s == 1.0 and q[0] == 0xFE and q[-1] == 0x7E
 
 
-def test_mfma_ceiling_depends_on_operand_values(gpu):
+def test_diag_mfma_rate_depends_on_operand_values(gpu):
     """Independent MFMAs over registers: zeros run near the published peak, random bf16 data
     well below it (the board's power limit), and both are plausible rates for this chip."""
     from aster_amd import _capi, gemm as AG
@@ -147,15 +147,15 @@ def test_mfma_ceiling_depends_on_operand_values(gpu):
     bits = (x.view(np.uint32) >> 16).astype(np.uint16)
     buf = GpuBuffer(bits.nbytes)
     buf.copy_from_host(bits)
-    random_tf = AG.mfma_ceiling(buf.ptr_value, bits.nbytes, "bf16", target_ms=100)
+    random_tf = AG.mfma_rate(buf.ptr_value, bits.nbytes, "bf16", target_ms=100)
     buf.copy_from_host(np.zeros_like(bits))
-    zeros_tf = AG.mfma_ceiling(buf.ptr_value, bits.nbytes, "bf16", target_ms=100)
-    fp8_tf = AG.mfma_ceiling(buf.ptr_value, bits.nbytes, "fp8_e4m3", target_ms=50)
-    fp4_tf = AG.mfma_ceiling(buf.ptr_value, bits.nbytes, "mxfp4", target_ms=50)
+    zeros_tf = AG.mfma_rate(buf.ptr_value, bits.nbytes, "bf16", target_ms=100)
+    fp8_tf = AG.mfma_rate(buf.ptr_value, bits.nbytes, "fp8_e4m3", target_ms=50)
+    fp4_tf = AG.mfma_rate(buf.ptr_value, bits.nbytes, "mxfp4", target_ms=50)
     buf.free()
     assert 500.0 < random_tf < zeros_tf <= 2600.0
     assert zeros_tf < fp8_tf <= 5200.0 and fp8_tf < fp4_tf <= 10500.0
     with pytest.raises(_capi.AsterGemmError):
-        AG.mfma_ceiling(0, 4096, "bf16")
+        AG.mfma_rate(0, 4096, "bf16")
     with pytest.raises(_capi.AsterGemmError):
-        AG.mfma_ceiling(1 << 20, 100, "bf16")
+        AG.mfma_rate(1 << 20, 100, "bf16")

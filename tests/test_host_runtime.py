@@ -25,13 +25,13 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in astergemm.h but not exported"
     assert declared == set(_capi.SIGNATURES), declared ^ set(_capi.SIGNATURES)
-    assert lib.astergemm_abi_version() == 1
+    assert lib.astergemm_abi_version() == _capi.ABI_VERSION
 
 
 def test_struct_sizes_match_header_layout():
     # 6 x int64 + 16 x int32 ; pointers ; see include/astergemm.h
     assert ctypes.sizeof(_capi.Config) == 6 * 8 + 16 * 4
-    assert ctypes.sizeof(_capi.Operands) == 8 * 8
+    assert ctypes.sizeof(_capi.Operands) == 10 * 8
     assert ctypes.sizeof(_capi.KernelInfo) == 13 * 4 + 4 + 2 * 8 + 64
 
 
@@ -142,6 +142,108 @@ def test_compile_gemm_writes_descriptor(tmp_path):
     (tmp_path / "bad.hsaco").write_text("{}")
     with pytest.raises(ValueError):
         gemm._read_descriptor(str(tmp_path / "bad.hsaco"))
+
+
+def test_descriptor_says_when_the_mapping_is_not_honoured(tmp_path):
+    import dataclasses
+
+    from aster_amd.gemm_config import OperandPath, WeakScaledMappedGemmInstance
+
+    # the library's own 256 x 256, 2 x 4 waves geometry: honoured
+    cfg = make_instance(512, 512, 256)
+    path, asm = gemm.compile_gemm(cfg, str(tmp_path / "a.hsaco"))
+    desc = json.load(open(path))
+    assert desc["mapping_honoured"] is True and desc["mapping_not_honoured"] == {}
+    assert "mapping_honoured: true" in asm
+    assert desc["mapping_fixed_by_kernel"]["pipeline_strategy"] == 1
+    # the reference's best label geometry (128 x 256 tile, 1 x 4 waves) has no pre-built kernel:
+    # the library's choice runs and the descriptor says which requested values it does not have
+    cfg = make_instance(512, 512, 256, wg_tile=(128, 256), waves=(1, 4), pipeline_strategy=11)
+    path, asm = gemm.compile_gemm(cfg, str(tmp_path / "b.hsaco"))
+    desc = json.load(open(path))
+    assert desc["mapping_honoured"] is False
+    assert desc["mapping_not_honoured"]["wg_tile"]["requested"] == [128, 256]
+    assert desc["mapping_not_honoured"]["waves"] == {"requested": [1, 4], "kernel": desc["waves"]}
+    assert "mapping_honoured: false" in asm and "wg_tile: requested [128, 256]" in asm
+    # a direct_b request on a shape no pre-shuffled kernel takes falls back to row-major B
+    m = dataclasses.replace(make_instance(512, 520 // 8 * 8 + 248, 264).mapping,
+                            operand_path=OperandPath.DIRECT_B)
+    cfg = WeakScaledMappedGemmInstance(make_instance(512, 768, 264).spec, m)
+    c, info = gemm.select_for_instance(cfg)
+    rep = gemm.mapping_report(cfg, c, info)
+    if c.operand_path == _capi.OPERAND_LDS:
+        assert rep.not_honoured["operand_path"] == {"requested": "direct_b", "kernel": "lds"}
+    else:
+        assert "operand_path" not in rep.not_honoured
+
+
+def test_execute_checks_host_operand_sizes_before_touching_the_gpu(tmp_path):
+    cfg = make_instance(256, 256, 256)
+    path, _ = gemm.compile_gemm(cfg, str(tmp_path / "k.hsaco"))
+    A = np.zeros((256, 256), np.uint16)
+    B = np.zeros((256, 256), np.uint16)
+    # (no GPU here: any of these would fail in hip_init if the check came later)
+    with pytest.raises(ValueError, match="A holds"):
+        gemm.execute_gemm_hsaco(cfg, path, 1, A[:128], B, skip_gpu_check=True)
+    with pytest.raises(ValueError, match="B holds"):
+        gemm.execute_gemm_hsaco(cfg, path, 1, A, np.zeros((256, 128), np.uint16), skip_gpu_check=True)
+    with pytest.raises(ValueError, match="storage type"):
+        gemm.execute_gemm_hsaco(cfg, path, 1, A.view(np.uint8), B, skip_gpu_check=True)
+    with pytest.raises(ValueError, match="storage type"):
+        gemm.execute_gemm_hsaco(cfg, path, 1, A.astype(np.float32), B, skip_gpu_check=True)
+    q = make_instance(256, 256, 256, dtype_ab="mxfp4")
+    a4 = np.zeros((256, 128), np.uint8)
+    mx = np.full((256, 8), 127, np.uint8)
+    with pytest.raises(ValueError, match="mx_a is required"):
+        gemm.check_host_operands(q, a4, a4)
+    with pytest.raises(ValueError, match="mx_b must be"):
+        gemm.check_host_operands(q, a4, a4, mx_a=mx, mx_b=mx[:, :4])
+    gemm.check_host_operands(q, a4, a4, mx_a=mx, mx_b=mx)
+    b = make_instance(256, 256, 256, has_bias=True)
+    with pytest.raises(ValueError, match="bias"):
+        gemm.check_host_operands(b, A, B, bias=np.zeros(255, np.float32))
+
+
+def test_workspace_query_and_caller_workspace_checks():
+    # shapes that are not cut into K ranges need no workspace
+    assert gemm.GemmPlan.create(8192, 8192, 8192).workspace_bytes() == 0
+    assert gemm.GemmPlan.create(16, 14336, 4096).workspace_bytes() == 0
+    # split K on the 128 x 128 kernel: 8 ranges of 128 x 4096 fp32 partial sums
+    p = gemm.GemmPlan.create(128, 4096, 14336)
+    assert p.info.name.decode().startswith("splitk_") and p.workspace_bytes() == 8 * 128 * 4096 * 4
+    # decode rows of 28 KiB: 7 ranges of 4 KiB
+    d = gemm.GemmPlan.create(16, 4096, 14336)
+    assert d.workspace_bytes() == 7 * 16 * 4096 * 4
+    # a workspace that is too small, or misaligned, is refused before anything is launched
+    with pytest.raises(_capi.AsterGemmError, match="workspace of"):
+        d.run(4096, 4096, 4096, workspace=4096, workspace_bytes=d.workspace_bytes() - 1)
+    with pytest.raises(_capi.AsterGemmError, match="dWorkspace must be 16-byte aligned"):
+        d.run(4096, 4096, 4096, workspace=4096 + 4, workspace_bytes=d.workspace_bytes())
+
+
+def test_reported_grid_is_the_launched_grid_of_the_k_range_kernels():
+    # S K ranges x R row ranges, one workgroup per CU: the description comes from the same
+    # function the launcher uses (the number of CUs is 0 without a device: one row range)
+    def krange_grid(M, N, S, cus):
+        mh = 2 if M > 32 else 1
+        slots = (cus // 16) * 8 if mh == 2 else cus
+        rows = min(max(slots // S, 1), (N + 15) // 16)
+        g = mh * S * rows
+        return (g + 15) // 16 * 16 if mh == 2 else g
+
+    for (M, N, K, S) in ((16, 4096, 14336, 7), (16, 4096, 28672, 7), (64, 4096, 14336, 7),
+                         (16, 8192, 28672, 7)):
+        p = gemm.GemmPlan.create(M, N, K, family=_capi.KERNEL_SKINNY)
+        assert p.workspace_bytes() == S * M * N * 4
+        assert p.info.grid_x == krange_grid(M, N, S, cus=0)
+
+
+def test_runtime_seam_function_free_and_cluster_launch():
+    lib = _capi.load()
+    assert lib.aster_rt_function_free(None) == 0
+    # a cluster larger than (1,1,1) is refused on gfx950 before the function handle is used
+    rc = lib.aster_rt_module_launch_kernel_ex(None, 1, 1, 1, 64, 1, 1, 2, 1, 1, 0, None, None)
+    assert rc == -95 and "cluster launch" in _capi.last_error()
 
 
 # ---- array roles and kernel-argument packing (reference:

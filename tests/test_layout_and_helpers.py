@@ -143,3 +143,71 @@ def test_coop_2d_split_bruteforce():
                 assert covered >= set(itertools.product(range(num_tiles), range(kt)))
     assert coop_2d_split(8, 4, 1) == (4, 1, 2, 1)
     assert coop_2d_split(2, 8, 2) == (4, 2, 1, 1)
+
+
+def test_make_coop_load_plan_covers_the_workgroup_tile_with_clamped_starts():
+    from aster_amd.coop import make_coop_load_plan
+    from aster_amd.layout import Layout
+
+    # the reference's shape of use: tiles of 1 KiB in LDS, 16 rows of a row-major operand in
+    # global memory, kt K tiles of 64 bytes each
+    for num_tiles in (1, 3, 8, 12, 16):
+        for kt in (1, 2, 4):
+            for num_waves in (1, 2, 4, 8):
+                g = Layout((num_tiles, kt), (16 * 8192, 64))
+                l = Layout((num_tiles, kt), (kt * 1024, 1024))
+                ws, wk, cs, ck = coop_2d_split(num_tiles, num_waves, kt)
+                seen = set()
+                for w in range(num_waves):
+                    plan = make_coop_load_plan(w, num_waves=num_waves, wg_tile_global=g, wg_tile_lds=l)
+                    assert plan.global_layout.sizes == (cs, ck) == plan.lds_layout.sizes
+                    assert plan.unroll_axes == ("s", "k")
+                    # clamped start in tile units, then the layout's strides (coop.py:77-83)
+                    s0 = coop_wave_start(w // wk, cs, num_tiles)
+                    k0 = coop_wave_start(w % wk, ck, kt)
+                    assert plan.global_wave_off == s0 * 16 * 8192 + k0 * 64
+                    assert plan.lds_wave_off == s0 * kt * 1024 + k0 * 1024
+                    for go, lo in plan.transfers():
+                        # global and LDS offsets name the same tile
+                        s, k = divmod(lo, kt * 1024)[0], (lo % (kt * 1024)) // 1024
+                        assert go == s * 16 * 8192 + k * 64 and s < num_tiles and k < kt
+                        seen.add((s, k))
+                assert seen == set(itertools.product(range(num_tiles), range(kt)))
+    # hand-evaluated: 8 tiles, 4 waves, 1 K tile -> two adjacent tiles per wave; wave 3 starts at 6
+    plan = make_coop_load_plan(3, num_waves=4, wg_tile_global=Layout((8, 1), (100, 7)),
+                               wg_tile_lds=Layout((8, 1), (1024, 1024)))
+    assert plan.transfers() == [(600, 6144), (700, 7168)]
+    # 3 tiles on 4 waves: the split is (1 x 4) over K?  kt = 1, so ws = 4 wastes one wave, which
+    # redoes the last tile instead of running past the end
+    plans = [make_coop_load_plan(w, num_waves=4, wg_tile_global=Layout((3, 1), (10, 1)),
+                                 wg_tile_lds=Layout((3, 1), (1, 1))) for w in range(4)]
+    assert [p.global_wave_off for p in plans] == [0, 10, 20, 20]
+    with pytest.raises(AssertionError):
+        make_coop_load_plan(0, num_waves=2, wg_tile_global=Layout((4, 1), (1, 1)),
+                            wg_tile_lds=Layout((4, 2), (2, 1)))
+    with pytest.raises(ValueError):
+        make_coop_load_plan(4, num_waves=4, wg_tile_global=Layout((4, 1), (1, 1)),
+                            wg_tile_lds=Layout((4, 1), (1, 1)))
+
+
+@pytest.mark.parametrize("tile_rows,num_waves", [(256, 8), (256, 4), (128, 4)])
+def test_stream_kernel_staging_is_the_interleaved_coop_plan(tile_rows, num_waves):
+    """What the stream kernels do (gemm_stream_kernel.hpp: LH = BM / 8 / NW transfers per wave
+    and ring slot, transfer j of wave w from operand rows (j * NW + w) * 8 to LDS offset
+    (j * NW + w) * 8 * 128 of the slot) is the plan `coop_2d_split` gives for BM / 8 tiles of
+    8 rows, one K tile, interleaved over the waves."""
+    from aster_amd.coop import stream_kernel_load_plan
+
+    ld = 16384
+    lh = tile_rows // 8 // num_waves
+    assert coop_2d_split(tile_rows // 8, num_waves, 1) == (num_waves, 1, lh, 1)
+    everything = []
+    for w in range(num_waves):
+        plan = stream_kernel_load_plan(w, tile_rows=tile_rows, num_waves=num_waves, ld_bytes=ld)
+        assert plan.global_layout.sizes == (lh, 1)
+        kernel = [((j * num_waves + w) * 8 * ld, (j * num_waves + w) * 8 * 128) for j in range(lh)]
+        assert plan.transfers() == kernel
+        everything += kernel
+    # the slot is filled exactly once: every 1 KiB of it, every 8-row group of the tile
+    assert sorted(lo for _, lo in everything) == [t * 1024 for t in range(tile_rows // 8)]
+    assert sorted(go for go, _ in everything) == [t * 8 * ld for t in range(tile_rows // 8)]
