@@ -23,6 +23,7 @@ SCALE_NONE, SCALE_TENSOR, SCALE_MX32 = 0, 1, 2
 KERNEL_AUTO, KERNEL_TILE, KERNEL_SKINNY = 0, 1, 2
 OPERAND_LDS, OPERAND_DIRECT_B = 0, 1
 ABI_VERSION = 2
+NOALLOC_SCRATCH_BYTES = 16 << 20
 
 DTYPE_NAMES = {"f16": F16, "bf16": BF16, "fp8_e4m3": FP8_E4M3, "mxfp4": MXFP4, "f32": F32}
 
@@ -109,6 +110,7 @@ SIGNATURES = {
     "astergemm_variant_count": (C.c_int, []),
     "astergemm_variant_info": (C.c_int, [C.c_int, C.POINTER(Config), C.POINTER(KernelInfo)]),
     "astergemm_run": (C.c_int, [C.POINTER(Config), C.POINTER(Operands), _P]),
+    "astergemm_run_noalloc": (C.c_int, [C.POINTER(Config), C.POINTER(Operands), _P]),
     "astergemm_workspace_bytes": (C.c_int, [C.POINTER(Config), C.POINTER(C.c_size_t)]),
     "astergemm_bench_rotate": (C.c_int, [C.POINTER(Config), C.POINTER(Operands), C.c_int, C.c_int,
                                          C.POINTER(C.c_int64), C.c_void_p]),

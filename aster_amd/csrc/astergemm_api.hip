@@ -357,6 +357,33 @@ int build_args(const Variant& v, const astergemm_config& c, const astergemm_oper
   return 0;
 }
 
+// ---- the entry point that allocates nothing ------------------------------------------------
+// Partial sums of rows cut into K ranges go to this array instead of an allocation.  Its name is
+// a host-side handle only: the device address is looked up once per device.
+static __device__ __attribute__((used)) __align__(256) unsigned char scratch[ASTERGEMM_NOALLOC_SCRATCH_BYTES];
+std::atomic<void*> g_scratch_ptr[64];
+
+// Device address of `scratch` on the current device (looked up on first use), or nullptr with
+// the error set.
+void* scratch_address() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    hip_fail(hipGetLastError(), "hipGetDevice", __FILE__, __LINE__);
+    return nullptr;
+  }
+  std::atomic<void*>& slot = g_scratch_ptr[dev & 63];
+  void* p = slot.load(std::memory_order_acquire);
+  if (!p) {
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) {
+      hip_fail(e, "hipGetSymbolAddress(scratch)", __FILE__, __LINE__);
+      return nullptr;
+    }
+    slot.store(p, std::memory_order_release);
+  }
+  return p;
+}
+
 // Start / stop events of a timed region; destroyed on every return path.
 struct EventPair {
   hipEvent_t e0 = nullptr, e1 = nullptr;
@@ -450,6 +477,40 @@ int astergemm_workspace_bytes(const astergemm_config* cfg, size_t* bytes) {
   const Variant* v = choose(*cfg, &index);
   if (!v) return g_choose_rc;
   *bytes = (cfg->M == 0 || cfg->N == 0) ? 0 : workspace_need(*v, *cfg);
+  return 0;
+}
+
+int astergemm_run_noalloc(const astergemm_config* cfg, const astergemm_operands* ops,
+                          void* stream) {
+  if (!cfg || !ops) {
+    set_error("astergemm_run_noalloc: null argument");
+    return ASTERGEMM_EINVAL;
+  }
+  int index = -1;
+  const Variant* v = choose(*cfg, &index);
+  if (!v) return g_choose_rc;
+  if (cfg->M == 0 || cfg->N == 0) return 0;
+  const size_t need = workspace_need(*v, *cfg);
+  if (need > (size_t)ASTERGEMM_NOALLOC_SCRATCH_BYTES) {
+    set_error("astergemm_run_noalloc: %s needs %zu bytes of partial sums for this config, the "
+              "built-in scratch holds %zu; use astergemm_run with a workspace",
+              v->name, need, (size_t)ASTERGEMM_NOALLOC_SCRATCH_BYTES);
+    return ASTERGEMM_EINVAL;
+  }
+  astergemm_operands o = *ops;
+  o.dWorkspace = nullptr;
+  o.workspace_bytes = 0;
+  if (need) {
+    void* p = scratch_address();
+    if (!p) return ASTERGEMM_EHIP;
+    o.dWorkspace = p;
+    o.workspace_bytes = (size_t)ASTERGEMM_NOALLOC_SCRATCH_BYTES;
+  }
+  GemmArgs a;
+  if (int rc = build_args(*v, *cfg, o, &a)) return rc;
+  (void)hipGetLastError();
+  const int e = v->launch(a, grid_of(*v, *cfg), (hipStream_t)stream);
+  if (e != 0) return hip_fail((hipError_t)e, v->name, __FILE__, __LINE__);
   return 0;
 }
 
@@ -623,6 +684,8 @@ int aster_rt_init(void) {
     set_error("aster_rt_init: no HIP device");
     return ASTERGEMM_ENODEV;
   }
+  // the built-in scratch of astergemm_run_noalloc, for the device that is current now
+  if (!scratch_address()) return ASTERGEMM_EHIP;
   return 0;
 }
 int aster_rt_peek_at_last_error(void) { return (int)hipPeekAtLastError(); }

@@ -236,6 +236,16 @@ class GemmPlan:
         _capi.check(_capi.load().astergemm_run(ctypes.byref(self.config), ctypes.byref(ops),
                                                ctypes.c_void_p(stream) if stream else None))
 
+    def run_noalloc(self, dA: int, dB: int, dC: int, *, scale_a: int = None, scale_b: int = None,
+                    mx_a: int = None, mx_b: int = None, bias: int = None,
+                    stream: int = None) -> None:
+        """`run` through the entry point that never allocates device memory: K-range partial
+        sums go to the library's built-in scratch (`_capi.NOALLOC_SCRATCH_BYTES` per device)."""
+        ops = self._operands(dA, dB, dC, scale_a, scale_b, mx_a, mx_b, bias)
+        _capi.check(_capi.load().astergemm_run_noalloc(
+            ctypes.byref(self.config), ctypes.byref(ops),
+            ctypes.c_void_p(stream) if stream else None))
+
     def bench(self, dA: int, dB: int, dC: int, iters: int, *, scale_a: int = None,
               scale_b: int = None, mx_a: int = None, mx_b: int = None, bias: int = None,
               flush_bytes: int = 0, stream: int = None) -> List[int]:

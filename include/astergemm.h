@@ -186,6 +186,21 @@ int astergemm_run(const astergemm_config* cfg, const astergemm_operands* ops,
  * caller-owned form of what split K adds here.                              */
 int astergemm_workspace_bytes(const astergemm_config* cfg, size_t* bytes);
 
+/* astergemm_run for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc): it
+ * never calls hipMalloc / hipFree or an allocating routine.  No counterpart in
+ * the reference.  ops->dWorkspace is ignored: the partial sums of K ranges go
+ * to a scratch array built into the library, ASTERGEMM_NOALLOC_SCRATCH_BYTES
+ * per device, held until the process ends; a config that needs more is refused
+ * with ASTERGEMM_EINVAL.  Every call on a device shares that array, whatever
+ * its stream: calls that overlap on one device race (calls on one stream are
+ * ordered and safe).  Nothing in the array has to start at zero: every launch
+ * writes all the planes it later adds.  The array's address is looked up on
+ * the first call on a device, or by aster_rt_init for the current device.     */
+#define ASTERGEMM_NOALLOC_SCRATCH_BYTES (16u << 20)
+int astergemm_run_noalloc(const astergemm_config* cfg, const astergemm_operands* ops,
+                          void* stream);
+
 /* Replaces execute_fn's timed loop (execution/core.py:690-703): `iters`
  * launches, each bracketed by its own HIP event pair on `stream`;
  * times_ns[i] = int(ms * 1e6).  If flush_bytes > 0 a streaming kernel over a

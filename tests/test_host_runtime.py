@@ -211,6 +211,7 @@ def test_workspace_query_and_caller_workspace_checks():
     # split K on the 128 x 128 kernel: 8 ranges of 128 x 4096 fp32 partial sums
     p = gemm.GemmPlan.create(128, 4096, 14336)
     assert p.info.name.decode().startswith("splitk_") and p.workspace_bytes() == 8 * 128 * 4096 * 4
+    assert p.workspace_bytes() == _capi.NOALLOC_SCRATCH_BYTES
     # decode rows of 28 KiB: 7 ranges of 4 KiB
     d = gemm.GemmPlan.create(16, 4096, 14336)
     assert d.workspace_bytes() == 7 * 16 * 4096 * 4
@@ -219,6 +220,13 @@ def test_workspace_query_and_caller_workspace_checks():
         d.run(4096, 4096, 4096, workspace=4096, workspace_bytes=d.workspace_bytes() - 1)
     with pytest.raises(_capi.AsterGemmError, match="dWorkspace must be 16-byte aligned"):
         d.run(4096, 4096, 4096, workspace=4096 + 4, workspace_bytes=d.workspace_bytes())
+    # the entry point that allocates nothing refuses what its scratch cannot hold
+    big = gemm.GemmPlan.create(512, 4096, 14336)
+    assert big.workspace_bytes() > _capi.NOALLOC_SCRATCH_BYTES
+    with pytest.raises(_capi.AsterGemmError, match="built-in scratch"):
+        big.run_noalloc(4096, 4096, 4096)
+    with pytest.raises(_capi.AsterGemmError, match="non-null"):
+        gemm.GemmPlan.create(256, 256, 256).run_noalloc(None, None, None)
 
 
 def test_reported_grid_is_the_launched_grid_of_the_k_range_kernels():

@@ -1,0 +1,92 @@
+"""The entry point that allocates nothing (`astergemm_run_noalloc`) against `astergemm_run`.
+
+Shapes whose rows are cut into K ranges keep their fp32 partial sums in a scratch array built
+into the library instead of an allocated workspace; the results must be the same bits.  Two calls
+in a row share the array, the second smaller than the first; a shape that needs no workspace and
+one that needs more than the array holds are covered as well.
+"""
+import ctypes
+
+import numpy as np
+import pytest
+
+from aster_amd import _capi, gemm as AG
+from aster_amd.execution import GpuBuffer
+from oracle import formats as F, gemm as G
+
+pytestmark = pytest.mark.gpu
+
+
+def _bf16(rng, shape, std):
+    return F.f32_to_bf16_bits((rng.standard_normal(shape) * std).astype(np.float32))
+
+
+def _both_ways(M, N, K, seed):
+    rng = np.random.default_rng(seed)
+    a, b = _bf16(rng, (M, K), 1.0), _bf16(rng, (N, K), 0.02)
+    plan = AG.GemmPlan.create(M, N, K, "bf16", "bf16")
+    bufs = [GpuBuffer(a.nbytes), GpuBuffer(b.nbytes), GpuBuffer(M * N * 2), GpuBuffer(M * N * 2)]
+    bufs[0].copy_from_host(a)
+    bufs[1].copy_from_host(b)
+    outs = []
+    for i, run in enumerate((plan.run, plan.run_noalloc)):
+        out = np.full((M, N), 0x7FC1, np.uint16)
+        bufs[2 + i].copy_from_host(out)
+        print(f"{run.__name__} {plan.info.name.decode()} M={M} N={N} K={K} "
+              f"workspace={plan.workspace_bytes()}", flush=True)
+        run(bufs[0].ptr_value, bufs[1].ptr_value, bufs[2 + i].ptr_value)
+        bufs[2 + i].copy_to_host(out)
+        outs.append(out)
+    for bf in bufs:
+        bf.free()
+    want = G.gemm(a, b, G.BF16, G.BF16)
+    return plan, outs[0], outs[1], want
+
+
+def test_noalloc_matches_run_on_two_calls_in_a_row(gpu):
+    # split K on the 128 x 128 kernel: 8 K ranges x 128 x 4096 x 4 bytes = the whole 16 MiB array
+    plan, ref, got, want = _both_ways(128, 4096, 14336, seed=7)
+    assert plan.workspace_bytes() == _capi.NOALLOC_SCRATCH_BYTES
+    assert np.array_equal(ref, got)
+    assert G.rel_l2(F.bf16_bits_to_f32(got), F.bf16_bits_to_f32(want)) <= 1e-3
+    # then a smaller one through the same array: a decode shape in K ranges
+    plan, ref, got, want = _both_ways(16, 520, 14336, seed=8)
+    assert 0 < plan.workspace_bytes() < _capi.NOALLOC_SCRATCH_BYTES
+    assert np.array_equal(ref, got)
+    assert G.rel_l2(F.bf16_bits_to_f32(got), F.bf16_bits_to_f32(want)) <= 1e-3
+    # and a shape without K ranges: the array is not touched at all
+    plan, ref, got, want = _both_ways(264, 520, 512, seed=9)
+    assert plan.workspace_bytes() == 0
+    assert np.array_equal(ref, got)
+
+
+def test_noalloc_refuses_what_the_scratch_cannot_hold(gpu):
+    plan = AG.GemmPlan.create(512, 4096, 14336, "bf16", "bf16")
+    assert plan.workspace_bytes() > _capi.NOALLOC_SCRATCH_BYTES
+    with pytest.raises(_capi.AsterGemmError) as err:
+        plan.run_noalloc(256, 256, 256)     # refused before any pointer is used
+    assert err.value.code == -22 and "scratch" in str(err.value)
+
+
+def test_caller_workspace_matches_the_library_workspace(gpu):
+    M, N, K = 96, 1000, 16384
+    rng = np.random.default_rng(11)
+    a, b = _bf16(rng, (M, K), 1.0), _bf16(rng, (N, K), 0.02)
+    plan = AG.GemmPlan.create(M, N, K, "bf16", "bf16")
+    need = plan.workspace_bytes()
+    assert need > 0
+    bufs = [GpuBuffer(a.nbytes), GpuBuffer(b.nbytes), GpuBuffer(M * N * 2), GpuBuffer(need)]
+    bufs[0].copy_from_host(a)
+    bufs[1].copy_from_host(b)
+    out_lib, out_own = np.zeros((M, N), np.uint16), np.zeros((M, N), np.uint16)
+    plan.run(bufs[0].ptr_value, bufs[1].ptr_value, bufs[2].ptr_value)
+    bufs[2].copy_to_host(out_lib)
+    plan.run(bufs[0].ptr_value, bufs[1].ptr_value, bufs[2].ptr_value, workspace=bufs[3].ptr_value,
+             workspace_bytes=need)
+    bufs[2].copy_to_host(out_own)
+    assert np.array_equal(out_lib, out_own)
+    with pytest.raises(_capi.AsterGemmError):
+        plan.run(bufs[0].ptr_value, bufs[1].ptr_value, bufs[2].ptr_value,
+                 workspace=bufs[3].ptr_value, workspace_bytes=need - 4)
+    for bf in bufs:
+        bf.free()
