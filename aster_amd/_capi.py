@@ -21,7 +21,7 @@ F16, BF16, FP8_E4M3, MXFP4, F32 = 0, 1, 2, 3, 4
 SCALE_NONE, SCALE_TENSOR, SCALE_MX32 = 0, 1, 2
 # astergemm_kernel_family
 KERNEL_AUTO, KERNEL_TILE, KERNEL_SKINNY = 0, 1, 2
-OPERAND_LDS, OPERAND_DIRECT_B = 0, 1
+OPERAND_LDS, OPERAND_DIRECT_B, OPERAND_DIRECT_B_K8 = 0, 1, 2
 ABI_VERSION = 2
 NOALLOC_SCRATCH_BYTES = 16 << 20
 
@@ -120,6 +120,7 @@ SIGNATURES = {
                                  C.POINTER(C.c_int64), _P]),
     "astergemm_diag_mfma_rate": (C.c_int, [C.c_int, _P, C.c_int64, C.c_int, C.POINTER(C.c_double), _P]),
     "astergemm_shuffle_weight_16": (C.c_int, [_P, _P, C.c_int64, C.c_int64]),
+    "astergemm_shuffle_weight_k8_16": (C.c_int, [_P, _P, C.c_int64, C.c_int64]),
     "astergemm_weight_crc32": (C.c_uint32, [_P, C.c_size_t]),
     "astergemm_weight_header_init": (C.c_int, [C.POINTER(WeightHeader), C.c_int, C.c_int, C.c_int64,
                                                C.c_int64, C.c_float]),

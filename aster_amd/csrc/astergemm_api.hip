@@ -87,8 +87,11 @@ const char* validate_problem(const astergemm_config& c) {
     return "dtype_c must be F32, BF16 or F16";
   if (c.scale_mode < ASTERGEMM_SCALE_NONE || c.scale_mode > ASTERGEMM_SCALE_MX32)
     return "bad scale_mode";
-  if (c.operand_path != ASTERGEMM_OPERAND_LDS && c.operand_path != ASTERGEMM_OPERAND_DIRECT_B)
+  if (c.operand_path < ASTERGEMM_OPERAND_LDS || c.operand_path > ASTERGEMM_OPERAND_DIRECT_B_K8)
     return "bad operand_path";
+  if (c.operand_path != ASTERGEMM_OPERAND_LDS && c.dtype_ab != ASTERGEMM_F16 &&
+      c.dtype_ab != ASTERGEMM_BF16)
+    return "pre-shuffled B is built for 16-bit operands";
   if ((c.dtype_ab == ASTERGEMM_MXFP4) != (c.scale_mode == ASTERGEMM_SCALE_MX32))
     return "MXFP4 operands and SCALE_MX32 go together";
   if (c.dtype_ab == ASTERGEMM_MXFP4 && c.K % 32 != 0) return "MXFP4 needs K % 32 == 0";
@@ -151,6 +154,7 @@ const Variant* choose(const astergemm_config& c, int* index_out) {
     }
   }
   if (c.operand_path == ASTERGEMM_OPERAND_DIRECT_B) family = ASTERGEMM_KERNEL_SKINNY;
+  if (c.operand_path == ASTERGEMM_OPERAND_DIRECT_B_K8) family = ASTERGEMM_KERNEL_TILE;
 
   const Variant* best = nullptr;
   int best_index = -1;
@@ -672,6 +676,22 @@ int astergemm_shuffle_weight_16(const uint16_t* src, uint16_t* dst, int64_t N, i
           for (int kh = 0; kh < 2; ++kh)
             for (int kw = 0; kw < 4; ++kw)
               dst[o++] = src[(nb * 16 + nl) * K + kb * 32 + kh * 16 + g * 4 + kw];
+  return 0;
+}
+
+int astergemm_shuffle_weight_k8_16(const uint16_t* src, uint16_t* dst, int64_t N, int64_t K) {
+  if (!src || !dst || N < 0 || K < 0 || N % 16 != 0 || K % 32 != 0) {
+    set_error("astergemm_shuffle_weight_k8_16: need N %% 16 == 0 and K %% 32 == 0");
+    return ASTERGEMM_EINVAL;
+  }
+  // dst order (nb, kb, lane group g, row n, 8 consecutive K) <- src (nb, n, kb, g, k)
+  const int64_t kblocks = K / 32;
+  int64_t o = 0;
+  for (int64_t nb = 0; nb < N / 16; ++nb)
+    for (int64_t kb = 0; kb < kblocks; ++kb)
+      for (int g = 0; g < 4; ++g)
+        for (int nl = 0; nl < 16; ++nl)
+          for (int kw = 0; kw < 8; ++kw) dst[o++] = src[(nb * 16 + nl) * K + kb * 32 + g * 8 + kw];
   return 0;
 }
 

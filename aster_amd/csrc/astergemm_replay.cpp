@@ -10,7 +10,8 @@
 //   astergemm_replay --m 8192 --n 8192 --k 8192 --ab bf16 --c bf16 --iters 100
 //                    [--warmup 20] [--tile 256] [--family tile|skinny|auto]
 //                    [--variant ID] [--flush BYTES] [--bias] [--json] [--calib BYTES]
-//                    [--direct-b]   (B taken as pre-shuffled; timing only, the fill is random)
+//                    [--direct-b | --direct-b-k8]   (B taken as pre-shuffled in the reference's order /
+//                                    in K8 order; timing only, the fill is random)
 //   astergemm_replay --quantize fp8|mxfp4 --m ROWS --k K --iters 100
 //                    (operand quantiser on a ROWS x K fp32 source instead of a GEMM)
 //
@@ -153,6 +154,7 @@ int main(int argc, char** argv) {
     else if (a == "--flush") flush = atoll(val());
     else if (a == "--calib") calib = atoll(val());
     else if (a == "--direct-b") cfg.operand_path = ASTERGEMM_OPERAND_DIRECT_B;
+    else if (a == "--direct-b-k8") cfg.operand_path = ASTERGEMM_OPERAND_DIRECT_B_K8;
     else if (a == "--bias") cfg.has_bias = 1;
     else if (a == "--json") json = 1;
     else if (a == "--quantize") quantize = val();

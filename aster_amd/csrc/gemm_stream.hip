@@ -4,6 +4,7 @@
 #include "gemm_stream_kernel.hpp"
 #include "gemm_stream8_kernel.hpp"
 #include "gemm_stream4_kernel.hpp"
+#include "gemm_streamdb_kernel.hpp"
 
 namespace astergemm {
 namespace {
@@ -43,6 +44,39 @@ const char* check_stream_whole_k(const astergemm_config& c) {
         (const void*)gemm_stream_kernel<DT, OUT, BM, BN, WM, WN>,                \
         launch_stream<DT, OUT, BM, BN, WM, WN>,                                  \
         (WM * WN == 8 || BM == 128) ? check_stream : check_stream_whole_k        \
+  }
+
+// ---- B pre-shuffled, loaded straight into MFMA operands (gemm_streamdb_kernel.hpp) ---------
+template <int DT, int OUT, int NSLOT, int NBUF>
+int launch_streamdb(const GemmArgs& a, int grid, hipStream_t s) {
+  constexpr int lds = 5 * 256 * kRowBytes;  // the epilogue stages through up to 160 KiB
+  auto k = gemm_streamdb_kernel<DT, OUT, NSLOT, NBUF>;
+  static std::atomic<uint64_t> attr_devs{0};
+  if (int e = lds_attr_once(attr_devs, (const void*)k, lds)) return e;
+  // what the kernel's indexing assumes: whole 16-row blocks of B and whole K-steps
+  if (a.N % 16 != 0 || a.N < 16 || a.M < 8 || a.M % 8 != 0 || a.K % 64 != 0 || a.tail_granules != 0 ||
+      a.ldb_bytes != (int64_t)a.K * 2)
+    return (int)hipErrorInvalidValue;
+  hipLaunchKernelGGL(k, dim3(grid), dim3(512), lds, s, a);
+  return (int)hipGetLastError();
+}
+
+const char* check_streamdb(const astergemm_config& c) {
+  if (c.M % 8 != 0 || c.M < 8) return "M must be a multiple of 8";
+  if (c.N % 16 != 0 || c.N < 16) return "pre-shuffled B needs N % 16 == 0";
+  if (c.K % 64 != 0) return "pre-shuffled B in K8 order needs K % 64 == 0";
+  if (c.ldb != 0 && c.ldb != c.K) return "pre-shuffled B is packed (ldb = K)";
+  if (c.ldc % 8 != 0) return "ldc must be a multiple of 8 elements";
+  if (c.N * c.K * 2 >= ((int64_t)1 << 32)) return "pre-shuffled B must stay below 4 GiB";
+  return nullptr;
+}
+
+#define AG_STREAMDB(name, DT, OUT, NSLOT, NBUF, RANK)                            \
+  Variant {                                                                      \
+    name, ASTERGEMM_KERNEL_TILE, DT, OUT, 256, 256, kRowBytes, 2, 4, NSLOT, RANK, \
+        5 * 256 * kRowBytes, (const void*)gemm_streamdb_kernel<DT, OUT, NSLOT, NBUF>, \
+        launch_streamdb<DT, OUT, NSLOT, NBUF>, check_streamdb,                   \
+        ASTERGEMM_OPERAND_DIRECT_B_K8                                            \
   }
 
 // ---- split K on the 128x128 kernel --------------------------------------------------------
@@ -161,10 +195,22 @@ const char* check_stream4(const astergemm_config& c) {
 
 #define AG_STREAM4(name, DT, OUT)                                                \
   Variant {                                                                      \
-    name, ASTERGEMM_KERNEL_TILE, DT, OUT, 256, 256, kRowBytes, 2, 2, 2, 2,       \
+    name, ASTERGEMM_KERNEL_TILE, DT, OUT, 256, 256, kRowBytes, 2, 2, 2, 1,       \
         4 * 256 * kRowBytes + 4 * 256 * 16,                                      \
         (const void*)gemm_stream4_kernel<DT, OUT, 256, 256, 2, 2>,               \
         launch_stream4<DT, OUT, 256, 256, 2, 2>, check_stream4                   \
+  }
+// The same kernel with eight waves (2 x 4, wave tile 128 x 64, two waves per SIMD): with the
+// accumulators in the accumulation registers it allocates without spills (128 + 116), and a
+// second wave on every SIMD covers the waits of the first.  p50, one box, four -> eight waves:
+// 4096 x 14336 x 4096 134.2 -> 125.3 us, 8192^3 246.8 -> 243.1, 16384 x 16384 x 4096 550.5 ->
+// 533.3, 4096^3 38.1 -> 37.3; the same bits.  Preferred (rank 2 over 1).
+#define AG_STREAM4_W8(name, DT, OUT, RANK)                                       \
+  Variant {                                                                      \
+    name, ASTERGEMM_KERNEL_TILE, DT, OUT, 256, 256, kRowBytes, 2, 4, 2, RANK,    \
+        4 * 256 * kRowBytes + 4 * 256 * 16,                                      \
+        (const void*)gemm_stream4_kernel<DT, OUT, 256, 256, 2, 4>,               \
+        launch_stream4<DT, OUT, 256, 256, 2, 4>, check_stream4                   \
   }
 #define AG_STREAM4_128(name, DT, OUT)                                            \
   Variant {                                                                      \
@@ -173,6 +219,127 @@ const char* check_stream4(const astergemm_config& c) {
         (const void*)gemm_stream4_kernel<DT, OUT, 128, 128, 2, 2>,               \
         launch_stream4<DT, OUT, 128, 128, 2, 2>, check_stream4                   \
   }
+
+// ---- whole rounds of 256 x 256 tiles, the rest in 128 x 128 tiles ---------------------------
+//
+// One workgroup of the 256 x 256 kernels runs per CU, so a tile count that is not a multiple of
+// the CU count leaves the last round partly empty (4096 x 14336: 896 tiles on 256 CUs = 3.5
+// rounds, paid as 4).  The problem is cut along N or M: the part whose 256 x 256 tiles fill
+// whole rounds goes to the 256 x 256 kernel, the remaining columns (or rows) to the 128 x 128
+// kernel of the same family, two workgroups per CU, right behind it on the same stream.
+// Measured on 4096 x 14336 x 4096, p50 on one box, 256 x 256 alone -> with the cut: MXFP4 136.3 ->
+// 134.7 us, bf16 350.2 -> 343.4 us, fp8 179.2 -> 180.0 us (128 x 128 alone: 141.9, 393.7, 203.5).
+// The gain is far below the 12 % of the empty half round: the chip is power limited, and the CUs
+// that stay busy in a half-empty round run at a higher clock.
+struct TailSplit {
+  int along = 0;      // 0 = no split, 1 = along N, 2 = along M
+  int64_t first = 0;  // columns (rows) of the 256 x 256 part
+};
+
+inline TailSplit tail_split_of(int64_t M, int64_t N, int cus) {
+  TailSplit best;
+  if (cus <= 0) cus = 256;
+  const int64_t tm = (M + 255) / 256, tn = (N + 255) / 256;
+  const double whole = (double)((tm * tn + cus - 1) / cus);
+  double best_cost = whole * 0.93;  // a split has to save at least 7 %
+  for (int along = 1; along <= 2; ++along) {
+    const int64_t cut_tiles = along == 1 ? tn : tm, other = along == 1 ? tm : tn;
+    const int64_t extent = along == 1 ? N : M;
+    // the largest number of tile columns (rows) that gives whole rounds
+    for (int64_t t1 = cut_tiles - 1; t1 >= 1; --t1) {
+      if ((t1 * other) % cus != 0) continue;
+      const int64_t rest = extent - t1 * 256;
+      const int64_t rest128 = (rest + 127) / 128 * (((along == 1 ? M : N) + 127) / 128);
+      const double cost = (double)(t1 * other / cus) +
+                          0.55 * (double)((rest128 + 2 * cus - 1) / (2 * cus));
+      if (cost < best_cost) {
+        best_cost = cost;
+        best.along = along;
+        best.first = t1 * 256;
+      }
+      break;
+    }
+  }
+  return best;
+}
+
+// the two sub-problems of a split: `part1` the first `ts.first` columns (rows), `part2` the rest
+inline void tail_parts(const GemmArgs& a, const TailSplit& ts, int out_bytes, GemmArgs* part1,
+                       GemmArgs* part2) {
+  *part1 = a;
+  *part2 = a;
+  if (ts.along == 1) {
+    part1->N = (int32_t)ts.first;
+    part2->N = a.N - (int32_t)ts.first;
+    part2->B = a.B + ts.first * a.ldb_bytes;
+    if (a.mx_b) part2->mx_b = a.mx_b + ts.first * a.mx_ld;
+    if (a.bias) part2->bias = a.bias + ts.first;
+    part2->C = (uint8_t*)a.C + ts.first * out_bytes;
+  } else {
+    part1->M = (int32_t)ts.first;
+    part2->M = a.M - (int32_t)ts.first;
+    part2->A = a.A + ts.first * a.lda_bytes;
+    if (a.mx_a) part2->mx_a = a.mx_a + ts.first * a.mx_ld;
+    part2->C = (uint8_t*)a.C + ts.first * a.ldc * out_bytes;
+  }
+  part1->tiles_m = (part1->M + 255) / 256;
+  part1->tiles_n = (part1->N + 255) / 256;
+  part2->tiles_m = (part2->M + 127) / 128;
+  part2->tiles_n = (part2->N + 127) / 128;
+}
+
+// KIND 0: 16-bit operands, 1: fp8, 2: MXFP4
+template <int KIND, int DT, int OUT>
+int launch_stream_tail(const GemmArgs& a, int grid, hipStream_t s) {
+  (void)grid;
+  const TailSplit ts = tail_split_of(a.M, a.N, device_cus());
+  if (ts.along == 0) return (int)hipErrorInvalidValue;
+  GemmArgs p1, p2;
+  tail_parts(a, ts, OUT == ASTERGEMM_F32 ? 4 : 2, &p1, &p2);
+  const int g1 = p1.tiles_m * p1.tiles_n, g2 = p2.tiles_m * p2.tiles_n;
+  int rc;
+  if constexpr (KIND == 0) {
+    if ((rc = launch_stream<DT, OUT, 256, 256, 2, 4>(p1, g1, s)) != 0) return rc;
+    return launch_stream<DT, OUT, 128, 128, 2, 2>(p2, g2, s);
+  } else if constexpr (KIND == 1) {
+    if ((rc = launch_stream8<DT, OUT, 256, 256, 2, 4>(p1, g1, s)) != 0) return rc;
+    return launch_stream8<DT, OUT, 128, 128, 2, 2>(p2, g2, s);
+  } else {
+    if ((rc = launch_stream4<DT, OUT, 256, 256, 2, 4>(p1, g1, s)) != 0) return rc;
+    return launch_stream4<DT, OUT, 128, 128, 2, 2>(p2, g2, s);
+  }
+}
+
+const char* check_stream_tail(const astergemm_config& c) {
+  if (c.dtype_ab == ASTERGEMM_MXFP4) {
+    if (const char* why = check_stream4(c)) return why;
+  } else if (const char* why = check_stream(c)) {
+    return why;
+  }
+  if (tail_split_of(c.M, c.N, device_cus()).along == 0)
+    return "no cut along M or N gives whole rounds of 256 x 256 tiles plus a cheaper rest";
+  return nullptr;
+}
+
+int grid_stream_tail(const astergemm_config& c, int cus) {
+  const TailSplit ts = tail_split_of(c.M, c.N, cus);
+  if (ts.along == 0) return (int)(((c.M + 255) / 256) * ((c.N + 255) / 256));
+  const int64_t m1 = ts.along == 2 ? ts.first : c.M, n1 = ts.along == 1 ? ts.first : c.N;
+  const int64_t m2 = ts.along == 2 ? c.M - ts.first : c.M, n2 = ts.along == 1 ? c.N - ts.first : c.N;
+  return (int)(((m1 + 255) / 256) * ((n1 + 255) / 256) + ((m2 + 127) / 128) * ((n2 + 127) / 128));
+}
+
+// rank 3: preferred over the plain 256 x 256 kernel wherever its check passes
+#define AG_STREAM_TAIL(name, KIND, DT, OUT, WM, WN, LDS, FUNC)                   \
+  Variant {                                                                      \
+    name, ASTERGEMM_KERNEL_TILE, DT, OUT, 256, 256, kRowBytes, WM, WN, 3, 3, LDS, \
+        (const void*)FUNC<DT, OUT, 256, 256, WM, WN>, launch_stream_tail<KIND, DT, OUT>, \
+        check_stream_tail, ASTERGEMM_OPERAND_LDS, nullptr, grid_stream_tail      \
+  }
+#define AG_STREAM_TAIL_SET(prefix, KIND, DT, WM, WN, LDS, FUNC)                  \
+  AG_STREAM_TAIL(prefix "_bf16", KIND, DT, ASTERGEMM_BF16, WM, WN, LDS, FUNC),   \
+      AG_STREAM_TAIL(prefix "_f32", KIND, DT, ASTERGEMM_F32, WM, WN, LDS, FUNC), \
+      AG_STREAM_TAIL(prefix "_f16", KIND, DT, ASTERGEMM_F16, WM, WN, LDS, FUNC)
 
 #define AG_STREAM_SET(prefix, DT)                                                      \
   AG_STREAM(prefix "_256x256_w2x4_bf16", DT, ASTERGEMM_BF16, 256, 256, 2, 4),          \
@@ -192,6 +359,20 @@ const Variant kStreamVariants[] = {
     AG_STREAM_SPLITK_SET("splitk_mxfp4", 2, ASTERGEMM_MXFP4, 4 * 128 * kRowBytes + 4 * 128 * 16,
                          gemm_stream4_splitk_kernel),
     AG_STREAM_SET("stream_f16", ASTERGEMM_F16),
+    AG_STREAMDB("streamdb_bf16_256x256_w2x4_bf16", ASTERGEMM_BF16, ASTERGEMM_BF16, 5, 5, 2),
+    AG_STREAMDB("streamdb_bf16_256x256_w2x4_f32", ASTERGEMM_BF16, ASTERGEMM_F32, 5, 5, 2),
+    AG_STREAMDB("streamdb_bf16_256x256_w2x4_f16", ASTERGEMM_BF16, ASTERGEMM_F16, 5, 5, 2),
+    AG_STREAMDB("streamdb_f16_256x256_w2x4_bf16", ASTERGEMM_F16, ASTERGEMM_BF16, 5, 5, 2),
+    AG_STREAMDB("streamdb_f16_256x256_w2x4_f32", ASTERGEMM_F16, ASTERGEMM_F32, 5, 5, 2),
+    AG_STREAMDB("streamdb_f16_256x256_w2x4_f16", ASTERGEMM_F16, ASTERGEMM_F16, 5, 5, 2),
+    AG_STREAM_TAIL_SET("stream_bf16_256x256_w2x4_tail128", 0, ASTERGEMM_BF16, 2, 4, 5 * 256 * kRowBytes,
+                       gemm_stream_kernel),
+    AG_STREAM_TAIL_SET("stream_f16_256x256_w2x4_tail128", 0, ASTERGEMM_F16, 2, 4, 5 * 256 * kRowBytes,
+                       gemm_stream_kernel),
+    AG_STREAM_TAIL_SET("stream_fp8_256x256_w2x4_tail128", 1, ASTERGEMM_FP8_E4M3, 2, 4,
+                       5 * 256 * kRowBytes, gemm_stream8_kernel),
+    AG_STREAM_TAIL_SET("stream_mxfp4_256x256_w2x4_tail128", 2, ASTERGEMM_MXFP4, 2, 4,
+                       4 * 256 * kRowBytes + 4 * 256 * 16, gemm_stream4_kernel),
     AG_STREAM8("stream_fp8_256x256_w2x4_bf16", ASTERGEMM_FP8_E4M3, ASTERGEMM_BF16),
     AG_STREAM8("stream_fp8_256x256_w2x4_f32", ASTERGEMM_FP8_E4M3, ASTERGEMM_F32),
     AG_STREAM8("stream_fp8_256x256_w2x4_f16", ASTERGEMM_FP8_E4M3, ASTERGEMM_F16),
@@ -201,6 +382,9 @@ const Variant kStreamVariants[] = {
     AG_STREAM4("stream_mxfp4_256x256_w2x2_bf16", ASTERGEMM_MXFP4, ASTERGEMM_BF16),
     AG_STREAM4("stream_mxfp4_256x256_w2x2_f32", ASTERGEMM_MXFP4, ASTERGEMM_F32),
     AG_STREAM4("stream_mxfp4_256x256_w2x2_f16", ASTERGEMM_MXFP4, ASTERGEMM_F16),
+    AG_STREAM4_W8("stream_mxfp4_256x256_w2x4_bf16", ASTERGEMM_MXFP4, ASTERGEMM_BF16, 2),
+    AG_STREAM4_W8("stream_mxfp4_256x256_w2x4_f32", ASTERGEMM_MXFP4, ASTERGEMM_F32, 2),
+    AG_STREAM4_W8("stream_mxfp4_256x256_w2x4_f16", ASTERGEMM_MXFP4, ASTERGEMM_F16, 2),
     AG_STREAM4_128("stream_mxfp4_128x128_w2x2_bf16", ASTERGEMM_MXFP4, ASTERGEMM_BF16),
     AG_STREAM4_128("stream_mxfp4_128x128_w2x2_f32", ASTERGEMM_MXFP4, ASTERGEMM_F32),
     AG_STREAM4_128("stream_mxfp4_128x128_w2x2_f16", ASTERGEMM_MXFP4, ASTERGEMM_F16),

@@ -22,10 +22,12 @@
 // the last read of B(k): it certifies everything transferred for K-step k+1 and frees the
 // slots of K-step k, whose refills (K-step k+2) are issued right behind it.
 //
-// The kernel runs four waves per workgroup (one per SIMD, 128x128 of C each): two MFMAs per
-// accumulator and trip plus the scale registers do not fit next to 128 accumulators in the
-// 256 registers a wave gets at two waves per SIMD, while one wave per SIMD has 256
-// accumulation registers for the 64 accumulators and 256 architectural ones for the rest.
+// Wave grid: 2 x 4 (eight waves, wave tile 128 x 64, two waves per SIMD) is the default; 2 x 2
+// (four waves, one per SIMD, 128 x 128 of C each, a third fewer LDS reads per MFMA) is built as
+// well and is slower: with one wave per SIMD nothing covers a wave's wait at the barrier.
+// Either way the accumulators live in the accumulation registers (64 or 32 tiles x 4), which
+// leaves the architectural registers to fragments, scales and addresses; with one pool of 256
+// registers the eight-wave form does not allocate.
 #pragma once
 #include "gemm_stream_kernel.hpp"
 

@@ -3,10 +3,11 @@
 // scale, MXFP4 nibbles with their e8m0 plane), behind a fixed 128-byte little-endian header.
 // Host code only: parsing, validation, the checksum and the header -> astergemm_config step.
 //
-// The pre-shuffled layout is the reference's shuffle_weight order
+// The pre-shuffled layouts are the reference's shuffle_weight order
 // (contrib/kittens/test/kittens_helpers.py:90-119), which its execute_fn applies on every call
-// (contrib/kittens/test/test_102_gemm_python_multitile_g2s_directb_cdna4.py:440-467); a file
-// written once replaces that per-call host permutation.
+// (contrib/kittens/test/test_102_gemm_python_multitile_g2s_directb_cdna4.py:440-467), read by
+// the decode kernels, and the K8 order of astergemm_shuffle_weight_k8_16, read by the 256 x 256
+// stream kernel with direct B; a file written once replaces that per-call host permutation.
 #include <cstring>
 
 #include "astergemm_internal.h"
@@ -67,10 +68,10 @@ extern "C" int astergemm_weight_header_init(astergemm_weight_header* h, int dtyp
   if (N <= 0 || K <= 0) return fail("N and K must be positive");
   if (dtype == ASTERGEMM_MXFP4 && K % 32 != 0) return fail("MXFP4 needs K % 32 == 0");
   if (astergemm::row_bytes(dtype, K) % 16 != 0) return fail("a row must be a multiple of 16 bytes");
-  if (layout == ASTERGEMM_OPERAND_DIRECT_B) {
+  if (layout == ASTERGEMM_OPERAND_DIRECT_B || layout == ASTERGEMM_OPERAND_DIRECT_B_K8) {
     if (dtype != ASTERGEMM_F16 && dtype != ASTERGEMM_BF16)
-      return fail("the pre-shuffled layout holds 16-bit elements");
-    if (N % 16 != 0 || K % 32 != 0) return fail("the pre-shuffled layout needs N % 16 == 0, K % 32 == 0");
+      return fail("the pre-shuffled layouts hold 16-bit elements");
+    if (N % 16 != 0 || K % 32 != 0) return fail("the pre-shuffled layouts need N % 16 == 0, K % 32 == 0");
   } else if (layout != ASTERGEMM_OPERAND_LDS) {
     return fail("unknown layout");
   }

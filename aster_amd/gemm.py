@@ -32,6 +32,9 @@ _DTYPE_ID = {"f16": _capi.F16, "bf16": _capi.BF16, "fp8_e4m3": _capi.FP8_E4M3,
              "mxfp4": _capi.MXFP4, "f32": _capi.F32}
 _SCALE_ID = {"none": _capi.SCALE_NONE, "tensor": _capi.SCALE_TENSOR, "mx32": _capi.SCALE_MX32}
 _OUT_NP = {"f32": np.float32, "bf16": np.uint16, "f16": np.float16}
+_OPERAND_PATH_ID = {"lds": _capi.OPERAND_LDS, "direct_b": _capi.OPERAND_DIRECT_B,
+                    "direct_b_k8": _capi.OPERAND_DIRECT_B_K8}
+_OPERAND_PATH_NAME = {v: k for k, v in _OPERAND_PATH_ID.items()}
 
 
 def config_from_instance(cfg: WeakScaledMappedGemmInstance, *, use_mapping: bool = True,
@@ -55,8 +58,6 @@ def config_from_instance(cfg: WeakScaledMappedGemmInstance, *, use_mapping: bool
         c.wg_tile_n = twg[DIM_N] * spec.mfma_shape[DIM_N]
         c.waves_m = mapping.num_waves_per_workgroup[DIM_M]
         c.waves_n = mapping.num_waves_per_workgroup[DIM_N]
-        if mapping.direct_b and not mapping.direct_a:
-            c.operand_path = _capi.OPERAND_DIRECT_B
     return c
 
 
@@ -98,8 +99,8 @@ def mapping_report(cfg: WeakScaledMappedGemmInstance, c: _capi.Config,
         miss["wg_tile"] = {"requested": want_tile, "kernel": [info.wg_tile_m, info.wg_tile_n]}
     if [info.waves_m, info.waves_n] != want_waves:
         miss["waves"] = {"requested": want_waves, "kernel": [info.waves_m, info.waves_n]}
-    ran_path = "direct_b" if c.operand_path == _capi.OPERAND_DIRECT_B else "lds"
-    if mapping.operand_path.value != ran_path:
+    ran_path = _OPERAND_PATH_NAME[c.operand_path]
+    if mapping.operand_path.value != ran_path.replace("_k8", ""):
         miss["operand_path"] = {"requested": mapping.operand_path.value, "kernel": ran_path}
     fixed = {}
     for k in _COMPILER_KNOBS:
@@ -111,24 +112,26 @@ def mapping_report(cfg: WeakScaledMappedGemmInstance, c: _capi.Config,
 
 def select_for_instance(cfg: WeakScaledMappedGemmInstance) -> Tuple[_capi.Config, _capi.KernelInfo]:
     """Honour the instance's mapping when a variant with that geometry exists, otherwise let the
-    library choose (`mapping_report` tells which happened).  A `direct_b` request that no kernel
-    takes for this shape falls back to plain row-major B."""
-    c = config_from_instance(cfg, use_mapping=True)
-    try:
-        return c, select(c)
-    except _capi.AsterGemmError as e:
-        if e.code != -95:
-            raise
-    if c.operand_path == _capi.OPERAND_DIRECT_B:
-        # keep the operand path, drop the geometry
-        c2 = config_from_instance(cfg, use_mapping=False)
-        c2.operand_path = _capi.OPERAND_DIRECT_B
-        try:
-            return c2, select(c2)
-        except _capi.AsterGemmError as e:
-            if e.code != -95:
-                raise
+    library choose (`mapping_report` tells which happened).  A `direct_b` mapping gets a kernel
+    that reads pre-shuffled B when one takes the shape -- the decode kernels in the reference's
+    `shuffle_weight` order, else the 256 x 256 stream kernel in `shuffle_weight_k8` order (the
+    returned config's `operand_path` says which; `execute_gemm_hsaco` shuffles accordingly) --
+    and falls back to plain row-major B otherwise."""
+    want_direct = cfg.mapping.direct_b and not cfg.mapping.direct_a
+    paths = [_capi.OPERAND_DIRECT_B, _capi.OPERAND_DIRECT_B_K8] if want_direct else []
+    for use_mapping in (True, False):
+        for path in paths + [_capi.OPERAND_LDS]:
+            if not use_mapping and path == _capi.OPERAND_LDS and not want_direct:
+                break
+            c = config_from_instance(cfg, use_mapping=use_mapping)
+            c.operand_path = path
+            try:
+                return c, select(c)
+            except _capi.AsterGemmError as e:
+                if e.code != -95:
+                    raise
     c = config_from_instance(cfg, use_mapping=False)
+    c.operand_path = _capi.OPERAND_LDS
     return c, select(c)
 
 
@@ -157,7 +160,7 @@ def compile_gemm(cfg: WeakScaledMappedGemmInstance, output_hsaco_path: str, **kw
         "vgprs": info.vgprs,
         "wg_tile": [info.wg_tile_m, info.wg_tile_n, info.wg_tile_k],
         "waves": [info.waves_m, info.waves_n],
-        "operand_path": "direct_b" if c.operand_path == _capi.OPERAND_DIRECT_B else "lds",
+        "operand_path": _OPERAND_PATH_NAME[c.operand_path],
         "mapping_honoured": rep.honoured,
         "mapping_not_honoured": rep.not_honoured,
         "mapping_fixed_by_kernel": rep.fixed_by_kernel,
@@ -195,9 +198,11 @@ class GemmPlan:
                ldb: int = 0, ldc: int = 0, family: int = _capi.KERNEL_AUTO, wg_tile=(0, 0),
                variant: int = 0, operand_path: str = "lds") -> "GemmPlan":
         """`operand_path` follows GemmMappingSpec.operand_path of the reference: "lds" = B is
-        plain row-major [N, ldb]; "direct_b" = B was pre-shuffled with `shuffle_weight`."""
+        plain row-major [N, ldb]; "direct_b" = B was pre-shuffled with `shuffle_weight` (the
+        reference's order, read by the decode kernels); "direct_b_k8" = pre-shuffled with
+        `shuffle_weight_k8` (read by the 256 x 256 stream kernel)."""
         c = _capi.Config()
-        c.operand_path = {"lds": _capi.OPERAND_LDS, "direct_b": _capi.OPERAND_DIRECT_B}[operand_path]
+        c.operand_path = _OPERAND_PATH_ID[operand_path]
         c.M, c.N, c.K = M, N, K
         c.lda, c.ldb, c.ldc = lda, ldb, ldc
         c.dtype_ab, c.dtype_c = _DTYPE_ID[dtype_ab], _DTYPE_ID[dtype_c]
@@ -366,13 +371,14 @@ def execute_gemm_hsaco(cfg: WeakScaledMappedGemmInstance, hsaco_path: str, num_i
                            f"{info.name.decode()!r}")
     M, N, K = cfg.spec.gemm_size
     out_np = _OUT_NP[cfg.spec.dtype_c]
-    if c.operand_path == _capi.OPERAND_DIRECT_B:
+    if c.operand_path != _capi.OPERAND_LDS:
         # single point of truth, as in the reference's execute_fn
         # (test_102_gemm_python_multitile_g2s_directb_cdna4.py:446-467): the caller passes B
-        # row-major and the pre-shuffle happens here, only when the kernel that runs wants it
-        from .kittens_helpers import shuffle_weight
+        # row-major and the pre-shuffle happens here, in the order the kernel that runs reads
+        from .kittens_helpers import shuffle_weight, shuffle_weight_k8
 
-        B = shuffle_weight(np.ascontiguousarray(B).reshape(N, K))
+        shuffle = shuffle_weight if c.operand_path == _capi.OPERAND_DIRECT_B else shuffle_weight_k8
+        B = shuffle(np.ascontiguousarray(B).reshape(N, K))
     C_host = np.zeros(M * N, dtype=out_np)
 
     def up(arr, dtype=None):

@@ -531,8 +531,8 @@ class Cdna4GemmInstance(WeakScaledMappedGemmInstance):
 
 def make_instance(M: int, N: int, K: int, *, dtype_ab: str = "bf16", dtype_c: str = "bf16",
                   wg_tile=(256, 256), waves=(2, 4), pipeline_strategy: int = 1,
-                  has_bias: bool = False, scale_mode: Optional[str] = None
-                  ) -> WeakScaledMappedGemmInstance:
+                  has_bias: bool = False, scale_mode: Optional[str] = None,
+                  operand_path: "OperandPath" = None) -> WeakScaledMappedGemmInstance:
     """Instance for one of the HIP kernels' native tilings: M and N must be
     multiples of the workgroup tile (the weak-scale rule)."""
     tm, tn = wg_tile
@@ -547,6 +547,7 @@ def make_instance(M: int, N: int, K: int, *, dtype_ab: str = "bf16", dtype_c: st
         num_tiles_per_wave=[tm // mfma[0] // waves[0], tn // mfma[1] // waves[1], 1],
         pipeline_strategy=pipeline_strategy,
         mcpu="gfx950",
+        **({} if operand_path is None else {"operand_path": operand_path}),
     )
     return WeakScaledMappedGemmInstance(spec, mapping)
 

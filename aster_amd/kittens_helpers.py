@@ -69,3 +69,27 @@ def unshuffle_weight(Bs: np.ndarray) -> np.ndarray:
     N, K = Bs.shape
     view = Bs.reshape(N // 16, K // 32, 4, 16, 2, 4)
     return np.ascontiguousarray(view.transpose(0, 3, 1, 4, 2, 5)).reshape(N, K)
+
+
+def shuffle_weight_k8(B: np.ndarray) -> np.ndarray:
+    """Pre-shuffle B[N, K] (2-byte elements) for the 16x16x32 MFMA read with 16-byte operand
+    loads: view B as (n_block, n_lane=16, k_block, lane_group=4, k_within=8) and store it in
+    the order (n_block, k_block, lane_group, n_lane, k_within).  Lane d of block (nb, kb) then
+    finds B[nb*16 + d%16, kb*32 + (d//16)*8 + 0..7] contiguous.  The reference's
+    `shuffle_weight` (kittens_helpers.py:90-119) is the same idea for A fragments read with
+    two ds_read_b64 (K elements {4g..4g+3} and {16+4g..16+4g+3} per lane); this is the order
+    for ds_read_b128, which the HIP stream kernel with operand_path direct_b_k8 uses."""
+    N, K = B.shape
+    if N % 16 != 0:
+        raise AssertionError(f"N={N} must be multiple of 16")
+    if K % 32 != 0:
+        raise AssertionError(f"K={K} must be multiple of 32")
+    view = B.reshape(N // 16, 16, K // 32, 4, 8)
+    return np.ascontiguousarray(view.transpose(0, 2, 3, 1, 4)).reshape(N, K)
+
+
+def unshuffle_weight_k8(Bs: np.ndarray) -> np.ndarray:
+    """Inverse of `shuffle_weight_k8`."""
+    N, K = Bs.shape
+    view = Bs.reshape(N // 16, K // 32, 4, 16, 8)
+    return np.ascontiguousarray(view.transpose(0, 3, 1, 2, 4)).reshape(N, K)

@@ -24,9 +24,10 @@ import numpy as np
 from . import _capi
 from .execution import GpuBuffer
 from .gemm import GemmPlan
-from .kittens_helpers import shuffle_weight
+from .kittens_helpers import shuffle_weight, shuffle_weight_k8
 
-_LAYOUT_ID = {"lds": _capi.OPERAND_LDS, "direct_b": _capi.OPERAND_DIRECT_B}
+_LAYOUT_ID = {"lds": _capi.OPERAND_LDS, "direct_b": _capi.OPERAND_DIRECT_B,
+              "direct_b_k8": _capi.OPERAND_DIRECT_B_K8}
 _LAYOUT_NAME = {v: k for k, v in _LAYOUT_ID.items()}
 _DTYPE_NAME = {v: k for k, v in _capi.DTYPE_NAMES.items()}
 
@@ -95,7 +96,7 @@ class WeightArtifact:
     @classmethod
     def from_f32(cls, w: np.ndarray, dtype: str, *, layout: str = "lds") -> "WeightArtifact":
         """Pack an fp32 matrix W[N, K]: f16 / bf16 are rounded on the host (and pre-shuffled
-        for layout "direct_b"); fp8 and MXFP4 go through the GPU quantisers."""
+        for the layouts "direct_b" and "direct_b_k8"); fp8 and MXFP4 go through the GPU quantisers."""
         w = np.ascontiguousarray(w, dtype=np.float32)
         if w.ndim != 2:
             raise ValueError("from_f32: W must be [N, K]")
@@ -104,6 +105,8 @@ class WeightArtifact:
             bits = w.astype(np.float16).view(np.uint16) if dtype == "f16" else _bf16_bits(w)
             if layout == "direct_b":
                 bits = shuffle_weight(bits)
+            elif layout == "direct_b_k8":
+                bits = shuffle_weight_k8(bits)
             return cls.from_storage(bits, dtype, N, K, layout=layout)
         from . import quantize as Q
         if dtype == "fp8_e4m3":

@@ -82,9 +82,16 @@ typedef enum astergemm_kernel_family {
  * global load is its MFMA operand and B never passes through LDS.            */
 typedef enum astergemm_operand_path {
   ASTERGEMM_OPERAND_LDS = 0,      /* B[N, ldb] row-major as described below   */
-  ASTERGEMM_OPERAND_DIRECT_B = 1  /* B packed [N, K] and pre-shuffled with
-                                     astergemm_shuffle_weight_16 (16-bit
-                                     operands; skinny kernels only)          */
+  ASTERGEMM_OPERAND_DIRECT_B = 1, /* B packed [N, K] and pre-shuffled with
+                                     astergemm_shuffle_weight_16, the
+                                     reference's order (16-bit operands; the
+                                     decode kernels, M <= 16)                */
+  ASTERGEMM_OPERAND_DIRECT_B_K8 = 2 /* B packed [N, K] and pre-shuffled with
+                                     astergemm_shuffle_weight_k8_16: 8
+                                     consecutive K per lane, the order of the
+                                     16x16x32 MFMA and of 16-byte LDS reads
+                                     (16-bit operands; the 256 x 256 stream
+                                     kernel, N % 16 == 0, K % 64 == 0)       */
 } astergemm_operand_path;
 
 /* ---- problem + mapping --------------------------------------------------
@@ -236,6 +243,15 @@ int astergemm_tune(const astergemm_config* cfg, const astergemm_operands* ops, i
  * (reference: shuffle_weight, contrib/kittens/test/kittens_helpers.py:90-119). */
 int astergemm_shuffle_weight_16(const uint16_t* src, uint16_t* dst, int64_t N,
                                 int64_t K);
+/* The same pre-shuffle for the 16x16x32 MFMA of gfx950 read with 16-byte
+ * operand loads: chunk (nb, kb) of 1 KiB holds rows 16 nb .. + 15 and K
+ * elements 32 kb .. + 31, lane 16 g + n of a wave finds its eight consecutive
+ * K elements 32 kb + 8 g .. + 7 of row 16 nb + n at byte 16 (16 g + n).  The
+ * reference's shuffle_weight (kittens_helpers.py:90-119) pairs the K elements
+ * {4g..4g+3} and {16+4g..16+4g+3} instead, because its kernels read A with two
+ * ds_read_b64 (test_102_gemm_python_multitile_g2s_directb_cdna4.py:178-188). */
+int astergemm_shuffle_weight_k8_16(const uint16_t* src, uint16_t* dst, int64_t N,
+                                   int64_t K);
 
 /* ---- operand quantisers (device to device, on `stream`) -------------------
  * They write the bytes the fp8 / MXFP4 GEMM paths read (dtype_ab
@@ -284,8 +300,10 @@ int astergemm_quantize_mxfp4(const void* dSrc, int src_dtype, int64_t rows, int6
  *
  * File = this 128-byte little-endian header, then the payload at
  * payload_offset (N rows; layout ASTERGEMM_OPERAND_LDS = row-major,
- * ASTERGEMM_OPERAND_DIRECT_B = astergemm_shuffle_weight_16 order, 16-bit
- * dtypes only), then for MXFP4 the e8m0 plane [N, K/32] at scales_offset.
+ * ASTERGEMM_OPERAND_DIRECT_B = astergemm_shuffle_weight_16 order,
+ * ASTERGEMM_OPERAND_DIRECT_B_K8 = astergemm_shuffle_weight_k8_16 order, the
+ * pre-shuffled ones for 16-bit dtypes only), then for MXFP4 the e8m0 plane
+ * [N, K/32] at scales_offset.
  * Sections start on 256-byte boundaries.  FP8 carries its tensor scale in the
  * header.  Checksums are CRC-32 (the zlib polynomial) of each section.       */
 #define ASTERGEMM_WEIGHT_VERSION 1u

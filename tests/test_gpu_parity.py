@@ -7,6 +7,7 @@ same way); the reference's own bar `assert_allclose(rtol=1e-2, atol=1e-2)` on
 its own test shapes; bit-exact where the arithmetic is exact (known answers,
 power-of-two scaling, identity operand, run-to-run determinism).
 """
+import ctypes
 import json
 import os
 
@@ -28,12 +29,12 @@ _OUT_NP = {"f32": np.float32, "bf16": np.uint16, "f16": np.uint16}
 
 def run_gemm(a, b, M, N, K, dtype_ab, dtype_c, *, scale_a=None, scale_b=None, mx_a=None, mx_b=None,
              bias=None, lda=0, ldb=0, ldc=0, family=_capi.KERNEL_AUTO, wg_tile=(0, 0),
-             operand_path="lds"):
+             operand_path="lds", variant=0):
     """Upload, launch once through astergemm_run, download.  Returns the raw
     output storage [M, ldc or N] and the kernel name."""
     plan = AG.GemmPlan.create(M, N, K, dtype_ab, dtype_c, has_bias=bias is not None, lda=lda,
                               ldb=ldb, ldc=ldc, family=family, wg_tile=wg_tile,
-                              operand_path=operand_path)
+                              operand_path=operand_path, variant=variant)
     ldc_eff = ldc or N
     out = np.full((M, ldc_eff), 0x7FC1 if dtype_c != "f32" else np.nan, dtype=_OUT_NP[dtype_c])
     bufs = []
@@ -804,6 +805,41 @@ def test_config5_full_size_mxfp4_row_sample_determinism_and_scaling(gpu):
     assert np.array_equal(F.bf16_bits_to_f32(outx2), F.bf16_bits_to_f32(out) * 2.0)
 
 
+def _variant_id(name):
+    lib = _capi.load()
+    cfg, info = _capi.Config(), _capi.KernelInfo()
+    cfg.M = cfg.N = cfg.K = 512
+    for i in range(lib.astergemm_variant_count()):
+        _capi.check(lib.astergemm_variant_info(i, ctypes.byref(cfg), ctypes.byref(info)))
+        if info.name.decode() == name:
+            return info.variant
+    raise KeyError(name)
+
+
+@pytest.mark.parametrize("M,N", [(512, 32768 + 520), (33288, 512), (1024, 16384 + 264)])
+@pytest.mark.parametrize("dtype_ab,dtype_c,K", [("bf16", "bf16", 264), ("f16", "f32", 128),
+                                                ("fp8_e4m3", "bf16", 384), ("mxfp4", "bf16", 512)])
+def test_whole_rounds_plus_tail_split(gpu, M, N, dtype_ab, dtype_c, K):
+    # 256 x 256 tiles that do not fill whole rounds of the 256 CUs: the columns (rows) that do go
+    # to the 256 x 256 kernel, the rest to the 128 x 128 kernel; bias and scales follow the cut
+    a, b, ex = operands(M, N, K, dtype_ab, a_std=1.0, b_std=1.0 if dtype_ab != "bf16" else 0.02)
+    bias = np.random.default_rng(3).standard_normal(N).astype(np.float32)
+    out, name = run_gemm(a, b, M, N, K, dtype_ab, dtype_c, bias=bias, wg_tile=(256, 256), **ex)
+    assert "tail128" in name, name
+    want = G.gemm(a, b, _DT[dtype_ab], _DT[dtype_c], bias=bias, **ex)
+    check(out, want, dtype_c, N)
+    # the same bits as the two kernels give when each runs the whole problem
+    plain = name.replace("_tail128", "")
+    waves = plain.split("_")[3]
+    for vname, rows, cols in ((plain, slice(0, 256), slice(0, 256)),
+                              (plain.replace("256x256_" + waves, "128x128_w2x2"),
+                               slice(M - 128, M), slice(N - 128, N))):
+        whole, wname = run_gemm(a, b, M, N, K, dtype_ab, dtype_c, bias=bias,
+                                variant=_variant_id(vname), **ex)
+        assert wname == vname
+        assert np.array_equal(out[rows, cols], whole[rows, cols])
+
+
 def test_identity_operand_is_exact_at_full_width(gpu):
     # B = I: every output is one product plus zeros, so C == A bit for bit.
     M, N = 512, 8192
@@ -839,13 +875,19 @@ def test_every_tile_variant(gpu, vid, name, dtype_ab, dtype_c):
     M, N, K = 512, 768, 1536  # whole 256-tiles; 24 / 12 / 6 K-steps of 128 bytes (16-bit / fp8 / fp4)
     if name.startswith("splitk"):
         K = {"fp8_e4m3": 8192, "mxfp4": 8192}.get(dtype_ab, 4096)  # 64 (MXFP4: 32) steps of 128 bytes
+    if "tail128" in name:
+        M, N, K = 512, 32768 + 256, 512  # 2 x 129 tiles of 256 x 256: one whole round and a rest
     a, b, ex = operands(M, N, K, dtype_ab, seed=11, a_std=1.0, b_std=1.0 if dtype_ab != "bf16" else 0.05)
     bias = np.random.default_rng(12).standard_normal(N).astype(np.float32)
-    plan = AG.GemmPlan.create(M, N, K, dtype_ab, dtype_c, has_bias=True, variant=vid)
+    path, b_dev = "lds", b
+    if name.startswith("streamdb"):  # B pre-shuffled in K8 order
+        from aster_amd.kittens_helpers import shuffle_weight_k8
+        path, b_dev = "direct_b_k8", shuffle_weight_k8(np.ascontiguousarray(b).view(np.uint16))
+    plan = AG.GemmPlan.create(M, N, K, dtype_ab, dtype_c, has_bias=True, variant=vid, operand_path=path)
     assert plan.info.name.decode() == name
     out = np.zeros((M, N), dtype=_OUT_NP[dtype_c])
     bufs = {}
-    for key, arr in dict(a=a, b=b, c=out, bias=bias, **{k: np.asarray(v) for k, v in ex.items()}).items():
+    for key, arr in dict(a=a, b=b_dev, c=out, bias=bias, **{k: np.asarray(v) for k, v in ex.items()}).items():
         arr = np.ascontiguousarray(arr if arr.ndim else arr.reshape(1).astype(np.float32))
         bufs[key] = GpuBuffer(arr.nbytes)
         bufs[key].copy_from_host(arr)
@@ -968,6 +1010,24 @@ def test_mxfp4_stream_kernel_every_loop_phase(gpu, ksteps, tile):
     check(out, G.gemm_mxfp4(a, mxa, b, mxb, out_dtype=G.F32), "f32", N, bar=1e-5)
 
 
+@pytest.mark.parametrize("ksteps", [2, 4, 6, 8, 10, 12, 14])
+@pytest.mark.parametrize("dtype_c", ["f32", "bf16"])
+def test_mxfp4_stream_kernel_eight_waves_every_loop_phase(gpu, ksteps, dtype_c):
+    # the 256 x 256 kernel with 2 x 4 waves (wave tile 128 x 64): same loop phases, an edge tile
+    # in M and N, random nibbles and per-block scales
+    M, N, K = 264, 520, 256 * ksteps
+    rng = np.random.default_rng(61 + ksteps)
+    a = rng.integers(0, 256, (M, K // 2)).astype(np.uint8)
+    b = rng.integers(0, 256, (N, K // 2)).astype(np.uint8)
+    mxa = rng.integers(118, 134, (M, K // 32)).astype(np.uint8)
+    mxb = rng.integers(118, 134, (N, K // 32)).astype(np.uint8)
+    out, name = run_gemm(a, b, M, N, K, "mxfp4", dtype_c, mx_a=mxa, mx_b=mxb,
+                         variant=_variant_id(f"stream_mxfp4_256x256_w2x4_{dtype_c}"))
+    assert name == f"stream_mxfp4_256x256_w2x4_{dtype_c}"
+    want = G.gemm_mxfp4(a, mxa, b, mxb, out_dtype=_DT[dtype_c])
+    check(out, want, dtype_c, N, bar=1e-5 if dtype_c == "f32" else REL_L2_BAR)
+
+
 def test_mxfp4_stream_kernel_falls_back_for_odd_kstep_counts(gpu):
     assert AG.GemmPlan.create(512, 512, 768, "mxfp4", "bf16", wg_tile=(256, 256)).info.name.decode() \
         .startswith("tile_mxfp4")
@@ -994,6 +1054,55 @@ def test_skinny_direct_b_preshuffled_weights(gpu, M, N, K, dtype_ab, dtype_c):
     check(out, want, dtype_c, N, bar=1e-5 if dtype_c == "f32" else REL_L2_BAR)
     pad = out[:, N:]
     assert np.isnan(pad).all() if dtype_c == "f32" else (pad == 0x7FC1).all()
+
+
+# ---- B pre-shuffled in K8 order, loaded straight into MFMA operands (256 x 256 stream kernel) ---
+
+@pytest.mark.parametrize("M,N,K", [(256, 256, 64), (256, 256, 128), (512, 768, 576), (512, 512, 640),
+                                   (264, 528, 704), (1000, 1008, 896), (256, 512, 960),
+                                   (512, 256, 1280), (768, 1024, 1472), (2048, 2048, 4096)])
+@pytest.mark.parametrize("dtype_ab,dtype_c", [("bf16", "bf16"), ("f16", "f32")])
+def test_stream_direct_b_k8(gpu, M, N, K, dtype_ab, dtype_c):
+    # K steps of 64 elements: 1, 2, 9 (no steady group), 10 (one steady group exactly), 11, 14, 15,
+    # 20, 23, 64; edge tiles in M (multiple of 8) and N (multiple of 16)
+    from aster_amd.kittens_helpers import shuffle_weight_k8
+    a, b, _ = operands(M, N, K, dtype_ab)
+    bias = np.random.default_rng(4).standard_normal(N).astype(np.float32)
+    out, name = run_gemm(a, shuffle_weight_k8(b), M, N, K, dtype_ab, dtype_c, bias=bias,
+                         operand_path="direct_b_k8")
+    assert name.startswith("streamdb_")
+    check(out, G.gemm(a, b, _DT[dtype_ab], _DT[dtype_c], bias=bias), dtype_c, N)
+    # the same K order on both operands as the LDS kernel: same products, same sums
+    lds_out, lds_name = run_gemm(a, b, M, N, K, dtype_ab, dtype_c, bias=bias, wg_tile=(256, 256),
+                                 family=_capi.KERNEL_TILE)
+    if lds_name.startswith("stream_"):
+        assert G.rel_l2(G.output_to_f32(out, _DT[dtype_c]), G.output_to_f32(lds_out, _DT[dtype_c])) <= 1e-5
+
+
+def test_stream_direct_b_k8_full_size_row_sample(gpu, big):
+    from aster_amd.kittens_helpers import shuffle_weight_k8
+    M, N, K, a, b = big
+    out, name = run_gemm(a, shuffle_weight_k8(b), M, N, K, "bf16", "bf16", operand_path="direct_b_k8")
+    assert name == "streamdb_bf16_256x256_w2x4_bf16"
+    rows, cols = _sampled_rows_and_cols(M, N)
+    check(out[rows], G.gemm(a[rows], b, G.BF16, G.BF16), "bf16", N)
+    check(out[:, cols], G.gemm(a, b[cols], G.BF16, G.BF16), "bf16", len(cols))
+    out2, _ = run_gemm(a, shuffle_weight_k8(b), M, N, K, "bf16", "bf16", operand_path="direct_b_k8")
+    assert np.array_equal(out, out2)
+
+
+def test_direct_b_mapping_through_the_harness_seam(gpu, tmp_path):
+    # a DIRECT_B mapping on a compute-bound shape: compile_gemm selects the kernel that reads
+    # pre-shuffled B, execute_gemm_hsaco shuffles the row-major B it is given in that kernel's order
+    cfg = make_instance(512, 768, 640, operand_path=OperandPath.DIRECT_B)
+    path, asm = AG.compile_gemm(cfg, str(tmp_path / "k.hsaco"))
+    desc = json.load(open(path))
+    assert desc["kernel"].startswith("streamdb_") and desc["operand_path"] == "direct_b_k8"
+    assert desc["mapping_honoured"] is True
+    a, b, _ = operands(512, 768, 640, "bf16")
+    c_flat, times = AG.execute_gemm_hsaco(cfg, path, 3, a, b)
+    assert len(times) == 3
+    check(c_flat.reshape(512, 768), G.gemm(a, b, G.BF16, G.BF16), "bf16", 768)
 
 
 def test_direct_b_is_refused_where_it_is_not_implemented(gpu):

@@ -115,6 +115,31 @@ def test_shuffle_weight(N, K):
     assert np.array_equal(out, S)
 
 
+def test_shuffle_weight_k8_is_the_16x16x32_operand_order():
+    from aster_amd.kittens_helpers import shuffle_weight_k8, unshuffle_weight_k8
+    N, K = 48, 128
+    B = np.arange(N * K, dtype=np.uint16).reshape(N, K)
+    S = shuffle_weight_k8(B)
+    assert np.array_equal(np.sort(S.reshape(-1)), B.reshape(-1))
+    assert np.array_equal(unshuffle_weight_k8(S), B)
+    # lane d of block (nb, kb) reads 8 contiguous elements = B[nb*16 + d%16, kb*32 + (d//16)*8 + 0..7]:
+    # the K positions lane d of a wave feeds to v_mfma_f32_16x16x32 (k = 8 * (lane / 16) .. + 7,
+    # the 16-bit form of the reference's fp8 fragment map, indexing.mlir:202-218)
+    flat = S.reshape(-1)
+    for nb in range(N // 16):
+        for kb in range(K // 32):
+            for d in range(64):
+                base = (nb * (K // 32) + kb) * 512 + d * 8
+                want = B[nb * 16 + d % 16, kb * 32 + (d // 16) * 8:][:8]
+                assert np.array_equal(flat[base: base + 8], want)
+    out = np.empty_like(B)
+    _capi.check(_capi.load().astergemm_shuffle_weight_k8_16(B.ctypes.data, out.ctypes.data, N, K))
+    assert np.array_equal(out, S)
+    # it differs from the reference's order exactly in the K pairing inside a 32-wide block
+    assert not np.array_equal(S, shuffle_weight(B))
+    assert _capi.load().astergemm_shuffle_weight_k8_16(B.ctypes.data, out.ctypes.data, 15, 32) == -22
+
+
 def test_shuffle_weight_rejects_bad_shapes():
     with pytest.raises(AssertionError):
         shuffle_weight(np.zeros((15, 32), np.float16))

@@ -127,6 +127,7 @@ def test_packing_rules():
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype,layout,M,N,K", [("bf16", "lds", 16, 512, 4096), ("bf16", "direct_b", 16, 512, 4096),
+                                                ("bf16", "direct_b_k8", 264, 512, 1024),
                                                 ("f16", "lds", 40, 264, 256), ("fp8_e4m3", "lds", 16, 512, 4096),
                                                 ("fp8_e4m3", "lds", 300, 256, 512), ("mxfp4", "lds", 64, 256, 1024)])
 def test_artifact_to_gemm_matches_the_oracle(tmp_path, dtype, layout, M, N, K):
@@ -171,5 +172,7 @@ def test_artifact_to_gemm_matches_the_oracle(tmp_path, dtype, layout, M, N, K):
     d_out.copy_to_host(out)
     if layout == "direct_b":
         assert dev.plan(M, "f32").info.name.decode().startswith("skinnyd")
+    if layout == "direct_b_k8":
+        assert dev.plan(M, "f32").info.name.decode().startswith("streamdb")
     assert G.rel_l2(out, G.output_to_f32(want, G.F32)) <= bar
     dev.free()
