@@ -137,13 +137,13 @@ const Variant* choose(const astergemm_config& c, int* index_out) {
                ((c.K % 512 == 0 && c.K <= 16 * 4096) || (c.K % 8192 == 0 && c.K <= 16 * 8192))))
                  ? ASTERGEMM_KERNEL_SKINNY
                  : ASTERGEMM_KERNEL_TILE;
-  // 32 < M <= 64 on rows the decode kernels cut into K ranges: their paired workgroups are
-  // behind split K on the 128 x 128 kernel where that is available (cold weights, bf16
-  // 64x4096x14336: 39.0 against 34.1 us, 64x8192x28672: 131 against 93; fp8 only from 28 KiB
-  // rows on: 71 against 60 us, level below that); for M <= 32 they stay ahead (28.7 against 32.3)
+  // 32 < M <= 64 on rows of more than 32 KiB: the decode kernel's K ranges of 4 KiB leave more
+  // partial sums than split K on the 128 x 128 kernel (bf16 64x8192x28672: 107 against 94 us;
+  // 64x4096x28672 level at 57.5 against 58.5); up to 32 KiB the decode kernel is ahead
+  // (64x8192x16384: 60 against 81 us, 64x14336x8192: 53 against 63, fp8 64x8192x28672: 56
+  // against 60)
   if (c.family == ASTERGEMM_KERNEL_AUTO && family == ASTERGEMM_KERNEL_SKINNY && c.M > 32 &&
-      ((is16 && row_bytes(c.dtype_ab, c.K) > 8192) ||
-       (c.dtype_ab == ASTERGEMM_FP8_E4M3 && row_bytes(c.dtype_ab, c.K) >= 28672))) {
+      (is16 || c.dtype_ab == ASTERGEMM_FP8_E4M3) && row_bytes(c.dtype_ab, c.K) > 32768) {
     for (int i = 0; i < total_variants(); ++i) {
       const Variant* v = variant_at(i);
       if (v->family == ASTERGEMM_KERNEL_TILE && v->rank == 4 && variant_matches_types(*v, c) &&

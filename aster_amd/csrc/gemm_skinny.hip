@@ -752,15 +752,15 @@ int splitk_workspace(size_t bytes, hipStream_t stream, float** out) {
   return 0;
 }
 
-// Grid of the K-range decode kernels: S K ranges x R row ranges, one workgroup per CU; above 32
-// activation rows two workgroups (MH = 2) share a row range, in whole pairs on each of the 8
-// XCDs.  The launchers and the description of a variant both come here.
+// Grid of the K-range decode kernels: S K ranges x R row ranges, one workgroup per CU; with
+// mh = 2 two workgroups share a row range, in whole pairs on each of the 8 XCDs.  The launchers
+// and the description of a variant both come here.
 struct KRangeGrid {
   int mh, rows, grid;
 };
-inline KRangeGrid krange_grid(int64_t M, int64_t N, int S, int cus) {
+inline KRangeGrid krange_grid(int mh, int64_t N, int S, int cus) {
   KRangeGrid g;
-  g.mh = M > 32 ? 2 : 1;
+  g.mh = mh;
   const int nblocks = (int)((N + 15) / 16);
   const int slots = g.mh == 2 ? (cus / 16) * 8 : cus;
   int R = slots / S;
@@ -1027,8 +1027,7 @@ int launch_skinny_fp4m_t(const GemmArgs& a0, int S, hipStream_t s) {
   const int cus = device_cus();
   if (cus <= 0) return (int)hipErrorNoDevice;
   GemmArgs a = a0;
-  const KRangeGrid kg = krange_grid(a.M, a.N, S, cus);
-  if (kg.mh != MH) return (int)hipErrorInvalidValue;
+  const KRangeGrid kg = krange_grid(MH, a.N, S, cus);
   a.tiles_n = kg.rows;
   a.split_k = S;
   if (S > 1 && !a.workspace) {
@@ -1070,7 +1069,7 @@ int splits_skinny_fp4m(const astergemm_config& c) {
   return S < 1 ? 1 : S;
 }
 int grid_skinny_fp4m(const astergemm_config& c, int cus) {
-  return krange_grid(c.M, c.N, splits_skinny_fp4m(c), cus).grid;
+  return krange_grid(c.M > 32 ? 2 : 1, c.N, splits_skinny_fp4m(c), cus).grid;
 }
 
 #define AG_SKINNY_FP4M(name, OUT)                                                          \
@@ -1088,9 +1087,15 @@ int grid_skinny_fp4m(const astergemm_config& c, int cus) {
 // so 32 rows is the limit (64 rows x 8 KB would be the whole register file of the CU).
 // Every weight operand read back from the wave's LDS buffer feeds MT MFMAs; the partial
 // tiles of a row block are reduced after every block, tile mt by wave mt.
-// M > 32 (MH = 2): two workgroups on the same XCD (block ids 8 apart) take the same weight
-// rows and one half of the activation rows each.  They run side by side, so the second
-// read of a weight line is served by that XCD's L2 and HBM still sees every line once.
+// M > 32 has two forms.  Rows of exactly 8 KiB (and rows of more than 64 KiB): MH = 2, two
+// workgroups on the same XCD (block ids 8 apart) take the same weight rows and one half of the
+// activation rows each, the second read of a weight line served by that XCD's L2 (bf16 64 x
+// 14336 x 4096: 29.5 us).  Other rows take four activation tiles per wave (MT = 4) on K ranges
+// of 4 KiB (SPB = 4: the same 128 operand registers): one workgroup covers all 64 rows and
+// every weight byte is fetched once and multiplied four times (64 x 14336 x 8192: 52 us
+// against 63 for split K on the tile kernel); a 4 KiB row is a single range.  On an 8 KiB row
+// that form would pay for a workspace pass the paired form does not need (33.0 against
+// 29.5 us).
 template <int DT, int OUT, int SPB, int MT, int MH>
 __global__ __launch_bounds__(512) void gemm_skinny_regm_kernel(const GemmArgs p) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t slds[];
@@ -1101,7 +1106,7 @@ __global__ __launch_bounds__(512) void gemm_skinny_regm_kernel(const GemmArgs p)
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int li = lane & 15, lq = lane >> 4;
   uint8_t* tbuf = slds + wave * 8192;            // 4 steps x 2 KiB, private to the wave
-  constexpr int NBS = 2;                         // blocks between workgroup barriers
+  constexpr int NBS = MT >= 4 ? 1 : 2;           // blocks between workgroup barriers (NBS * MT <= 8)
   f32x4* red = (f32x4*)(slds + KW * 8192);       // [2][NBS][MT][KW][64]
 
   // block b runs on XCD b % 8; with MH = 2 blocks b and b + 8 share a row range.
@@ -1325,17 +1330,37 @@ __host__ inline int skinny_split_of(int64_t rb, int* spb) {
   return 0;
 }
 
+// How the decode kernel of up to 64 rows runs a problem: K ranges, steps per wave and range,
+// activation tiles per wave, workgroups per row range.  Shared by the launcher, the workspace
+// size and the reported grid.
+struct RegmPlan {
+  int S = 0, spb = 0, mt = 0, mh = 0;
+};
+inline RegmPlan regm_plan_of(int64_t M, int64_t rb) {
+  RegmPlan r;
+  int spb = 0;
+  const int S = skinny_split_of(rb, &spb);
+  if (S == 0) return r;
+  if (M > 32 && rb != 8192 && rb % 512 == 0 && (rb + 4095) / 4096 <= 16) {
+    r.S = (int)((rb + 4095) / 4096), r.spb = 4, r.mt = 4, r.mh = 1;
+    return r;
+  }
+  r.S = S, r.spb = spb;
+  r.mt = (M <= 16 && S > 1) ? 1 : 2;
+  r.mh = M > 32 ? 2 : 1;
+  return r;
+}
+
 template <int DT, int OUT, int SPB, int MT, int MH>
 int launch_skinny_regm_t(const GemmArgs& a0, int S, hipStream_t s) {
   auto k = gemm_skinny_regm_kernel<DT, OUT, SPB, MT, MH>;
-  constexpr int lds = 8 * 8192 + 2 * 2 * MT * 8 * 64 * 16;
+  constexpr int lds = 8 * 8192 + 2 * (MT >= 4 ? 1 : 2) * MT * 8 * 64 * 16;
   static std::atomic<uint64_t> attr_devs{0};
   if (int e = lds_attr_once(attr_devs, (const void*)k, lds)) return e;
   const int cus = device_cus();
   if (cus <= 0) return (int)hipErrorNoDevice;
   GemmArgs a = a0;
-  const KRangeGrid kg = krange_grid(a.M, a.N, S, cus);
-  if (kg.mh != MH) return (int)hipErrorInvalidValue;
+  const KRangeGrid kg = krange_grid(MH, a.N, S, cus);
   a.tiles_n = kg.rows;
   a.split_k = S;
   if (S > 1 && !a.workspace) {
@@ -1349,17 +1374,17 @@ int launch_skinny_regm_t(const GemmArgs& a0, int S, hipStream_t s) {
 template <int DT, int OUT>
 int launch_skinny_regm(const GemmArgs& a, int grid, hipStream_t s) {
   (void)grid;
-  int spb = 0;
-  const int S = skinny_split_of(row_bytes(DT, a.K), &spb);
-  if (S == 0) return (int)hipErrorInvalidValue;
-  if (a.M <= 16 && S > 1)
-    return spb == 8 ? launch_skinny_regm_t<DT, OUT, 8, 1, 1>(a, S, s)
-                    : launch_skinny_regm_t<DT, OUT, 4, 1, 1>(a, S, s);
-  if (a.M <= 32)
-    return spb == 8 ? launch_skinny_regm_t<DT, OUT, 8, 2, 1>(a, S, s)
-                    : launch_skinny_regm_t<DT, OUT, 4, 2, 1>(a, S, s);
-  return spb == 8 ? launch_skinny_regm_t<DT, OUT, 8, 2, 2>(a, S, s)
-                  : launch_skinny_regm_t<DT, OUT, 4, 2, 2>(a, S, s);
+  const RegmPlan r = regm_plan_of(a.M, row_bytes(DT, a.K));
+  if (r.S == 0) return (int)hipErrorInvalidValue;
+  if (r.mt == 4) return launch_skinny_regm_t<DT, OUT, 4, 4, 1>(a, r.S, s);
+  if (r.mt == 1)
+    return r.spb == 8 ? launch_skinny_regm_t<DT, OUT, 8, 1, 1>(a, r.S, s)
+                      : launch_skinny_regm_t<DT, OUT, 4, 1, 1>(a, r.S, s);
+  if (r.mh == 1)
+    return r.spb == 8 ? launch_skinny_regm_t<DT, OUT, 8, 2, 1>(a, r.S, s)
+                      : launch_skinny_regm_t<DT, OUT, 4, 2, 1>(a, r.S, s);
+  return r.spb == 8 ? launch_skinny_regm_t<DT, OUT, 8, 2, 2>(a, r.S, s)
+                    : launch_skinny_regm_t<DT, OUT, 4, 2, 2>(a, r.S, s);
 }
 
 const char* check_skinny_regm(const astergemm_config& c) {
@@ -1375,12 +1400,12 @@ const char* check_skinny_regm(const astergemm_config& c) {
 }
 
 int splits_skinny_regm(const astergemm_config& c) {
-  int spb = 0;
-  const int S = skinny_split_of(row_bytes(c.dtype_ab, c.K), &spb);
-  return S < 1 ? 1 : S;
+  const RegmPlan r = regm_plan_of(c.M, row_bytes(c.dtype_ab, c.K));
+  return r.S < 1 ? 1 : r.S;
 }
 int grid_skinny_regm(const astergemm_config& c, int cus) {
-  return krange_grid(c.M, c.N, splits_skinny_regm(c), cus).grid;
+  const RegmPlan r = regm_plan_of(c.M, row_bytes(c.dtype_ab, c.K));
+  return krange_grid(r.mh < 1 ? 1 : r.mh, c.N, r.S < 1 ? 1 : r.S, cus).grid;
 }
 
 #define AG_SKINNY_LDSM(name, DT, OUT)                                                      \

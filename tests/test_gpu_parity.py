@@ -244,8 +244,9 @@ def test_skinny_resident_activations(gpu, M, N, K, dtype_ab, dtype_c):
                                    (50, 24, 4096), (64, 14337, 2048), (48, 4104, 4096), (64, 136, 4096)])
 @pytest.mark.parametrize("dtype_ab,dtype_c", [("bf16", "f32"), ("f16", "f16"), ("bf16", "bf16")])
 def test_skinny_resident_activations_up_to_64_rows(gpu, M, N, K, dtype_ab, dtype_c):
-    """16 < M <= 64 with K in {2048, 4096}: two activation tiles per wave, and above 32 rows
-    two workgroups per row range (one half of the activation rows each)."""
+    """16 < M <= 64 with K in {2048, 4096}: two activation tiles per wave; above 32 rows four
+    tiles per wave on 4 KiB rows, and two workgroups per row range (one half of the activation
+    rows each) on 8 KiB rows."""
     a, b, _ = operands(M, N, K, dtype_ab, seed=61, b_std=0.05)
     bias = np.random.default_rng(62).standard_normal(N).astype(np.float32)
     ldc = (N + 11) & ~3
@@ -260,7 +261,7 @@ def test_skinny_resident_activations_up_to_64_rows(gpu, M, N, K, dtype_ab, dtype
 @pytest.mark.parametrize("M,N,K", [(16, 4096, 14336), (1, 8, 6144), (33, 777, 14336), (64, 4096, 14336),
                                    (16, 1000, 28672), (64, 24, 10240), (7, 4104, 32768), (40, 2050, 12288),
                                    (16, 4096, 11008), (16, 5120, 13824), (33, 100, 2304), (64, 520, 6400),
-                                   (5, 64, 3840)])
+                                   (5, 64, 3840), (40, 136, 40960), (64, 520, 8192)])
 @pytest.mark.parametrize("dtype_ab,dtype_c", [("bf16", "f32"), ("f16", "f16"), ("bf16", "bf16")])
 def test_skinny_resident_activations_long_rows(gpu, M, N, K, dtype_ab, dtype_c):
     """Rows that are not 4 or 8 KiB (down-projections): the persistent kernel runs one K range
@@ -575,14 +576,16 @@ def test_split_k_fp8_and_mxfp4(gpu, M, N, K, dtype_ab, dtype_c):
 
 def test_long_rows_above_32_activation_rows_take_split_k(gpu):
     """AUTO on rows the decode kernels cut into K ranges: M <= 32 stays with them, 32 < M <= 64
-    goes to split K on the 128 x 128 kernel where the shape allows it (N % 8 == 0)."""
-    for (M, N, K, dt, want) in ((32, 4096, 14336, "bf16", "skinnyx_bf16_m64"),
-                                (48, 4096, 14336, "bf16", "splitk_bf16"),
-                                (64, 4096, 14336, "f16", "splitk_f16"),
-                                (64, 4100, 14336, "bf16", "skinnyx_bf16_m64"),
+    goes to split K on the 128 x 128 kernel for rows of more than 32 KiB where the shape allows
+    it (N % 8 == 0)."""
+    for (M, N, K, dt, want) in ((32, 4096, 28672, "bf16", "skinnyx_bf16_m64"),
+                                (48, 4096, 14336, "bf16", "skinnyx_bf16_m64"),
+                                (48, 4096, 28672, "bf16", "splitk_bf16"),
+                                (64, 4096, 20480, "f16", "splitk_f16"),
+                                (64, 4100, 28672, "bf16", "skinnyx_bf16_m64"),
                                 (64, 14336, 4096, "bf16", "skinnyx_bf16_m64"),
-                                (64, 4096, 14336, "fp8_e4m3", "skinnyx_fp8_m64"),
-                                (64, 4096, 28672, "fp8_e4m3", "splitk_fp8")):
+                                (64, 4096, 28672, "fp8_e4m3", "skinnyx_fp8_m64"),
+                                (64, 4096, 40960, "fp8_e4m3", "splitk_fp8")):
         a, b, extra = operands(M, N, K, dt, seed=93, b_std=0.05)
         out, name = run_gemm(a, b, M, N, K, dt, "f32", **extra)
         assert name.startswith(want), (M, N, K, dt, name)

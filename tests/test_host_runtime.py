@@ -232,18 +232,22 @@ def test_workspace_query_and_caller_workspace_checks():
 def test_reported_grid_is_the_launched_grid_of_the_k_range_kernels():
     # S K ranges x R row ranges, one workgroup per CU: the description comes from the same
     # function the launcher uses (the number of CUs is 0 without a device: one row range)
-    def krange_grid(M, N, S, cus):
-        mh = 2 if M > 32 else 1
+    def krange_grid(mh, N, S, cus):
         slots = (cus // 16) * 8 if mh == 2 else cus
         rows = min(max(slots // S, 1), (N + 15) // 16)
         g = mh * S * rows
         return (g + 15) // 16 * 16 if mh == 2 else g
 
-    for (M, N, K, S) in ((16, 4096, 14336, 7), (16, 4096, 28672, 7), (64, 4096, 14336, 7),
-                         (16, 8192, 28672, 7)):
+    # (M, N, K, K ranges, workgroups per row range): over 32 rows one workgroup covers all
+    # activation rows (four tiles per wave on 4 KiB ranges) except on rows of exactly 8 KiB or of
+    # more than 16 such ranges, which keep two workgroups per row range
+    for (M, N, K, S, mh) in ((16, 4096, 14336, 7, 1), (16, 4096, 28672, 7, 1), (64, 4096, 14336, 7, 1),
+                             (16, 8192, 28672, 7, 1), (64, 14336, 4096, 1, 2), (33, 520, 2048, 1, 1),
+                             (64, 14336, 8192, 4, 1), (64, 512, 3072, 2, 1), (64, 4096, 40960, 10, 2)):
         p = gemm.GemmPlan.create(M, N, K, family=_capi.KERNEL_SKINNY)
-        assert p.workspace_bytes() == S * M * N * 4
-        assert p.info.grid_x == krange_grid(M, N, S, cus=0)
+        assert p.info.name.decode().startswith("skinnyx_bf16_m64")
+        assert p.workspace_bytes() == (S * M * N * 4 if S > 1 else 0)
+        assert p.info.grid_x == krange_grid(mh, N, S, cus=0)
 
 
 def test_runtime_seam_function_free_and_cluster_launch():
