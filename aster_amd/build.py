@@ -10,6 +10,7 @@ tree.  `python -m aster_amd.build` rebuilds it.
 from __future__ import annotations
 
 import os
+import re
 import subprocess
 import sys
 from concurrent.futures import ThreadPoolExecutor
@@ -44,12 +45,103 @@ COMMON_FLAGS = [
 
 
 def _compile(src: str) -> str:
-    obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
-    cmd = [HIPCC, *COMMON_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    """Compile one source; the device assembly is kept beside the object and checked for the
+    hazard `scan_mfma_hazards` describes."""
+    stem = os.path.splitext(src)[0]
+    obj = os.path.join(OBJ_DIR, stem + ".o")
+    cmd = [HIPCC, *COMMON_FLAGS, "-save-temps=obj", "-c", os.path.join(CSRC, src), "-o", obj]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError(f"hipcc failed on {src}:\n{proc.stdout}\n{proc.stderr}")
+    asm = os.path.join(OBJ_DIR, stem + "-hip-amdgcn-amd-amdhsa-gfx950.s")
+    if not os.path.exists(asm):
+        raise RuntimeError(f"hipcc left no device assembly for {src} (expected {asm})")
+    with open(asm) as f:
+        found = scan_mfma_hazards(f.read())
+    for name in os.listdir(OBJ_DIR):  # the other intermediates are large and of no use
+        if name.startswith(stem + "-") and name.endswith((".hipi", ".bc", ".out", ".resolution.txt")):
+            os.remove(os.path.join(OBJ_DIR, name))
+    if found:
+        lines = "\n".join(f"  {asm}:{no}: {mfma}\n      written at line {wno}: {writer}"
+                          for (no, mfma, wno, writer) in found[:20])
+        raise RuntimeError(f"{src}: {len(found)} inline-asm MFMA(s) read a register a VALU instruction "
+                           f"wrote fewer than {MFMA_WAIT_STATES} wait states earlier:\n{lines}")
     return obj
+
+
+# ---- a hazard the compiler cannot see -----------------------------------------------------
+#
+# The stream kernels write some MFMAs as inline asm (to tie the accumulator to the accumulation
+# registers).  The compiler's hazard recogniser does not look inside inline asm: where register
+# allocation places a copy (v_mov, v_accvgpr_mov, v_and ...) into a source register right in front
+# of such an MFMA, it inserts no wait states and the MFMA reads the register before the copy has
+# landed: wrong sums, no error (seen on gfx950 with one v_mov_b64 directly in front of a
+# v_mfma_scale_f32_16x16x128_f8f6f4).  The kernels keep such copies out of their K loops and put
+# `s_nop 1` in front of the MFMAs elsewhere; this scan of the generated assembly is the proof.
+
+MFMA_WAIT_STATES = 2
+
+_REG_RANGE = re.compile(r"([va])\[(\d+):(\d+)\]$")
+_REG_ONE = re.compile(r"([va])(\d+)$")
+
+
+def _regs(tok: str) -> set:
+    tok = tok.strip().rstrip(",")
+    m = _REG_RANGE.match(tok)
+    if m:
+        return {(m.group(1), i) for i in range(int(m.group(2)), int(m.group(3)) + 1)}
+    m = _REG_ONE.match(tok)
+    return {(m.group(1), int(m.group(2)))} if m else set()
+
+
+def scan_mfma_hazards(asm_text: str, wait_states: int = MFMA_WAIT_STATES):
+    """[(line, mfma text, writer line, writer text)] for every MFMA inside an inline-asm block of
+    gfx9 assembly text whose A, B, C or scale registers were written by a VALU instruction fewer
+    than `wait_states` wait states earlier (an instruction is one wait state, `s_nop n` is n + 1)."""
+    found = []
+    hist = []      # (wait states, registers written by a VALU instruction, text, line)
+    in_asm = False
+    for no, raw in enumerate(asm_text.split("\n"), 1):
+        l = raw.strip()
+        if l.startswith(";;#ASMSTART"):
+            in_asm = True
+            continue
+        if l.startswith(";;#ASMEND"):
+            in_asm = False
+            continue
+        if not l or l[0] in ";." :
+            continue
+        if l.endswith(":"):
+            if not l.startswith(".L"):
+                hist = []          # a new function
+            continue
+        op = l.split()[0]
+        args = l[len(op):].split(";")[0]
+        toks = [t for t in re.split(r",\s*", args.strip()) if t]
+        if op.startswith("v_mfma") or op.startswith("v_smfmac"):
+            if in_asm:
+                srcs = set()
+                for t in toks[1:]:
+                    if t.split():
+                        srcs |= _regs(t.split()[0])
+                ws = 0
+                for (w, written, text, wno) in reversed(hist):
+                    if ws >= wait_states:
+                        break
+                    if written & srcs:
+                        found.append((no, l[:110], wno, text[:90]))
+                    ws += w
+            hist.append((1, set(), l, no))
+        else:
+            w, written = 1, set()
+            if op == "s_nop":
+                w = int(toks[0], 0) + 1 if toks else 1
+            elif op.startswith("v_") and not op.startswith(("v_cmp", "v_readlane", "v_readfirstlane")):
+                written = _regs(toks[0]) if toks else set()
+            hist.append((w, written, l, no))
+        if len(hist) > 8:
+            hist.pop(0)
+    return found
 
 
 def _genco(src: str) -> str:

@@ -212,6 +212,51 @@ const char* check_stream4(const astergemm_config& c) {
         (const void*)gemm_stream4_kernel<DT, OUT, 256, 256, 2, 4>,               \
         launch_stream4<DT, OUT, 256, 256, 2, 4>, check_stream4                   \
   }
+// Tile walk: one workgroup per CU takes its tiles round-robin as one long K loop, the next
+// tile's first K-steps arriving during the last trips and the epilogue of the current one
+// (see gemm_stream4_body).  16 KiB of LDS outside the ring stage the epilogue.
+template <int DT, int OUT>
+int launch_stream4_walk(const GemmArgs& a, int grid, hipStream_t s) {
+  (void)grid;
+  constexpr int lds = 4 * 256 * kRowBytes + 4 * 256 * 16 + 8 * 2048;
+  if ((((uintptr_t)a.mx_a | (uintptr_t)a.mx_b) & 15) != 0 || a.mx_ld % 16 != 0)
+    return (int)hipErrorInvalidValue;
+  // what the kernel assumes: slot parities that carry over from tile to tile, and whole tiles
+  // (its epilogue stores without bounds checks)
+  if (a.ksteps % 4 != 0 || a.M % 256 != 0 || a.N % 256 != 0) return (int)hipErrorInvalidValue;
+  auto k = gemm_stream4_walk_kernel<DT, OUT, 256, 256, 2, 4>;
+  static std::atomic<uint64_t> attr_devs{0};
+  if (int e = lds_attr_once(attr_devs, (const void*)k, lds)) return e;
+  const int cus = device_cus();
+  if (cus <= 0) return (int)hipErrorNoDevice;
+  const int tiles = a.tiles_m * a.tiles_n;
+  hipLaunchKernelGGL(k, dim3(tiles < cus ? tiles : cus), dim3(512), lds, s, a);
+  return (int)hipGetLastError();
+}
+
+const char* check_stream4_walk(const astergemm_config& c) {
+  if (const char* why = check_stream4(c)) return why;
+  if (c.K % 1024 != 0) return "the tile walk needs K to be a multiple of 1024";
+  if (c.M % 256 != 0 || c.N % 256 != 0) return "the tile walk needs M and N to be multiples of 256";
+  const int cus = device_cus();
+  if (cus > 0 && ((c.M + 255) / 256) * ((c.N + 255) / 256) <= cus)
+    return "the tile walk pays from two tiles per workgroup on";
+  return nullptr;
+}
+
+int grid_stream4_walk(const astergemm_config& c, int cus) {
+  const int64_t tiles = ((c.M + 255) / 256) * ((c.N + 255) / 256);
+  return (int)(cus > 0 && tiles > cus ? cus : tiles);
+}
+
+#define AG_STREAM4_WALK(name, DT, OUT)                                           \
+  Variant {                                                                      \
+    name, ASTERGEMM_KERNEL_TILE, DT, OUT, 256, 256, kRowBytes, 2, 4, 2, 3,       \
+        4 * 256 * kRowBytes + 4 * 256 * 16 + 8 * 2048,                           \
+        (const void*)gemm_stream4_walk_kernel<DT, OUT, 256, 256, 2, 4>,          \
+        launch_stream4_walk<DT, OUT>, check_stream4_walk, ASTERGEMM_OPERAND_LDS, \
+        nullptr, grid_stream4_walk                                               \
+  }
 #define AG_STREAM4_128(name, DT, OUT)                                            \
   Variant {                                                                      \
     name, ASTERGEMM_KERNEL_TILE, DT, OUT, 128, 128, kRowBytes, 2, 2, 2, 2,       \
@@ -305,7 +350,10 @@ int launch_stream_tail(const GemmArgs& a, int grid, hipStream_t s) {
     if ((rc = launch_stream8<DT, OUT, 256, 256, 2, 4>(p1, g1, s)) != 0) return rc;
     return launch_stream8<DT, OUT, 128, 128, 2, 2>(p2, g2, s);
   } else {
-    if ((rc = launch_stream4<DT, OUT, 256, 256, 2, 4>(p1, g1, s)) != 0) return rc;
+    // the whole rounds as a tile walk where its conditions hold (see launch_stream4_walk)
+    const bool walk = p1.ksteps % 4 == 0 && p1.M % 256 == 0 && p1.N % 256 == 0 && g1 > device_cus();
+    rc = walk ? launch_stream4_walk<DT, OUT>(p1, g1, s) : launch_stream4<DT, OUT, 256, 256, 2, 4>(p1, g1, s);
+    if (rc != 0) return rc;
     return launch_stream4<DT, OUT, 128, 128, 2, 2>(p2, g2, s);
   }
 }
@@ -326,7 +374,12 @@ int grid_stream_tail(const astergemm_config& c, int cus) {
   if (ts.along == 0) return (int)(((c.M + 255) / 256) * ((c.N + 255) / 256));
   const int64_t m1 = ts.along == 2 ? ts.first : c.M, n1 = ts.along == 1 ? ts.first : c.N;
   const int64_t m2 = ts.along == 2 ? c.M - ts.first : c.M, n2 = ts.along == 1 ? c.N - ts.first : c.N;
-  return (int)(((m1 + 255) / 256) * ((n1 + 255) / 256) + ((m2 + 127) / 128) * ((n2 + 127) / 128));
+  int64_t g1 = ((m1 + 255) / 256) * ((n1 + 255) / 256);
+  // MXFP4: the whole rounds run as a tile walk, one workgroup per CU (see launch_stream_tail)
+  if (c.dtype_ab == ASTERGEMM_MXFP4 && c.K % 1024 == 0 && m1 % 256 == 0 && n1 % 256 == 0 && cus > 0 &&
+      g1 > cus)
+    g1 = cus;
+  return (int)(g1 + ((m2 + 127) / 128) * ((n2 + 127) / 128));
 }
 
 // rank 3: preferred over the plain 256 x 256 kernel wherever its check passes
@@ -385,6 +438,9 @@ const Variant kStreamVariants[] = {
     AG_STREAM4_W8("stream_mxfp4_256x256_w2x4_bf16", ASTERGEMM_MXFP4, ASTERGEMM_BF16, 2),
     AG_STREAM4_W8("stream_mxfp4_256x256_w2x4_f32", ASTERGEMM_MXFP4, ASTERGEMM_F32, 2),
     AG_STREAM4_W8("stream_mxfp4_256x256_w2x4_f16", ASTERGEMM_MXFP4, ASTERGEMM_F16, 2),
+    AG_STREAM4_WALK("stream_mxfp4_256x256_w2x4_walk_bf16", ASTERGEMM_MXFP4, ASTERGEMM_BF16),
+    AG_STREAM4_WALK("stream_mxfp4_256x256_w2x4_walk_f32", ASTERGEMM_MXFP4, ASTERGEMM_F32),
+    AG_STREAM4_WALK("stream_mxfp4_256x256_w2x4_walk_f16", ASTERGEMM_MXFP4, ASTERGEMM_F16),
     AG_STREAM4_128("stream_mxfp4_128x128_w2x2_bf16", ASTERGEMM_MXFP4, ASTERGEMM_BF16),
     AG_STREAM4_128("stream_mxfp4_128x128_w2x2_f32", ASTERGEMM_MXFP4, ASTERGEMM_F32),
     AG_STREAM4_128("stream_mxfp4_128x128_w2x2_f16", ASTERGEMM_MXFP4, ASTERGEMM_F16),

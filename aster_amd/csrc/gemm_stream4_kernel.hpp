@@ -37,8 +37,72 @@
 namespace astergemm {
 namespace {
 
-template <int DT, int OUT, int BM, int BN, int WM, int WN>
-__device__ __forceinline__ void gemm_stream4_body(const GemmArgs& p, int bid) {
+// Epilogue of the tile walk: a wave stages its 16-row slabs in 2 KiB of its own, outside the
+// ring (which is already receiving the next tile), so no barrier is needed: LDS operations of
+// one wave execute in order.  A slab row is 128 bytes (64 16-bit or 32 fp32 columns), 16-byte
+// granule g of row r sits at granule g ^ (r & 7).  M and N are whole tiles.
+template <int OUT, int TM, int TN>
+__device__ __forceinline__ void walk_epilogue(const GemmArgs& p, f32x4 (&acc)[TM][TN], uint8_t* stage,
+                                              int wrow0, int wcol0) {
+  static_assert(TN == 4, "64 columns per wave");
+  float scale = 1.0f;  // fetched per tile (scalar loads): nothing to keep across the K loop
+  if (p.scale_a) scale *= *p.scale_a;
+  if (p.scale_b) scale *= *p.scale_b;
+  int lane;
+  asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lane));
+  const int li = lane & 15, lq = lane >> 4;
+  constexpr int OB = (OUT == ASTERGEMM_F32) ? 4 : 2;
+  constexpr int PASSES = 64 * OB / 128;          // 128-byte column ranges of the wave tile
+  constexpr int TPP = TN / PASSES;               // 16-column tiles per pass
+  float bias_v[TN][4];
+#pragma unroll
+  for (int n = 0; n < TN; ++n)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      int col = wcol0 + n * 16 + 4 * lq + e;
+      col = col < p.N ? col : p.N - 1;
+      bias_v[n][e] = p.bias ? p.bias[col] : 0.f;
+    }
+#pragma unroll
+  for (int m = 0; m < TM; ++m) {
+#pragma unroll
+    for (int ps = 0; ps < PASSES; ++ps) {
+#pragma unroll
+      for (int t = 0; t < TPP; ++t) {
+        const int n = ps * TPP + t;
+        f32x4 v = acc[m][n] * scale;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] += bias_v[n][e];
+        if constexpr (OUT == ASTERGEMM_F32) {
+          *(f32x4*)(stage + li * 128 + (((t * 4 + lq) ^ (li & 7)) << 4)) = v;
+        } else {
+          const u16x4 h = cast4_16<OUT>(v);
+          *(u16x4*)(stage + li * 128 + (((t * 2 + (lq >> 1)) ^ (li & 7)) << 4) + (lq & 1) * 8) = h;
+        }
+      }
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        const int c = t * 64 + lane;
+        const int r = c >> 3, cc = c & 7;
+        const i32x4 d = *(const i32x4*)(stage + r * 128 + ((cc ^ (r & 7)) << 4));
+        const int col = wcol0 + (ps * 128 + cc * 16) / OB;
+        uint8_t* out = (uint8_t*)p.C + ((int64_t)(wrow0 + m * 16 + r) * p.ldc + col) * OB;
+        // whole tiles only (the launcher checks): every store is issued, so that the count
+        // the next tile's first barrier leaves outstanding is exact
+        __builtin_nontemporal_store(d, (i32x4*)out);
+      }
+    }
+  }
+}
+
+// WALK: the workgroup takes tiles bid, bid + stride, ... below `total` as one long K loop: the
+// last two trips of a tile bring in K-steps 0 and 1 (and scale chunks 0 and 1) of the next tile
+// where a longer row would have brought K-steps nk and nk+1, so the next tile starts with its
+// operands in LDS, and the epilogue in between touches no ring memory.  Needs nk % 4 == 0 (slot
+// and scale-buffer parities carry over).
+template <int DT, int OUT, int BM, int BN, int WM, int WN, bool WALK = false>
+__device__ __forceinline__ void gemm_stream4_body(const GemmArgs& p, int bid, int stride = 0,
+                                                  int total = 0) {
   constexpr int NW = WM * WN;
   constexpr int TM = BM / WM / 16;
   constexpr int TN = BN / WN / 16;
@@ -62,21 +126,54 @@ __device__ __forceinline__ void gemm_stream4_body(const GemmArgs& p, int bid) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wm = wave / WN, wn = wave % WN;
 
-  int tile_m, tile_n;
-  map_tile(bid, p.tiles_m, p.tiles_n, p.group_m, tile_m, tile_n);
-  const int row0 = tile_m * BM, col0 = tile_n * BN;
-
   // ---- global -> LDS, tiles: identical to the other stream kernels ---------------------------
   const int lane = threadIdx.x & 63;
   const int lrow = lane >> 3;
   const int g_lane = (lane & 7) ^ (((wave * 8 + lrow) >> 1) & 7);
   const unsigned a_off = (unsigned)(lrow * (int)p.lda_bytes + g_lane * 16);
   const unsigned b_off = (unsigned)(lrow * (int)p.ldb_bytes + g_lane * 16);
-  const uint8_t* a_base[LH];
-  const uint8_t* b_base[LH];
-  group_bases<LH, NW>(p.A, p.lda_bytes, row0 + wave * 8, p.M, a_base);
-  group_bases<LH, NW>(p.B, p.ldb_bytes, col0 + wave * 8, p.N, b_base);
   const int nk = p.ksteps;
+
+  // what depends on the tile: where its rows start and where its transfers read
+  struct Src {
+    int row0, col0;
+    const uint8_t* a[LH];
+    const uint8_t* b[LH];
+    const uint8_t* sc[NSC];
+    unsigned sc_off[NSC];
+  };
+  uint8_t* sc_lds[NSC];
+#pragma unroll
+  for (int i = 0; i < NSC; ++i) sc_lds[i] = lds + (wave + i * NW < NSR ? SC_A : SC_B) + ((wave + i * NW) % NSR) * 64 * 16;
+  auto load_tile = [&](int id, Src& t) {
+    int tile_m, tile_n;
+    map_tile(id, p.tiles_m, p.tiles_n, p.group_m, tile_m, tile_n);
+    t.row0 = tile_m * BM, t.col0 = tile_n * BN;
+    if constexpr (WALK) {
+      // whole tiles: transfer j starts 8 * NW rows behind transfer j - 1, one base is enough
+      t.a[0] = p.A + (int64_t)(t.row0 + wave * 8) * p.lda_bytes;
+      t.b[0] = p.B + (int64_t)(t.col0 + wave * 8) * p.ldb_bytes;
+    } else {
+      group_bases<LH, NW>(p.A, p.lda_bytes, t.row0 + wave * 8, p.M, t.a);
+      group_bases<LH, NW>(p.B, p.ldb_bytes, t.col0 + wave * 8, p.N, t.b);
+    }
+    // scales: transfer x = wave + i * NW (0..7): x < 4 covers A rows [64x, +64), else B rows
+    // [64(x-4), +64); lane L brings the 16 scale bytes of row L for chunk c (K-steps 2c and
+    // 2c+1) to [buffer c mod 2][row][16]
+#pragma unroll
+    for (int i = 0; i < NSC; ++i) {
+      const int x = wave + i * NW;
+      const bool is_a = x < NSR;
+      t.sc[i] = is_a ? p.mx_a + (int64_t)t.row0 * p.mx_ld : p.mx_b + (int64_t)t.col0 * p.mx_ld;
+      // rows past the end of an edge tile re-read the operand's last row
+      const int first = is_a ? t.row0 : t.col0, rows = is_a ? p.M : p.N;
+      int r = (x % NSR) * 64 + lane;
+      if constexpr (!WALK) r = first + r < rows ? r : rows - 1 - first;  // the walk has whole tiles
+      t.sc_off[i] = (unsigned)(r * p.mx_ld);
+    }
+  };
+  Src cur;
+  load_tile(bid, cur);
 
   auto g2s = [&](const uint8_t* base, unsigned voff, uint8_t* dst) {
     const unsigned m0v = (unsigned)(size_t)AG_LDS(dst);
@@ -85,37 +182,19 @@ __device__ __forceinline__ void gemm_stream4_body(const GemmArgs& p, int bid) {
                  : "s"(m0v), "v"(voff), "s"(base)
                  : "memory", "m0");
   };
-  auto issue_a1 = [&](int k, int slot, int j) {  // slot: 0..1
-    g2s(a_base[j] + (int64_t)k * kRowBytes, a_off,
-        lds + slot * SLOT + (j * NW + wave) * 8 * kRowBytes);
+  // K-step k of tile t into ring slot `slot` (A: 0..1, B: 2..3)
+  auto issue_a1 = [&](const Src& t, int k, int slot, int j) {
+    const uint8_t* base = WALK ? t.a[0] + (int64_t)j * (8 * NW) * p.lda_bytes : t.a[j];
+    g2s(base + (int64_t)k * kRowBytes, a_off, lds + slot * SLOT + (j * NW + wave) * 8 * kRowBytes);
   };
-  auto issue_b1 = [&](int k, int slot, int j) {  // slot: 2..3
-    g2s(b_base[j] + (int64_t)k * kRowBytes, b_off,
-        lds + slot * SLOT + (j * NW + wave) * 8 * kRowBytes);
+  auto issue_b1 = [&](const Src& t, int k, int slot, int j) {
+    const uint8_t* base = WALK ? t.b[0] + (int64_t)j * (8 * NW) * p.ldb_bytes : t.b[j];
+    g2s(base + (int64_t)k * kRowBytes, b_off, lds + slot * SLOT + (j * NW + wave) * 8 * kRowBytes);
   };
-
-  // ---- global -> LDS, scales: wave w < 4 brings A rows [64w, 64w+64), wave w >= 4 brings B
-  // rows [64(w-4), +64); lane L brings the 16 scale bytes of row L for chunk c (K-steps 2c
-  // and 2c+1) to [buffer c mod 2][row][16] ----------------------------------------------------
-  // transfer t = wave + i * NW (0..7): t < 4 covers A rows [64t, +64), else B rows [64(t-4), +64)
-  const uint8_t* sc_base[NSC];
-  uint8_t* sc_lds[NSC];
-  unsigned sc_off[NSC];
+  // scale chunk c of tile t into scale buffer `buf`
+  auto issue_scales = [&](const Src& t, int c, int buf) {
 #pragma unroll
-  for (int i = 0; i < NSC; ++i) {
-    const int t = wave + i * NW;
-    const bool is_a = t < NSR;
-    sc_base[i] = is_a ? p.mx_a + (int64_t)row0 * p.mx_ld : p.mx_b + (int64_t)col0 * p.mx_ld;
-    // rows past the end of an edge tile re-read the operand's last row
-    const int first = is_a ? row0 : col0, rows = is_a ? p.M : p.N;
-    int r = (t % NSR) * 64 + lane;
-    r = first + r < rows ? r : rows - 1 - first;
-    sc_off[i] = (unsigned)(r * p.mx_ld);
-    sc_lds[i] = lds + (is_a ? SC_A : SC_B) + (t % NSR) * 64 * 16;
-  }
-  auto issue_scales = [&](int c) {
-#pragma unroll
-    for (int i = 0; i < NSC; ++i) g2s(sc_base[i] + c * 16, sc_off[i], sc_lds[i] + (c & 1) * BM * 16);
+    for (int i = 0; i < NSC; ++i) g2s(t.sc[i] + c * 16, t.sc_off[i], sc_lds[i] + buf * BM * 16);
   };
   // in place: bytes b[0..15] of this lane's row -> pairs {b[8h+q], b[8h+4+q]}, h = K-step
   // parity, q = 0..3
@@ -175,17 +254,17 @@ __device__ __forceinline__ void gemm_stream4_body(const GemmArgs& p, int bid) {
 
   // ---- prologue: scales of chunks 0 and 1 and tiles of K-steps 0 and 1 issued; chunk 0
   // re-packed; A-row fragments and the first B-row fragment of K-step 0 read --------------------
-  issue_scales(0);
+  issue_scales(cur, 0, 0);
 #pragma unroll
-  for (int j = 0; j < LH; ++j) issue_a1(0, 0, j);
+  for (int j = 0; j < LH; ++j) issue_a1(cur, 0, 0, j);
 #pragma unroll
-  for (int j = 0; j < LH; ++j) issue_b1(0, 2, j);
-  if (nk > 2) issue_scales(1);
+  for (int j = 0; j < LH; ++j) issue_b1(cur, 0, 2, j);
+  if (nk > 2) issue_scales(cur, 1, 1);
   if (nk > 1) {
 #pragma unroll
-    for (int j = 0; j < LH; ++j) issue_a1(1, 1, j);
+    for (int j = 0; j < LH; ++j) issue_a1(cur, 1, 1, j);
 #pragma unroll
-    for (int j = 0; j < LH; ++j) issue_b1(1, 3, j);
+    for (int j = 0; j < LH; ++j) issue_b1(cur, 1, 3, j);
   }
   // the first transfer (scales of chunk 0) has landed for this wave: re-pack it
   if (nk > 2) __builtin_amdgcn_s_waitcnt(waitcnt_imm(4 * LH + NSC, 15));
@@ -198,20 +277,28 @@ __device__ __forceinline__ void gemm_stream4_body(const GemmArgs& p, int bid) {
   else __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
-  using K0 = std::integral_constant<int, 0>;
-  read_b(0, K0{});
-  read_sb(0, K0{});
-  {
+  // fragments of K-step 0 (slot 0, scale buffer 0): all A rows and the first B row
+  auto first_reads = [&]() {
+    using K0 = std::integral_constant<int, 0>;
+    read_b(0, K0{});
+    read_sb(0, K0{});
     const uint8_t* s = lds + a_rd;
     const uint8_t* ps = lds + sa_rd + sc_rd;
+    if constexpr (WALK) {
+      // used once per tile: recomputed from a lane index the optimiser cannot see through,
+      // instead of living in a register (or a spill slot) across the K loop
+      int l2;
+      asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(l2));
+      ps = lds + sa_rd + (unsigned)((l2 & 15) * 16 + (l2 >> 4) * 2);
+    }
     static_for<0, TM>([&](auto mc) {
       constexpr int m = decltype(mc)::value;
       fa_lo[m] = *(const i32x4*)(s + rd0 + m * 16 * kRowBytes);
       fa_hi[m] = *(const i32x4*)(s + rd1 + m * 16 * kRowBytes);
       sa[m] = *(const unsigned short*)(ps + m * 16 * 16);
     });
-  }
-  __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_sched_barrier(0);
+  };
 
   // ---- K loop: trip k multiplies K-step k; pair i = (n, m) is the two MFMAs of tile (m, n) ----
   // (slot numbers for TM = 8; group n is slots 8n .. 8n+7)
@@ -230,7 +317,22 @@ __device__ __forceinline__ void gemm_stream4_body(const GemmArgs& p, int bid) {
   // Every condition of a part is a compile-time flag, so that each part is straight-line
   // code: ODD = k is odd; LD = K-step k+2 exists (tile transfers); RD = K-step k+1 exists
   // (reads, re-pack, barrier); SC = K-step k+3 exists (scale transfer, odd trips only).
-  auto part = [&](int k, auto first, auto odd_c, auto ld_c, auto rd_c, auto sc_c) {
+  // Tile transfers read tile `lt` at K-step k + 2 - kshift, scale transfers tile `lsc` at chunk
+  // (k + 3) / 2 - cshift: both shifts are 0 inside a tile; when the last trips of a tile bring
+  // in the next one they are nk and nk / 2.  Where transfers land, and everything that is
+  // read, follows k alone.
+  // GUARD: two wait states in front of every MFMA.  The MFMAs are inline asm, which the
+  // compiler's hazard recogniser does not look into: where it places a register copy right in
+  // front of one (it does in the straight-line parts of the tile walk, not in the K loop), the
+  // MFMA would read the register before the copy has landed.
+  constexpr int NST = TM * 2 * (OUT == ASTERGEMM_F32 ? 2 : 1);  // stores of walk_epilogue per wave
+  bool stores_behind = false;
+  auto part = [&](int k, auto first, auto odd_c, auto ld_c, auto rd_c, auto sc_c, const Src& lt,
+                  int kshift, const Src& lsc, int cshift, auto guard_c) {
+    constexpr bool GUARD = decltype(guard_c)::value != 0;
+    // trip 0 of the tile walk: the stores of the previous tile's epilogue are younger than every
+    // transfer this barrier has to certify, so they may stay outstanding
+    constexpr bool AFTER_STORES = decltype(guard_c)::value == 2;
     constexpr bool FIRST = decltype(first)::value;
     constexpr bool odd = decltype(odd_c)::value;
     constexpr bool do_ld = decltype(ld_c)::value;
@@ -255,16 +357,19 @@ __device__ __forceinline__ void gemm_stream4_body(const GemmArgs& p, int bid) {
         // a trip rotate an accumulator through fresh registers, which costs copies at the
         // loop edge and more registers than there are.  Same destination and addend is also
         // the form the hardware chains without software wait states.
-        if constexpr (!HI)
-          asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 "
-                       "op_sel_hi:[0,0,0] cbsz:4 blgp:4"
-                       : ACC_CONSTRAINT(acc[m][n])
-                       : "v"(b4), "v"(a4), "v"(sb[n & 1]), "v"(sa[m]));
-        else
-          asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 "
-                       "op_sel:[1,1,0] op_sel_hi:[0,0,0] cbsz:4 blgp:4"
-                       : ACC_CONSTRAINT(acc[m][n])
-                       : "v"(b4), "v"(a4), "v"(sb[n & 1]), "v"(sa[m]));
+#define AG_MFMA4(PRE, SEL)                                                              \
+  asm volatile(PRE "v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 " SEL       \
+               "op_sel_hi:[0,0,0] cbsz:4 blgp:4"                                         \
+               : ACC_CONSTRAINT(acc[m][n])                                               \
+               : "v"(b4), "v"(a4), "v"(sb[n & 1]), "v"(sa[m]))
+        if constexpr (GUARD) {
+          if constexpr (!HI) AG_MFMA4("s_nop 1\n\t", "");
+          else AG_MFMA4("s_nop 1\n\t", "op_sel:[1,1,0] ");
+        } else {
+          if constexpr (!HI) AG_MFMA4("", "");
+          else AG_MFMA4("", "op_sel:[1,1,0] ");
+        }
+#undef AG_MFMA4
         // ---- one or two side instructions behind every MFMA --------------------------------
         if constexpr (decltype(jc)::value == 0) {
           if constexpr (I % TM == 0 && n + 1 < TN) read_b(k, std::integral_constant<int, n + 1>{});
@@ -273,7 +378,7 @@ __device__ __forceinline__ void gemm_stream4_body(const GemmArgs& p, int bid) {
             if (odd && do_rd) repack_scales((k + 1) >> 1);
           }
           if constexpr (I >= BAR && I < BAR + LH) {
-            if (do_ld) issue_b1(k + 2, 2 + (k & 1), I - BAR);
+            if (do_ld) issue_b1(lt, k + 2 - kshift, 2 + (k & 1), I - BAR);
           }
           if constexpr (I == (TN - 1) * TM) {
             const int kn = k + 1;
@@ -288,12 +393,12 @@ __device__ __forceinline__ void gemm_stream4_body(const GemmArgs& p, int bid) {
           }
         } else {
           if constexpr (I >= BAR && I < BAR + LH) {
-            if (do_ld) issue_a1(k + 2, k & 1, I - BAR);
+            if (do_ld) issue_a1(lt, k + 2 - kshift, k & 1, I - BAR);
           }
           if constexpr (I == BAR + LH - 1) {
             // chunk (k+3)/2 covers K-steps k+3 and k+4; its buffer held chunk (k-1)/2
             // (K-steps k-1 and k), last read before this trip's barrier
-            if (odd && do_sc) issue_scales((k + 3) >> 1);
+            if (odd && do_sc) issue_scales(lsc, ((k + 3) >> 1) - cshift, ((k + 3) >> 1) & 1);
           }
         }
         // refill in place for K-step k+1: the first-MFMA operands of a couple are dead after
@@ -312,7 +417,12 @@ __device__ __forceinline__ void gemm_stream4_body(const GemmArgs& p, int bid) {
       });
       if constexpr (I == BAR - 1) {
         if (do_rd) {
-          __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
+          if constexpr (AFTER_STORES) {
+            if (stores_behind) __builtin_amdgcn_s_waitcnt(waitcnt_imm(NST, 0));
+            else __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
+          } else {
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
+          }
           __builtin_amdgcn_s_barrier();
           asm volatile("" ::: "memory");
         }
@@ -323,35 +433,102 @@ __device__ __forceinline__ void gemm_stream4_body(const GemmArgs& p, int bid) {
   static_assert(BAR > (TN - 2) * TM + 1 && BAR + LH <= NMF, "schedule positions");
   using T = std::true_type;
   using F = std::false_type;
-  // nk is even.  part(k, first-half?, odd, LD, RD, SC)
-  int k = 0;
-  part(0, T{}, F{}, F{}, T{}, F{});
+  using G0 = std::integral_constant<int, 0>;  // guard_c: no wait states in front of the MFMAs
+  using G1 = std::integral_constant<int, 1>;  // two wait states
+  using G2 = std::integral_constant<int, 2>;  // two wait states, trip 0 of the tile walk
+  // nk is even.  part(k, first-half?, odd, LD, RD, SC, tile source, K shift, scale source, chunk shift)
+  if constexpr (!WALK) {
+    first_reads();
+    int k = 0;
+    part(0, T{}, F{}, F{}, T{}, F{}, cur, 0, cur, 0, G0{});
 #pragma unroll 1
-  for (; k + 4 < nk; k += 2) {
-    part(k, F{}, F{}, T{}, T{}, F{});
-    part(k + 1, T{}, T{}, F{}, T{}, F{});
-    part(k + 1, F{}, T{}, T{}, T{}, T{});
-    part(k + 2, T{}, F{}, F{}, T{}, F{});
+    for (; k + 4 < nk; k += 2) {
+      part(k, F{}, F{}, T{}, T{}, F{}, cur, 0, cur, 0, G0{});
+      part(k + 1, T{}, T{}, F{}, T{}, F{}, cur, 0, cur, 0, G0{});
+      part(k + 1, F{}, T{}, T{}, T{}, T{}, cur, 0, cur, 0, G0{});
+      part(k + 2, T{}, F{}, F{}, T{}, F{}, cur, 0, cur, 0, G0{});
+    }
+    if (nk >= 4) {  // k = nk - 4: the last scale chunk is already on its way
+      part(k, F{}, F{}, T{}, T{}, F{}, cur, 0, cur, 0, G0{});
+      part(k + 1, T{}, T{}, F{}, T{}, F{}, cur, 0, cur, 0, G0{});
+      part(k + 1, F{}, T{}, T{}, T{}, F{}, cur, 0, cur, 0, G0{});
+      part(k + 2, T{}, F{}, F{}, T{}, F{}, cur, 0, cur, 0, G0{});
+      k += 2;
+    }
+    // k = nk - 2: nothing left to transfer; the last trip has nothing left to read
+    part(k, F{}, F{}, F{}, T{}, F{}, cur, 0, cur, 0, G0{});
+    part(k + 1, T{}, T{}, F{}, F{}, F{}, cur, 0, cur, 0, G0{});
+    part(k + 1, F{}, T{}, F{}, F{}, F{}, cur, 0, cur, 0, G0{});
+    __builtin_amdgcn_sched_barrier(0);
+    stream_epilogue<OUT, BM, BN, WM, WN>(p, acc, lds, wave, cur.row0, cur.col0);
+  } else {
+    // One path for every tile, so that the accumulators never meet a join: the last tile of a
+    // workgroup brings in its own first two K-steps again, into slots nothing reads any more.
+    int tile = bid;
+    for (;;) {
+      // zeroed here, not behind the epilogue: nothing of the accumulators crosses the back edge.
+      // The zero is made here as well (opaque, so that it is not kept across the loop in
+      // registers the loop does not have).
+      float z;
+      asm volatile("v_mov_b32 %0, 0" : "=v"(z));
+      const f32x4 zero = {z, z, z, z};
+#pragma unroll
+      for (int m = 0; m < TM; ++m)
+#pragma unroll
+        for (int n = 0; n < TN; ++n) {
+          acc[m][n] = zero;
+          asm volatile("" : ACC_CONSTRAINT(acc[m][n]));
+        }
+      // what the barrier of the last trip (the prologue, for the first tile) certified
+      first_reads();
+      int k = 0;
+      part(0, T{}, F{}, F{}, T{}, F{}, cur, 0, cur, 0, G2{});
+#pragma unroll 1
+      for (; k + 4 < nk; k += 2) {
+        part(k, F{}, F{}, T{}, T{}, F{}, cur, 0, cur, 0, G0{});
+        part(k + 1, T{}, T{}, F{}, T{}, F{}, cur, 0, cur, 0, G0{});
+        part(k + 1, F{}, T{}, T{}, T{}, T{}, cur, 0, cur, 0, G0{});
+        part(k + 2, T{}, F{}, F{}, T{}, F{}, cur, 0, cur, 0, G0{});
+      }
+      // k = nk - 4 (nk % 4 == 0, so nk >= 4): chunk nk / 2 is chunk 0 of the next tile, K-steps
+      // nk and nk + 1 are its K-steps 0 and 1; the last trip keeps its barrier (which certifies
+      // K-step 0 and the re-packed scales of the next tile) but reads nothing: fragments held
+      // across the epilogue would not fit in the registers next to it
+      const bool more = tile + stride < total;
+      Src nxt;
+      load_tile(more ? tile + stride : tile, nxt);
+      part(k, F{}, F{}, T{}, T{}, F{}, cur, 0, cur, 0, G1{});
+      part(k + 1, T{}, T{}, F{}, T{}, F{}, cur, 0, cur, 0, G1{});
+      part(k + 1, F{}, T{}, T{}, T{}, T{}, cur, 0, nxt, nk >> 1, G1{});
+      part(k + 2, T{}, F{}, F{}, T{}, F{}, cur, 0, cur, 0, G1{});
+      k += 2;
+      part(k, F{}, F{}, T{}, T{}, F{}, nxt, nk, nxt, nk >> 1, G1{});
+      part(k + 1, T{}, T{}, F{}, T{}, F{}, cur, 0, cur, 0, G1{});
+      part(k + 1, F{}, T{}, T{}, F{}, T{}, nxt, nk, nxt, nk >> 1, G1{});
+      __builtin_amdgcn_sched_barrier(0);
+      walk_epilogue<OUT, TM, TN>(p, acc, lds + SC_B + 2 * BM * 16 + wave * 2048,
+                                 cur.row0 + wm * TM * 16, cur.col0 + wn * TN * 16);
+      __builtin_amdgcn_sched_barrier(0);
+      if (!more) break;
+      cur = nxt;
+      tile += stride;
+      stores_behind = true;
+    }
+    // the transfers the last tile issued into the ring must have landed before the workgroup
+    // gives its LDS back
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
   }
-  if (nk >= 4) {  // k = nk - 4: the last scale chunk is already on its way
-    part(k, F{}, F{}, T{}, T{}, F{});
-    part(k + 1, T{}, T{}, F{}, T{}, F{});
-    part(k + 1, F{}, T{}, T{}, T{}, F{});
-    part(k + 2, T{}, F{}, F{}, T{}, F{});
-    k += 2;
-  }
-  // k = nk - 2: nothing left to transfer; the last trip has nothing left to read
-  part(k, F{}, F{}, F{}, T{}, F{});
-  part(k + 1, T{}, T{}, F{}, F{}, F{});
-  part(k + 1, F{}, T{}, F{}, F{}, F{});
-  __builtin_amdgcn_sched_barrier(0);
-
-  stream_epilogue<OUT, BM, BN, WM, WN>(p, acc, lds, wave, row0, col0);
 }
 
 template <int DT, int OUT, int BM, int BN, int WM, int WN>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_stream4_kernel(const GemmArgs p) {
   gemm_stream4_body<DT, OUT, BM, BN, WM, WN>(p, blockIdx.x);
+}
+
+// Tile walk: gridDim.x workgroups (one per CU) share the tiles_m x tiles_n tiles round-robin.
+template <int DT, int OUT, int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(WM* WN * 64) void gemm_stream4_walk_kernel(const GemmArgs p) {
+  gemm_stream4_body<DT, OUT, BM, BN, WM, WN, true>(p, blockIdx.x, gridDim.x, p.tiles_m * p.tiles_n);
 }
 
 // Split K (see gemm_stream_splitk_kernel): copy s of the tile grid multiplies K steps

@@ -880,6 +880,8 @@ def test_every_tile_variant(gpu, vid, name, dtype_ab, dtype_c):
         K = {"fp8_e4m3": 8192, "mxfp4": 8192}.get(dtype_ab, 4096)  # 64 (MXFP4: 32) steps of 128 bytes
     if "tail128" in name:
         M, N, K = 512, 32768 + 256, 512  # 2 x 129 tiles of 256 x 256: one whole round and a rest
+    if "_walk_" in name:
+        M, N, K = 512, 32768 + 256, 1024  # 258 tiles: more than one per workgroup, four K-steps
     a, b, ex = operands(M, N, K, dtype_ab, seed=11, a_std=1.0, b_std=1.0 if dtype_ab != "bf16" else 0.05)
     bias = np.random.default_rng(12).standard_normal(N).astype(np.float32)
     path, b_dev = "lds", b
@@ -1029,6 +1031,31 @@ def test_mxfp4_stream_kernel_eight_waves_every_loop_phase(gpu, ksteps, dtype_c):
     assert name == f"stream_mxfp4_256x256_w2x4_{dtype_c}"
     want = G.gemm_mxfp4(a, mxa, b, mxb, out_dtype=_DT[dtype_c])
     check(out, want, dtype_c, N, bar=1e-5 if dtype_c == "f32" else REL_L2_BAR)
+
+
+@pytest.mark.parametrize("K", [1024, 2048, 3072])
+@pytest.mark.parametrize("dtype_c", ["bf16", "f32"])
+def test_mxfp4_tile_walk_equals_the_plain_kernel(gpu, K, dtype_c):
+    """The tile walk (one workgroup per CU takes several tiles as one long K loop, the next tile's
+    first K-steps arriving during the last trips of the current one) on more tiles than any
+    device has CUs: the same bits as the one-tile-per-workgroup kernel, and sampled rows against
+    the oracle.  The walk takes whole tiles only."""
+    M, N = 4352, 4608   # 17 x 18 = 306 tiles of 256 x 256
+    rng = np.random.default_rng(7 + K)
+    a = rng.integers(0, 256, (M, K // 2)).astype(np.uint8)
+    b = rng.integers(0, 256, (N, K // 2)).astype(np.uint8)
+    mxa = rng.integers(118, 134, (M, K // 32)).astype(np.uint8)
+    mxb = rng.integers(118, 134, (N, K // 32)).astype(np.uint8)
+    bias = rng.standard_normal(N).astype(np.float32)
+    plain, pname = run_gemm(a, b, M, N, K, "mxfp4", dtype_c, mx_a=mxa, mx_b=mxb, bias=bias,
+                            variant=_variant_id(f"stream_mxfp4_256x256_w2x4_{dtype_c}"))
+    walk, wname = run_gemm(a, b, M, N, K, "mxfp4", dtype_c, mx_a=mxa, mx_b=mxb, bias=bias,
+                           variant=_variant_id(f"stream_mxfp4_256x256_w2x4_walk_{dtype_c}"))
+    assert pname == f"stream_mxfp4_256x256_w2x4_{dtype_c}" and wname == f"stream_mxfp4_256x256_w2x4_walk_{dtype_c}"
+    assert np.array_equal(walk.view(np.uint8), plain.view(np.uint8))
+    rows = np.unique(np.concatenate([rng.integers(0, M, 12), [0, 255, 256, M - 1]]))
+    want = G.gemm_mxfp4(a[rows], mxa[rows], b, mxb, out_dtype=_DT[dtype_c], bias=bias)
+    check(walk[rows], want, dtype_c, N, bar=1e-5 if dtype_c == "f32" else REL_L2_BAR)
 
 
 def test_mxfp4_stream_kernel_falls_back_for_odd_kstep_counts(gpu):

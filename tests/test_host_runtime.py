@@ -345,3 +345,23 @@ def test_make_inputs_storage_types():
     from oracle import formats as F
     want = F.f32_to_bf16_bits(BH.init_array((256, 64), "hpl", "A").astype(np.float32))
     assert np.array_equal(a, want)
+
+
+def test_build_scan_finds_a_register_copy_in_front_of_an_inline_asm_mfma():
+    # the compiler's hazard recogniser does not look inside inline asm; the build scans the device
+    # assembly instead (aster_amd/build.py: scan_mfma_hazards)
+    from aster_amd.build import scan_mfma_hazards
+    mfma = ("\t;;#ASMSTART\n{pre}\tv_mfma_scale_f32_16x16x128_f8f6f4 a[36:39], v[68:71], v[36:39], a[36:39], "
+            "v32, v95 op_sel_hi:[0,0,0] cbsz:4 blgp:4\n\t;;#ASMEND\n")
+    copy = "\tv_mov_b64_e32 v[38:39], v[36:37]\n\tv_mov_b64_e32 v[36:37], v[34:35]\n"
+    found = scan_mfma_hazards(copy + mfma.format(pre=""))
+    assert [(f[0], f[2]) for f in found] == [(4, 2), (4, 1)]
+    # two wait states in between, of any kind, are enough
+    assert scan_mfma_hazards(copy + mfma.format(pre="\ts_nop 1\n")) == []
+    assert scan_mfma_hazards(copy + "\ts_add_u32 s0, s1, s2\n\ts_nop 0\n" + mfma.format(pre="")) == []
+    # scale and accumulator registers count as sources; other registers do not
+    assert len(scan_mfma_hazards("\tv_and_b32_e32 v95, 0xffff, v95\n" + mfma.format(pre=""))) == 1
+    assert len(scan_mfma_hazards("\tv_accvgpr_mov_b32 a37, a5\n" + mfma.format(pre=""))) == 1
+    assert scan_mfma_hazards("\tv_mov_b32_e32 v40, v41\n" + mfma.format(pre="")) == []
+    # MFMAs the compiler emitted itself are its own business
+    assert scan_mfma_hazards(copy + "\tv_mfma_f32_16x16x32_bf16 a[0:3], v[36:39], v[4:7], a[0:3]\n") == []
