@@ -89,9 +89,9 @@ const char* validate_problem(const astergemm_config& c) {
     return "bad scale_mode";
   if (c.operand_path < ASTERGEMM_OPERAND_LDS || c.operand_path > ASTERGEMM_OPERAND_DIRECT_B_K8)
     return "bad operand_path";
-  if (c.operand_path != ASTERGEMM_OPERAND_LDS && c.dtype_ab != ASTERGEMM_F16 &&
+  if (c.operand_path == ASTERGEMM_OPERAND_DIRECT_B_K8 && c.dtype_ab != ASTERGEMM_F16 &&
       c.dtype_ab != ASTERGEMM_BF16)
-    return "pre-shuffled B is built for 16-bit operands";
+    return "B pre-shuffled in K8 order is built for 16-bit operands";
   if ((c.dtype_ab == ASTERGEMM_MXFP4) != (c.scale_mode == ASTERGEMM_SCALE_MX32))
     return "MXFP4 operands and SCALE_MX32 go together";
   if (c.dtype_ab == ASTERGEMM_MXFP4 && c.K % 32 != 0) return "MXFP4 needs K % 32 == 0";
@@ -692,6 +692,37 @@ int astergemm_shuffle_weight_k8_16(const uint16_t* src, uint16_t* dst, int64_t N
       for (int g = 0; g < 4; ++g)
         for (int nl = 0; nl < 16; ++nl)
           for (int kw = 0; kw < 8; ++kw) dst[o++] = src[(nb * 16 + nl) * K + kb * 32 + g * 8 + kw];
+  return 0;
+}
+
+int astergemm_shuffle_weight_8(const uint8_t* src, uint8_t* dst, int64_t N, int64_t row_bytes_) {
+  if (!src || !dst || N < 0 || row_bytes_ < 0 || N % 16 != 0 || row_bytes_ % 128 != 0) {
+    set_error("astergemm_shuffle_weight_8: need N %% 16 == 0 and rows of whole 128-byte steps");
+    return ASTERGEMM_EINVAL;
+  }
+  // dst order (nb, step, half u, lane group q, row n, 16 bytes) <- src (nb, n, step, 4u + q, 16 bytes)
+  const int64_t steps = row_bytes_ / 128;
+  uint8_t* o = dst;
+  for (int64_t nb = 0; nb < N / 16; ++nb)
+    for (int64_t st = 0; st < steps; ++st)
+      for (int u = 0; u < 2; ++u)
+        for (int q = 0; q < 4; ++q)
+          for (int nl = 0; nl < 16; ++nl, o += 16)
+            memcpy(o, src + (nb * 16 + nl) * row_bytes_ + st * 128 + (4 * u + q) * 16, 16);
+  return 0;
+}
+
+int astergemm_shuffle_scales_e8m0(const uint8_t* src, uint8_t* dst, int64_t N, int64_t K) {
+  if (!src || !dst || N < 0 || K < 0 || N % 16 != 0 || K % 256 != 0) {
+    set_error("astergemm_shuffle_scales_e8m0: need N %% 16 == 0 and K %% 256 == 0");
+    return ASTERGEMM_EINVAL;
+  }
+  // dst order (nb, step, row n, 8 bytes) <- src (nb, n, step, 8 bytes)
+  const int64_t steps = K / 256, ld = K / 32;
+  uint8_t* o = dst;
+  for (int64_t nb = 0; nb < N / 16; ++nb)
+    for (int64_t st = 0; st < steps; ++st)
+      for (int nl = 0; nl < 16; ++nl, o += 8) memcpy(o, src + (nb * 16 + nl) * ld + st * 8, 8);
   return 0;
 }
 

@@ -1657,6 +1657,258 @@ const char* check_skinny_direct(const astergemm_config& c) {
         check_skinny_direct, ASTERGEMM_OPERAND_DIRECT_B                                     \
   }
 
+// ---- M <= 16, fp8 or MXFP4 weights pre-shuffled (operand path "direct B") ------------------
+//
+// The same idea for the one-byte and nibble types, whose MFMA (16x16x128) takes pieces lq and
+// 4 + lq of a 128-byte step of a row: B arrives in STEP ORDER (astergemm_shuffle_weight_8),
+// row block nb (16 rows), step s, half u in one KiB at ((nb * steps + s) * 2 + u) * 1024, lane
+// 16 q + n of a wave finding bytes [(4u + q) * 16, + 16) of row 16 nb + n, step s, at byte
+// 16 (16 q + n).  A lane's 16-byte load of a KiB is therefore its operand piece (fp8: the two
+// halves of a step are the two halves of one operand; MXFP4: one operand each), a unit of SU
+// steps is 2 SU KiB in a row, and a wave's slice of a row block (SPB steps) is contiguous.
+// The MXFP4 scale plane arrives in the matching order (astergemm_shuffle_scales_e8m0): the
+// 8 e8m0 bytes of row 16 nb + n, step s at (nb * steps + s) * 128 + 8 n, so the scales a wave
+// needs for a step are one line.  Activations are plain row-major and go through the wave's
+// LDS buffer once, as in gemm_skinny_reg_kernel / gemm_skinny_fp4_kernel; persistent grid, N in
+// multiples of 8 rows, three register sets (a loaded register is the operand, so a set is busy
+// until its MFMAs have issued), reduction through LDS every four row blocks.
+// SPB = steps per wave and row (row bytes / 1024), SU = steps per unit.
+template <int DT, int OUT, int SPB, int SU>
+__global__ __launch_bounds__(512) void gemm_skinny_directb_kernel(const GemmArgs p) {
+  static_assert(DT == ASTERGEMM_FP8_E4M3 || DT == ASTERGEMM_MXFP4, "one-byte and nibble operands");
+  extern __shared__ __attribute__((aligned(1024))) uint8_t slds[];
+  constexpr bool FP4 = DT == ASTERGEMM_MXFP4;
+  constexpr int KW = 8;
+  constexpr int UPB = SPB / SU;                  // units per row block
+  constexpr int NL = 2 * SU;                     // loads (KiB) per unit
+  constexpr int NBS = 4;                         // row blocks between workgroup barriers
+  static_assert(SPB % SU == 0, "whole units");
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int li = lane & 15, lq = lane >> 4;
+  f32x4* red = (f32x4*)slds;                     // [2][NBS][KW][64]
+  uint8_t* tbuf = slds + 2 * NBS * KW * 1024 + wave * 8192;  // the activations' way into operand order
+
+  const int g = gridDim.x;
+  const int per = (((p.N + g - 1) / g) + 7) & ~7;
+  const int r0 = blockIdx.x * per;
+  const int r1 = (r0 + per) < p.N ? (r0 + per) : p.N;
+  if (r0 >= p.N) return;
+  const int nb0 = r0 >> 4;
+  const int nblk = ((r1 - 1) >> 4) - nb0 + 1;
+  const int total = nblk * UPB;
+  const int64_t steps = (int64_t)SPB * KW;       // 128-byte steps of a row
+  const int64_t blk_bytes = steps * 2048;        // payload of one row block
+
+  const uint8_t* wbase = p.B + (int64_t)nb0 * blk_bytes + (int64_t)wave * SPB * 2048 + lane * 16;
+  const uint8_t* sbase = FP4 ? p.mx_b + ((int64_t)nb0 * steps + wave * SPB) * 128 + li * 8 : nullptr;
+  const uint8_t* idle = p.A + lane * 16;         // nothing to fetch: lines that stay in L2
+  auto issue = [&](int j, i32x4(&dst)[NL], i32x2(&sc)[SU]) {  // flat index j = block * UPB + t
+    int blk = j / UPB;
+    const int t = j % UPB;
+    blk = blk < nblk ? blk : nblk - 1;
+    const int n = (nb0 + blk) * 16 + li;
+    const bool dead = j >= total || n < r0 || n >= r1;
+    const uint8_t* src = dead ? idle : wbase + (int64_t)blk * blk_bytes + t * (NL * 1024);
+    const int step = dead ? 0 : 1024;            // idle lanes re-read one line of x
+#pragma unroll
+    for (int u = 0; u < NL; ++u) dst[u] = __builtin_nontemporal_load((const i32x4*)(src + u * step));
+    if constexpr (FP4) {
+      // scale bytes of a row of the block exist even where the row belongs to a neighbour
+      const uint8_t* ssrc = sbase + ((int64_t)blk * steps + t * SU) * 128;
+#pragma unroll
+      for (int s2 = 0; s2 < SU; ++s2) sc[s2] = *(const i32x2*)(ssrc + s2 * 128);
+    }
+  };
+
+  // x (and its scales): operand registers for the SPB * 2 pieces of a row block, fetched as
+  // whole lines and turned around in the wave's LDS buffer
+  i32x4 x[SPB * 2];
+  int xs[FP4 ? SPB * 2 : 1];
+  {
+    const int lrow = lane >> 3, lpiece = lane & 7;
+    const int wr_off = lrow * 128 + ((lpiece ^ lrow) << 4);
+    if constexpr (FP4) {
+      const int m = li < p.M ? li : p.M - 1;
+      const uint8_t* xsrc = p.mx_a + (int64_t)m * p.mx_ld + wave * (SPB * 8);
+#pragma unroll
+      for (int s2 = 0; s2 < SPB; ++s2) {
+        const i32x2 v = *(const i32x2*)(xsrc + s2 * 8);
+        xs[s2 * 2] = (int)((unsigned)v[0] >> (8 * lq));
+        xs[s2 * 2 + 1] = (int)((unsigned)v[1] >> (8 * lq));
+      }
+    }
+    static_for<0, UPB>([&](auto T) {
+      constexpr int t = decltype(T)::value;
+      i32x4 xw[NL];
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        int m = h * 8 + lrow;
+        m = m < p.M ? m : p.M - 1;
+        const uint8_t* src =
+            p.A + (int64_t)m * p.lda_bytes + (int64_t)wave * SPB * 128 + t * (SU * 128) + lpiece * 16;
+#pragma unroll
+        for (int s2 = 0; s2 < SU; ++s2) xw[s2 * 2 + h] = *(const i32x4*)(src + s2 * 128);
+      }
+#pragma unroll
+      for (int i = 0; i < NL; ++i)
+        *(i32x4*)(tbuf + (i >> 1) * 2048 + (i & 1) * 1024 + wr_off) = xw[i];
+#pragma unroll
+      for (int i = 0; i < NL; ++i)               // piece 4u + lq of step s: i = 2 s + u
+        x[t * NL + i] = *(const i32x4*)(tbuf + (i >> 1) * 2048 + li * 128 +
+                                        (((4 * (i & 1) + lq) ^ (li & 7)) << 4));
+    });
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  i32x4 w0[NL], w1[NL], w2[NL];
+  i32x2 s0[SU], s1[SU], s2r[SU];
+  issue(0, w0, s0);
+  issue(1, w1, s1);
+  issue(2, w2, s2r);
+  __builtin_amdgcn_sched_barrier(0);
+
+  float scale = 1.0f;
+  if (p.scale_a) scale *= *p.scale_a;
+  if (p.scale_b) scale *= *p.scale_b;
+
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  int parity = 0;
+  auto block_end = [&](int blk) {
+    const int slot = blk & (NBS - 1);
+    red[((parity * NBS + slot) * KW + wave) * 64 + lane] = acc;
+    acc = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (slot != NBS - 1 && blk != nblk - 1) return;
+    __syncthreads();
+    if (wave <= slot) {
+      const f32x4* src = red + ((parity * NBS + wave) * KW) * 64 + lane;
+      f32x4 v = src[0];
+#pragma unroll
+      for (int k = 1; k < KW; ++k) v += src[k * 64];
+      const int m = li, n = (nb0 + blk - slot + wave) * 16 + 4 * lq;
+      if (m < p.M && n >= r0 && n < r1) {
+        v *= scale;
+        if (p.bias)
+          for (int r = 0; r < 4; ++r) v[r] += p.bias[n + r];
+        const int64_t idx = (int64_t)m * p.ldc + n;
+        const bool vec_ok = (p.ldc & 3) == 0;
+        if constexpr (OUT == ASTERGEMM_F32) {
+          float* o = (float*)p.C + idx;
+          if (vec_ok) *(f32x4*)o = v;
+          else
+            for (int r = 0; r < 4; ++r) o[r] = v[r];
+        } else {
+          unsigned short h[4];
+          for (int r = 0; r < 4; ++r) {
+            if constexpr (OUT == ASTERGEMM_BF16) h[r] = sk_f32_to_bf16(v[r]);
+            else {
+              _Float16 hh = (_Float16)v[r];
+              h[r] = __builtin_bit_cast(unsigned short, hh);
+            }
+          }
+          unsigned short* o = (unsigned short*)p.C + idx;
+          if (vec_ok) *(u16x4*)o = u16x4{h[0], h[1], h[2], h[3]};
+          else
+            for (int r = 0; r < 4; ++r) o[r] = h[r];
+        }
+      }
+    }
+    parity ^= 1;
+  };
+  // T = unit index inside the row block (compile time: selects the x registers)
+  auto mma = [&](int blk, auto T, const i32x4(&w)[NL], const i32x2(&sc)[SU]) {
+    constexpr int t = decltype(T)::value;
+    if constexpr (FP4) {
+#pragma unroll
+      for (int i = 0; i < NL; ++i) {             // i = 2 s + u: scale byte 4u + lq of step s
+        const int ws = (int)((unsigned)sc[i >> 1][i & 1] >> (8 * lq));
+        const i32x4 xv = x[t * NL + i];
+        acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+            i32x8{w[i][0], w[i][1], w[i][2], w[i][3], 0, 0, 0, 0},
+            i32x8{xv[0], xv[1], xv[2], xv[3], 0, 0, 0, 0}, acc, 4, 4, 0, ws, 0, xs[t * NL + i]);
+      }
+    } else {
+#pragma unroll
+      for (int s2 = 0; s2 < SU; ++s2) {
+        const i32x4 lo = w[2 * s2], hi = w[2 * s2 + 1];
+        const i32x4 xl = x[t * NL + 2 * s2], xh = x[t * NL + 2 * s2 + 1];
+        acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+            i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]},
+            i32x8{xl[0], xl[1], xl[2], xl[3], xh[0], xh[1], xh[2], xh[3]}, acc, 0, 0, 0, 0, 0, 0);
+      }
+    }
+    if (t == UPB - 1) block_end(blk);
+  };
+
+  // flat steps in groups of lcm(3, UPB) so that register set and x indices are static
+  constexpr int TRIP = (UPB % 3 == 0) ? UPB : 3 * UPB;
+  auto step = [&](int j, auto IC) {
+    constexpr int i = decltype(IC)::value;
+    auto body = [&](i32x4(&w)[NL], i32x2(&sc)[SU]) {
+      mma((j + i) / UPB, std::integral_constant<int, i % UPB>{}, w, sc);
+      __builtin_amdgcn_sched_barrier(0);
+      issue(j + i + 3, w, sc);
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    if constexpr (i % 3 == 0) body(w0, s0);
+    else if constexpr (i % 3 == 1) body(w1, s1);
+    else body(w2, s2r);
+  };
+  int j = 0;
+  for (; j + TRIP <= total; j += TRIP) static_for<0, TRIP>([&](auto IC) { step(j, IC); });
+  // remainder: fewer than TRIP steps, j is a multiple of TRIP (so of 3 and of UPB)
+  static_for<0, TRIP>([&](auto IC) {
+    if (j + decltype(IC)::value < total) step(j, IC);
+  });
+}
+
+template <int DT, int OUT, int SPB, int SU>
+int launch_skinny_directb_t(const GemmArgs& a, hipStream_t s) {
+  auto k = gemm_skinny_directb_kernel<DT, OUT, SPB, SU>;
+  constexpr int lds = 2 * 4 * 8 * 64 * 16 + 8 * 8192;
+  static std::atomic<uint64_t> attr_devs{0};
+  if (int e = lds_attr_once(attr_devs, (const void*)k, lds)) return e;
+  const int cus = device_cus();
+  if (cus <= 0) return (int)hipErrorNoDevice;
+  // what the kernel's indexing assumes: whole row blocks, packed rows of SPB * 8 steps
+  if (a.N % 16 != 0 || row_bytes(DT, a.K) != (int64_t)SPB * 1024 || a.ldb_bytes != row_bytes(DT, a.K))
+    return (int)hipErrorInvalidValue;
+  if (DT == ASTERGEMM_MXFP4 && (((uintptr_t)a.mx_b | (uintptr_t)a.mx_a) & 7) != 0)
+    return (int)hipErrorInvalidValue;
+  const int nblocks = (int)(a.N / 16);
+  const int g = nblocks < cus ? nblocks : cus;
+  hipLaunchKernelGGL(k, dim3(g), dim3(512), lds, s, a);
+  return (int)hipGetLastError();
+}
+
+template <int DT, int OUT>
+int launch_skinny_directb(const GemmArgs& a, int grid, hipStream_t s) {
+  (void)grid;
+  switch (row_bytes(DT, a.K)) {
+    case 2048: return launch_skinny_directb_t<DT, OUT, 2, 2>(a, s);
+    case 4096: return launch_skinny_directb_t<DT, OUT, 4, 4>(a, s);
+    case 8192: return launch_skinny_directb_t<DT, OUT, 8, 4>(a, s);
+  }  // 16 KiB rows: 128 activation registers next to three weight sets do not allocate
+  return (int)hipErrorInvalidValue;
+}
+
+const char* check_skinny_directb(const astergemm_config& c) {
+  if (c.M > 16) return "pre-shuffled B is supported for M <= 16";
+  const int64_t rb = row_bytes(c.dtype_ab, c.K);
+  if (rb != 2048 && rb != 4096 && rb != 8192)
+    return c.dtype_ab == ASTERGEMM_MXFP4 ? "pre-shuffled MXFP4 B is supported for K = 4096, 8192 or 16384"
+                                          : "pre-shuffled fp8 B is supported for K = 2048, 4096 or 8192";
+  if (c.N % 16 != 0) return "pre-shuffled B needs N % 16 == 0";
+  if (c.ldb != 0 && c.ldb != c.K) return "pre-shuffled B is packed (ldb = K)";
+  return nullptr;
+}
+
+#define AG_SKINNY_DIRECTB(name, DT, OUT)                                                      \
+  Variant {                                                                                   \
+    name, ASTERGEMM_KERNEL_SKINNY, DT, OUT, 16, 16, 512, 1, 8, 1, 1, 131072,                  \
+        (const void*)gemm_skinny_directb_kernel<DT, OUT, 4, 4>, launch_skinny_directb<DT, OUT>, \
+        check_skinny_directb, ASTERGEMM_OPERAND_DIRECT_B                                      \
+  }
+
 template <int DT, int OUT, int MT, int NB, int KW, int U>
 int launch_skinny(const GemmArgs& a, int grid, hipStream_t s) {
   hipLaunchKernelGGL((gemm_skinny_kernel<DT, OUT, MT, NB, KW, U>), dim3(grid), dim3(KW * 64), 0,
@@ -1739,6 +1991,12 @@ const Variant kSkinnyVariants[] = {
     AG_SKINNY_DIRECT("skinnyd_f16_m16_bf16", ASTERGEMM_F16, ASTERGEMM_BF16),
     AG_SKINNY_DIRECT("skinnyd_f16_m16_f32", ASTERGEMM_F16, ASTERGEMM_F32),
     AG_SKINNY_DIRECT("skinnyd_f16_m16_f16", ASTERGEMM_F16, ASTERGEMM_F16),
+    AG_SKINNY_DIRECTB("skinnyd_fp8_m16_bf16", ASTERGEMM_FP8_E4M3, ASTERGEMM_BF16),
+    AG_SKINNY_DIRECTB("skinnyd_fp8_m16_f32", ASTERGEMM_FP8_E4M3, ASTERGEMM_F32),
+    AG_SKINNY_DIRECTB("skinnyd_fp8_m16_f16", ASTERGEMM_FP8_E4M3, ASTERGEMM_F16),
+    AG_SKINNY_DIRECTB("skinnyd_mxfp4_m16_bf16", ASTERGEMM_MXFP4, ASTERGEMM_BF16),
+    AG_SKINNY_DIRECTB("skinnyd_mxfp4_m16_f32", ASTERGEMM_MXFP4, ASTERGEMM_F32),
+    AG_SKINNY_DIRECTB("skinnyd_mxfp4_m16_f16", ASTERGEMM_MXFP4, ASTERGEMM_F16),
 };
 
 }  // namespace

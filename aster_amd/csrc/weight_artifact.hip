@@ -69,9 +69,14 @@ extern "C" int astergemm_weight_header_init(astergemm_weight_header* h, int dtyp
   if (dtype == ASTERGEMM_MXFP4 && K % 32 != 0) return fail("MXFP4 needs K % 32 == 0");
   if (astergemm::row_bytes(dtype, K) % 16 != 0) return fail("a row must be a multiple of 16 bytes");
   if (layout == ASTERGEMM_OPERAND_DIRECT_B || layout == ASTERGEMM_OPERAND_DIRECT_B_K8) {
-    if (dtype != ASTERGEMM_F16 && dtype != ASTERGEMM_BF16)
-      return fail("the pre-shuffled layouts hold 16-bit elements");
-    if (N % 16 != 0 || K % 32 != 0) return fail("the pre-shuffled layouts need N % 16 == 0, K % 32 == 0");
+    const bool is16 = dtype == ASTERGEMM_F16 || dtype == ASTERGEMM_BF16;
+    if (!is16 && layout == ASTERGEMM_OPERAND_DIRECT_B_K8)
+      return fail("the K8 pre-shuffled layout holds 16-bit elements");
+    if (is16 && (N % 16 != 0 || K % 32 != 0))
+      return fail("the pre-shuffled layouts need N % 16 == 0, K % 32 == 0");
+    // fp8 / MXFP4: step order (astergemm_shuffle_weight_8, astergemm_shuffle_scales_e8m0)
+    if (!is16 && (N % 16 != 0 || astergemm::row_bytes(dtype, K) % 128 != 0))
+      return fail("the pre-shuffled layout of fp8 / MXFP4 needs N % 16 == 0 and rows of whole 128-byte steps");
   } else if (layout != ASTERGEMM_OPERAND_LDS) {
     return fail("unknown layout");
   }

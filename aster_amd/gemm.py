@@ -375,10 +375,16 @@ def execute_gemm_hsaco(cfg: WeakScaledMappedGemmInstance, hsaco_path: str, num_i
         # single point of truth, as in the reference's execute_fn
         # (test_102_gemm_python_multitile_g2s_directb_cdna4.py:446-467): the caller passes B
         # row-major and the pre-shuffle happens here, in the order the kernel that runs reads
-        from .kittens_helpers import shuffle_weight, shuffle_weight_k8
+        from .kittens_helpers import (shuffle_scales_e8m0, shuffle_weight, shuffle_weight_bytes,
+                                      shuffle_weight_k8)
 
-        shuffle = shuffle_weight if c.operand_path == _capi.OPERAND_DIRECT_B else shuffle_weight_k8
-        B = shuffle(np.ascontiguousarray(B).reshape(N, K))
+        if cfg.spec.dtype_ab in ("fp8_e4m3", "mxfp4"):   # byte rows in step order (+ the e8m0 plane)
+            B = shuffle_weight_bytes(np.ascontiguousarray(B).reshape(N, -1).view(np.uint8))
+            if mx_b is not None:
+                mx_b = shuffle_scales_e8m0(np.asarray(mx_b, dtype=np.uint8).reshape(N, K // 32))
+        else:
+            shuffle = shuffle_weight if c.operand_path == _capi.OPERAND_DIRECT_B else shuffle_weight_k8
+            B = shuffle(np.ascontiguousarray(B).reshape(N, K))
     C_host = np.zeros(M * N, dtype=out_np)
 
     def up(arr, dtype=None):

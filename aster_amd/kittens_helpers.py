@@ -93,3 +93,52 @@ def unshuffle_weight_k8(Bs: np.ndarray) -> np.ndarray:
     N, K = Bs.shape
     view = Bs.reshape(N // 16, K // 32, 4, 16, 8)
     return np.ascontiguousarray(view.transpose(0, 3, 1, 2, 4)).reshape(N, K)
+
+
+def shuffle_weight_bytes(B: np.ndarray) -> np.ndarray:
+    """Pre-shuffle the byte rows of an fp8 (B[N, K] uint8) or MXFP4 (B[N, K/2] uint8 nibble
+    pairs) weight matrix into STEP ORDER, the operand order of the 16x16x128 MFMA, which takes
+    the 16-byte pieces q and 4 + q of a 128-byte step of a row: view B as (n_block, n_lane=16,
+    step, half=2, lane_group=4, 16 bytes) and store it in the order (n_block, step, half,
+    lane_group, n_lane, 16 bytes).  Lane d of the KiB (nb, step, half) then finds bytes
+    [(4 half + d // 16) * 16, + 16) of row 16 nb + d % 16 at byte 16 d.  The reference's
+    `shuffle_weight` (kittens_helpers.py:90-119) is the same idea for 2-byte elements and the
+    16x16x16 MFMA; it has no byte-type form."""
+    B = np.ascontiguousarray(B)
+    if B.dtype.itemsize != 1 or B.ndim != 2:
+        raise AssertionError("shuffle_weight_bytes takes a 2-D array of one-byte elements")
+    N, rb = B.shape
+    if N % 16 != 0:
+        raise AssertionError(f"N={N} must be multiple of 16")
+    if rb % 128 != 0:
+        raise AssertionError(f"rows of {rb} bytes are not whole 128-byte steps")
+    view = B.reshape(N // 16, 16, rb // 128, 2, 4, 16)
+    return np.ascontiguousarray(view.transpose(0, 2, 3, 4, 1, 5)).reshape(N, rb)
+
+
+def unshuffle_weight_bytes(Bs: np.ndarray) -> np.ndarray:
+    """Inverse of `shuffle_weight_bytes`."""
+    N, rb = Bs.shape
+    view = np.ascontiguousarray(Bs).reshape(N // 16, rb // 128, 2, 4, 16, 16)
+    return np.ascontiguousarray(view.transpose(0, 4, 1, 2, 3, 5)).reshape(N, rb)
+
+
+def shuffle_scales_e8m0(S: np.ndarray) -> np.ndarray:
+    """The e8m0 plane S[N, K/32] of pre-shuffled MXFP4 weights in the matching order: view it as
+    (n_block, n_lane=16, step, 8 bytes) and store (n_block, step, n_lane, 8 bytes), so that the
+    scales of a row block and 256-element step are one 128-byte line."""
+    S = np.ascontiguousarray(S, dtype=np.uint8)
+    N, nb = S.shape
+    if N % 16 != 0:
+        raise AssertionError(f"N={N} must be multiple of 16")
+    if nb % 8 != 0:
+        raise AssertionError(f"{nb} scale bytes per row are not whole 256-element steps")
+    view = S.reshape(N // 16, 16, nb // 8, 8)
+    return np.ascontiguousarray(view.transpose(0, 2, 1, 3)).reshape(N, nb)
+
+
+def unshuffle_scales_e8m0(Ss: np.ndarray) -> np.ndarray:
+    """Inverse of `shuffle_scales_e8m0`."""
+    N, nb = Ss.shape
+    view = np.ascontiguousarray(Ss).reshape(N // 16, nb // 8, 16, 8)
+    return np.ascontiguousarray(view.transpose(0, 2, 1, 3)).reshape(N, nb)

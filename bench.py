@@ -461,6 +461,11 @@ def main() -> int:
             sets = [dict(dA=a.data_ptr(), dB=w.data_ptr(), dC=c.data_ptr(), **kw) for w in wts]
             p.bench_rotate(sets, 48)
             rot_ns = p.bench_rotate(sets, 240) / 240.0
+            # the same bytes read as weights pre-shuffled into the MFMA's operand order
+            # (operand_path direct_b; values do not matter for the timing)
+            pd = AG.GemmPlan.create(16, 14336, 4096, dt, "bf16", operand_path="direct_b")
+            pd.bench_rotate(sets, 48)
+            rot_d_ns = pd.bench_rotate(sets, 240) / 240.0
             del wts, sets
             others.append({"workload": f"{dt} skinny GEMM M=16 N=14336 K=4096 -> bf16, LLC flushed "
                                        "before every launch",
@@ -469,7 +474,9 @@ def main() -> int:
                            "frac": round(p.info.bytes / p50 / PEAK_HBM_GBPS, 4),
                            f"us_back_to_back_{nsets}_weight_sets": round(rot_ns / 1e3, 2),
                            "gbps_back_to_back": round(p.info.bytes / rot_ns, 1),
-                           "frac_back_to_back": round(p.info.bytes / rot_ns / PEAK_HBM_GBPS, 4)})
+                           "frac_back_to_back": round(p.info.bytes / rot_ns / PEAK_HBM_GBPS, 4),
+                           "kernel_weights_pre_shuffled": pd.info.name.decode(),
+                           "us_back_to_back_weights_pre_shuffled": round(rot_d_ns / 1e3, 2)})
         # the same M = 16 shape with the weights pre-shuffled into MFMA operand order
         # (the reference's operand_path = direct_b); values do not matter for the timing
         del a, b, c

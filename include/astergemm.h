@@ -82,10 +82,13 @@ typedef enum astergemm_kernel_family {
  * global load is its MFMA operand and B never passes through LDS.            */
 typedef enum astergemm_operand_path {
   ASTERGEMM_OPERAND_LDS = 0,      /* B[N, ldb] row-major as described below   */
-  ASTERGEMM_OPERAND_DIRECT_B = 1, /* B packed [N, K] and pre-shuffled with
-                                     astergemm_shuffle_weight_16, the
-                                     reference's order (16-bit operands; the
-                                     decode kernels, M <= 16)                */
+  ASTERGEMM_OPERAND_DIRECT_B = 1, /* B packed [N, K] and pre-shuffled: 16-bit
+                                     operands with astergemm_shuffle_weight_16,
+                                     the reference's order; fp8 and MXFP4
+                                     payloads with astergemm_shuffle_weight_8
+                                     (MXFP4: dMxB pre-shuffled as well, with
+                                     astergemm_shuffle_scales_e8m0).  The
+                                     decode kernels, M <= 16                 */
   ASTERGEMM_OPERAND_DIRECT_B_K8 = 2 /* B packed [N, K] and pre-shuffled with
                                      astergemm_shuffle_weight_k8_16: 8
                                      consecutive K per lane, the order of the
@@ -253,6 +256,21 @@ int astergemm_shuffle_weight_16(const uint16_t* src, uint16_t* dst, int64_t N,
 int astergemm_shuffle_weight_k8_16(const uint16_t* src, uint16_t* dst, int64_t N,
                                    int64_t K);
 
+/* The pre-shuffle for the one-byte and nibble types (fp8 e4m3, MXFP4 payload),
+ * whose 16x16x128 MFMA takes the 16-byte pieces q and 4 + q of a 128-byte step
+ * of a row: rows of `row_bytes` bytes (K for fp8, K / 2 for MXFP4; whole
+ * 128-byte steps), N % 16 == 0.  Row block nb (16 rows), step s, half u is one
+ * KiB at ((nb * steps + s) * 2 + u) * 1024 in which lane 16 q + n of a wave
+ * finds bytes [(4u + q) * 16, + 16) of row 16 nb + n, step s, at byte
+ * 16 (16 q + n).  The reference has no counterpart for these types; it is the
+ * generalisation of its shuffle_weight (kittens_helpers.py:90-119) to the
+ * operand order of v_mfma_scale_f32_16x16x128_f8f6f4. */
+int astergemm_shuffle_weight_8(const uint8_t* src, uint8_t* dst, int64_t N, int64_t row_bytes);
+/* The e8m0 plane [N, K/32] of pre-shuffled MXFP4 weights in the matching
+ * order: the 8 scale bytes of row 16 nb + n, step s (256 elements) at
+ * (nb * steps + s) * 128 + 8 n.  N % 16 == 0, K % 256 == 0. */
+int astergemm_shuffle_scales_e8m0(const uint8_t* src, uint8_t* dst, int64_t N, int64_t K);
+
 /* ---- operand quantisers (device to device, on `stream`) -------------------
  * They write the bytes the fp8 / MXFP4 GEMM paths read (dtype_ab
  * ASTERGEMM_FP8_E4M3 / ASTERGEMM_MXFP4), so that a caller holding activations
@@ -301,9 +319,10 @@ int astergemm_quantize_mxfp4(const void* dSrc, int src_dtype, int64_t rows, int6
  * File = this 128-byte little-endian header, then the payload at
  * payload_offset (N rows; layout ASTERGEMM_OPERAND_LDS = row-major,
  * ASTERGEMM_OPERAND_DIRECT_B = astergemm_shuffle_weight_16 order,
- * ASTERGEMM_OPERAND_DIRECT_B_K8 = astergemm_shuffle_weight_k8_16 order, the
- * pre-shuffled ones for 16-bit dtypes only), then for MXFP4 the e8m0 plane
- * [N, K/32] at scales_offset.
+ * ASTERGEMM_OPERAND_DIRECT_B_K8 = astergemm_shuffle_weight_k8_16 order, 16-bit
+ * dtypes only; for fp8 and MXFP4 ASTERGEMM_OPERAND_DIRECT_B =
+ * astergemm_shuffle_weight_8 order), then for MXFP4 the e8m0 plane [N, K/32]
+ * at scales_offset (layout DIRECT_B: in astergemm_shuffle_scales_e8m0 order).
  * Sections start on 256-byte boundaries.  FP8 carries its tensor scale in the
  * header.  Checksums are CRC-32 (the zlib polynomial) of each section.       */
 #define ASTERGEMM_WEIGHT_VERSION 1u

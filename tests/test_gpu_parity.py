@@ -1086,6 +1086,41 @@ def test_skinny_direct_b_preshuffled_weights(gpu, M, N, K, dtype_ab, dtype_c):
     assert np.isnan(pad).all() if dtype_c == "f32" else (pad == 0x7FC1).all()
 
 
+@pytest.mark.parametrize("M,N", [(16, 14336), (1, 16), (5, 784), (13, 6000), (16, 48), (9, 4112),
+                                 (16, 4096 + 16 * 7)])
+@pytest.mark.parametrize("dtype_ab,K,dtype_c", [("fp8_e4m3", 4096, "bf16"), ("fp8_e4m3", 2048, "f32"),
+                                                ("fp8_e4m3", 8192, "f16"), ("mxfp4", 8192, "bf16"),
+                                                ("mxfp4", 4096, "f32"), ("mxfp4", 16384, "f32")])
+def test_skinny_direct_b_preshuffled_fp8_and_mxfp4_weights(gpu, M, N, dtype_ab, K, dtype_c):
+    """operand_path = direct_b for the one-byte and nibble types: the payload rows in the step
+    order of `shuffle_weight_bytes`, the MXFP4 scale plane in the order of `shuffle_scales_e8m0`;
+    the result must equal the oracle's GEMM on the unshuffled weights, and the kernel that reads
+    the same weights row-major through LDS to summation order.  Row ranges that start or end
+    inside a 16-row block, single-workgroup grids, bias and a padded output pitch."""
+    from aster_amd.kittens_helpers import shuffle_scales_e8m0, shuffle_weight_bytes
+    a, b, ex = operands(M, N, K, dtype_ab, seed=57, b_std=0.05)
+    bias = np.random.default_rng(58).standard_normal(N).astype(np.float32)
+    ldc = (N + 11) & ~3
+    ex_dev = dict(ex)
+    if dtype_ab == "mxfp4":
+        ex_dev["mx_b"] = shuffle_scales_e8m0(ex["mx_b"])
+    out, name = run_gemm(a, shuffle_weight_bytes(np.asarray(b).view(np.uint8)), M, N, K, dtype_ab, dtype_c,
+                         bias=bias, ldc=ldc, operand_path="direct_b", **ex_dev)
+    assert name.startswith("skinnyd_" + ("fp8" if dtype_ab == "fp8_e4m3" else "mxfp4"))
+    want = G.gemm(a, b, _DT[dtype_ab], _DT[dtype_c], bias=bias, **ex)
+    if dtype_c == "f32" or M * N >= 4096:
+        check(out, want, dtype_c, N, bar=1e-4 if dtype_c == "f32" else REL_L2_BAR)
+    else:  # few outputs: bound every element (see test_skinny_fp8_resident_activations)
+        got, ref = G.output_to_f32(out[:, :N], _DT[dtype_c]), G.output_to_f32(want, _DT[dtype_c])
+        assert np.all(np.abs(got - ref) <= 2.0 ** -6 * np.abs(ref) + 1e-4 * np.abs(ref).max())
+    pad = out[:, N:]
+    assert np.isnan(pad).all() if dtype_c == "f32" else (pad == 0x7FC1).all()
+    plain, pname = run_gemm(a, b, M, N, K, dtype_ab, dtype_c, bias=bias, ldc=ldc, **ex)
+    assert not pname.startswith("skinnyd")
+    assert G.rel_l2(G.output_to_f32(out[:, :N], _DT[dtype_c]), G.output_to_f32(plain[:, :N], _DT[dtype_c])) \
+        <= (1e-5 if dtype_c == "f32" else REL_L2_BAR)
+
+
 # ---- B pre-shuffled in K8 order, loaded straight into MFMA operands (256 x 256 stream kernel) ---
 
 @pytest.mark.parametrize("M,N,K", [(256, 256, 64), (256, 256, 128), (512, 768, 576), (512, 512, 640),

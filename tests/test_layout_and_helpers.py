@@ -236,3 +236,42 @@ def test_stream_kernel_staging_is_the_interleaved_coop_plan(tile_rows, num_waves
     # the slot is filled exactly once: every 1 KiB of it, every 8-row group of the tile
     assert sorted(lo for _, lo in everything) == [t * 1024 for t in range(tile_rows // 8)]
     assert sorted(go for go, _ in everything) == [t * 8 * ld for t in range(tile_rows // 8)]
+
+
+def test_shuffle_weight_bytes_is_the_operand_order_of_the_16x16x128_mfma():
+    # lane 16 q + n of the KiB (row block nb, step s, half u) holds bytes [(4u + q) * 16, + 16) of
+    # row 16 nb + n, step s; the C-ABI function writes the same bytes; the inverse restores them
+    import ctypes
+    from aster_amd import _capi
+    from aster_amd.kittens_helpers import (shuffle_scales_e8m0, shuffle_weight_bytes,
+                                           unshuffle_scales_e8m0, unshuffle_weight_bytes)
+    rng = np.random.default_rng(5)
+    N, rb = 48, 384
+    b = rng.integers(0, 256, (N, rb)).astype(np.uint8)
+    sh = shuffle_weight_bytes(b)
+    flat = sh.reshape(-1)
+    steps = rb // 128
+    for (nb, st, u, q, n) in ((0, 0, 0, 0, 0), (2, 1, 1, 3, 15), (1, 2, 0, 2, 7), (2, 2, 1, 0, 9)):
+        at = ((nb * steps + st) * 2 + u) * 1024 + (16 * q + n) * 16
+        assert np.array_equal(flat[at:at + 16], b[16 * nb + n, st * 128 + (4 * u + q) * 16:][:16])
+    assert np.array_equal(unshuffle_weight_bytes(sh), b)
+    out = np.empty_like(b)
+    _capi.check(_capi.load().astergemm_shuffle_weight_8(b.ctypes.data, out.ctypes.data, N, rb))
+    assert np.array_equal(out, sh)
+    with pytest.raises(AssertionError):
+        shuffle_weight_bytes(b[:40])
+    with pytest.raises(AssertionError):
+        shuffle_weight_bytes(b[:, :200])
+    # the scale plane: the 8 bytes of row 16 nb + n, step s at (nb * steps + s) * 128 + 8 n
+    K = 768
+    mx = rng.integers(0, 256, (N, K // 32)).astype(np.uint8)
+    ss = shuffle_scales_e8m0(mx)
+    sflat, ssteps = ss.reshape(-1), K // 256
+    for (nb, st, n) in ((0, 0, 0), (2, 2, 15), (1, 1, 6)):
+        at = (nb * ssteps + st) * 128 + 8 * n
+        assert np.array_equal(sflat[at:at + 8], mx[16 * nb + n, st * 8:][:8])
+    assert np.array_equal(unshuffle_scales_e8m0(ss), mx)
+    out = np.empty_like(mx)
+    _capi.check(_capi.load().astergemm_shuffle_scales_e8m0(mx.ctypes.data, out.ctypes.data, N, K))
+    assert np.array_equal(out, ss)
+    assert _capi.load().astergemm_shuffle_scales_e8m0(mx.ctypes.data, out.ctypes.data, N, K + 32) != 0

@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 
 from aster_amd import _capi, weights as W
-from aster_amd.kittens_helpers import shuffle_weight
+from aster_amd.kittens_helpers import shuffle_scales_e8m0, shuffle_weight, shuffle_weight_bytes
 
 
 def _bf16(x):
@@ -41,10 +41,11 @@ def test_crc32_is_the_zlib_polynomial():
 
 
 @pytest.mark.parametrize("dtype,layout", [("bf16", "lds"), ("f16", "direct_b"), ("fp8_e4m3", "lds"),
-                                           ("mxfp4", "lds")])
+                                           ("mxfp4", "lds"), ("fp8_e4m3", "direct_b"),
+                                           ("mxfp4", "direct_b")])
 def test_save_load_round_trip(tmp_path, dtype, layout):
     rng = np.random.default_rng(5)
-    N, K = 48, 128
+    N, K = 48, 256
     scales, ts = None, 1.0
     if dtype in ("bf16", "f16"):
         bits = rng.integers(0, 1 << 16, (N, K), dtype=np.uint16)
@@ -108,8 +109,10 @@ def test_corrupt_files_are_refused_with_a_reason(tmp_path):
 
 
 def test_packing_rules():
-    with pytest.raises(_capi.AsterGemmError, match="16-bit"):
+    with pytest.raises(_capi.AsterGemmError, match="128-byte steps"):
         W.WeightArtifact.from_storage(np.zeros((16, 32), np.uint8), "fp8_e4m3", 16, 32, layout="direct_b")
+    with pytest.raises(_capi.AsterGemmError, match="16-bit"):
+        W.WeightArtifact.from_storage(np.zeros((16, 128), np.uint8), "fp8_e4m3", 16, 128, layout="direct_b_k8")
     with pytest.raises(_capi.AsterGemmError, match="N % 16"):
         W.WeightArtifact.from_storage(np.zeros((8, 32), np.uint16), "bf16", 8, 32, layout="direct_b")
     with pytest.raises(ValueError, match="scale plane"):
@@ -129,7 +132,9 @@ def test_packing_rules():
 @pytest.mark.parametrize("dtype,layout,M,N,K", [("bf16", "lds", 16, 512, 4096), ("bf16", "direct_b", 16, 512, 4096),
                                                 ("bf16", "direct_b_k8", 264, 512, 1024),
                                                 ("f16", "lds", 40, 264, 256), ("fp8_e4m3", "lds", 16, 512, 4096),
-                                                ("fp8_e4m3", "lds", 300, 256, 512), ("mxfp4", "lds", 64, 256, 1024)])
+                                                ("fp8_e4m3", "lds", 300, 256, 512), ("mxfp4", "lds", 64, 256, 1024),
+                                                ("fp8_e4m3", "direct_b", 16, 528, 4096),
+                                                ("mxfp4", "direct_b", 9, 528, 8192)])
 def test_artifact_to_gemm_matches_the_oracle(tmp_path, dtype, layout, M, N, K):
     from aster_amd import quantize as Q
     from aster_amd.execution import GpuBuffer
@@ -153,7 +158,9 @@ def test_artifact_to_gemm_matches_the_oracle(tmp_path, dtype, layout, M, N, K):
     elif dtype == "fp8_e4m3":
         xs, sx = F.quantize_fp8_tensor(x)
         wq, sw = F.quantize_fp8_tensor(w)
-        assert np.array_equal(np.asarray(art.payload).reshape(N, K), wq) and art.tensor_scale == sw
+        stored = np.asarray(art.payload).reshape(N, K)
+        assert np.array_equal(stored, shuffle_weight_bytes(wq) if layout == "direct_b" else wq)
+        assert art.tensor_scale == sw
         d_sx = GpuBuffer(4); d_sx.copy_from_host(np.array([sx], np.float32))
         kw["scale_x"] = d_sx.ptr_value
         want = G.gemm_fp8(xs, wq, sx, sw, out_dtype=G.F32)
@@ -161,8 +168,9 @@ def test_artifact_to_gemm_matches_the_oracle(tmp_path, dtype, layout, M, N, K):
     else:
         xs, mx = F.quantize_mxfp4(x)
         wq, ws = F.quantize_mxfp4(w)
-        assert np.array_equal(np.asarray(art.payload).reshape(N, K // 2), wq)
-        assert np.array_equal(np.asarray(art.scales).reshape(N, K // 32), ws)
+        stored, plane = np.asarray(art.payload).reshape(N, K // 2), np.asarray(art.scales).reshape(N, K // 32)
+        assert np.array_equal(stored, shuffle_weight_bytes(wq) if layout == "direct_b" else wq)
+        assert np.array_equal(plane, shuffle_scales_e8m0(ws) if layout == "direct_b" else ws)
         d_mx = GpuBuffer(mx.nbytes); d_mx.copy_from_host(mx)
         kw["mx_x"] = d_mx.ptr_value
         want = G.gemm_mxfp4(xs, mx, wq, ws, out_dtype=G.F32)
