@@ -118,7 +118,9 @@ def select_for_instance(cfg: WeakScaledMappedGemmInstance) -> Tuple[_capi.Config
     returned config's `operand_path` says which; `execute_gemm_hsaco` shuffles accordingly) --
     and falls back to plain row-major B otherwise."""
     want_direct = cfg.mapping.direct_b and not cfg.mapping.direct_a
-    paths = [_capi.OPERAND_DIRECT_B, _capi.OPERAND_DIRECT_B_K8] if want_direct else []
+    paths = [_capi.OPERAND_DIRECT_B] if want_direct else []
+    if want_direct and cfg.spec.dtype_ab in ("bf16", "f16"):
+        paths.append(_capi.OPERAND_DIRECT_B_K8)          # the K8 order holds 16-bit elements
     for use_mapping in (True, False):
         for path in paths + [_capi.OPERAND_LDS]:
             if not use_mapping and path == _capi.OPERAND_LDS and not want_direct:

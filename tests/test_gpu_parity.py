@@ -1170,6 +1170,23 @@ def test_direct_b_mapping_through_the_harness_seam(gpu, tmp_path):
     check(c_flat.reshape(512, 768), G.gemm(a, b, G.BF16, G.BF16), "bf16", 768)
 
 
+@pytest.mark.parametrize("dtype_ab,K", [("fp8_e4m3", 4096), ("mxfp4", 8192)])
+def test_direct_b_mapping_of_a_decode_shape_with_byte_operands(gpu, tmp_path, dtype_ab, K):
+    # the same seam for fp8 / MXFP4 on a decode shape: the DIRECT_B mapping selects the kernel that
+    # reads the payload in step order, execute_gemm_hsaco shuffles the row-major payload (and the
+    # MXFP4 scale plane) it is given
+    M, N = 16, 528
+    cfg = make_instance(M, N, K, dtype_ab=dtype_ab, dtype_c="f32", wg_tile=(16, 16), waves=(1, 1),
+                        operand_path=OperandPath.DIRECT_B)
+    path, asm = AG.compile_gemm(cfg, str(tmp_path / "k.hsaco"))
+    desc = json.load(open(path))
+    assert desc["kernel"].startswith("skinnyd_") and desc["operand_path"] == "direct_b"
+    a, b, ex = operands(M, N, K, dtype_ab, seed=91, b_std=0.05)
+    c_flat, times = AG.execute_gemm_hsaco(cfg, path, 2, a, b, **ex)
+    want = G.gemm(a, b, _DT[dtype_ab], G.F32, **ex)
+    check(c_flat.reshape(M, N), want, "f32", N, bar=1e-4)
+
+
 def test_direct_b_is_refused_where_it_is_not_implemented(gpu):
     for kw in (dict(M=128, N=256, K=4096), dict(M=16, N=256, K=1024), dict(M=16, N=24, K=4096)):
         with pytest.raises(_capi.AsterGemmError):
