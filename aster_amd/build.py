@@ -64,8 +64,9 @@ def _compile(src: str) -> str:
     if found:
         lines = "\n".join(f"  {asm}:{no}: {mfma}\n      written at line {wno}: {writer}"
                           for (no, mfma, wno, writer) in found[:20])
-        raise RuntimeError(f"{src}: {len(found)} inline-asm MFMA(s) read a register a VALU instruction "
-                           f"wrote fewer than {MFMA_WAIT_STATES} wait states earlier:\n{lines}")
+        raise RuntimeError(f"{src}: {len(found)} inline-asm instruction(s) read a register a VALU instruction "
+                           f"wrote too few wait states earlier (MFMA sources: {MFMA_WAIT_STATES}, scalar "
+                           f"bases of vector-memory instructions: {VMEM_SGPR_WAIT_STATES}):\n{lines}")
     return obj
 
 
@@ -80,9 +81,27 @@ def _compile(src: str) -> str:
 # `s_nop 1` in front of the MFMAs elsewhere; this scan of the generated assembly is the proof.
 
 MFMA_WAIT_STATES = 2
+# The same blind spot for the transfers (global_load_lds_* / buffer_load_* written as inline asm with
+# a scalar base): an SGPR written by a VALU instruction (v_readlane restoring a spilled SGPR,
+# v_readfirstlane, a compare into an SGPR pair) must not be read by a vector-memory instruction
+# for five wait states.
+VMEM_SGPR_WAIT_STATES = 5
 
 _REG_RANGE = re.compile(r"([va])\[(\d+):(\d+)\]$")
 _REG_ONE = re.compile(r"([va])(\d+)$")
+
+
+_SREG_RANGE = re.compile(r"s\[(\d+):(\d+)\]$")
+_SREG_ONE = re.compile(r"s(\d+)$")
+
+
+def _sregs(tok: str) -> set:
+    tok = tok.strip().rstrip(",")
+    m = _SREG_RANGE.match(tok)
+    if m:
+        return {("s", i) for i in range(int(m.group(1)), int(m.group(2)) + 1)}
+    m = _SREG_ONE.match(tok)
+    return {("s", int(m.group(1)))} if m else set()
 
 
 def _regs(tok: str) -> set:
@@ -95,9 +114,11 @@ def _regs(tok: str) -> set:
 
 
 def scan_mfma_hazards(asm_text: str, wait_states: int = MFMA_WAIT_STATES):
-    """[(line, mfma text, writer line, writer text)] for every MFMA inside an inline-asm block of
-    gfx9 assembly text whose A, B, C or scale registers were written by a VALU instruction fewer
-    than `wait_states` wait states earlier (an instruction is one wait state, `s_nop n` is n + 1)."""
+    """[(line, instruction text, writer line, writer text)] for every MFMA inside an inline-asm block
+    of gfx9 assembly text whose A, B, C or scale registers were written by a VALU instruction fewer
+    than `wait_states` wait states earlier (an instruction is one wait state, `s_nop n` is n + 1),
+    and for every vector-memory instruction inside an inline-asm block whose SGPR operands were
+    written by a VALU instruction fewer than VMEM_SGPR_WAIT_STATES wait states earlier."""
     found = []
     hist = []      # (wait states, registers written by a VALU instruction, text, line)
     in_asm = False
@@ -136,10 +157,25 @@ def scan_mfma_hazards(asm_text: str, wait_states: int = MFMA_WAIT_STATES):
             w, written = 1, set()
             if op == "s_nop":
                 w = int(toks[0], 0) + 1 if toks else 1
-            elif op.startswith("v_") and not op.startswith(("v_cmp", "v_readlane", "v_readfirstlane")):
+            elif op.startswith(("v_readlane", "v_readfirstlane")) or \
+                    (op.startswith("v_cmp") and toks and toks[0].startswith("s")):
+                written = _sregs(toks[0]) if toks else set()
+            elif op.startswith("v_") and not op.startswith("v_cmp"):
                 written = _regs(toks[0]) if toks else set()
+            if in_asm and op.startswith(("global_load", "global_store", "buffer_load", "buffer_store")):
+                srcs = set()
+                for t in toks:
+                    if t.split():
+                        srcs |= _sregs(t.split()[0])
+                ws = 0
+                for (w2, written2, text, wno) in reversed(hist):
+                    if ws >= VMEM_SGPR_WAIT_STATES:
+                        break
+                    if written2 & srcs:
+                        found.append((no, l[:110], wno, text[:90]))
+                    ws += w2
             hist.append((w, written, l, no))
-        if len(hist) > 8:
+        if len(hist) > 12:
             hist.pop(0)
     return found
 

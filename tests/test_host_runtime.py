@@ -365,3 +365,9 @@ def test_build_scan_finds_a_register_copy_in_front_of_an_inline_asm_mfma():
     assert scan_mfma_hazards("\tv_mov_b32_e32 v40, v41\n" + mfma.format(pre="")) == []
     # MFMAs the compiler emitted itself are its own business
     assert scan_mfma_hazards(copy + "\tv_mfma_f32_16x16x32_bf16 a[0:3], v[36:39], v[4:7], a[0:3]\n") == []
+    # a spilled scalar base restored by v_readlane right in front of an inline-asm transfer
+    g2s = ("\t;;#ASMSTART\n\ts_mov_b32 m0, s12\n\ts_nop 0\n\tglobal_load_lds_dwordx4 v9, s[4:5]\n"
+           "\t;;#ASMEND\n")
+    assert len(scan_mfma_hazards("\tv_readlane_b32 s4, v127, 3\n\tv_readlane_b32 s5, v127, 4\n" + g2s)) == 2
+    assert scan_mfma_hazards("\tv_readlane_b32 s4, v127, 3\n\ts_nop 3\n" + g2s) == []
+    assert scan_mfma_hazards("\ts_add_u32 s4, s6, s7\n" + g2s) == []
