@@ -238,15 +238,17 @@ const char* check_stream4_walk(const astergemm_config& c) {
   if (const char* why = check_stream4(c)) return why;
   if (c.K % 1024 != 0) return "the tile walk needs K to be a multiple of 1024";
   if (c.M % 256 != 0 || c.N % 256 != 0) return "the tile walk needs M and N to be multiples of 256";
-  const int cus = device_cus();
-  if (cus > 0 && ((c.M + 255) / 256) * ((c.N + 255) / 256) <= cus)
+  int cus = device_cus();
+  if (cus <= 0) cus = 256;                       // no device to ask: describe the MI355X
+  if (((c.M + 255) / 256) * ((c.N + 255) / 256) <= cus)
     return "the tile walk pays from two tiles per workgroup on";
   return nullptr;
 }
 
 int grid_stream4_walk(const astergemm_config& c, int cus) {
   const int64_t tiles = ((c.M + 255) / 256) * ((c.N + 255) / 256);
-  return (int)(cus > 0 && tiles > cus ? cus : tiles);
+  if (cus <= 0) cus = 256;
+  return (int)(tiles > cus ? cus : tiles);
 }
 
 #define AG_STREAM4_WALK(name, DT, OUT)                                           \
@@ -376,8 +378,8 @@ int grid_stream_tail(const astergemm_config& c, int cus) {
   const int64_t m2 = ts.along == 2 ? c.M - ts.first : c.M, n2 = ts.along == 1 ? c.N - ts.first : c.N;
   int64_t g1 = ((m1 + 255) / 256) * ((n1 + 255) / 256);
   // MXFP4: the whole rounds run as a tile walk, one workgroup per CU (see launch_stream_tail)
-  if (c.dtype_ab == ASTERGEMM_MXFP4 && c.K % 1024 == 0 && m1 % 256 == 0 && n1 % 256 == 0 && cus > 0 &&
-      g1 > cus)
+  if (cus <= 0) cus = 256;
+  if (c.dtype_ab == ASTERGEMM_MXFP4 && c.K % 1024 == 0 && m1 % 256 == 0 && n1 % 256 == 0 && g1 > cus)
     g1 = cus;
   return (int)(g1 + ((m2 + 127) / 128) * ((n2 + 127) / 128));
 }
