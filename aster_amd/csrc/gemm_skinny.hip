@@ -37,6 +37,33 @@ __device__ __forceinline__ unsigned short sk_f32_to_bf16(float f) {
   return (unsigned short)(u >> 16);
 }
 
+// C[m][n .. n + ncols) = cast(v): the four neighbours one lane owns; one vector store where the
+// row pitch keeps it aligned and all four columns exist.
+template <int OUT>
+__device__ __forceinline__ void sk_store_row4(void* C, int64_t ldc, int m, int n, const f32x4& v, int ncols) {
+  const int64_t idx = (int64_t)m * ldc + n;
+  const bool vec_ok = (ldc & 3) == 0 && ncols == 4;
+  if constexpr (OUT == ASTERGEMM_F32) {
+    float* o = (float*)C + idx;
+    if (vec_ok) *(f32x4*)o = v;
+    else
+      for (int r = 0; r < ncols; ++r) o[r] = v[r];
+  } else {
+    unsigned short h[4];
+    for (int r = 0; r < 4; ++r) {
+      if constexpr (OUT == ASTERGEMM_BF16) h[r] = sk_f32_to_bf16(v[r]);
+      else {
+        const _Float16 hh = (_Float16)v[r];
+        h[r] = __builtin_bit_cast(unsigned short, hh);
+      }
+    }
+    unsigned short* o = (unsigned short*)C + idx;
+    if (vec_ok) *(u16x4*)o = u16x4{h[0], h[1], h[2], h[3]};
+    else
+      for (int r = 0; r < ncols; ++r) o[r] = h[r];
+  }
+}
+
 template <int I, int N, class Fn>
 __device__ __forceinline__ void static_for(Fn&& f) {
   if constexpr (I < N) {
@@ -134,7 +161,6 @@ __global__ __launch_bounds__(KW * 64) void gemm_skinny_kernel(const GemmArgs p) 
   float scale = 1.0f;
   if (p.scale_a) scale *= *p.scale_a;
   if (p.scale_b) scale *= *p.scale_b;
-  const bool vec_ok = (p.ldc & 3) == 0;
   // Lane l of tile (t, b) owns C[t*16 + l%16][n0 + b*16 + 4*(l/16) + 0..3].
   for (int e = threadIdx.x; e < MT * NB * 64; e += KW * 64) {
     const int tb = e >> 6, l = e & 63;
@@ -149,26 +175,7 @@ __global__ __launch_bounds__(KW * 64) void gemm_skinny_kernel(const GemmArgs p) 
     const int ncols = (p.N - n) < 4 ? (p.N - n) : 4;
     if (p.bias)
       for (int r = 0; r < ncols; ++r) v[r] += p.bias[n + r];
-    const int64_t idx = (int64_t)m * p.ldc + n;
-    if constexpr (OUT == ASTERGEMM_F32) {
-      float* o = (float*)p.C + idx;
-      if (vec_ok && ncols == 4) *(f32x4*)o = v;
-      else
-        for (int r = 0; r < ncols; ++r) o[r] = v[r];
-    } else {
-      unsigned short h[4];
-      for (int r = 0; r < 4; ++r) {
-        if constexpr (OUT == ASTERGEMM_BF16) h[r] = sk_f32_to_bf16(v[r]);
-        else {
-          _Float16 hh = (_Float16)v[r];
-          h[r] = __builtin_bit_cast(unsigned short, hh);
-        }
-      }
-      unsigned short* o = (unsigned short*)p.C + idx;
-      if (vec_ok && ncols == 4) *(u16x4*)o = u16x4{h[0], h[1], h[2], h[3]};
-      else
-        for (int r = 0; r < ncols; ++r) o[r] = h[r];
-    }
+    sk_store_row4<OUT>(p.C, p.ldc, m, n, v, ncols);
   }
 }
 
@@ -312,27 +319,7 @@ __global__ __launch_bounds__(512) void gemm_skinny_reg_kernel(const GemmArgs p) 
         const int ncols = (r1 - n) < 4 ? (r1 - n) : 4;
         if (p.bias)
           for (int r = 0; r < ncols; ++r) v[r] += p.bias[n + r];
-        const int64_t idx = (int64_t)m * p.ldc + n;
-        const bool vec_ok = (p.ldc & 3) == 0 && ncols == 4;
-        if constexpr (OUT == ASTERGEMM_F32) {
-          float* o = (float*)p.C + idx;
-          if (vec_ok) *(f32x4*)o = v;
-          else
-            for (int r = 0; r < ncols; ++r) o[r] = v[r];
-        } else {
-          unsigned short h[4];
-          for (int r = 0; r < 4; ++r) {
-            if constexpr (OUT == ASTERGEMM_BF16) h[r] = sk_f32_to_bf16(v[r]);
-            else {
-              _Float16 hh = (_Float16)v[r];
-              h[r] = __builtin_bit_cast(unsigned short, hh);
-            }
-          }
-          unsigned short* o = (unsigned short*)p.C + idx;
-          if (vec_ok) *(u16x4*)o = u16x4{h[0], h[1], h[2], h[3]};
-          else
-            for (int r = 0; r < ncols; ++r) o[r] = h[r];
-        }
+        sk_store_row4<OUT>(p.C, p.ldc, m, n, v, ncols);
       }
     }
     parity ^= 1;
@@ -532,27 +519,7 @@ __global__ __launch_bounds__(512) void gemm_skinny_fp4_kernel(const GemmArgs p) 
         const int ncols = (r1 - n) < 4 ? (r1 - n) : 4;
         if (p.bias)
           for (int r = 0; r < ncols; ++r) v[r] += p.bias[n + r];
-        const int64_t idx = (int64_t)m * p.ldc + n;
-        const bool vec_ok = (p.ldc & 3) == 0 && ncols == 4;
-        if constexpr (OUT == ASTERGEMM_F32) {
-          float* o = (float*)p.C + idx;
-          if (vec_ok) *(f32x4*)o = v;
-          else
-            for (int r = 0; r < ncols; ++r) o[r] = v[r];
-        } else {
-          unsigned short h[4];
-          for (int r = 0; r < 4; ++r) {
-            if constexpr (OUT == ASTERGEMM_BF16) h[r] = sk_f32_to_bf16(v[r]);
-            else {
-              _Float16 hh = (_Float16)v[r];
-              h[r] = __builtin_bit_cast(unsigned short, hh);
-            }
-          }
-          unsigned short* o = (unsigned short*)p.C + idx;
-          if (vec_ok) *(u16x4*)o = u16x4{h[0], h[1], h[2], h[3]};
-          else
-            for (int r = 0; r < ncols; ++r) o[r] = h[r];
-        }
+        sk_store_row4<OUT>(p.C, p.ldc, m, n, v, ncols);
       }
     }
     parity ^= 1;
@@ -688,27 +655,7 @@ __global__ __launch_bounds__(256) void skinny_splitk_reduce_kernel(const float* 
     v *= scale;
     if (bias)
       for (int r = 0; r < ncols; ++r) v[r] += bias[n + r];
-    const int64_t o = (int64_t)m * ldc + n;
-    const bool vec_ok = (ldc & 3) == 0 && ncols == 4;
-    if constexpr (OUT == ASTERGEMM_F32) {
-      float* out = (float*)C + o;
-      if (vec_ok) *(f32x4*)out = v;
-      else
-        for (int r = 0; r < ncols; ++r) out[r] = v[r];
-    } else {
-      unsigned short h[4];
-      for (int r = 0; r < 4; ++r) {
-        if constexpr (OUT == ASTERGEMM_BF16) h[r] = sk_f32_to_bf16(v[r]);
-        else {
-          const _Float16 hh = (_Float16)v[r];
-          h[r] = __builtin_bit_cast(unsigned short, hh);
-        }
-      }
-      unsigned short* out = (unsigned short*)C + o;
-      if (vec_ok) *(u16x4*)out = u16x4{h[0], h[1], h[2], h[3]};
-      else
-        for (int r = 0; r < ncols; ++r) out[r] = h[r];
-    }
+    sk_store_row4<OUT>(C, ldc, m, n, v, ncols);
   }
 }
 
@@ -926,27 +873,7 @@ __global__ __launch_bounds__(512) void gemm_skinny_fp4m_kernel(const GemmArgs p)
         const int ncols = (r1 - n) < 4 ? (r1 - n) : 4;
         if (p.bias)
           for (int r = 0; r < ncols; ++r) v[r] += p.bias[n + r];
-        const int64_t idx = (int64_t)m * p.ldc + n;
-        const bool vec_ok = (p.ldc & 3) == 0 && ncols == 4;
-        if constexpr (OUT == ASTERGEMM_F32) {
-          float* o = (float*)p.C + idx;
-          if (vec_ok) *(f32x4*)o = v;
-          else
-            for (int r = 0; r < ncols; ++r) o[r] = v[r];
-        } else {
-          unsigned short h[4];
-          for (int r = 0; r < 4; ++r) {
-            if constexpr (OUT == ASTERGEMM_BF16) h[r] = sk_f32_to_bf16(v[r]);
-            else {
-              _Float16 hh = (_Float16)v[r];
-              h[r] = __builtin_bit_cast(unsigned short, hh);
-            }
-          }
-          unsigned short* o = (unsigned short*)p.C + idx;
-          if (vec_ok) *(u16x4*)o = u16x4{h[0], h[1], h[2], h[3]};
-          else
-            for (int r = 0; r < ncols; ++r) o[r] = h[r];
-        }
+        sk_store_row4<OUT>(p.C, p.ldc, m, n, v, ncols);
       }
     }
     parity ^= 1;
@@ -1241,27 +1168,7 @@ __global__ __launch_bounds__(512) void gemm_skinny_regm_kernel(const GemmArgs p)
         const int ncols = (r1 - n) < 4 ? (r1 - n) : 4;
         if (p.bias)
           for (int r = 0; r < ncols; ++r) v[r] += p.bias[n + r];
-        const int64_t idx = (int64_t)m * p.ldc + n;
-        const bool vec_ok = (p.ldc & 3) == 0 && ncols == 4;
-        if constexpr (OUT == ASTERGEMM_F32) {
-          float* o = (float*)p.C + idx;
-          if (vec_ok) *(f32x4*)o = v;
-          else
-            for (int r = 0; r < ncols; ++r) o[r] = v[r];
-        } else {
-          unsigned short h[4];
-          for (int r = 0; r < 4; ++r) {
-            if constexpr (OUT == ASTERGEMM_BF16) h[r] = sk_f32_to_bf16(v[r]);
-            else {
-              _Float16 hh = (_Float16)v[r];
-              h[r] = __builtin_bit_cast(unsigned short, hh);
-            }
-          }
-          unsigned short* o = (unsigned short*)p.C + idx;
-          if (vec_ok) *(u16x4*)o = u16x4{h[0], h[1], h[2], h[3]};
-          else
-            for (int r = 0; r < ncols; ++r) o[r] = h[r];
-        }
+        sk_store_row4<OUT>(p.C, p.ldc, m, n, v, ncols);
       }
     }
     parity ^= 1;
@@ -1561,27 +1468,7 @@ __global__ __launch_bounds__(512) void gemm_skinny_direct_kernel(const GemmArgs 
         v *= scale;
         if (p.bias)
           for (int r = 0; r < 4; ++r) v[r] += p.bias[n + r];
-        const int64_t idx = (int64_t)m * p.ldc + n;
-        const bool vec_ok = (p.ldc & 3) == 0;
-        if constexpr (OUT == ASTERGEMM_F32) {
-          float* o = (float*)p.C + idx;
-          if (vec_ok) *(f32x4*)o = v;
-          else
-            for (int r = 0; r < 4; ++r) o[r] = v[r];
-        } else {
-          unsigned short h[4];
-          for (int r = 0; r < 4; ++r) {
-            if constexpr (OUT == ASTERGEMM_BF16) h[r] = sk_f32_to_bf16(v[r]);
-            else {
-              _Float16 hh = (_Float16)v[r];
-              h[r] = __builtin_bit_cast(unsigned short, hh);
-            }
-          }
-          unsigned short* o = (unsigned short*)p.C + idx;
-          if (vec_ok) *(u16x4*)o = u16x4{h[0], h[1], h[2], h[3]};
-          else
-            for (int r = 0; r < 4; ++r) o[r] = h[r];
-        }
+        sk_store_row4<OUT>(p.C, p.ldc, m, n, v, 4);
       }
     }
     parity ^= 1;
@@ -1789,27 +1676,7 @@ __global__ __launch_bounds__(512) void gemm_skinny_directb_kernel(const GemmArgs
         v *= scale;
         if (p.bias)
           for (int r = 0; r < 4; ++r) v[r] += p.bias[n + r];
-        const int64_t idx = (int64_t)m * p.ldc + n;
-        const bool vec_ok = (p.ldc & 3) == 0;
-        if constexpr (OUT == ASTERGEMM_F32) {
-          float* o = (float*)p.C + idx;
-          if (vec_ok) *(f32x4*)o = v;
-          else
-            for (int r = 0; r < 4; ++r) o[r] = v[r];
-        } else {
-          unsigned short h[4];
-          for (int r = 0; r < 4; ++r) {
-            if constexpr (OUT == ASTERGEMM_BF16) h[r] = sk_f32_to_bf16(v[r]);
-            else {
-              _Float16 hh = (_Float16)v[r];
-              h[r] = __builtin_bit_cast(unsigned short, hh);
-            }
-          }
-          unsigned short* o = (unsigned short*)p.C + idx;
-          if (vec_ok) *(u16x4*)o = u16x4{h[0], h[1], h[2], h[3]};
-          else
-            for (int r = 0; r < 4; ++r) o[r] = h[r];
-        }
+        sk_store_row4<OUT>(p.C, p.ldc, m, n, v, 4);
       }
     }
     parity ^= 1;
