@@ -25,7 +25,7 @@ struct GemmArgs {
   int32_t ksteps;        // K-loop trip count (128 bytes of a row per step)
   int32_t tail_granules; // valid 16-byte granules of the last step, 0 = all 8
   int32_t tiles_m, tiles_n;
-  int32_t group_m;       // tile rows per rasterisation group
+  int32_t group_m;       // tile rows per rasterisation group; < 0: band order (see map_tile)
   int32_t split_k;       // skinny path: K slices per output row block
   float* workspace;      // fp32 partials [split_k][M][N] when a row is cut into K ranges; set by
                          // the caller of a launcher = use this buffer, null = the library's own

@@ -333,6 +333,9 @@ inline void tail_parts(const GemmArgs& a, const TailSplit& ts, int out_bytes, Ge
   part1->tiles_n = (part1->N + 255) / 256;
   part2->tiles_m = (part2->M + 127) / 128;
   part2->tiles_n = (part2->N + 127) / 128;
+  // the tile order is a property of each part's own tile grid (see map_tile)
+  part1->group_m = (part1->tiles_m % 8 == 0 && part1->tiles_n % 32 == 0) ? -1 : 8;
+  part2->group_m = (part2->tiles_m % 8 == 0 && part2->tiles_n % 32 == 0) ? -1 : 8;
 }
 
 // KIND 0: 16-bit operands, 1: fp8, 2: MXFP4

@@ -72,6 +72,18 @@ __device__ __forceinline__ u16x4 cast4_16(f32x4 v) {
 // A and B panels through that XCD's L2.
 __device__ __forceinline__ void map_tile(int bid, int tiles_m, int tiles_n,
                                          int group_m, int& tm, int& tn) {
+  if (group_m < 0) {
+    // band order (tiles_m % 8 == 0, tiles_n % 8 == 0): all eight XCDs work on the same band of
+    // eight tile rows, XCD x on its own tiles_n / 8 tile columns of it, so that a band of A is
+    // fetched from HBM once and reaches the other seven XCDs from the last-level cache
+    const int xcd = bid & 7, idx = bid >> 3;
+    const int cols = tiles_n >> 3;               // tile columns of an XCD
+    const int per_band = 8 * cols;               // tiles of an XCD in one band
+    const int band = idx / per_band, j = idx - band * per_band;
+    tm = band * 8 + (j & 7);
+    tn = xcd * cols + (j >> 3);
+    return;
+  }
   const int total = tiles_m * tiles_n;
   const int q = total >> 3, rem = total & 7;
   const int xcd = bid & 7, idx = bid >> 3;

@@ -853,6 +853,42 @@ def test_identity_operand_is_exact_at_full_width(gpu):
     assert np.array_equal(out, a)
 
 
+@pytest.mark.parametrize("dtype_ab,M", [("bf16", 2048), ("fp8_e4m3", 2048), ("mxfp4", 4096)])
+def test_band_tile_order_writes_every_tile_once(gpu, dtype_ab, M):
+    # B = I at a size whose tile grid divides by 8 x 32 (all XCDs on one band of eight tile
+    # rows; the MXFP4 case has more tiles than CUs and goes through the tile walk): each output
+    # is one product plus zeros, so C is A's values bit for bit and a tile that is skipped,
+    # written twice from the wrong place or swapped with another shows
+    N = K = 8192
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    ex = {}
+    if dtype_ab == "bf16":
+        a = F.f32_to_bf16_bits(x)
+        b = np.zeros((N, K), np.uint16)
+        b[np.arange(N), np.arange(N)] = 0x3F80
+        want = a
+    elif dtype_ab == "fp8_e4m3":
+        a = F.e4m3_encode(x)
+        b = np.zeros((N, K), np.uint8)
+        b[np.arange(N), np.arange(N)] = F.e4m3_encode_scalar(1.0)
+        ex = dict(scale_a=np.float32(1), scale_b=np.float32(1))
+        want = F.f32_to_bf16_bits(F.e4m3_decode(a))
+    else:
+        a, mxa = F.quantize_mxfp4(x)
+        codes = np.zeros((N, K), np.uint8)
+        codes[np.arange(N), np.arange(N)] = F.e2m1_encode(np.ones(1, np.float32))[0]
+        b = F.pack_nibbles(codes)
+        ex = dict(mx_a=mxa, mx_b=np.full((N, K // 32), 127, np.uint8))
+        want = F.f32_to_bf16_bits(F.dequantize_mxfp4(a, mxa))
+    out, name = run_gemm(a, b, M, N, K, dtype_ab, "bf16", **ex)
+    assert name.startswith("stream_") and "256x256" in name, name
+    if dtype_ab == "mxfp4":
+        assert "_walk_" in name, name
+    # as values: a negative zero of A comes out as the accumulator's positive zero
+    assert np.array_equal(F.bf16_bits_to_f32(out), F.bf16_bits_to_f32(want))
+
+
 # ---- every pre-built tile variant, selected by its id ---------------------------------------
 
 def _tile_variants():
