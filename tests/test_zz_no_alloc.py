@@ -3,7 +3,8 @@
 Shapes whose rows are cut into K ranges keep their fp32 partial sums in a scratch array built
 into the library instead of an allocated workspace; the results must be the same bits.  Two calls
 in a row share the array, the second smaller than the first; a shape that needs no workspace and
-one that needs more than the array holds are covered as well.
+one that needs more than the array holds are covered as well, and so is a HIP graph that holds
+two launches of it and is replayed on fresh activations.
 """
 import ctypes
 
@@ -90,3 +91,82 @@ def test_caller_workspace_matches_the_library_workspace(gpu):
                  workspace=bufs[3].ptr_value, workspace_bytes=need - 4)
     for bf in bufs:
         bf.free()
+
+
+def _hip():
+    lib = ctypes.CDLL("libamdhip64.so")
+    for name, args in (("hipStreamBeginCapture", [ctypes.c_void_p, ctypes.c_int]),
+                       ("hipStreamEndCapture", [ctypes.c_void_p, ctypes.POINTER(ctypes.c_void_p)]),
+                       ("hipGraphInstantiate", [ctypes.POINTER(ctypes.c_void_p), ctypes.c_void_p,
+                                                ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t]),
+                       ("hipGraphLaunch", [ctypes.c_void_p, ctypes.c_void_p]),
+                       ("hipGraphExecDestroy", [ctypes.c_void_p]),
+                       ("hipGraphDestroy", [ctypes.c_void_p])):
+        fn = getattr(lib, name)
+        fn.argtypes, fn.restype = args, ctypes.c_int
+    return lib
+
+
+def test_noalloc_launches_replay_from_a_graph(gpu):
+    # two decode projections in a row, h = x W1^T (no K ranges) and y = h W2^T (rows cut into K
+    # ranges: partial sums in the built-in scratch array), captured once in global capture mode
+    # (a hipMalloc or a synchronizing call inside the capture would fail it) and replayed on
+    # three different x, with eager launches and synchronizations in between; every replay must
+    # give the bits of the eager pair on the same x
+    M, H, D = 16, 4096, 14336
+    rng = np.random.default_rng(21)
+    w1, w2 = _bf16(rng, (D, H), 0.02), _bf16(rng, (H, D), 0.02)
+    xs = [_bf16(rng, (M, H), 1.0) for _ in range(3)]
+    up = AG.GemmPlan.create(M, D, H, "bf16", "bf16")
+    down = AG.GemmPlan.create(M, H, D, "bf16", "bf16")
+    assert up.workspace_bytes() == 0 and 0 < down.workspace_bytes() <= _capi.NOALLOC_SCRATCH_BYTES
+    dx, dw1, dw2 = GpuBuffer(xs[0].nbytes), GpuBuffer(w1.nbytes), GpuBuffer(w2.nbytes)
+    dh, dy = GpuBuffer(M * D * 2), GpuBuffer(M * H * 2)
+    dw1.copy_from_host(w1)
+    dw2.copy_from_host(w2)
+    rt, hip = _capi.load(), _hip()
+
+    def eager_pair(x):
+        dx.copy_from_host(x)
+        up.run(dx.ptr_value, dw1.ptr_value, dh.ptr_value)
+        down.run(dh.ptr_value, dw2.ptr_value, dy.ptr_value)
+        y = np.zeros((M, H), np.uint16)
+        dy.copy_to_host(y)
+        return y
+
+    want = [eager_pair(x) for x in xs]
+    assert not np.array_equal(want[0], want[1])
+    # the eager calls above were also the first calls on this device: set-up is behind us
+    up.run_noalloc(dx.ptr_value, dw1.ptr_value, dh.ptr_value)
+    down.run_noalloc(dh.ptr_value, dw2.ptr_value, dy.ptr_value)
+    _capi.check(rt.aster_rt_device_synchronize())
+
+    stream, graph, gexec = ctypes.c_void_p(), ctypes.c_void_p(), ctypes.c_void_p()
+    _capi.check(rt.aster_rt_stream_create(ctypes.byref(stream)))
+    print("capture", up.info.name.decode(), down.info.name.decode(), flush=True)
+    assert hip.hipStreamBeginCapture(stream, 0) == 0        # hipStreamCaptureModeGlobal
+    try:
+        up.run_noalloc(dx.ptr_value, dw1.ptr_value, dh.ptr_value, stream=stream.value)
+        down.run_noalloc(dh.ptr_value, dw2.ptr_value, dy.ptr_value, stream=stream.value)
+    finally:
+        rc = hip.hipStreamEndCapture(stream, ctypes.byref(graph))
+    assert rc == 0 and graph.value
+    assert hip.hipGraphInstantiate(ctypes.byref(gexec), graph, None, None, 0) == 0
+    try:
+        for i in (2, 0, 1):
+            # eager work between the replays: another x through the allocating entry point
+            assert np.array_equal(eager_pair(xs[(i + 1) % 3]), want[(i + 1) % 3])
+            dx.copy_from_host(xs[i])
+            dy.copy_from_host(np.full((M, H), 0x7FC1, np.uint16))
+            print("replay on x", i, flush=True)
+            assert hip.hipGraphLaunch(gexec, stream) == 0
+            _capi.check(rt.aster_rt_stream_synchronize(stream))
+            y = np.zeros((M, H), np.uint16)
+            dy.copy_to_host(y)
+            assert np.array_equal(y, want[i]), f"replay on x{i}"
+    finally:
+        hip.hipGraphExecDestroy(gexec)
+        hip.hipGraphDestroy(graph)
+        _capi.check(rt.aster_rt_stream_destroy(stream))
+        for bf in (dx, dw1, dw2, dh, dy):
+            bf.free()
