@@ -181,6 +181,12 @@ const Variant* choose(const astergemm_config& c, int* index_out) {
       else if (!fits) better = v->tile_m > best->tile_m;
       else if (v->rank >= 2 || best->rank >= 2) better = v->rank > best->rank;
       else better = v->tile_m < best->tile_m || (v->tile_m == best->tile_m && v->rank > best->rank);
+    } else if (c.operand_path == ASTERGEMM_OPERAND_DIRECT_B_K8) {
+      // pre-shuffled B straight into operands: the 128 x 256 form (four waves side by side, two
+      // workgroups per CU, no B line fetched by two waves) is ahead of the 256 x 256 form on
+      // every shape measured (8192^3 744 against 757 us, 16384 x 16384 x 4096 1508 against 1566,
+      // 4096 x 14336 x 4096 336 against 370, 2048^3 29.5 against 45.5)
+      better = v->tile_m < best->tile_m;
     } else {
       // Measured on MI355X (256 CUs): the 256 x 256 kernels (one workgroup per CU) win once
       // they nearly fill the chip; below that the 128 x 128 stream kernel (rank 2, two

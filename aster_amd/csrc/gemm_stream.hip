@@ -47,17 +47,17 @@ const char* check_stream_whole_k(const astergemm_config& c) {
   }
 
 // ---- B pre-shuffled, loaded straight into MFMA operands (gemm_streamdb_kernel.hpp) ---------
-template <int DT, int OUT, int NSLOT, int NBUF>
+template <int DT, int OUT, int NSLOT, int NBUF, int WM>
 int launch_streamdb(const GemmArgs& a, int grid, hipStream_t s) {
-  constexpr int lds = 5 * 256 * kRowBytes;  // the epilogue stages through up to 160 KiB
-  auto k = gemm_streamdb_kernel<DT, OUT, NSLOT, NBUF>;
+  constexpr int lds = 5 * 128 * WM * kRowBytes;  // the epilogue stages through the ring
+  auto k = gemm_streamdb_kernel<DT, OUT, NSLOT, NBUF, WM>;
   static std::atomic<uint64_t> attr_devs{0};
   if (int e = lds_attr_once(attr_devs, (const void*)k, lds)) return e;
   // what the kernel's indexing assumes: whole 16-row blocks of B and whole K-steps
   if (a.N % 16 != 0 || a.N < 16 || a.M < 8 || a.M % 8 != 0 || a.K % 64 != 0 || a.tail_granules != 0 ||
       a.ldb_bytes != (int64_t)a.K * 2)
     return (int)hipErrorInvalidValue;
-  hipLaunchKernelGGL(k, dim3(grid), dim3(512), lds, s, a);
+  hipLaunchKernelGGL(k, dim3(grid), dim3(WM * 256), lds, s, a);
   return (int)hipGetLastError();
 }
 
@@ -71,11 +71,12 @@ const char* check_streamdb(const astergemm_config& c) {
   return nullptr;
 }
 
-#define AG_STREAMDB(name, DT, OUT, NSLOT, NBUF, RANK)                            \
+#define AG_STREAMDB(name, DT, OUT, NSLOT, NBUF, WM, RANK)                        \
   Variant {                                                                      \
-    name, ASTERGEMM_KERNEL_TILE, DT, OUT, 256, 256, kRowBytes, 2, 4, NSLOT, RANK, \
-        5 * 256 * kRowBytes, (const void*)gemm_streamdb_kernel<DT, OUT, NSLOT, NBUF>, \
-        launch_streamdb<DT, OUT, NSLOT, NBUF>, check_streamdb,                   \
+    name, ASTERGEMM_KERNEL_TILE, DT, OUT, 128 * WM, 256, kRowBytes, WM, 4, NSLOT, RANK, \
+        5 * 128 * WM * kRowBytes,                                                \
+        (const void*)gemm_streamdb_kernel<DT, OUT, NSLOT, NBUF, WM>,             \
+        launch_streamdb<DT, OUT, NSLOT, NBUF, WM>, check_streamdb,               \
         ASTERGEMM_OPERAND_DIRECT_B_K8                                            \
   }
 
@@ -417,12 +418,18 @@ const Variant kStreamVariants[] = {
     AG_STREAM_SPLITK_SET("splitk_mxfp4", 2, ASTERGEMM_MXFP4, 4 * 128 * kRowBytes + 4 * 128 * 16,
                          gemm_stream4_splitk_kernel),
     AG_STREAM_SET("stream_f16", ASTERGEMM_F16),
-    AG_STREAMDB("streamdb_bf16_256x256_w2x4_bf16", ASTERGEMM_BF16, ASTERGEMM_BF16, 5, 5, 2),
-    AG_STREAMDB("streamdb_bf16_256x256_w2x4_f32", ASTERGEMM_BF16, ASTERGEMM_F32, 5, 5, 2),
-    AG_STREAMDB("streamdb_bf16_256x256_w2x4_f16", ASTERGEMM_BF16, ASTERGEMM_F16, 5, 5, 2),
-    AG_STREAMDB("streamdb_f16_256x256_w2x4_bf16", ASTERGEMM_F16, ASTERGEMM_BF16, 5, 5, 2),
-    AG_STREAMDB("streamdb_f16_256x256_w2x4_f32", ASTERGEMM_F16, ASTERGEMM_F32, 5, 5, 2),
-    AG_STREAMDB("streamdb_f16_256x256_w2x4_f16", ASTERGEMM_F16, ASTERGEMM_F16, 5, 5, 2),
+    AG_STREAMDB("streamdb_bf16_256x256_w2x4_bf16", ASTERGEMM_BF16, ASTERGEMM_BF16, 5, 5, 2, 2),
+    AG_STREAMDB("streamdb_bf16_256x256_w2x4_f32", ASTERGEMM_BF16, ASTERGEMM_F32, 5, 5, 2, 2),
+    AG_STREAMDB("streamdb_bf16_256x256_w2x4_f16", ASTERGEMM_BF16, ASTERGEMM_F16, 5, 5, 2, 2),
+    AG_STREAMDB("streamdb_f16_256x256_w2x4_bf16", ASTERGEMM_F16, ASTERGEMM_BF16, 5, 5, 2, 2),
+    AG_STREAMDB("streamdb_f16_256x256_w2x4_f32", ASTERGEMM_F16, ASTERGEMM_F32, 5, 5, 2, 2),
+    AG_STREAMDB("streamdb_f16_256x256_w2x4_f16", ASTERGEMM_F16, ASTERGEMM_F16, 5, 5, 2, 2),
+    AG_STREAMDB("streamdb_bf16_128x256_w1x4_bf16", ASTERGEMM_BF16, ASTERGEMM_BF16, 5, 5, 1, 1),
+    AG_STREAMDB("streamdb_bf16_128x256_w1x4_f32", ASTERGEMM_BF16, ASTERGEMM_F32, 5, 5, 1, 1),
+    AG_STREAMDB("streamdb_bf16_128x256_w1x4_f16", ASTERGEMM_BF16, ASTERGEMM_F16, 5, 5, 1, 1),
+    AG_STREAMDB("streamdb_f16_128x256_w1x4_bf16", ASTERGEMM_F16, ASTERGEMM_BF16, 5, 5, 1, 1),
+    AG_STREAMDB("streamdb_f16_128x256_w1x4_f32", ASTERGEMM_F16, ASTERGEMM_F32, 5, 5, 1, 1),
+    AG_STREAMDB("streamdb_f16_128x256_w1x4_f16", ASTERGEMM_F16, ASTERGEMM_F16, 5, 5, 1, 1),
     AG_STREAM_TAIL_SET("stream_bf16_256x256_w2x4_tail128", 0, ASTERGEMM_BF16, 2, 4, 5 * 256 * kRowBytes,
                        gemm_stream_kernel),
     AG_STREAM_TAIL_SET("stream_f16_256x256_w2x4_tail128", 0, ASTERGEMM_F16, 2, 4, 5 * 256 * kRowBytes,

@@ -1,5 +1,7 @@
 // Stream kernel with B straight from global memory into MFMA operand registers ("direct B"),
-// 16-bit operands, 256x256 workgroup tile, 2x4 waves: the operand path of the reference's best
+// 16-bit operands, 256x256 workgroup tile with 2x4 waves or 128x256 with 1x4 waves (the
+// reference's own best mapping: no two waves of a workgroup fetch the same B, two workgroups
+// of four waves per CU): the operand path of the reference's best
 // gfx950 kernel (contrib/kittens/test/test_102_gemm_python_multitile_g2s_directb_cdna4.py:75-324:
 // A through LDS by direct-to-LDS transfers, B pre-shuffled on the host so that one
 // global_load_dwordx4 per lane is an MFMA operand) on this build's staging, swizzle, tile map
@@ -36,13 +38,13 @@
 namespace astergemm {
 namespace {
 
-template <int DT, int OUT, int NSLOT, int NBUF>
+template <int DT, int OUT, int NSLOT, int NBUF, int WM>
 __device__ __forceinline__ void gemm_streamdb_body(const GemmArgs& p, int bid) {
-  constexpr int BM = 256, BN = 256, WM = 2, WN = 4;
+  constexpr int BM = 128 * WM, BN = 256, WN = 4;
   constexpr int NW = WM * WN;
   constexpr int TM = BM / WM / 16;      // 8
   constexpr int TN = BN / WN / 16;      // 4
-  constexpr int SLOT = BM * kRowBytes;  // 32 KiB: A rows of one K-step
+  constexpr int SLOT = BM * kRowBytes;  // 32 (16) KiB: A rows of one K-step
   constexpr int LH = BM / 8 / NW;       // 4 transfers of 1 KiB per wave and slot
   // NSLOT A slots in LDS, NBUF B register buffers of one MFMA substep each; the loop is unrolled
   // over NSLOT trips, after which slot and buffer numbers repeat
@@ -55,6 +57,7 @@ __device__ __forceinline__ void gemm_streamdb_body(const GemmArgs& p, int bid) {
   constexpr int MS = 2 * TM;            // m-steps per K-step
   constexpr int BAR = MS - (RA - 1);    // m-step whose first slot carries the barrier
   static_assert(DT == ASTERGEMM_BF16 || DT == ASTERGEMM_F16, "16-bit operands");
+  static_assert(WM == 1 || WM == 2, "one or two wave rows of 128 rows each");
   static_assert(MS % RA == 0, "the A fragment ring is in phase at every K-step");
   static_assert(TN == 4 && LH == 4, "side-instruction schedule below");
 
@@ -260,9 +263,11 @@ __device__ __forceinline__ void gemm_streamdb_body(const GemmArgs& p, int bid) {
   stream_epilogue<OUT, BM, BN, WM, WN>(p, acc, lds, wave, row0, col0);
 }
 
-template <int DT, int OUT, int NSLOT, int NBUF>
-__global__ __launch_bounds__(512) void gemm_streamdb_kernel(const GemmArgs p) {
-  gemm_streamdb_body<DT, OUT, NSLOT, NBUF>(p, blockIdx.x);
+// WM = 1: four waves and 80 KiB per workgroup, two workgroups per CU (at most 256 registers per
+// wave, which the second launch bound asks for)
+template <int DT, int OUT, int NSLOT, int NBUF, int WM = 2>
+__global__ __launch_bounds__(WM * 256, 2) void gemm_streamdb_kernel(const GemmArgs p) {
+  gemm_streamdb_body<DT, OUT, NSLOT, NBUF, WM>(p, blockIdx.x);
 }
 
 }  // namespace

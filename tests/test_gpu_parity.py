@@ -1163,15 +1163,17 @@ def test_skinny_direct_b_preshuffled_fp8_and_mxfp4_weights(gpu, M, N, dtype_ab, 
                                    (264, 528, 704), (1000, 1008, 896), (256, 512, 960),
                                    (512, 256, 1280), (768, 1024, 1472), (2048, 2048, 4096)])
 @pytest.mark.parametrize("dtype_ab,dtype_c", [("bf16", "bf16"), ("f16", "f32")])
-def test_stream_direct_b_k8(gpu, M, N, K, dtype_ab, dtype_c):
+@pytest.mark.parametrize("tile_m", [256, 128])
+def test_stream_direct_b_k8(gpu, M, N, K, dtype_ab, dtype_c, tile_m):
     # K steps of 64 elements: 1, 2, 9 (no steady group), 10 (one steady group exactly), 11, 14, 15,
-    # 20, 23, 64; edge tiles in M (multiple of 8) and N (multiple of 16)
+    # 20, 23, 64; edge tiles in M (multiple of 8) and N (multiple of 16).  tile_m 128 is the
+    # reference's own best mapping: 128 x 256 tiles, four waves side by side
     from aster_amd.kittens_helpers import shuffle_weight_k8
     a, b, _ = operands(M, N, K, dtype_ab)
     bias = np.random.default_rng(4).standard_normal(N).astype(np.float32)
     out, name = run_gemm(a, shuffle_weight_k8(b), M, N, K, dtype_ab, dtype_c, bias=bias,
-                         operand_path="direct_b_k8")
-    assert name.startswith("streamdb_")
+                         operand_path="direct_b_k8", wg_tile=(tile_m, 256))
+    assert name.startswith(f"streamdb_{dtype_ab}_{tile_m}x256_w{tile_m // 128}x4_")
     check(out, G.gemm(a, b, _DT[dtype_ab], _DT[dtype_c], bias=bias), dtype_c, N)
     # the same K order on both operands as the LDS kernel: same products, same sums
     lds_out, lds_name = run_gemm(a, b, M, N, K, dtype_ab, dtype_c, bias=bias, wg_tile=(256, 256),
@@ -1184,12 +1186,28 @@ def test_stream_direct_b_k8_full_size_row_sample(gpu, big):
     from aster_amd.kittens_helpers import shuffle_weight_k8
     M, N, K, a, b = big
     out, name = run_gemm(a, shuffle_weight_k8(b), M, N, K, "bf16", "bf16", operand_path="direct_b_k8")
-    assert name == "streamdb_bf16_256x256_w2x4_bf16"
+    assert name == "streamdb_bf16_128x256_w1x4_bf16"
     rows, cols = _sampled_rows_and_cols(M, N)
     check(out[rows], G.gemm(a[rows], b, G.BF16, G.BF16), "bf16", N)
     check(out[:, cols], G.gemm(a, b[cols], G.BF16, G.BF16), "bf16", len(cols))
     out2, _ = run_gemm(a, shuffle_weight_k8(b), M, N, K, "bf16", "bf16", operand_path="direct_b_k8")
     assert np.array_equal(out, out2)
+
+
+def test_the_reference_best_mapping_is_honoured_as_it_stands(gpu, tmp_path):
+    # the mapping of the reference's best gfx950 label (128 x 256 workgroup tile = 8 x 16 MFMA
+    # tiles, four waves in a 1 x 4 grid, B pre-shuffled and loaded straight into operands) selects
+    # a kernel of exactly that geometry; nothing of the request is reported as dropped
+    M, N, K = 1024, 1536, 1024
+    cfg = make_instance(M, N, K, wg_tile=(128, 256), waves=(1, 4), operand_path=OperandPath.DIRECT_B)
+    path, _ = AG.compile_gemm(cfg, str(tmp_path / "k.hsaco"))
+    desc = json.load(open(path))
+    assert desc["kernel"] == "streamdb_bf16_128x256_w1x4_bf16", desc
+    assert desc["mapping_honoured"] is True and not desc.get("mapping_not_honoured")
+    assert desc["grid"] == (M // 128) * (N // 256) and desc["block"] == 256
+    a, b, _ = operands(M, N, K, "bf16")
+    c_flat, times = AG.execute_gemm_hsaco(cfg, path, 2, a, b)
+    check(c_flat.reshape(M, N), G.gemm(a, b, G.BF16, G.BF16), "bf16", N)
 
 
 def test_direct_b_mapping_through_the_harness_seam(gpu, tmp_path):
