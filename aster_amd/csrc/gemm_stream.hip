@@ -158,6 +158,50 @@ int launch_stream8(const GemmArgs& a, int grid, hipStream_t s) {
   return (int)hipGetLastError();
 }
 
+// The 256 x 256 fp8 kernel as a tile walk (see gemm_stream8_body): one workgroup per CU.
+template <int DT, int OUT>
+int launch_stream8_walk(const GemmArgs& a, int grid, hipStream_t s) {
+  (void)grid;
+  constexpr int lds = 5 * 256 * kRowBytes;
+  // what the kernel assumes: whole tiles (its epilogue stores without bounds checks), whole
+  // K-steps and enough of them for the steady form of trip 0
+  if (a.M % 256 != 0 || a.N % 256 != 0 || a.tail_granules != 0 || a.ksteps < 4)
+    return (int)hipErrorInvalidValue;
+  auto k = gemm_stream8_walk_kernel<DT, OUT, 256, 256, 2, 4>;
+  static std::atomic<uint64_t> attr_devs{0};
+  if (int e = lds_attr_once(attr_devs, (const void*)k, lds)) return e;
+  const int cus = device_cus();
+  if (cus <= 0) return (int)hipErrorNoDevice;
+  const int tiles = a.tiles_m * a.tiles_n;
+  hipLaunchKernelGGL(k, dim3(tiles < cus ? tiles : cus), dim3(512), lds, s, a);
+  return (int)hipGetLastError();
+}
+
+const char* check_stream8_walk(const astergemm_config& c) {
+  if (const char* why = check_stream_whole_k(c)) return why;
+  if (c.K < 512) return "the tile walk needs at least four K-steps";
+  if (c.M % 256 != 0 || c.N % 256 != 0) return "the tile walk needs M and N to be multiples of 256";
+  int cus = device_cus();
+  if (cus <= 0) cus = 256;                       // no device to ask: describe the MI355X
+  if (((c.M + 255) / 256) * ((c.N + 255) / 256) <= cus)
+    return "the tile walk pays from two tiles per workgroup on";
+  return nullptr;
+}
+
+int grid_stream_walk(const astergemm_config& c, int cus) {
+  const int64_t tiles = ((c.M + 255) / 256) * ((c.N + 255) / 256);
+  if (cus <= 0) cus = 256;
+  return (int)(tiles > cus ? cus : tiles);
+}
+
+#define AG_STREAM8_WALK(name, DT, OUT, RANK)                                     \
+  Variant {                                                                      \
+    name, ASTERGEMM_KERNEL_TILE, DT, OUT, 256, 256, kRowBytes, 2, 4, 3, RANK,    \
+        5 * 256 * kRowBytes,                                                     \
+        (const void*)gemm_stream8_walk_kernel<DT, OUT, 256, 256, 2, 4>,          \
+        launch_stream8_walk<DT, OUT>, check_stream8_walk, ASTERGEMM_OPERAND_LDS, \
+        nullptr, grid_stream_walk                                                \
+  }
 #define AG_STREAM8(name, DT, OUT)                                                \
   Variant {                                                                      \
     name, ASTERGEMM_KERNEL_TILE, DT, OUT, 256, 256, kRowBytes, 2, 4, 3, 2,       \
@@ -353,7 +397,11 @@ int launch_stream_tail(const GemmArgs& a, int grid, hipStream_t s) {
     if ((rc = launch_stream<DT, OUT, 256, 256, 2, 4>(p1, g1, s)) != 0) return rc;
     return launch_stream<DT, OUT, 128, 128, 2, 2>(p2, g2, s);
   } else if constexpr (KIND == 1) {
-    if ((rc = launch_stream8<DT, OUT, 256, 256, 2, 4>(p1, g1, s)) != 0) return rc;
+    // the whole rounds as a tile walk where its conditions hold (see launch_stream8_walk)
+    const bool walk = p1.M % 256 == 0 && p1.N % 256 == 0 && p1.tail_granules == 0 &&
+                      p1.ksteps >= 4 && g1 > device_cus();
+    rc = walk ? launch_stream8_walk<DT, OUT>(p1, g1, s) : launch_stream8<DT, OUT, 256, 256, 2, 4>(p1, g1, s);
+    if (rc != 0) return rc;
     return launch_stream8<DT, OUT, 128, 128, 2, 2>(p2, g2, s);
   } else {
     // the whole rounds as a tile walk where its conditions hold (see launch_stream4_walk)
@@ -381,9 +429,12 @@ int grid_stream_tail(const astergemm_config& c, int cus) {
   const int64_t m1 = ts.along == 2 ? ts.first : c.M, n1 = ts.along == 1 ? ts.first : c.N;
   const int64_t m2 = ts.along == 2 ? c.M - ts.first : c.M, n2 = ts.along == 1 ? c.N - ts.first : c.N;
   int64_t g1 = ((m1 + 255) / 256) * ((n1 + 255) / 256);
-  // MXFP4: the whole rounds run as a tile walk, one workgroup per CU (see launch_stream_tail)
+  // MXFP4, fp8: the whole rounds run as a tile walk, one workgroup per CU (see launch_stream_tail)
   if (cus <= 0) cus = 256;
   if (c.dtype_ab == ASTERGEMM_MXFP4 && c.K % 1024 == 0 && m1 % 256 == 0 && n1 % 256 == 0 && g1 > cus)
+    g1 = cus;
+  if (c.dtype_ab == ASTERGEMM_FP8_E4M3 && c.K % 128 == 0 && c.K >= 512 && m1 % 256 == 0 &&
+      n1 % 256 == 0 && g1 > cus)
     g1 = cus;
   return (int)(g1 + ((m2 + 127) / 128) * ((n2 + 127) / 128));
 }
@@ -441,6 +492,9 @@ const Variant kStreamVariants[] = {
     AG_STREAM8("stream_fp8_256x256_w2x4_bf16", ASTERGEMM_FP8_E4M3, ASTERGEMM_BF16),
     AG_STREAM8("stream_fp8_256x256_w2x4_f32", ASTERGEMM_FP8_E4M3, ASTERGEMM_F32),
     AG_STREAM8("stream_fp8_256x256_w2x4_f16", ASTERGEMM_FP8_E4M3, ASTERGEMM_F16),
+    AG_STREAM8_WALK("stream_fp8_256x256_w2x4_walk_bf16", ASTERGEMM_FP8_E4M3, ASTERGEMM_BF16, 3),
+    AG_STREAM8_WALK("stream_fp8_256x256_w2x4_walk_f32", ASTERGEMM_FP8_E4M3, ASTERGEMM_F32, 3),
+    AG_STREAM8_WALK("stream_fp8_256x256_w2x4_walk_f16", ASTERGEMM_FP8_E4M3, ASTERGEMM_F16, 3),
     AG_STREAM8_128("stream_fp8_128x128_w2x2_bf16", ASTERGEMM_FP8_E4M3, ASTERGEMM_BF16),
     AG_STREAM8_128("stream_fp8_128x128_w2x2_f32", ASTERGEMM_FP8_E4M3, ASTERGEMM_F32),
     AG_STREAM8_128("stream_fp8_128x128_w2x2_f16", ASTERGEMM_FP8_E4M3, ASTERGEMM_F16),

@@ -37,64 +37,6 @@
 namespace astergemm {
 namespace {
 
-// Epilogue of the tile walk: a wave stages its 16-row slabs in 2 KiB of its own, outside the
-// ring (which is already receiving the next tile), so no barrier is needed: LDS operations of
-// one wave execute in order.  A slab row is 128 bytes (64 16-bit or 32 fp32 columns), 16-byte
-// granule g of row r sits at granule g ^ (r & 7).  M and N are whole tiles.
-template <int OUT, int TM, int TN>
-__device__ __forceinline__ void walk_epilogue(const GemmArgs& p, f32x4 (&acc)[TM][TN], uint8_t* stage,
-                                              int wrow0, int wcol0) {
-  static_assert(TN == 4, "64 columns per wave");
-  float scale = 1.0f;  // fetched per tile (scalar loads): nothing to keep across the K loop
-  if (p.scale_a) scale *= *p.scale_a;
-  if (p.scale_b) scale *= *p.scale_b;
-  int lane;
-  asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lane));
-  const int li = lane & 15, lq = lane >> 4;
-  constexpr int OB = (OUT == ASTERGEMM_F32) ? 4 : 2;
-  constexpr int PASSES = 64 * OB / 128;          // 128-byte column ranges of the wave tile
-  constexpr int TPP = TN / PASSES;               // 16-column tiles per pass
-  float bias_v[TN][4];
-#pragma unroll
-  for (int n = 0; n < TN; ++n)
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      int col = wcol0 + n * 16 + 4 * lq + e;
-      col = col < p.N ? col : p.N - 1;
-      bias_v[n][e] = p.bias ? p.bias[col] : 0.f;
-    }
-#pragma unroll
-  for (int m = 0; m < TM; ++m) {
-#pragma unroll
-    for (int ps = 0; ps < PASSES; ++ps) {
-#pragma unroll
-      for (int t = 0; t < TPP; ++t) {
-        const int n = ps * TPP + t;
-        f32x4 v = acc[m][n] * scale;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] += bias_v[n][e];
-        if constexpr (OUT == ASTERGEMM_F32) {
-          *(f32x4*)(stage + li * 128 + (((t * 4 + lq) ^ (li & 7)) << 4)) = v;
-        } else {
-          const u16x4 h = cast4_16<OUT>(v);
-          *(u16x4*)(stage + li * 128 + (((t * 2 + (lq >> 1)) ^ (li & 7)) << 4) + (lq & 1) * 8) = h;
-        }
-      }
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        const int c = t * 64 + lane;
-        const int r = c >> 3, cc = c & 7;
-        const i32x4 d = *(const i32x4*)(stage + r * 128 + ((cc ^ (r & 7)) << 4));
-        const int col = wcol0 + (ps * 128 + cc * 16) / OB;
-        uint8_t* out = (uint8_t*)p.C + ((int64_t)(wrow0 + m * 16 + r) * p.ldc + col) * OB;
-        // whole tiles only (the launcher checks): every store is issued, so that the count
-        // the next tile's first barrier leaves outstanding is exact
-        __builtin_nontemporal_store(d, (i32x4*)out);
-      }
-    }
-  }
-}
-
 // WALK: the workgroup takes tiles bid, bid + stride, ... below `total` as one long K loop: the
 // last two trips of a tile bring in K-steps 0 and 1 (and scale chunks 0 and 1) of the next tile
 // where a longer row would have brought K-steps nk and nk+1, so the next tile starts with its

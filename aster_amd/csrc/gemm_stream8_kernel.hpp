@@ -21,14 +21,23 @@
 // the 16-bit kernel.  Slot offsets are scalars that rotate from trip to trip, so the loop
 // body is a single trip (the register allocator does not cope with six unrolled ones at
 // this register pressure).
+//
+// WALK: one workgroup per CU takes tiles bid, bid + stride, ... below `total` in one launch.  When
+// the K loop of a tile is over and every wave has left the ring (one barrier), the first two
+// K-steps of the next tile are requested into slots A0, A1, B0, B1 and arrive while the
+// epilogue runs out of the third A slot (4 KiB per wave, no barrier); the epilogue's stores are
+// left in flight: the waits of the next tile's start count them as still outstanding (the
+// vector-memory counter retires in issue order), so only the barrier of trip 1, whose transfers
+// were requested behind the stores, waits for them.  Whole tiles, whole K-steps, at least four.
 #pragma once
 #include "gemm_stream_kernel.hpp"
 
 namespace astergemm {
 namespace {
 
-template <int DT, int OUT, int BM, int BN, int WM, int WN>
-__device__ __forceinline__ void gemm_stream8_body(const GemmArgs& p, int bid) {
+template <int DT, int OUT, int BM, int BN, int WM, int WN, bool WALK = false>
+__device__ __forceinline__ void gemm_stream8_body(const GemmArgs& p, int bid, int stride = 0,
+                                                  int total = 0) {
   constexpr int NW = WM * WN;
   constexpr int TM = BM / WM / 16;
   constexpr int TN = BN / WN / 16;
@@ -42,15 +51,14 @@ __device__ __forceinline__ void gemm_stream8_body(const GemmArgs& p, int bid) {
   static_assert(DT == ASTERGEMM_FP8_E4M3, "fp8 operands");
   static_assert(BM % (8 * NW) == 0 && (8 * NW) % 16 == 0, "tile rows per wave");
   static_assert((TM == 8 || TM == 4) && TN == 4 && LH == 4, "side-instruction schedule below");
+  // vector stores of one wave's walk epilogue (two per 16-row slab and 128 bytes of row)
+  constexpr int NST = TM * 2 * (OUT == ASTERGEMM_F32 ? 2 : 1);
+  static_assert(2 * LH + NST <= 63, "the counted waits fit the vmcnt field");
 
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wm = wave / WN, wn = wave % WN;
-
-  int tile_m, tile_n;
-  map_tile(bid, p.tiles_m, p.tiles_n, p.group_m, tile_m, tile_n);
-  const int row0 = tile_m * BM, col0 = tile_n * BN;
 
   // ---- global -> LDS: identical to the 16-bit stream kernel --------------------------------
   const int lane = threadIdx.x & 63;
@@ -58,10 +66,24 @@ __device__ __forceinline__ void gemm_stream8_body(const GemmArgs& p, int bid) {
   const int g_lane = (lane & 7) ^ (((wave * 8 + lrow) >> 1) & 7);
   const unsigned a_off = (unsigned)(lrow * (int)p.lda_bytes + g_lane * 16);
   const unsigned b_off = (unsigned)(lrow * (int)p.ldb_bytes + g_lane * 16);
+  // what depends on the tile
+  int row0, col0;
   const uint8_t* a_base[LH];
   const uint8_t* b_base[LH];
-  group_bases<LH, NW>(p.A, p.lda_bytes, row0 + wave * 8, p.M, a_base);
-  group_bases<LH, NW>(p.B, p.ldb_bytes, col0 + wave * 8, p.N, b_base);
+  auto set_tile = [&](int id) {
+    int tile_m, tile_n;
+    map_tile(id, p.tiles_m, p.tiles_n, p.group_m, tile_m, tile_n);
+    row0 = tile_m * BM, col0 = tile_n * BN;
+    if constexpr (WALK) {
+      // whole tiles: transfer j starts 8 * NW rows behind transfer j - 1, one base is enough
+      a_base[0] = p.A + (int64_t)(row0 + wave * 8) * p.lda_bytes;
+      b_base[0] = p.B + (int64_t)(col0 + wave * 8) * p.ldb_bytes;
+    } else {
+      group_bases<LH, NW>(p.A, p.lda_bytes, row0 + wave * 8, p.M, a_base);
+      group_bases<LH, NW>(p.B, p.ldb_bytes, col0 + wave * 8, p.N, b_base);
+    }
+  };
+  set_tile(bid);
   const int nk = p.ksteps - (p.tail_granules ? 1 : 0);  // whole 128-byte steps
 
   auto g2s = [&](const uint8_t* base, unsigned voff, uint8_t* dst) {
@@ -72,12 +94,12 @@ __device__ __forceinline__ void gemm_stream8_body(const GemmArgs& p, int bid) {
                  : "memory", "m0");
   };
   auto issue_a1 = [&](int k, int slot, int j) {  // slot: 0..2
-    g2s(a_base[j] + (int64_t)k * kRowBytes, a_off,
-        lds + slot * SLOT + (j * NW + wave) * 8 * kRowBytes);
+    const uint8_t* base = WALK ? a_base[0] + (int64_t)j * (8 * NW) * p.lda_bytes : a_base[j];
+    g2s(base + (int64_t)k * kRowBytes, a_off, lds + slot * SLOT + (j * NW + wave) * 8 * kRowBytes);
   };
   auto issue_b1 = [&](int k, int slot, int j) {  // slot: 3..4
-    g2s(b_base[j] + (int64_t)k * kRowBytes, b_off,
-        lds + slot * SLOT + (j * NW + wave) * 8 * kRowBytes);
+    const uint8_t* base = WALK ? b_base[0] + (int64_t)j * (8 * NW) * p.ldb_bytes : b_base[j];
+    g2s(base + (int64_t)k * kRowBytes, b_off, lds + slot * SLOT + (j * NW + wave) * 8 * kRowBytes);
   };
   auto issue_a = [&](int k, int slot) {
 #pragma unroll
@@ -119,38 +141,49 @@ __device__ __forceinline__ void gemm_stream8_body(const GemmArgs& p, int bid) {
   };
 
   f32x4 acc[TM][TN];
+  auto zero_acc = [&]() {
 #pragma unroll
-  for (int m = 0; m < TM; ++m)
+    for (int m = 0; m < TM; ++m)
 #pragma unroll
-    for (int n = 0; n < TN; ++n) {
-      acc[m][n] = f32x4{0.f, 0.f, 0.f, 0.f};
-      // opaque to the optimiser: otherwise the first MFMA of every tile reads one shared
-      // zero tuple and writes a fresh one, and 128 accumulators + 4 no longer fit
-      asm volatile("" : "+v"(acc[m][n]));
-    }
-
-  // ---- prologue: A(0) B(0) A(1) B(1) issued; A-row fragments and the first B-row fragment
-  // of K-step 0 read -----------------------------------------------------------------------------
-  issue_a(0, a_slot(0));
-  issue_b(0, b_slot(0));
-  if (nk > 1) {
-    issue_a(1, a_slot(1));
-    issue_b(1, b_slot(1));
-    __builtin_amdgcn_s_waitcnt(waitcnt_imm(2 * LH, 15));
-  } else {
-    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
-  }
-  __builtin_amdgcn_s_barrier();
-  asm volatile("" ::: "memory");
+      for (int n = 0; n < TN; ++n) {
+        acc[m][n] = f32x4{0.f, 0.f, 0.f, 0.f};
+        // opaque to the optimiser: otherwise the first MFMA of every tile reads one shared
+        // zero tuple and writes a fresh one, and 128 accumulators + 4 no longer fit
+        asm volatile("" : "+v"(acc[m][n]));
+      }
+  };
   using K0 = std::integral_constant<int, 0>;
-  read_b(b_slot(0), K0{});
-  {
+  // A-row fragments and the first B-row fragment of K-step 0 (slots 0 and 3)
+  auto first_reads = [&]() {
+    read_b(b_slot(0), K0{});
     const uint8_t* sa = lds + ((unsigned)(a_slot(0) * SLOT) + a_rd);
     const uint8_t* p0 = sa + rd0;
     const uint8_t* p1 = sa + rd1;
     static_for<0, TM>([&](auto m) { read_a(m, p0, p1); });
+  };
+  bool stores_behind = false;  // walk: the previous tile's stores are still counted
+
+  // ---- prologue: A(0) B(0) A(1) B(1) issued; A-row fragments and the first B-row fragment
+  // of K-step 0 read -----------------------------------------------------------------------------
+  if constexpr (!WALK) zero_acc();
+  issue_a(0, a_slot(0));
+  issue_b(0, b_slot(0));
+  if constexpr (!WALK) {
+    if (nk > 1) {
+      issue_a(1, a_slot(1));
+      issue_b(1, b_slot(1));
+      __builtin_amdgcn_s_waitcnt(waitcnt_imm(2 * LH, 15));
+    } else {
+      __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
+    }
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    first_reads();
+    __builtin_amdgcn_sched_barrier(0);
+  } else {
+    issue_a(1, a_slot(1));
+    issue_b(1, b_slot(1));
   }
-  __builtin_amdgcn_sched_barrier(0);
 
   // ---- K loop: trip k multiplies K-step k ------------------------------------------------------
   //   MFMA  0         + B-row fragment 1 of K-step k          (8: fragment 2, 16: fragment 3)
@@ -164,9 +197,11 @@ __device__ __forceinline__ void gemm_stream8_body(const GemmArgs& p, int bid) {
   // k+1, so that the loop header comes right after the full wait and the barrier and the
   // compiler's own wait counts inside the body stay exact.
   // ia = k mod 3, ib = k mod 2.  FIRST: MFMAs 0..BAR-1 and the barrier; else MFMAs BAR..31.
-  auto part = [&](int k, int ia, int ib, auto first, auto steady) {
+  // W0: trip 0 of a walked tile, whose barrier may leave the previous tile's stores in flight
+  auto part = [&](int k, int ia, int ib, auto first, auto steady, auto w0) {
     constexpr bool FIRST = decltype(first)::value;
     constexpr bool STEADY = decltype(steady)::value;
+    constexpr bool W0 = decltype(w0)::value;
     const bool do_ld = STEADY || k + 2 < nk;
     const bool do_rd = STEADY || k + 1 < nk;
     const int a_next = ia == 2 ? 0 : ia + 1;       // slot of A(k+1)
@@ -186,8 +221,15 @@ __device__ __forceinline__ void gemm_stream8_body(const GemmArgs& p, int bid) {
       if constexpr (I == BAR - 1) {
         __builtin_amdgcn_sched_barrier(0);
         if (do_rd) {
-          if constexpr (STEADY) __builtin_amdgcn_s_waitcnt(waitcnt_imm(LH, 0));
-          else __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
+          if constexpr (W0) {
+            // younger than A(1), B(1): the stores, then the LH transfers of A(2)
+            if (stores_behind) __builtin_amdgcn_s_waitcnt(waitcnt_imm(LH + NST, 0));
+            else __builtin_amdgcn_s_waitcnt(waitcnt_imm(LH, 0));
+          } else if constexpr (STEADY) {
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(LH, 0));
+          } else {
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
+          }
           __builtin_amdgcn_s_barrier();
           asm volatile("" ::: "memory");
         }
@@ -213,31 +255,79 @@ __device__ __forceinline__ void gemm_stream8_body(const GemmArgs& p, int bid) {
                 "schedule positions");
   using T = std::true_type;
   using F = std::false_type;
-  int k = 0, ia = 0, ib = 0;
-  part(0, 0, 0, T{}, F{});
+  // the K loop of one tile, from MFMA 0 of trip 0 to the last MFMA
+  auto k_loop = [&](auto w0) {
+    int k = 0, ia = 0, ib = 0;
+    part(0, 0, 0, T{}, w0, w0);  // a walked tile has K-steps 1 and 2 to read and to request
 #pragma unroll 1
-  for (; k + 3 < nk; ++k) {
-    part(k, ia, ib, F{}, T{});
-    ia = ia == 2 ? 0 : ia + 1;
-    ib ^= 1;
-    part(k + 1, ia, ib, T{}, T{});
-  }
+    for (; k + 3 < nk; ++k) {
+      part(k, ia, ib, F{}, T{}, F{});
+      ia = ia == 2 ? 0 : ia + 1;
+      ib ^= 1;
+      part(k + 1, ia, ib, T{}, T{}, F{});
+    }
 #pragma unroll 1
-  for (; k < nk; ++k) {
-    part(k, ia, ib, F{}, F{});
-    ia = ia == 2 ? 0 : ia + 1;
-    ib ^= 1;
-    if (k + 1 < nk) part(k + 1, ia, ib, T{}, F{});
+    for (; k < nk; ++k) {
+      part(k, ia, ib, F{}, F{}, F{});
+      ia = ia == 2 ? 0 : ia + 1;
+      ib ^= 1;
+      if (k + 1 < nk) part(k + 1, ia, ib, T{}, F{}, F{});
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  if constexpr (!WALK) {
+    k_loop(F{});
+    if (p.tail_granules) stream_k_tail<DT, BM, BN, WM, WN>(p, acc, wave, row0, col0, nk);
+    stream_epilogue<OUT, BM, BN, WM, WN>(p, acc, lds, wave, row0, col0);
+  } else {
+    // One path for every tile (the accumulators never meet a join): the last tile of a workgroup
+    // requests its own first two K-steps again, into slots nothing reads any more.
+    int tile = bid;
+    for (;;) {
+      zero_acc();
+      // A(0), B(0) have landed; A(1), B(1) and, behind them, the stores may be in flight
+      if (stores_behind) __builtin_amdgcn_s_waitcnt(waitcnt_imm(2 * LH + NST, 15));
+      else __builtin_amdgcn_s_waitcnt(waitcnt_imm(2 * LH, 15));
+      // also: every wave is through its epilogue, whose staging memory trip 0 gives to A(2)
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      first_reads();
+      __builtin_amdgcn_sched_barrier(0);
+      k_loop(T{});
+      // every wave has left the ring before anything is requested into it
+      __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      const bool more = tile + stride < total;
+      const int wrow0 = row0 + wm * TM * 16, wcol0 = col0 + wn * TN * 16;
+      set_tile(more ? tile + stride : tile);
+      issue_a(0, a_slot(0));
+      issue_b(0, b_slot(0));
+      issue_a(1, a_slot(1));
+      issue_b(1, b_slot(1));
+      __builtin_amdgcn_sched_barrier(0);
+      walk_epilogue<OUT, TM, TN>(p, acc, lds + 2 * SLOT + wave * 4096, wrow0, wcol0);
+      __builtin_amdgcn_sched_barrier(0);
+      if (!more) break;
+      tile += stride;
+      stores_behind = true;
+    }
+    // the transfers the last tile requested must have landed before the workgroup gives its
+    // LDS back
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
   }
-  __builtin_amdgcn_sched_barrier(0);
-
-  if (p.tail_granules) stream_k_tail<DT, BM, BN, WM, WN>(p, acc, wave, row0, col0, nk);
-  stream_epilogue<OUT, BM, BN, WM, WN>(p, acc, lds, wave, row0, col0);
 }
 
 template <int DT, int OUT, int BM, int BN, int WM, int WN>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_stream8_kernel(const GemmArgs p) {
   gemm_stream8_body<DT, OUT, BM, BN, WM, WN>(p, blockIdx.x);
+}
+
+// Tile walk: grid = one workgroup per CU, workgroup b takes tiles b, b + grid, ...
+template <int DT, int OUT, int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(WM* WN * 64) void gemm_stream8_walk_kernel(const GemmArgs p) {
+  gemm_stream8_body<DT, OUT, BM, BN, WM, WN, true>(p, blockIdx.x, gridDim.x,
+                                                  p.tiles_m * p.tiles_n);
 }
 
 // Split K (see gemm_stream_splitk_kernel): copy s of the tile grid multiplies K steps

@@ -764,7 +764,7 @@ def test_config3_full_size_fp8_row_sample_determinism_and_scaling(gpu):
     M = N = K = 8192
     a, b, ex = operands(M, N, K, "fp8_e4m3", a_std=1.0, b_std=1.0)
     out, name = run_gemm(a, b, M, N, K, "fp8_e4m3", "bf16", **ex)
-    assert name == "stream_fp8_256x256_w2x4_bf16"
+    assert name == "stream_fp8_256x256_w2x4_walk_bf16"   # 1024 tiles: four per workgroup
     rows, cols = _sampled_rows_and_cols(M, N)
     check(out[rows], G.gemm_fp8(a[rows], b, ex["scale_a"], ex["scale_b"], out_dtype=G.BF16), "bf16", N)
     check(out[:, cols], G.gemm_fp8(a, b[cols], ex["scale_a"], ex["scale_b"], out_dtype=G.BF16),
@@ -853,10 +853,11 @@ def test_identity_operand_is_exact_at_full_width(gpu):
     assert np.array_equal(out, a)
 
 
-@pytest.mark.parametrize("dtype_ab,M", [("bf16", 2048), ("fp8_e4m3", 2048), ("mxfp4", 4096)])
+@pytest.mark.parametrize("dtype_ab,M", [("bf16", 2048), ("fp8_e4m3", 2048), ("fp8_e4m3", 4096),
+                                        ("mxfp4", 4096)])
 def test_band_tile_order_writes_every_tile_once(gpu, dtype_ab, M):
     # B = I at a size whose tile grid divides by 8 x 32 (all XCDs on one band of eight tile
-    # rows; the MXFP4 case has more tiles than CUs and goes through the tile walk): each output
+    # rows; with 4096 rows there are more tiles than CUs and the tile walks run): each output
     # is one product plus zeros, so C is A's values bit for bit and a tile that is skipped,
     # written twice from the wrong place or swapped with another shows
     N = K = 8192
@@ -883,8 +884,7 @@ def test_band_tile_order_writes_every_tile_once(gpu, dtype_ab, M):
         want = F.f32_to_bf16_bits(F.dequantize_mxfp4(a, mxa))
     out, name = run_gemm(a, b, M, N, K, dtype_ab, "bf16", **ex)
     assert name.startswith("stream_") and "256x256" in name, name
-    if dtype_ab == "mxfp4":
-        assert "_walk_" in name, name
+    assert ("_walk_" in name) == (M == 4096), name
     # as values: a negative zero of A comes out as the accumulator's positive zero
     assert np.array_equal(F.bf16_bits_to_f32(out), F.bf16_bits_to_f32(want))
 
@@ -1092,6 +1092,28 @@ def test_mxfp4_tile_walk_equals_the_plain_kernel(gpu, K, dtype_c):
     rows = np.unique(np.concatenate([rng.integers(0, M, 12), [0, 255, 256, M - 1]]))
     want = G.gemm_mxfp4(a[rows], mxa[rows], b, mxb, out_dtype=_DT[dtype_c], bias=bias)
     check(walk[rows], want, dtype_c, N, bar=1e-5 if dtype_c == "f32" else REL_L2_BAR)
+
+
+@pytest.mark.parametrize("K", [512, 640, 768, 896, 2048])
+@pytest.mark.parametrize("dtype_c", ["bf16", "f32"])
+def test_fp8_tile_walk_equals_the_plain_kernel(gpu, K, dtype_c):
+    """The fp8 tile walk (one workgroup per CU takes several tiles in one launch; the next tile's
+    first two K-steps arrive during the epilogue, whose stores stay in flight into the next tile)
+    on more tiles than any device has CUs, K-step counts 4, 5, 6, 7 (every phase of the three A
+    and two B slots at the end of a tile) and 16: the same bits as the one-tile-per-workgroup
+    kernel, and sampled rows against the oracle.  The walk takes whole tiles only."""
+    M, N = 4352, 4608   # 17 x 18 = 306 tiles of 256 x 256
+    a, b, ex = operands(M, N, K, "fp8_e4m3", seed=5 + K, a_std=1.0, b_std=1.0)
+    bias = np.random.default_rng(K).standard_normal(N).astype(np.float32)
+    plain, pname = run_gemm(a, b, M, N, K, "fp8_e4m3", dtype_c, bias=bias,
+                            variant=_variant_id(f"stream_fp8_256x256_w2x4_{dtype_c}"), **ex)
+    walk, wname = run_gemm(a, b, M, N, K, "fp8_e4m3", dtype_c, bias=bias,
+                           variant=_variant_id(f"stream_fp8_256x256_w2x4_walk_{dtype_c}"), **ex)
+    assert pname == f"stream_fp8_256x256_w2x4_{dtype_c}" and wname == f"stream_fp8_256x256_w2x4_walk_{dtype_c}"
+    assert np.array_equal(walk.view(np.uint8), plain.view(np.uint8))
+    rows = np.unique(np.concatenate([np.random.default_rng(1).integers(0, M, 12), [0, 255, 256, M - 1]]))
+    want = G.gemm_fp8(a[rows], b, ex["scale_a"], ex["scale_b"], out_dtype=_DT[dtype_c], bias=bias)
+    check(walk[rows], want, dtype_c, N)
 
 
 def test_mxfp4_stream_kernel_falls_back_for_odd_kstep_counts(gpu):

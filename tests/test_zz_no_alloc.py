@@ -94,7 +94,10 @@ def test_caller_workspace_matches_the_library_workspace(gpu):
 
 
 def _hip():
-    lib = ctypes.CDLL("libamdhip64.so")
+    # the HIP runtime the library itself is linked against, found through the library's own handle
+    # (another copy of libamdhip64 may be loaded in this process, e.g. the one torch ships, and a
+    # stream of one runtime means nothing to the other)
+    lib = _capi.load()
     for name, args in (("hipStreamBeginCapture", [ctypes.c_void_p, ctypes.c_int]),
                        ("hipStreamEndCapture", [ctypes.c_void_p, ctypes.POINTER(ctypes.c_void_p)]),
                        ("hipGraphInstantiate", [ctypes.POINTER(ctypes.c_void_p), ctypes.c_void_p,
