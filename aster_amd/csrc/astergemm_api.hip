@@ -89,9 +89,8 @@ const char* validate_problem(const astergemm_config& c) {
     return "bad scale_mode";
   if (c.operand_path < ASTERGEMM_OPERAND_LDS || c.operand_path > ASTERGEMM_OPERAND_DIRECT_B_K8)
     return "bad operand_path";
-  if (c.operand_path == ASTERGEMM_OPERAND_DIRECT_B_K8 && c.dtype_ab != ASTERGEMM_F16 &&
-      c.dtype_ab != ASTERGEMM_BF16)
-    return "B pre-shuffled in K8 order is built for 16-bit operands";
+  if (c.operand_path == ASTERGEMM_OPERAND_DIRECT_B_K8 && c.dtype_ab == ASTERGEMM_FP8_E4M3)
+    return "B pre-shuffled for the stream kernels is built for 16-bit and MXFP4 operands";
   if ((c.dtype_ab == ASTERGEMM_MXFP4) != (c.scale_mode == ASTERGEMM_SCALE_MX32))
     return "MXFP4 operands and SCALE_MX32 go together";
   if (c.dtype_ab == ASTERGEMM_MXFP4 && c.K % 32 != 0) return "MXFP4 needs K % 32 == 0";
@@ -733,6 +732,24 @@ int astergemm_shuffle_scales_e8m0(const uint8_t* src, uint8_t* dst, int64_t N, i
   for (int64_t nb = 0; nb < N / 16; ++nb)
     for (int64_t st = 0; st < steps; ++st)
       for (int nl = 0; nl < 16; ++nl, o += 8) memcpy(o, src + (nb * 16 + nl) * ld + st * 8, 8);
+  return 0;
+}
+
+int astergemm_shuffle_scales_e8m0_lanes(const uint8_t* src, uint8_t* dst, int64_t N, int64_t K) {
+  if (!src || !dst || N < 0 || K < 0 || N % 64 != 0 || K % 256 != 0) {
+    set_error("astergemm_shuffle_scales_e8m0_lanes: need N %% 64 == 0 and K %% 256 == 0");
+    return ASTERGEMM_EINVAL;
+  }
+  // dst order (nb4, step, lane group q, row i, tile t, half h) <- src (nb4, t, i, step, 4 h + q)
+  const int64_t steps = K / 256, ld = K / 32;
+  uint8_t* o = dst;
+  for (int64_t nb4 = 0; nb4 < N / 64; ++nb4)
+    for (int64_t st = 0; st < steps; ++st)
+      for (int q = 0; q < 4; ++q)
+        for (int i = 0; i < 16; ++i)
+          for (int t = 0; t < 4; ++t)
+            for (int h = 0; h < 2; ++h)
+              *o++ = src[(nb4 * 64 + t * 16 + i) * ld + st * 8 + 4 * h + q];
   return 0;
 }
 

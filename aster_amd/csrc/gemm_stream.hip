@@ -5,6 +5,7 @@
 #include "gemm_stream8_kernel.hpp"
 #include "gemm_stream4_kernel.hpp"
 #include "gemm_streamdb_kernel.hpp"
+#include "gemm_stream4db_kernel.hpp"
 
 namespace astergemm {
 namespace {
@@ -78,6 +79,42 @@ const char* check_streamdb(const astergemm_config& c) {
         (const void*)gemm_streamdb_kernel<DT, OUT, NSLOT, NBUF, WM>,             \
         launch_streamdb<DT, OUT, NSLOT, NBUF, WM>, check_streamdb,               \
         ASTERGEMM_OPERAND_DIRECT_B_K8                                            \
+  }
+
+// ---- MXFP4, B pre-shuffled (payload in step order, scale plane in lane order) and loaded
+// straight into MFMA operands: 128 x 256 tiles, four waves (gemm_stream4db_kernel.hpp) ---------
+template <int DT, int OUT>
+int launch_stream4db(const GemmArgs& a, int grid, hipStream_t s) {
+  constexpr int lds = 4 * 128 * kRowBytes + 2 * 128 * 16;
+  auto k = gemm_stream4db_kernel<DT, OUT>;
+  static std::atomic<uint64_t> attr_devs{0};
+  if (int e = lds_attr_once(attr_devs, (const void*)k, lds)) return e;
+  // what the kernel's indexing assumes: whole 64-row groups of B, an even number of whole
+  // K-steps, packed B, A scale rows fetched in 16-byte granules
+  if (a.N % 64 != 0 || a.N < 64 || a.M < 8 || a.M % 8 != 0 || a.K % 512 != 0 || a.tail_granules != 0 ||
+      a.ldb_bytes != (int64_t)a.K / 2 || (((uintptr_t)a.mx_a | (uintptr_t)a.mx_b) & 15) != 0 ||
+      a.mx_ld % 16 != 0)
+    return (int)hipErrorInvalidValue;
+  hipLaunchKernelGGL(k, dim3(grid), dim3(256), lds, s, a);
+  return (int)hipGetLastError();
+}
+
+const char* check_stream4db(const astergemm_config& c) {
+  if (c.M % 8 != 0 || c.M < 8) return "M must be a multiple of 8";
+  if (c.N % 64 != 0 || c.N < 64) return "the pre-shuffled scale plane needs N % 64 == 0";
+  if (c.K % 512 != 0) return "K must be a multiple of 512";
+  if (c.ldb != 0 && c.ldb != c.K) return "pre-shuffled B is packed (ldb = K)";
+  if (c.ldc % 8 != 0) return "ldc must be a multiple of 8 elements";
+  if (c.N * (c.K / 2) >= ((int64_t)1 << 32)) return "pre-shuffled B must stay below 4 GiB";
+  return nullptr;
+}
+
+#define AG_STREAM4DB(name, DT, OUT)                                              \
+  Variant {                                                                      \
+    name, ASTERGEMM_KERNEL_TILE, DT, OUT, 128, 256, kRowBytes, 1, 4, 4, 2,       \
+        4 * 128 * kRowBytes + 2 * 128 * 16,                                      \
+        (const void*)gemm_stream4db_kernel<DT, OUT>, launch_stream4db<DT, OUT>,  \
+        check_stream4db, ASTERGEMM_OPERAND_DIRECT_B_K8                           \
   }
 
 // ---- split K on the 128x128 kernel --------------------------------------------------------
@@ -507,6 +544,9 @@ const Variant kStreamVariants[] = {
     AG_STREAM4_WALK("stream_mxfp4_256x256_w2x4_walk_bf16", ASTERGEMM_MXFP4, ASTERGEMM_BF16),
     AG_STREAM4_WALK("stream_mxfp4_256x256_w2x4_walk_f32", ASTERGEMM_MXFP4, ASTERGEMM_F32),
     AG_STREAM4_WALK("stream_mxfp4_256x256_w2x4_walk_f16", ASTERGEMM_MXFP4, ASTERGEMM_F16),
+    AG_STREAM4DB("streamdb_mxfp4_128x256_w1x4_bf16", ASTERGEMM_MXFP4, ASTERGEMM_BF16),
+    AG_STREAM4DB("streamdb_mxfp4_128x256_w1x4_f32", ASTERGEMM_MXFP4, ASTERGEMM_F32),
+    AG_STREAM4DB("streamdb_mxfp4_128x256_w1x4_f16", ASTERGEMM_MXFP4, ASTERGEMM_F16),
     AG_STREAM4_128("stream_mxfp4_128x128_w2x2_bf16", ASTERGEMM_MXFP4, ASTERGEMM_BF16),
     AG_STREAM4_128("stream_mxfp4_128x128_w2x2_f32", ASTERGEMM_MXFP4, ASTERGEMM_F32),
     AG_STREAM4_128("stream_mxfp4_128x128_w2x2_f16", ASTERGEMM_MXFP4, ASTERGEMM_F16),

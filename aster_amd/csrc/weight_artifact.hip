@@ -70,8 +70,13 @@ extern "C" int astergemm_weight_header_init(astergemm_weight_header* h, int dtyp
   if (astergemm::row_bytes(dtype, K) % 16 != 0) return fail("a row must be a multiple of 16 bytes");
   if (layout == ASTERGEMM_OPERAND_DIRECT_B || layout == ASTERGEMM_OPERAND_DIRECT_B_K8) {
     const bool is16 = dtype == ASTERGEMM_F16 || dtype == ASTERGEMM_BF16;
-    if (!is16 && layout == ASTERGEMM_OPERAND_DIRECT_B_K8)
-      return fail("the K8 pre-shuffled layout holds 16-bit elements");
+    if (dtype == ASTERGEMM_FP8_E4M3 && layout == ASTERGEMM_OPERAND_DIRECT_B_K8)
+      return fail("the stream kernels' pre-shuffled layout holds 16-bit or MXFP4 elements");
+    // MXFP4 for the stream kernel: payload in step order, scale plane in lane order
+    // (astergemm_shuffle_scales_e8m0_lanes)
+    if (dtype == ASTERGEMM_MXFP4 && layout == ASTERGEMM_OPERAND_DIRECT_B_K8 &&
+        (N % 64 != 0 || K % 256 != 0))
+      return fail("the stream kernels' pre-shuffled MXFP4 layout needs N % 64 == 0, K % 256 == 0");
     if (is16 && (N % 16 != 0 || K % 32 != 0))
       return fail("the pre-shuffled layouts need N % 16 == 0, K % 32 == 0");
     // fp8 / MXFP4: step order (astergemm_shuffle_weight_8, astergemm_shuffle_scales_e8m0)

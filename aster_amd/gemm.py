@@ -114,13 +114,14 @@ def select_for_instance(cfg: WeakScaledMappedGemmInstance) -> Tuple[_capi.Config
     """Honour the instance's mapping when a variant with that geometry exists, otherwise let the
     library choose (`mapping_report` tells which happened).  A `direct_b` mapping gets a kernel
     that reads pre-shuffled B when one takes the shape -- the decode kernels in the reference's
-    `shuffle_weight` order, else the 256 x 256 stream kernel in `shuffle_weight_k8` order (the
+    `shuffle_weight` order, else the stream kernels in `shuffle_weight_k8` order (MXFP4: step
+    order with the scale plane in lane order) (the
     returned config's `operand_path` says which; `execute_gemm_hsaco` shuffles accordingly) --
     and falls back to plain row-major B otherwise."""
     want_direct = cfg.mapping.direct_b and not cfg.mapping.direct_a
     paths = [_capi.OPERAND_DIRECT_B] if want_direct else []
-    if want_direct and cfg.spec.dtype_ab in ("bf16", "f16"):
-        paths.append(_capi.OPERAND_DIRECT_B_K8)          # the K8 order holds 16-bit elements
+    if want_direct and cfg.spec.dtype_ab in ("bf16", "f16", "mxfp4"):
+        paths.append(_capi.OPERAND_DIRECT_B_K8)          # the stream kernels: 16-bit and MXFP4
     for use_mapping in (True, False):
         for path in paths + [_capi.OPERAND_LDS]:
             if not use_mapping and path == _capi.OPERAND_LDS and not want_direct:
@@ -201,8 +202,10 @@ class GemmPlan:
                variant: int = 0, operand_path: str = "lds") -> "GemmPlan":
         """`operand_path` follows GemmMappingSpec.operand_path of the reference: "lds" = B is
         plain row-major [N, ldb]; "direct_b" = B was pre-shuffled with `shuffle_weight` (the
-        reference's order, read by the decode kernels); "direct_b_k8" = pre-shuffled with
-        `shuffle_weight_k8` (read by the 256 x 256 stream kernel)."""
+        reference's order, read by the decode kernels; fp8 / MXFP4: `shuffle_weight_bytes`, the
+        MXFP4 plane with `shuffle_scales_e8m0`); "direct_b_k8" = pre-shuffled for the stream
+        kernels: 16-bit operands with `shuffle_weight_k8`, MXFP4 with `shuffle_weight_bytes` and
+        the scale plane with `shuffle_scales_e8m0_lanes`."""
         c = _capi.Config()
         c.operand_path = _OPERAND_PATH_ID[operand_path]
         c.M, c.N, c.K = M, N, K
@@ -377,13 +380,15 @@ def execute_gemm_hsaco(cfg: WeakScaledMappedGemmInstance, hsaco_path: str, num_i
         # single point of truth, as in the reference's execute_fn
         # (test_102_gemm_python_multitile_g2s_directb_cdna4.py:446-467): the caller passes B
         # row-major and the pre-shuffle happens here, in the order the kernel that runs reads
-        from .kittens_helpers import (shuffle_scales_e8m0, shuffle_weight, shuffle_weight_bytes,
-                                      shuffle_weight_k8)
+        from .kittens_helpers import (shuffle_scales_e8m0, shuffle_scales_e8m0_lanes, shuffle_weight,
+                                      shuffle_weight_bytes, shuffle_weight_k8)
 
         if cfg.spec.dtype_ab in ("fp8_e4m3", "mxfp4"):   # byte rows in step order (+ the e8m0 plane)
             B = shuffle_weight_bytes(np.ascontiguousarray(B).reshape(N, -1).view(np.uint8))
-            if mx_b is not None:
-                mx_b = shuffle_scales_e8m0(np.asarray(mx_b, dtype=np.uint8).reshape(N, K // 32))
+            if mx_b is not None:   # decode kernels: step order; stream kernel: lane order
+                sc_shuffle = (shuffle_scales_e8m0 if c.operand_path == _capi.OPERAND_DIRECT_B
+                              else shuffle_scales_e8m0_lanes)
+                mx_b = sc_shuffle(np.asarray(mx_b, dtype=np.uint8).reshape(N, K // 32))
         else:
             shuffle = shuffle_weight if c.operand_path == _capi.OPERAND_DIRECT_B else shuffle_weight_k8
             B = shuffle(np.ascontiguousarray(B).reshape(N, K))

@@ -142,3 +142,27 @@ def unshuffle_scales_e8m0(Ss: np.ndarray) -> np.ndarray:
     N, nb = Ss.shape
     view = np.ascontiguousarray(Ss).reshape(N // 16, nb // 8, 16, 8)
     return np.ascontiguousarray(view.transpose(0, 2, 1, 3)).reshape(N, nb)
+
+
+def shuffle_scales_e8m0_lanes(S: np.ndarray) -> np.ndarray:
+    """The e8m0 plane S[N, K/32] of pre-shuffled MXFP4 weights in LANE ORDER, for the stream
+    kernel that loads B straight into MFMA operands: view it as (group of 64 rows, tile t=4,
+    row i=16, step, half h=2, lane group q=4) and store (group, step, q, i, t, h), so that lane
+    16 q + i of a wave finds, in the 8 bytes at 8 (16 q + i) of the 512 bytes of (group, step),
+    the scales of blocks q (h = 0) and 4 + q (h = 1) of its row in each of the wave's four
+    16-row tiles: the byte pairs the two MFMAs of a 256-element step select with op_sel."""
+    S = np.ascontiguousarray(S, dtype=np.uint8)
+    N, nb = S.shape
+    if N % 64 != 0:
+        raise AssertionError(f"N={N} must be multiple of 64")
+    if nb % 8 != 0:
+        raise AssertionError(f"{nb} scale bytes per row are not whole 256-element steps")
+    view = S.reshape(N // 64, 4, 16, nb // 8, 2, 4)
+    return np.ascontiguousarray(view.transpose(0, 3, 5, 2, 1, 4)).reshape(N, nb)
+
+
+def unshuffle_scales_e8m0_lanes(Ss: np.ndarray) -> np.ndarray:
+    """Inverse of `shuffle_scales_e8m0_lanes`."""
+    N, nb = Ss.shape
+    view = np.ascontiguousarray(Ss).reshape(N // 64, nb // 8, 4, 16, 4, 2)
+    return np.ascontiguousarray(view.transpose(0, 4, 3, 1, 5, 2)).reshape(N, nb)

@@ -24,8 +24,8 @@ import numpy as np
 from . import _capi
 from .execution import GpuBuffer
 from .gemm import GemmPlan
-from .kittens_helpers import (shuffle_scales_e8m0, shuffle_weight, shuffle_weight_bytes,
-                              shuffle_weight_k8)
+from .kittens_helpers import (shuffle_scales_e8m0, shuffle_scales_e8m0_lanes, shuffle_weight,
+                              shuffle_weight_bytes, shuffle_weight_k8)
 
 _LAYOUT_ID = {"lds": _capi.OPERAND_LDS, "direct_b": _capi.OPERAND_DIRECT_B,
               "direct_b_k8": _capi.OPERAND_DIRECT_B_K8}
@@ -72,7 +72,9 @@ class WeightArtifact:
         """`bits` is the matrix as a kernel reads it: [N, K] float16 / uint16 (bf16 bits) /
         uint8 (e4m3), or [N, K/2] uint8 nibbles with `scales` [N, K/32] for MXFP4.  For
         layout "direct_b" the bits must already be in `shuffle_weight` order (16-bit types) or
-        `shuffle_weight_bytes` order (fp8, MXFP4; the MXFP4 plane in `shuffle_scales_e8m0` order)."""
+        `shuffle_weight_bytes` order (fp8, MXFP4; the MXFP4 plane in `shuffle_scales_e8m0` order),
+        for "direct_b_k8" in `shuffle_weight_k8` order (16-bit types) or `shuffle_weight_bytes`
+        order with the plane in `shuffle_scales_e8m0_lanes` order (MXFP4)."""
         h = _capi.WeightHeader()
         _capi.check(_capi.load().astergemm_weight_header_init(
             ctypes.byref(h), _capi.DTYPE_NAMES[dtype], _LAYOUT_ID[layout], N, K,
@@ -111,8 +113,8 @@ class WeightArtifact:
                 bits = shuffle_weight_k8(bits)
             return cls.from_storage(bits, dtype, N, K, layout=layout)
         from . import quantize as Q
-        if layout == "direct_b_k8":
-            raise ValueError("layout direct_b_k8 holds 16-bit elements")
+        if layout == "direct_b_k8" and dtype != "mxfp4":
+            raise ValueError("layout direct_b_k8 holds 16-bit or MXFP4 elements")
         if dtype == "fp8_e4m3":
             q, s = Q.quantize_fp8_tensor(w)
             if layout == "direct_b":
@@ -120,9 +122,10 @@ class WeightArtifact:
             return cls.from_storage(q, dtype, N, K, layout=layout, tensor_scale=float(s))
         if dtype == "mxfp4":
             p, s = Q.quantize_mxfp4(w)
-            if layout == "direct_b":
+            if layout in ("direct_b", "direct_b_k8"):   # decode kernels / stream kernel
                 p = shuffle_weight_bytes(np.asarray(p).reshape(N, K // 2).view(np.uint8))
-                s = shuffle_scales_e8m0(np.asarray(s).reshape(N, K // 32))
+                sc_shuffle = shuffle_scales_e8m0 if layout == "direct_b" else shuffle_scales_e8m0_lanes
+                s = sc_shuffle(np.asarray(s).reshape(N, K // 32))
             return cls.from_storage(p, dtype, N, K, layout=layout, scales=s)
         raise ValueError(f"from_f32: unknown dtype {dtype!r}")
 

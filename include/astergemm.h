@@ -89,11 +89,17 @@ typedef enum astergemm_operand_path {
                                      (MXFP4: dMxB pre-shuffled as well, with
                                      astergemm_shuffle_scales_e8m0).  The
                                      decode kernels, M <= 16                 */
-  ASTERGEMM_OPERAND_DIRECT_B_K8 = 2 /* B packed [N, K] and pre-shuffled with
+  ASTERGEMM_OPERAND_DIRECT_B_K8 = 2 /* B packed [N, K] and pre-shuffled for the
+                                     stream kernels that load B straight into
+                                     MFMA operands.  MXFP4: payload with
+                                     astergemm_shuffle_weight_8, dMxB with
+                                     astergemm_shuffle_scales_e8m0_lanes
+                                     (128 x 256 tiles, N % 64 == 0,
+                                     K % 512 == 0).  16-bit operands: with
                                      astergemm_shuffle_weight_k8_16: 8
                                      consecutive K per lane, the order of the
                                      16x16x32 MFMA and of 16-byte LDS reads
-                                     (16-bit operands; the 256 x 256 stream
+                                     (the 128 x 256 and 256 x 256 stream
                                      kernel, N % 16 == 0, K % 64 == 0)       */
 } astergemm_operand_path;
 
@@ -270,6 +276,16 @@ int astergemm_shuffle_weight_8(const uint8_t* src, uint8_t* dst, int64_t N, int6
  * order: the 8 scale bytes of row 16 nb + n, step s (256 elements) at
  * (nb * steps + s) * 128 + 8 n.  N % 16 == 0, K % 256 == 0. */
 int astergemm_shuffle_scales_e8m0(const uint8_t* src, uint8_t* dst, int64_t N, int64_t K);
+/* The e8m0 plane [N, K/32] of pre-shuffled MXFP4 weights in lane order, for
+ * the stream kernel that loads B straight into MFMA operands
+ * (ASTERGEMM_OPERAND_DIRECT_B_K8): rows in groups of 64 (four 16-row tiles, the
+ * columns of one wave), group nb4 and step s (256 elements) are 512 bytes at
+ * (nb4 * steps + s) * 512 in which lane L = 16 q + i of a wave finds, at byte
+ * 8 L + 2 t + h, the scale of block 4 h + q of row 64 nb4 + 16 t + i: one
+ * 8-byte load per lane brings the scale bytes of both MFMAs of a step for the
+ * wave's four tiles.  N % 64 == 0, K % 256 == 0.  No counterpart in the
+ * reference (it has no scaled MFMA kernels). */
+int astergemm_shuffle_scales_e8m0_lanes(const uint8_t* src, uint8_t* dst, int64_t N, int64_t K);
 
 /* ---- operand quantisers (device to device, on `stream`) -------------------
  * They write the bytes the fp8 / MXFP4 GEMM paths read (dtype_ab
@@ -319,10 +335,12 @@ int astergemm_quantize_mxfp4(const void* dSrc, int src_dtype, int64_t rows, int6
  * File = this 128-byte little-endian header, then the payload at
  * payload_offset (N rows; layout ASTERGEMM_OPERAND_LDS = row-major,
  * ASTERGEMM_OPERAND_DIRECT_B = astergemm_shuffle_weight_16 order,
- * ASTERGEMM_OPERAND_DIRECT_B_K8 = astergemm_shuffle_weight_k8_16 order, 16-bit
- * dtypes only; for fp8 and MXFP4 ASTERGEMM_OPERAND_DIRECT_B =
- * astergemm_shuffle_weight_8 order), then for MXFP4 the e8m0 plane [N, K/32]
- * at scales_offset (layout DIRECT_B: in astergemm_shuffle_scales_e8m0 order).
+ * ASTERGEMM_OPERAND_DIRECT_B_K8 = astergemm_shuffle_weight_k8_16 order for the
+ * 16-bit dtypes; for fp8 and MXFP4 ASTERGEMM_OPERAND_DIRECT_B and for MXFP4
+ * ASTERGEMM_OPERAND_DIRECT_B_K8 = astergemm_shuffle_weight_8 order), then for
+ * MXFP4 the e8m0 plane [N, K/32] at scales_offset (layout DIRECT_B: in
+ * astergemm_shuffle_scales_e8m0 order, DIRECT_B_K8: in
+ * astergemm_shuffle_scales_e8m0_lanes order).
  * Sections start on 256-byte boundaries.  FP8 carries its tensor scale in the
  * header.  Checksums are CRC-32 (the zlib polynomial) of each section.       */
 #define ASTERGEMM_WEIGHT_VERSION 1u

@@ -920,15 +920,19 @@ def test_every_tile_variant(gpu, vid, name, dtype_ab, dtype_c):
         M, N, K = 512, 32768 + 256, 1024  # 258 tiles: more than one per workgroup, four K-steps
     a, b, ex = operands(M, N, K, dtype_ab, seed=11, a_std=1.0, b_std=1.0 if dtype_ab != "bf16" else 0.05)
     bias = np.random.default_rng(12).standard_normal(N).astype(np.float32)
-    path, b_dev = "lds", b
-    if name.startswith("streamdb"):  # B pre-shuffled in K8 order
+    path, b_dev, ex_dev = "lds", b, ex
+    if name.startswith("streamdb_mxfp4"):  # payload in step order, scale plane in lane order
+        from aster_amd.kittens_helpers import shuffle_scales_e8m0_lanes, shuffle_weight_bytes
+        path, b_dev = "direct_b_k8", shuffle_weight_bytes(b)
+        ex_dev = dict(ex, mx_b=shuffle_scales_e8m0_lanes(ex["mx_b"]))
+    elif name.startswith("streamdb"):  # B pre-shuffled in K8 order
         from aster_amd.kittens_helpers import shuffle_weight_k8
         path, b_dev = "direct_b_k8", shuffle_weight_k8(np.ascontiguousarray(b).view(np.uint16))
     plan = AG.GemmPlan.create(M, N, K, dtype_ab, dtype_c, has_bias=True, variant=vid, operand_path=path)
     assert plan.info.name.decode() == name
     out = np.zeros((M, N), dtype=_OUT_NP[dtype_c])
     bufs = {}
-    for key, arr in dict(a=a, b=b_dev, c=out, bias=bias, **{k: np.asarray(v) for k, v in ex.items()}).items():
+    for key, arr in dict(a=a, b=b_dev, c=out, bias=bias, **{k: np.asarray(v) for k, v in ex_dev.items()}).items():
         arr = np.ascontiguousarray(arr if arr.ndim else arr.reshape(1).astype(np.float32))
         bufs[key] = GpuBuffer(arr.nbytes)
         bufs[key].copy_from_host(arr)
@@ -1202,6 +1206,53 @@ def test_stream_direct_b_k8(gpu, M, N, K, dtype_ab, dtype_c, tile_m):
                                  family=_capi.KERNEL_TILE)
     if lds_name.startswith("stream_"):
         assert G.rel_l2(G.output_to_f32(out, _DT[dtype_c]), G.output_to_f32(lds_out, _DT[dtype_c])) <= 1e-5
+
+
+@pytest.mark.parametrize("M,N,K", [(128, 256, 512), (128, 256, 1024), (256, 512, 1536), (128, 256, 2048),
+                                   (136, 320, 2560), (264, 576, 3072), (128, 256, 3584), (512, 768, 4096),
+                                   (1000, 1088, 4608), (128, 64, 5120), (512, 512, 8192)])
+@pytest.mark.parametrize("dtype_c", ["f32", "bf16"])
+def test_mxfp4_stream_direct_b(gpu, M, N, K, dtype_c):
+    """MXFP4 with B pre-shuffled (payload in step order, e8m0 plane in lane order) and loaded
+    straight into MFMA operands: 128 x 256 tiles, four waves.  K-step counts 2, 4, 6 (no steady
+    group), 8 (one steady group exactly), 10, 12, 14, 16, 18, 20, 32; edge tiles in M (multiple
+    of 8) and N (multiple of 64).  Scales differ from row to row and block to block, so a wrong
+    scale byte (row, block, tile or half) shows.  Against the oracle, and the same bits as the
+    kernel that takes B row-major through LDS."""
+    from aster_amd.kittens_helpers import shuffle_scales_e8m0_lanes, shuffle_weight_bytes
+    rng = np.random.default_rng(K + M)
+    xa = rng.standard_normal((M, K)).astype(np.float32) * (2.0 ** rng.integers(-3, 4, (M, 1))).astype(np.float32)
+    xb = rng.standard_normal((N, K)).astype(np.float32) * (2.0 ** rng.integers(-3, 4, (N, 1))).astype(np.float32)
+    xa.reshape(M, K // 32, 32)[:] *= (2.0 ** rng.integers(-2, 3, (M, K // 32, 1))).astype(np.float32)
+    xb.reshape(N, K // 32, 32)[:] *= (2.0 ** rng.integers(-2, 3, (N, K // 32, 1))).astype(np.float32)
+    a, mxa = F.quantize_mxfp4(xa)
+    b, mxb = F.quantize_mxfp4(xb)
+    bias = rng.standard_normal(N).astype(np.float32)
+    out, name = run_gemm(a, shuffle_weight_bytes(b), M, N, K, "mxfp4", dtype_c, bias=bias, mx_a=mxa,
+                         mx_b=shuffle_scales_e8m0_lanes(mxb), operand_path="direct_b_k8")
+    assert name == f"streamdb_mxfp4_128x256_w1x4_{dtype_c}"
+    check(out, G.gemm_mxfp4(a, mxa, b, mxb, out_dtype=_DT[dtype_c], bias=bias), dtype_c, N,
+          bar=1e-5 if dtype_c == "f32" else REL_L2_BAR)
+    lds_out, lds_name = run_gemm(a, b, M, N, K, "mxfp4", dtype_c, bias=bias, mx_a=mxa, mx_b=mxb,
+                                 family=_capi.KERNEL_TILE)
+    if lds_name.startswith("stream_mxfp4"):   # the same products in the same order
+        assert np.array_equal(out.view(np.uint8), lds_out.view(np.uint8))
+
+
+def test_mxfp4_stream_direct_b_full_size_row_sample(gpu):
+    # configuration 5 at the size the bench times, weights pre-shuffled
+    from aster_amd.kittens_helpers import shuffle_scales_e8m0_lanes, shuffle_weight_bytes
+    M, N, K = 4096, 14336, 4096
+    a, b, ex = operands(M, N, K, "mxfp4", a_std=1.0, b_std=1.0)
+    out, name = run_gemm(a, shuffle_weight_bytes(b), M, N, K, "mxfp4", "bf16", mx_a=ex["mx_a"],
+                         mx_b=shuffle_scales_e8m0_lanes(ex["mx_b"]), operand_path="direct_b_k8")
+    assert name == "streamdb_mxfp4_128x256_w1x4_bf16"
+    rows, cols = _sampled_rows_and_cols(M, N)
+    check(out[rows], G.gemm_mxfp4(a[rows], ex["mx_a"][rows], b, ex["mx_b"], out_dtype=G.BF16), "bf16", N)
+    check(out[:, cols], G.gemm_mxfp4(a, ex["mx_a"], b[cols], ex["mx_b"][cols], out_dtype=G.BF16),
+          "bf16", len(cols))
+    plain, _ = run_gemm(a, b, M, N, K, "mxfp4", "bf16", **ex)
+    assert np.array_equal(out, plain)
 
 
 def test_stream_direct_b_k8_full_size_row_sample(gpu, big):

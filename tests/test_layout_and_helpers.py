@@ -275,3 +275,33 @@ def test_shuffle_weight_bytes_is_the_operand_order_of_the_16x16x128_mfma():
     _capi.check(_capi.load().astergemm_shuffle_scales_e8m0(mx.ctypes.data, out.ctypes.data, N, K))
     assert np.array_equal(out, ss)
     assert _capi.load().astergemm_shuffle_scales_e8m0(mx.ctypes.data, out.ctypes.data, N, K + 32) != 0
+
+
+def test_shuffle_scales_e8m0_lanes_is_what_a_lane_of_the_stream_kernel_loads():
+    # lane 16 q + i of a wave loads the 8 bytes at 8 (16 q + i) of the 512 bytes of (64-row group
+    # nb4, step s): byte 2 t + h is the scale of block 4 h + q of row 64 nb4 + 16 t + i, i.e. of
+    # the 32 K-elements that lane feeds into MFMA h of that step for its row in tile t; the C-ABI
+    # function writes the same bytes; the inverse restores the plane
+    from aster_amd import _capi
+    from aster_amd.kittens_helpers import shuffle_scales_e8m0_lanes, unshuffle_scales_e8m0_lanes
+    rng = np.random.default_rng(6)
+    N, K = 192, 768
+    mx = rng.integers(0, 256, (N, K // 32)).astype(np.uint8)
+    sh = shuffle_scales_e8m0_lanes(mx)
+    flat, steps = sh.reshape(-1), K // 256
+    for nb4 in range(N // 64):
+        for st in range(steps):
+            for lane in range(64):
+                q, i = lane // 16, lane % 16
+                got = flat[((nb4 * steps + st) * 64 + lane) * 8:][:8].reshape(4, 2)   # [t][h]
+                want = mx[64 * nb4 + 16 * np.arange(4) + i][:, st * 8 + 4 * np.arange(2) + q]
+                assert np.array_equal(got, want)
+    assert np.array_equal(unshuffle_scales_e8m0_lanes(sh), mx)
+    out = np.empty_like(mx)
+    lib = _capi.load()
+    _capi.check(lib.astergemm_shuffle_scales_e8m0_lanes(mx.ctypes.data, out.ctypes.data, N, K))
+    assert np.array_equal(out, sh)
+    assert lib.astergemm_shuffle_scales_e8m0_lanes(mx.ctypes.data, out.ctypes.data, N - 16, K) != 0
+    assert lib.astergemm_shuffle_scales_e8m0_lanes(mx.ctypes.data, out.ctypes.data, N, K + 32) != 0
+    with pytest.raises(AssertionError):
+        shuffle_scales_e8m0_lanes(mx[:48])

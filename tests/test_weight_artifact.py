@@ -8,7 +8,8 @@ import numpy as np
 import pytest
 
 from aster_amd import _capi, weights as W
-from aster_amd.kittens_helpers import shuffle_scales_e8m0, shuffle_weight, shuffle_weight_bytes
+from aster_amd.kittens_helpers import (shuffle_scales_e8m0, shuffle_scales_e8m0_lanes, shuffle_weight,
+                                       shuffle_weight_bytes)
 
 
 def _bf16(x):
@@ -134,7 +135,8 @@ def test_packing_rules():
                                                 ("f16", "lds", 40, 264, 256), ("fp8_e4m3", "lds", 16, 512, 4096),
                                                 ("fp8_e4m3", "lds", 300, 256, 512), ("mxfp4", "lds", 64, 256, 1024),
                                                 ("fp8_e4m3", "direct_b", 16, 528, 4096),
-                                                ("mxfp4", "direct_b", 9, 528, 8192)])
+                                                ("mxfp4", "direct_b", 9, 528, 8192),
+                                                ("mxfp4", "direct_b_k8", 264, 576, 2048)])
 def test_artifact_to_gemm_matches_the_oracle(tmp_path, dtype, layout, M, N, K):
     from aster_amd import quantize as Q
     from aster_amd.execution import GpuBuffer
@@ -169,8 +171,9 @@ def test_artifact_to_gemm_matches_the_oracle(tmp_path, dtype, layout, M, N, K):
         xs, mx = F.quantize_mxfp4(x)
         wq, ws = F.quantize_mxfp4(w)
         stored, plane = np.asarray(art.payload).reshape(N, K // 2), np.asarray(art.scales).reshape(N, K // 32)
-        assert np.array_equal(stored, shuffle_weight_bytes(wq) if layout == "direct_b" else wq)
-        assert np.array_equal(plane, shuffle_scales_e8m0(ws) if layout == "direct_b" else ws)
+        assert np.array_equal(stored, shuffle_weight_bytes(wq) if layout != "lds" else wq)
+        assert np.array_equal(plane, {"lds": lambda s: s, "direct_b": shuffle_scales_e8m0,
+                                      "direct_b_k8": shuffle_scales_e8m0_lanes}[layout](ws))
         d_mx = GpuBuffer(mx.nbytes); d_mx.copy_from_host(mx)
         kw["mx_x"] = d_mx.ptr_value
         want = G.gemm_mxfp4(xs, mx, wq, ws, out_dtype=G.F32)
