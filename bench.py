@@ -411,6 +411,24 @@ def main() -> int:
                            "traffic": MEASURED_TRAFFIC_BYTES.get(p.info.name.decode()),
                            "mfma_rate_measured_on_this_data": round(ceil_tf, 1),
                            "frac_of_measured_mfma_rate": round(tf / ceil_tf, 4)})
+            if dt == "mxfp4":
+                # the same product with the weights pre-shuffled (payload in step order, e8m0
+                # plane in lane order: operand_path direct_b_k8), the way the reference's best
+                # kernel takes its B; the permutations are done on the device here, the bits
+                # are those of kittens_helpers.shuffle_weight_bytes / shuffle_scales_e8m0_lanes
+                bs = b.view(n // 16, 16, k // 256, 2, 4, 16).permute(0, 2, 3, 4, 1, 5).contiguous()
+                sbs = keep["mx_b"].view(n // 64, 4, 16, k // 256, 2, 4).permute(0, 3, 5, 2, 1, 4).contiguous()
+                pd = AG.GemmPlan.create(m, n, k, dt, "bf16", operand_path="direct_b_k8")
+                c2 = torch.empty_like(c)
+                keep_d = {"mx_a": keep["mx_a"], "mx_b": sbs}
+                p50d, _, _ = event_timed_p50(pd, a, bs, c2, keep_d, 100, 20)
+                tfd = pd.info.flops / p50d * 1e-3
+                others[-1].update({"kernel_weights_pre_shuffled": pd.info.name.decode(),
+                                   "p50_us_weights_pre_shuffled": round(p50d / 1e3, 2),
+                                   "tflops_weights_pre_shuffled": round(tfd, 1),
+                                   "frac_weights_pre_shuffled": round(tfd / PEAK_TFLOPS[dt], 4),
+                                   "same_bits_as_row_major_weights": bool(torch.equal(c, c2))})
+                del bs, sbs, c2
         # the two gfx950 shapes the reference publishes its own kernels' numbers for (f16
         # operands, fp32 output; contrib/kittens/test/bench/best_known.json, quoted, not re-run)
         for (m, n, k, quoted) in ((4096, 4096, 4096, 1007.0), (2048, 4096, 4096, 846.3)):
