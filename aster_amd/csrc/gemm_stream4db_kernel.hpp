@@ -20,7 +20,8 @@
 //     block 4 h + q of row 64 nb4 + 16 t + i: one 8-byte load per wave and K-step brings the
 //     scales of the wave's four B tiles, and the MFMAs select their byte with op_sel.
 // A and its e8m0 plane are row-major.  A's scales go through LDS as in the LDS kernel (16 bytes
-// per row = one chunk of two K-steps, re-packed into byte pairs {block q, block 4 + q}), but by
+// per row = one chunk of two K-steps, re-packed into byte pairs {block q, block 4 + q}, here
+// one plane of 8 bytes per row for each of the two K-steps), but by
 // ordinary loads: a lane fetches one row's granule, re-packs it in registers and writes it
 // (waves 2 and 3 repeat what waves 0 and 1 do, which keeps the loop free of branches), so that
 // only the A tile transfers are counted by hand.
@@ -45,7 +46,7 @@ __device__ __forceinline__ void gemm_stream4db_body(const GemmArgs& p, int bid) 
   constexpr int NSLOT = 4;              // A ring
   constexpr int NBUF = 4;               // B register buffers of half a K-step each
   constexpr int LH = BM / 8 / NW;       // 4 transfers of 1 KiB per wave and slot
-  constexpr int SC_A = NSLOT * SLOT;    // A scales: [2 buffers][128 rows][16 bytes]
+  constexpr int SC_A = NSLOT * SLOT;    // A scales: [2 buffers][2 K-step parities][128 rows][8 bytes]
   constexpr int RA = 4;                 // A fragment ring
   constexpr int MS = 2 * TM;            // m-steps per K-step
   constexpr int BAR = MS - (RA - 1);    // m-step whose first MFMA follows the barrier
@@ -87,7 +88,7 @@ __device__ __forceinline__ void gemm_stream4db_body(const GemmArgs& p, int bid) 
   int sc_row = row0 + (wave & 1) * 64 + lane;
   sc_row = sc_row < p.M ? sc_row : p.M - 1;  // rows past the end of an edge tile re-read the last
   const uint8_t* sc_src = p.mx_a + (int64_t)sc_row * p.mx_ld;
-  uint8_t* sc_dst = lds + SC_A + ((wave & 1) * 64 + lane) * 16;
+  uint8_t* sc_dst = lds + SC_A + ((wave & 1) * 64 + lane) * 8;
   i32x4 sc_raw = {0, 0, 0, 0};
   auto load_scales = [&](int c) { sc_raw = *(const i32x4*)(sc_src + c * 16); };
   auto store_scales = [&](int c) {
@@ -97,7 +98,11 @@ __device__ __forceinline__ void gemm_stream4db_body(const GemmArgs& p, int bid) 
     r.y = (int)__builtin_amdgcn_perm((unsigned)sc_raw.y, (unsigned)sc_raw.x, 0x07030602u);
     r.z = (int)__builtin_amdgcn_perm((unsigned)sc_raw.w, (unsigned)sc_raw.z, 0x05010400u);
     r.w = (int)__builtin_amdgcn_perm((unsigned)sc_raw.w, (unsigned)sc_raw.z, 0x07030602u);
-    *(i32x4*)(sc_dst + (c & 1) * BM * 16) = r;
+    // the pairs of a K-step parity lie 8 bytes apart from row to row: the 16 rows of a tile are
+    // 128 contiguous bytes, which 64 lanes read without a bank conflict
+    typedef int i32x2 __attribute__((ext_vector_type(2)));
+    *(i32x2*)(sc_dst + (c & 1) * BM * 16) = i32x2{r.x, r.y};
+    *(i32x2*)(sc_dst + (c & 1) * BM * 16 + BM * 8) = i32x2{r.z, r.w};
   };
 
   // ---- B: global -> registers.  One buffer resource over the payload and one over the scale
@@ -141,19 +146,19 @@ __device__ __forceinline__ void gemm_stream4db_body(const GemmArgs& p, int bid) 
     rd_addr[s] = (unsigned)(size_t)AG_LDS(lds) + (unsigned)(li * kRowBytes + (((s * 4 + lq) ^ (li >> 1)) << 4));
     asm volatile("" : "+v"(rd_addr[s]));
   }
-  unsigned sc_addr = (unsigned)(size_t)AG_LDS(lds) + (unsigned)(SC_A + li * 16 + lq * 2);
+  unsigned sc_addr = (unsigned)(size_t)AG_LDS(lds) + (unsigned)(SC_A + li * 8 + lq * 2);
   asm volatile("" : "+v"(sc_addr));
   i32x4 fa[RA];
   int sa[TM];
   // fragment of m-step T (half T / TM, tile T % TM) of the K-step in ring slot KS; with the first
-  // half comes the tile's scale pair (scale buffer (k / 2) mod 2, byte 8 (k mod 2) of the row)
+  // half comes the tile's scale pair (scale buffer (k / 2) mod 2, parity plane k mod 2)
   auto read_a = [&](auto kslot, auto tt) {
     constexpr int KS = decltype(kslot)::value;
     constexpr int T = decltype(tt)::value;
     constexpr int OFF = KS * SLOT + (T % TM) * 16 * kRowBytes;
     fa[T % RA] = *(lvec_t)(size_t)(rd_addr[T / TM] + (unsigned)OFF);
     if constexpr (T < TM) {
-      constexpr int SOFF = ((KS >> 1) & 1) * BM * 16 + (KS & 1) * 8 + T * 16 * 16;
+      constexpr int SOFF = ((KS >> 1) & 1) * BM * 16 + (KS & 1) * BM * 8 + T * 16 * 8;
       sa[T] = *(lu16_t)(size_t)(sc_addr + (unsigned)SOFF);
     }
   };
