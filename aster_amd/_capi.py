@@ -124,6 +124,7 @@ SIGNATURES = {
     "astergemm_shuffle_weight_8": (C.c_int, [_P, _P, C.c_int64, C.c_int64]),
     "astergemm_shuffle_scales_e8m0": (C.c_int, [_P, _P, C.c_int64, C.c_int64]),
     "astergemm_shuffle_scales_e8m0_lanes": (C.c_int, [_P, _P, C.c_int64, C.c_int64]),
+    "astergemm_preshuffle": (C.c_int, [C.c_int, C.c_int, C.c_int64, C.c_int64, _P, _P, _P, _P, _P]),
     "astergemm_weight_crc32": (C.c_uint32, [_P, C.c_size_t]),
     "astergemm_weight_header_init": (C.c_int, [C.POINTER(WeightHeader), C.c_int, C.c_int, C.c_int64,
                                                C.c_int64, C.c_float]),

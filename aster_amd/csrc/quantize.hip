@@ -324,3 +324,112 @@ extern "C" int astergemm_quantize_mxfp4(const void* dSrc, int src_dtype, int64_t
   AG_HIP(hipGetLastError());
   return 0;
 }
+
+// ---- pre-shuffle of weights on the device ----------------------------------------------------
+//
+// Every pre-shuffled layout is a permutation of fixed-size units inside blocks of 16 (64) rows:
+// thread t writes destination unit t, fetched from where the host functions of the same name
+// take it.  MODE 0: 16-bit, the reference's shuffle_weight order (units of 8 bytes);
+// 1: 16-bit, K8 order (16 bytes); 2: byte rows in step order (16 bytes); 3: e8m0 plane in
+// step order (8 bytes); 4: e8m0 plane in lane order (1 byte).
+namespace astergemm {
+namespace {
+
+template <int MODE>
+__global__ __launch_bounds__(256) void preshuffle_kernel(const uint8_t* __restrict__ src,
+                                                         uint8_t* __restrict__ dst, int64_t units,
+                                                         int64_t rb) {
+  const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (t >= units) return;
+  if constexpr (MODE == 0) {
+    // dst (nb, kb, g, n, kh) <- src (nb, n, kb, kh, g), units of 4 elements
+    const int64_t kblocks = rb / 64;
+    const int kh = (int)(t & 1), n = (int)((t >> 1) & 15), g = (int)((t >> 5) & 3);
+    const int64_t kb = (t >> 7) % kblocks, nb = (t >> 7) / kblocks;
+    *(uint2*)(dst + t * 8) = *(const uint2*)(src + (nb * 16 + n) * rb + kb * 64 + kh * 32 + g * 8);
+  } else if constexpr (MODE == 1) {
+    // dst (nb, kb, g, n) <- src (nb, n, kb, g), units of 8 elements
+    const int64_t kblocks = rb / 64;
+    const int n = (int)(t & 15), g = (int)((t >> 4) & 3);
+    const int64_t kb = (t >> 6) % kblocks, nb = (t >> 6) / kblocks;
+    *(uint4*)(dst + t * 16) = *(const uint4*)(src + (nb * 16 + n) * rb + kb * 64 + g * 16);
+  } else if constexpr (MODE == 2) {
+    // dst (nb, step, u, q, n) <- src (nb, n, step, 4u + q), units of 16 bytes
+    const int64_t steps = rb / 128;
+    const int n = (int)(t & 15), q = (int)((t >> 4) & 3), u = (int)((t >> 6) & 1);
+    const int64_t st = (t >> 7) % steps, nb = (t >> 7) / steps;
+    *(uint4*)(dst + t * 16) = *(const uint4*)(src + (nb * 16 + n) * rb + st * 128 + (4 * u + q) * 16);
+  } else if constexpr (MODE == 3) {
+    // dst (nb, step, n) <- src (nb, n, step), units of 8 bytes; rb = K / 32 bytes
+    const int64_t steps = rb / 8;
+    const int n = (int)(t & 15);
+    const int64_t st = (t >> 4) % steps, nb = (t >> 4) / steps;
+    *(uint2*)(dst + t * 8) = *(const uint2*)(src + (nb * 16 + n) * rb + st * 8);
+  } else {
+    // dst (nb4, step, q, i, tile, h) <- src (nb4, tile, i, step, 4h + q), bytes; rb = K / 32 bytes
+    const int64_t steps = rb / 8;
+    const int h = (int)(t & 1), tl = (int)((t >> 1) & 3), i = (int)((t >> 3) & 15), q = (int)((t >> 7) & 3);
+    const int64_t st = (t >> 9) % steps, nb4 = (t >> 9) / steps;
+    dst[t] = src[(nb4 * 64 + tl * 16 + i) * rb + st * 8 + 4 * h + q];
+  }
+}
+
+template <int MODE>
+int preshuffle_launch(const void* src, void* dst, int64_t bytes, int unit, int64_t row_bytes_,
+                      hipStream_t s) {
+  const int64_t units = bytes / unit;
+  if (units == 0) return 0;
+  if ((units + 255) / 256 >= (int64_t)1 << 31) {
+    set_error("astergemm_preshuffle: matrix too large");
+    return ASTERGEMM_EINVAL;
+  }
+  (void)hipGetLastError();
+  hipLaunchKernelGGL(preshuffle_kernel<MODE>, dim3((unsigned)((units + 255) / 256)), dim3(256), 0, s,
+                     (const uint8_t*)src, (uint8_t*)dst, units, row_bytes_);
+  AG_HIP(hipGetLastError());
+  return 0;
+}
+
+}  // namespace
+}  // namespace astergemm
+
+extern "C" int astergemm_preshuffle(int dtype_ab, int operand_path, int64_t N, int64_t K,
+                                    const void* dSrc, void* dDst, const uint8_t* dMxSrc,
+                                    uint8_t* dMxDst, void* stream) {
+  using namespace astergemm;
+  const bool is16 = dtype_ab == ASTERGEMM_F16 || dtype_ab == ASTERGEMM_BF16;
+  const bool fp4 = dtype_ab == ASTERGEMM_MXFP4;
+  if (!is16 && !fp4 && dtype_ab != ASTERGEMM_FP8_E4M3) {
+    set_error("astergemm_preshuffle: dtype_ab must be F16, BF16, FP8_E4M3 or MXFP4");
+    return ASTERGEMM_EINVAL;
+  }
+  if (operand_path != ASTERGEMM_OPERAND_DIRECT_B && operand_path != ASTERGEMM_OPERAND_DIRECT_B_K8) {
+    set_error("astergemm_preshuffle: operand_path must be DIRECT_B or DIRECT_B_K8");
+    return ASTERGEMM_EINVAL;
+  }
+  const bool k8 = operand_path == ASTERGEMM_OPERAND_DIRECT_B_K8;
+  if (k8 && dtype_ab == ASTERGEMM_FP8_E4M3) {
+    set_error("astergemm_preshuffle: DIRECT_B_K8 holds 16-bit or MXFP4 weights");
+    return ASTERGEMM_EINVAL;
+  }
+  const int64_t rb = row_bytes(dtype_ab, K);
+  const int64_t rows_mod = (fp4 && k8) ? 64 : 16;
+  if (N < 0 || K < 0 || N % rows_mod != 0 || (is16 ? K % 32 != 0 : rb % 128 != 0) ||
+      (N > 0 && K > 0 && (!dSrc || !dDst || dSrc == dDst)) || ((((uintptr_t)dSrc) | ((uintptr_t)dDst)) & 15) ||
+      (fp4 && N > 0 && K > 0 && (!dMxSrc || !dMxDst || dMxSrc == dMxDst ||
+                                 ((((uintptr_t)dMxSrc) | ((uintptr_t)dMxDst)) & 7)))) {
+    set_error("astergemm_preshuffle: need N %% %d == 0, rows of whole %s, distinct 16-byte aligned "
+              "source and destination (MXFP4: and distinct 8-byte aligned scale planes)",
+              (int)rows_mod, is16 ? "32-element blocks" : "128-byte steps");
+    return ASTERGEMM_EINVAL;
+  }
+  if (N == 0 || K == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  int rc;
+  if (is16) rc = k8 ? preshuffle_launch<1>(dSrc, dDst, N * rb, 16, rb, s)
+                    : preshuffle_launch<0>(dSrc, dDst, N * rb, 8, rb, s);
+  else rc = preshuffle_launch<2>(dSrc, dDst, N * rb, 16, rb, s);
+  if (rc != 0 || !fp4) return rc;
+  return k8 ? preshuffle_launch<4>(dMxSrc, dMxDst, N * (K / 32), 1, K / 32, s)
+            : preshuffle_launch<3>(dMxSrc, dMxDst, N * (K / 32), 8, K / 32, s);
+}

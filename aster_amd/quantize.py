@@ -53,6 +53,20 @@ def quantize_mxfp4_device(d_src: int, rows: int, K: int, d_packed: int, d_scales
         ctypes.c_void_p(d_scales), _s(stream)))
 
 
+def preshuffle_device(d_src: int, d_dst: int, N: int, K: int, dtype_ab: str, operand_path: str, *,
+                      d_mx_src: Optional[int] = None, d_mx_dst: Optional[int] = None,
+                      stream: Optional[int] = None) -> None:
+    """Weights B[N, K] row-major in device memory -> the pre-shuffled order `operand_path`
+    ("direct_b" / "direct_b_k8") names for `dtype_ab`, device to device; for MXFP4 the e8m0
+    plane goes from `d_mx_src` to `d_mx_dst` in the matching order (the device form of
+    `kittens_helpers.shuffle_weight*` / `shuffle_scales_e8m0*`)."""
+    path = {"direct_b": _capi.OPERAND_DIRECT_B, "direct_b_k8": _capi.OPERAND_DIRECT_B_K8}[operand_path]
+    _capi.check(_capi.load().astergemm_preshuffle(
+        _capi.DTYPE_NAMES[dtype_ab], path, N, K, ctypes.c_void_p(d_src), ctypes.c_void_p(d_dst),
+        ctypes.c_void_p(d_mx_src) if d_mx_src else None,
+        ctypes.c_void_p(d_mx_dst) if d_mx_dst else None, _s(stream)))
+
+
 def _host_source(x: np.ndarray, dtype: Optional[str]):
     """(contiguous array, source dtype name): float32 and float16 arrays are taken as they are,
     uint16 arrays are bfloat16 bits when `dtype` says "bf16"."""

@@ -40,6 +40,7 @@ MEASURED_TRAFFIC_BYTES = {
     "stream_fp8_256x256_w2x4_walk_bf16": 9.47e8,  # 8192^3 as a tile walk: 8.12e8 read + 1.35e8 written
     "stream_mxfp4_256x256_w2x2_bf16": 3.22e8,   # 4096x14336x4096: 2.05e8 read + 1.17e8 written
     "stream_mxfp4_256x256_w2x4_tail128_bf16": 3.10e8,  # the same shape: 1.92e8 read + 1.18e8 written
+    "streamdb_mxfp4_128x256_w1x4_bf16": 3.13e8,  # the same shape, weights pre-shuffled: 1.96e8 + 1.17e8
 }
 
 
@@ -414,10 +415,13 @@ def main() -> int:
             if dt == "mxfp4":
                 # the same product with the weights pre-shuffled (payload in step order, e8m0
                 # plane in lane order: operand_path direct_b_k8), the way the reference's best
-                # kernel takes its B; the permutations are done on the device here, the bits
-                # are those of kittens_helpers.shuffle_weight_bytes / shuffle_scales_e8m0_lanes
-                bs = b.view(n // 16, 16, k // 256, 2, 4, 16).permute(0, 2, 3, 4, 1, 5).contiguous()
-                sbs = keep["mx_b"].view(n // 64, 4, 16, k // 256, 2, 4).permute(0, 3, 5, 2, 1, 4).contiguous()
+                # kernel takes its B; shuffled once, on the device (astergemm_preshuffle)
+                from aster_amd import quantize as Q
+                bs, sbs = torch.empty_like(b), torch.empty_like(keep["mx_b"])
+                torch.cuda.synchronize()
+                Q.preshuffle_device(b.data_ptr(), bs.data_ptr(), n, k, dt, "direct_b_k8",
+                                    d_mx_src=keep["mx_b"].data_ptr(), d_mx_dst=sbs.data_ptr())
+                torch.cuda.synchronize()
                 pd = AG.GemmPlan.create(m, n, k, dt, "bf16", operand_path="direct_b_k8")
                 c2 = torch.empty_like(c)
                 keep_d = {"mx_a": keep["mx_a"], "mx_b": sbs}
@@ -427,6 +431,7 @@ def main() -> int:
                                    "p50_us_weights_pre_shuffled": round(p50d / 1e3, 2),
                                    "tflops_weights_pre_shuffled": round(tfd, 1),
                                    "frac_weights_pre_shuffled": round(tfd / PEAK_TFLOPS[dt], 4),
+                                   "traffic_weights_pre_shuffled": MEASURED_TRAFFIC_BYTES.get(pd.info.name.decode()),
                                    "same_bits_as_row_major_weights": bool(torch.equal(c, c2))})
                 del bs, sbs, c2
         # the two gfx950 shapes the reference publishes its own kernels' numbers for (f16

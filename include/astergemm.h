@@ -323,6 +323,21 @@ int astergemm_quantize_mxfp4(const void* dSrc, int src_dtype, int64_t rows, int6
                              int64_t ld_src, uint8_t* dPacked, uint8_t* dScales,
                              void* stream);
 
+/* The pre-shuffles above on the device (device to device, on `stream`), for a
+ * caller whose weights are already in HBM (e.g. straight out of the quantisers):
+ * dSrc[N, K] row-major -> dDst in the order `operand_path` names for
+ * `dtype_ab`: DIRECT_B = astergemm_shuffle_weight_16 (16-bit) or
+ * astergemm_shuffle_weight_8 (fp8, MXFP4; dMxSrc -> dMxDst in
+ * astergemm_shuffle_scales_e8m0 order); DIRECT_B_K8 =
+ * astergemm_shuffle_weight_k8_16 (16-bit) or astergemm_shuffle_weight_8 with
+ * the plane in astergemm_shuffle_scales_e8m0_lanes order (MXFP4).  The same
+ * size rules as the host functions; source and destination distinct and
+ * 16-byte aligned (scale planes 8-byte; ignored unless MXFP4).  The reference
+ * shuffles on the host on every call
+ * (test_102_gemm_python_multitile_g2s_directb_cdna4.py:446-467).             */
+int astergemm_preshuffle(int dtype_ab, int operand_path, int64_t N, int64_t K, const void* dSrc,
+                         void* dDst, const uint8_t* dMxSrc, uint8_t* dMxDst, void* stream);
+
 /* ---- weight artefact files (host side) -------------------------------------
  * A weight matrix B[N, K] on disk in the bytes the kernels stream, so that
  * loading is one read + one upload: no conversion, no permutation.  The

@@ -266,3 +266,43 @@ def test_gemm_output_feeds_the_next_quantised_gemm():
     hq, hsc = F.quantize_mxfp4(F.bf16_bits_to_f32(hb))
     want = G.gemm_mxfp4(hq, hsc, w2p, w2s, out_dtype=G.F32)
     assert G.rel_l2(out, G.output_to_f32(want, G.F32)) <= 1e-5
+
+
+@pytest.mark.parametrize("dtype_ab,path", [("bf16", "direct_b"), ("f16", "direct_b_k8"), ("fp8_e4m3", "direct_b"),
+                                           ("mxfp4", "direct_b"), ("mxfp4", "direct_b_k8")])
+def test_preshuffle_on_the_device_writes_the_bytes_of_the_host_functions(gpu, dtype_ab, path):
+    # the five pre-shuffled layouts, device to device, against kittens_helpers (which the C host
+    # functions are tested against): same bytes; N, K with several row blocks and steps
+    from aster_amd import kittens_helpers as H
+    from aster_amd.execution import GpuBuffer
+    N, K = 192, 1280
+    rng = np.random.default_rng(8)
+    mx = rng.integers(0, 256, (N, K // 32)).astype(np.uint8)
+    if dtype_ab in ("bf16", "f16"):
+        b = rng.integers(0, 65536, (N, K)).astype(np.uint16)
+        want = (H.shuffle_weight if path == "direct_b" else H.shuffle_weight_k8)(b)
+    else:
+        b = rng.integers(0, 256, (N, K if dtype_ab == "fp8_e4m3" else K // 2)).astype(np.uint8)
+        want = H.shuffle_weight_bytes(b)
+    want_mx = (H.shuffle_scales_e8m0 if path == "direct_b" else H.shuffle_scales_e8m0_lanes)(mx)
+    d_b, d_o, d_mx, d_mo = GpuBuffer(b.nbytes), GpuBuffer(b.nbytes), GpuBuffer(mx.nbytes), GpuBuffer(mx.nbytes)
+    d_b.copy_from_host(b)
+    d_mx.copy_from_host(mx)
+    d_o.copy_from_host(np.zeros_like(b))
+    d_mo.copy_from_host(np.zeros_like(mx))
+    print(f"preshuffle {dtype_ab} {path}", flush=True)
+    Q.preshuffle_device(d_b.ptr_value, d_o.ptr_value, N, K, dtype_ab, path,
+                        d_mx_src=d_mx.ptr_value, d_mx_dst=d_mo.ptr_value)
+    got, got_mx = np.zeros_like(b), np.zeros_like(mx)
+    d_o.copy_to_host(got)
+    d_mo.copy_to_host(got_mx)
+    assert np.array_equal(got, want)
+    if dtype_ab == "mxfp4":
+        assert np.array_equal(got_mx, want_mx)
+    else:
+        assert not got_mx.any()     # no scale plane for these types: left alone
+    with pytest.raises(_capi.AsterGemmError):   # in place is refused
+        Q.preshuffle_device(d_b.ptr_value, d_b.ptr_value, N, K, dtype_ab, path,
+                            d_mx_src=d_mx.ptr_value, d_mx_dst=d_mo.ptr_value)
+    for bf in (d_b, d_o, d_mx, d_mo):
+        bf.free()
