@@ -89,8 +89,6 @@ const char* validate_problem(const astergemm_config& c) {
     return "bad scale_mode";
   if (c.operand_path < ASTERGEMM_OPERAND_LDS || c.operand_path > ASTERGEMM_OPERAND_DIRECT_B_K8)
     return "bad operand_path";
-  if (c.operand_path == ASTERGEMM_OPERAND_DIRECT_B_K8 && c.dtype_ab == ASTERGEMM_FP8_E4M3)
-    return "B pre-shuffled for the stream kernels is built for 16-bit and MXFP4 operands";
   if ((c.dtype_ab == ASTERGEMM_MXFP4) != (c.scale_mode == ASTERGEMM_SCALE_MX32))
     return "MXFP4 operands and SCALE_MX32 go together";
   if (c.dtype_ab == ASTERGEMM_MXFP4 && c.K % 32 != 0) return "MXFP4 needs K % 32 == 0";

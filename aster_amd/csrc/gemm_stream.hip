@@ -6,6 +6,7 @@
 #include "gemm_stream4_kernel.hpp"
 #include "gemm_streamdb_kernel.hpp"
 #include "gemm_stream4db_kernel.hpp"
+#include "gemm_stream8db_kernel.hpp"
 
 namespace astergemm {
 namespace {
@@ -115,6 +116,40 @@ const char* check_stream4db(const astergemm_config& c) {
         4 * 128 * kRowBytes + 2 * 128 * 16,                                      \
         (const void*)gemm_stream4db_kernel<DT, OUT>, launch_stream4db<DT, OUT>,  \
         check_stream4db, ASTERGEMM_OPERAND_DIRECT_B_K8                           \
+  }
+
+// ---- fp8, B pre-shuffled into step order and loaded straight into MFMA operands: 128 x 256
+// tiles, four waves (gemm_stream8db_kernel.hpp) -------------------------------------------------
+template <int DT, int OUT>
+int launch_stream8db(const GemmArgs& a, int grid, hipStream_t s) {
+  constexpr int lds = 4 * 128 * kRowBytes;
+  auto k = gemm_stream8db_kernel<DT, OUT>;
+  static std::atomic<uint64_t> attr_devs{0};
+  if (int e = lds_attr_once(attr_devs, (const void*)k, lds)) return e;
+  // what the kernel's indexing assumes: whole 16-row blocks of B, whole K-steps, packed B
+  if (a.N % 16 != 0 || a.N < 16 || a.M < 8 || a.M % 8 != 0 || a.K % 128 != 0 || a.tail_granules != 0 ||
+      a.ldb_bytes != (int64_t)a.K)
+    return (int)hipErrorInvalidValue;
+  hipLaunchKernelGGL(k, dim3(grid), dim3(256), lds, s, a);
+  return (int)hipGetLastError();
+}
+
+const char* check_stream8db(const astergemm_config& c) {
+  if (c.M % 8 != 0 || c.M < 8) return "M must be a multiple of 8";
+  if (c.N % 16 != 0 || c.N < 16) return "pre-shuffled B needs N % 16 == 0";
+  if (c.K % 128 != 0) return "pre-shuffled fp8 B needs K % 128 == 0";
+  if (c.ldb != 0 && c.ldb != c.K) return "pre-shuffled B is packed (ldb = K)";
+  if (c.ldc % 8 != 0) return "ldc must be a multiple of 8 elements";
+  if (c.N * c.K >= ((int64_t)1 << 32)) return "pre-shuffled B must stay below 4 GiB";
+  return nullptr;
+}
+
+#define AG_STREAM8DB(name, DT, OUT)                                              \
+  Variant {                                                                      \
+    name, ASTERGEMM_KERNEL_TILE, DT, OUT, 128, 256, kRowBytes, 1, 4, 4, 2,       \
+        4 * 128 * kRowBytes,                                                     \
+        (const void*)gemm_stream8db_kernel<DT, OUT>, launch_stream8db<DT, OUT>,  \
+        check_stream8db, ASTERGEMM_OPERAND_DIRECT_B_K8                           \
   }
 
 // ---- split K on the 128x128 kernel --------------------------------------------------------
@@ -547,6 +582,9 @@ const Variant kStreamVariants[] = {
     AG_STREAM4DB("streamdb_mxfp4_128x256_w1x4_bf16", ASTERGEMM_MXFP4, ASTERGEMM_BF16),
     AG_STREAM4DB("streamdb_mxfp4_128x256_w1x4_f32", ASTERGEMM_MXFP4, ASTERGEMM_F32),
     AG_STREAM4DB("streamdb_mxfp4_128x256_w1x4_f16", ASTERGEMM_MXFP4, ASTERGEMM_F16),
+    AG_STREAM8DB("streamdb_fp8_128x256_w1x4_bf16", ASTERGEMM_FP8_E4M3, ASTERGEMM_BF16),
+    AG_STREAM8DB("streamdb_fp8_128x256_w1x4_f32", ASTERGEMM_FP8_E4M3, ASTERGEMM_F32),
+    AG_STREAM8DB("streamdb_fp8_128x256_w1x4_f16", ASTERGEMM_FP8_E4M3, ASTERGEMM_F16),
     AG_STREAM4_128("stream_mxfp4_128x128_w2x2_bf16", ASTERGEMM_MXFP4, ASTERGEMM_BF16),
     AG_STREAM4_128("stream_mxfp4_128x128_w2x2_f32", ASTERGEMM_MXFP4, ASTERGEMM_F32),
     AG_STREAM4_128("stream_mxfp4_128x128_w2x2_f16", ASTERGEMM_MXFP4, ASTERGEMM_F16),

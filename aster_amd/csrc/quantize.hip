@@ -408,10 +408,6 @@ extern "C" int astergemm_preshuffle(int dtype_ab, int operand_path, int64_t N, i
     return ASTERGEMM_EINVAL;
   }
   const bool k8 = operand_path == ASTERGEMM_OPERAND_DIRECT_B_K8;
-  if (k8 && dtype_ab == ASTERGEMM_FP8_E4M3) {
-    set_error("astergemm_preshuffle: DIRECT_B_K8 holds 16-bit or MXFP4 weights");
-    return ASTERGEMM_EINVAL;
-  }
   const int64_t rb = row_bytes(dtype_ab, K);
   const int64_t rows_mod = (fp4 && k8) ? 64 : 16;
   if (N < 0 || K < 0 || N % rows_mod != 0 || (is16 ? K % 32 != 0 : rb % 128 != 0) ||

@@ -6,8 +6,9 @@
 // The pre-shuffled layouts are the reference's shuffle_weight order
 // (contrib/kittens/test/kittens_helpers.py:90-119), which its execute_fn applies on every call
 // (contrib/kittens/test/test_102_gemm_python_multitile_g2s_directb_cdna4.py:440-467), read by
-// the decode kernels, and the K8 order of astergemm_shuffle_weight_k8_16, read by the 256 x 256
-// stream kernel with direct B; a file written once replaces that per-call host permutation.
+// the decode kernels, and the orders read by the stream kernels with direct B (16-bit: the K8
+// order of astergemm_shuffle_weight_k8_16; fp8 and MXFP4: step order); a file written once
+// replaces that per-call host permutation.
 #include <cstring>
 
 #include "astergemm_internal.h"
@@ -70,8 +71,6 @@ extern "C" int astergemm_weight_header_init(astergemm_weight_header* h, int dtyp
   if (astergemm::row_bytes(dtype, K) % 16 != 0) return fail("a row must be a multiple of 16 bytes");
   if (layout == ASTERGEMM_OPERAND_DIRECT_B || layout == ASTERGEMM_OPERAND_DIRECT_B_K8) {
     const bool is16 = dtype == ASTERGEMM_F16 || dtype == ASTERGEMM_BF16;
-    if (dtype == ASTERGEMM_FP8_E4M3 && layout == ASTERGEMM_OPERAND_DIRECT_B_K8)
-      return fail("the stream kernels' pre-shuffled layout holds 16-bit or MXFP4 elements");
     // MXFP4 for the stream kernel: payload in step order, scale plane in lane order
     // (astergemm_shuffle_scales_e8m0_lanes)
     if (dtype == ASTERGEMM_MXFP4 && layout == ASTERGEMM_OPERAND_DIRECT_B_K8 &&

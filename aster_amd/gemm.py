@@ -114,14 +114,14 @@ def select_for_instance(cfg: WeakScaledMappedGemmInstance) -> Tuple[_capi.Config
     """Honour the instance's mapping when a variant with that geometry exists, otherwise let the
     library choose (`mapping_report` tells which happened).  A `direct_b` mapping gets a kernel
     that reads pre-shuffled B when one takes the shape -- the decode kernels in the reference's
-    `shuffle_weight` order, else the stream kernels in `shuffle_weight_k8` order (MXFP4: step
-    order with the scale plane in lane order) (the
+    `shuffle_weight` order, else the stream kernels in `shuffle_weight_k8` order (fp8: step
+    order; MXFP4: step order with the scale plane in lane order) (the
     returned config's `operand_path` says which; `execute_gemm_hsaco` shuffles accordingly) --
     and falls back to plain row-major B otherwise."""
     want_direct = cfg.mapping.direct_b and not cfg.mapping.direct_a
     paths = [_capi.OPERAND_DIRECT_B] if want_direct else []
-    if want_direct and cfg.spec.dtype_ab in ("bf16", "f16", "mxfp4"):
-        paths.append(_capi.OPERAND_DIRECT_B_K8)          # the stream kernels: 16-bit and MXFP4
+    if want_direct:
+        paths.append(_capi.OPERAND_DIRECT_B_K8)          # the stream kernels
     for use_mapping in (True, False):
         for path in paths + [_capi.OPERAND_LDS]:
             if not use_mapping and path == _capi.OPERAND_LDS and not want_direct:
@@ -204,8 +204,8 @@ class GemmPlan:
         plain row-major [N, ldb]; "direct_b" = B was pre-shuffled with `shuffle_weight` (the
         reference's order, read by the decode kernels; fp8 / MXFP4: `shuffle_weight_bytes`, the
         MXFP4 plane with `shuffle_scales_e8m0`); "direct_b_k8" = pre-shuffled for the stream
-        kernels: 16-bit operands with `shuffle_weight_k8`, MXFP4 with `shuffle_weight_bytes` and
-        the scale plane with `shuffle_scales_e8m0_lanes`."""
+        kernels: 16-bit operands with `shuffle_weight_k8`, fp8 with `shuffle_weight_bytes`, MXFP4
+        with `shuffle_weight_bytes` and the scale plane with `shuffle_scales_e8m0_lanes`."""
         c = _capi.Config()
         c.operand_path = _OPERAND_PATH_ID[operand_path]
         c.M, c.N, c.K = M, N, K

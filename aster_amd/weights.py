@@ -74,7 +74,7 @@ class WeightArtifact:
         layout "direct_b" the bits must already be in `shuffle_weight` order (16-bit types) or
         `shuffle_weight_bytes` order (fp8, MXFP4; the MXFP4 plane in `shuffle_scales_e8m0` order),
         for "direct_b_k8" in `shuffle_weight_k8` order (16-bit types) or `shuffle_weight_bytes`
-        order with the plane in `shuffle_scales_e8m0_lanes` order (MXFP4)."""
+        order (fp8; MXFP4, with the plane in `shuffle_scales_e8m0_lanes` order)."""
         h = _capi.WeightHeader()
         _capi.check(_capi.load().astergemm_weight_header_init(
             ctypes.byref(h), _capi.DTYPE_NAMES[dtype], _LAYOUT_ID[layout], N, K,
@@ -113,11 +113,9 @@ class WeightArtifact:
                 bits = shuffle_weight_k8(bits)
             return cls.from_storage(bits, dtype, N, K, layout=layout)
         from . import quantize as Q
-        if layout == "direct_b_k8" and dtype != "mxfp4":
-            raise ValueError("layout direct_b_k8 holds 16-bit or MXFP4 elements")
         if dtype == "fp8_e4m3":
             q, s = Q.quantize_fp8_tensor(w)
-            if layout == "direct_b":
+            if layout in ("direct_b", "direct_b_k8"):   # step order for both kernel sets
                 q = shuffle_weight_bytes(np.asarray(q).reshape(N, K).view(np.uint8))
             return cls.from_storage(q, dtype, N, K, layout=layout, tensor_scale=float(s))
         if dtype == "mxfp4":

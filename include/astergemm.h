@@ -95,7 +95,11 @@ typedef enum astergemm_operand_path {
                                      astergemm_shuffle_weight_8, dMxB with
                                      astergemm_shuffle_scales_e8m0_lanes
                                      (128 x 256 tiles, N % 64 == 0,
-                                     K % 512 == 0).  16-bit operands: with
+                                     K % 512 == 0).  fp8: with
+                                     astergemm_shuffle_weight_8, the same
+                                     bytes as DIRECT_B (128 x 256 tiles,
+                                     N % 16 == 0, K % 128 == 0).  16-bit
+                                     operands: with
                                      astergemm_shuffle_weight_k8_16: 8
                                      consecutive K per lane, the order of the
                                      16x16x32 MFMA and of 16-byte LDS reads
@@ -329,8 +333,8 @@ int astergemm_quantize_mxfp4(const void* dSrc, int src_dtype, int64_t rows, int6
  * `dtype_ab`: DIRECT_B = astergemm_shuffle_weight_16 (16-bit) or
  * astergemm_shuffle_weight_8 (fp8, MXFP4; dMxSrc -> dMxDst in
  * astergemm_shuffle_scales_e8m0 order); DIRECT_B_K8 =
- * astergemm_shuffle_weight_k8_16 (16-bit) or astergemm_shuffle_weight_8 with
- * the plane in astergemm_shuffle_scales_e8m0_lanes order (MXFP4).  The same
+ * astergemm_shuffle_weight_k8_16 (16-bit) or astergemm_shuffle_weight_8 (fp8;
+ * MXFP4, with the plane in astergemm_shuffle_scales_e8m0_lanes order).  The same
  * size rules as the host functions; source and destination distinct and
  * 16-byte aligned (scale planes 8-byte; ignored unless MXFP4).  The reference
  * shuffles on the host on every call
@@ -351,7 +355,7 @@ int astergemm_preshuffle(int dtype_ab, int operand_path, int64_t N, int64_t K, c
  * payload_offset (N rows; layout ASTERGEMM_OPERAND_LDS = row-major,
  * ASTERGEMM_OPERAND_DIRECT_B = astergemm_shuffle_weight_16 order,
  * ASTERGEMM_OPERAND_DIRECT_B_K8 = astergemm_shuffle_weight_k8_16 order for the
- * 16-bit dtypes; for fp8 and MXFP4 ASTERGEMM_OPERAND_DIRECT_B and for MXFP4
+ * 16-bit dtypes; for fp8 and MXFP4 both ASTERGEMM_OPERAND_DIRECT_B and
  * ASTERGEMM_OPERAND_DIRECT_B_K8 = astergemm_shuffle_weight_8 order), then for
  * MXFP4 the e8m0 plane [N, K/32] at scales_offset (layout DIRECT_B: in
  * astergemm_shuffle_scales_e8m0 order, DIRECT_B_K8: in

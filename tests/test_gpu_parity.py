@@ -925,6 +925,9 @@ def test_every_tile_variant(gpu, vid, name, dtype_ab, dtype_c):
         from aster_amd.kittens_helpers import shuffle_scales_e8m0_lanes, shuffle_weight_bytes
         path, b_dev = "direct_b_k8", shuffle_weight_bytes(b)
         ex_dev = dict(ex, mx_b=shuffle_scales_e8m0_lanes(ex["mx_b"]))
+    elif name.startswith("streamdb_fp8"):  # byte rows in step order
+        from aster_amd.kittens_helpers import shuffle_weight_bytes
+        path, b_dev = "direct_b_k8", shuffle_weight_bytes(b)
     elif name.startswith("streamdb"):  # B pre-shuffled in K8 order
         from aster_amd.kittens_helpers import shuffle_weight_k8
         path, b_dev = "direct_b_k8", shuffle_weight_k8(np.ascontiguousarray(b).view(np.uint16))
@@ -1255,6 +1258,47 @@ def test_mxfp4_stream_direct_b_full_size_row_sample(gpu):
     assert np.array_equal(out, plain)
 
 
+@pytest.mark.parametrize("M,N,K", [(128, 256, 128), (128, 256, 256), (136, 272, 384), (128, 256, 512),
+                                   (256, 512, 640), (128, 256, 896), (128, 256, 1024), (264, 528, 1152),
+                                   (128, 256, 1408), (512, 768, 1536), (128, 256, 1664), (1000, 1072, 2048),
+                                   (128, 64, 4096), (512, 512, 8192)])
+@pytest.mark.parametrize("dtype_c", ["f32", "bf16"])
+def test_fp8_stream_direct_b(gpu, M, N, K, dtype_c):
+    """fp8 with B pre-shuffled into step order and loaded straight into MFMA operands: 128 x 256
+    tiles, four waves, every load of the K loop counted by hand.  K-step counts 1..7 (no steady
+    group: every wait is for all loads), 8 (the first group and the last), 9, 11, 13 (first
+    group, then trips that wait for all), 12, 16, 32, 64 (steady groups between the first and
+    the last); edge tiles in M (multiple of 8) and N (multiple of 16).  Against the oracle, and
+    the same bits as the kernel that takes B row-major through LDS."""
+    from aster_amd.kittens_helpers import shuffle_weight_bytes
+    a, b, ex = operands(M, N, K, "fp8_e4m3", seed=K + M, b_std=0.05)
+    bias = np.random.default_rng(K).standard_normal(N).astype(np.float32)
+    out, name = run_gemm(a, shuffle_weight_bytes(b), M, N, K, "fp8_e4m3", dtype_c, bias=bias,
+                         operand_path="direct_b_k8", **ex)
+    assert name == f"streamdb_fp8_128x256_w1x4_{dtype_c}"
+    check(out, G.gemm_fp8(a, b, ex["scale_a"], ex["scale_b"], out_dtype=_DT[dtype_c], bias=bias), dtype_c, N,
+          bar=1e-4 if dtype_c == "f32" else REL_L2_BAR)
+    lds_out, lds_name = run_gemm(a, b, M, N, K, "fp8_e4m3", dtype_c, bias=bias, family=_capi.KERNEL_TILE,
+                                 wg_tile=(256, 256), **ex)
+    assert lds_name.startswith("stream_fp8_256x256")   # the same products in the same order
+    assert np.array_equal(out.view(np.uint8), lds_out.view(np.uint8))
+
+
+def test_fp8_stream_direct_b_full_size_row_sample(gpu):
+    # configuration 3 at the size the bench times, weights pre-shuffled: sampled rows against the
+    # oracle, every element against the kernel that takes B row-major
+    from aster_amd.kittens_helpers import shuffle_weight_bytes
+    M = N = K = 8192
+    a, b, ex = operands(M, N, K, "fp8_e4m3", a_std=1.0, b_std=1.0)
+    out, name = run_gemm(a, shuffle_weight_bytes(b), M, N, K, "fp8_e4m3", "bf16", operand_path="direct_b_k8",
+                         **ex)
+    assert name == "streamdb_fp8_128x256_w1x4_bf16"
+    rows, _ = _sampled_rows_and_cols(M, N)
+    check(out[rows], G.gemm_fp8(a[rows], b, ex["scale_a"], ex["scale_b"], out_dtype=G.BF16), "bf16", N)
+    plain, _ = run_gemm(a, b, M, N, K, "fp8_e4m3", "bf16", **ex)
+    assert np.array_equal(out, plain)
+
+
 def test_stream_direct_b_k8_full_size_row_sample(gpu, big):
     from aster_amd.kittens_helpers import shuffle_weight_k8
     M, N, K, a, b = big
@@ -1312,6 +1356,21 @@ def test_direct_b_mapping_of_a_decode_shape_with_byte_operands(gpu, tmp_path, dt
     c_flat, times = AG.execute_gemm_hsaco(cfg, path, 2, a, b, **ex)
     want = G.gemm(a, b, _DT[dtype_ab], G.F32, **ex)
     check(c_flat.reshape(M, N), want, "f32", N, bar=1e-4)
+
+
+def test_direct_b_mapping_of_a_compute_bound_fp8_shape(gpu, tmp_path):
+    # the reference's best mapping (128 x 256, waves 1 x 4, DIRECT_B) with fp8 operands: the stream
+    # kernel that loads the pre-shuffled payload straight into MFMA operands
+    M, N, K = 512, 768, 1152
+    cfg = make_instance(M, N, K, dtype_ab="fp8_e4m3", dtype_c="f32", wg_tile=(128, 256), waves=(1, 4),
+                        operand_path=OperandPath.DIRECT_B)
+    path, asm = AG.compile_gemm(cfg, str(tmp_path / "k.hsaco"))
+    desc = json.load(open(path))
+    assert desc["kernel"] == "streamdb_fp8_128x256_w1x4_f32" and desc["operand_path"] == "direct_b_k8"
+    assert desc["mapping_honoured"] is True
+    a, b, ex = operands(M, N, K, "fp8_e4m3", seed=93, b_std=0.05)
+    c_flat, times = AG.execute_gemm_hsaco(cfg, path, 2, a, b, **ex)
+    check(c_flat.reshape(M, N), G.gemm(a, b, G.FP8_E4M3, G.F32, **ex), "f32", N, bar=1e-4)
 
 
 def test_direct_b_is_refused_where_it_is_not_implemented(gpu):

@@ -269,7 +269,8 @@ def test_gemm_output_feeds_the_next_quantised_gemm():
 
 
 @pytest.mark.parametrize("dtype_ab,path", [("bf16", "direct_b"), ("f16", "direct_b_k8"), ("fp8_e4m3", "direct_b"),
-                                           ("mxfp4", "direct_b"), ("mxfp4", "direct_b_k8")])
+                                           ("fp8_e4m3", "direct_b_k8"), ("mxfp4", "direct_b"),
+                                           ("mxfp4", "direct_b_k8")])
 def test_preshuffle_on_the_device_writes_the_bytes_of_the_host_functions(gpu, dtype_ab, path):
     # the five pre-shuffled layouts, device to device, against kittens_helpers (which the C host
     # functions are tested against): same bytes; N, K with several row blocks and steps

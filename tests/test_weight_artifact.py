@@ -112,8 +112,10 @@ def test_corrupt_files_are_refused_with_a_reason(tmp_path):
 def test_packing_rules():
     with pytest.raises(_capi.AsterGemmError, match="128-byte steps"):
         W.WeightArtifact.from_storage(np.zeros((16, 32), np.uint8), "fp8_e4m3", 16, 32, layout="direct_b")
-    with pytest.raises(_capi.AsterGemmError, match="16-bit"):
-        W.WeightArtifact.from_storage(np.zeros((16, 128), np.uint8), "fp8_e4m3", 16, 128, layout="direct_b_k8")
+    with pytest.raises(_capi.AsterGemmError, match="128-byte steps"):
+        W.WeightArtifact.from_storage(np.zeros((16, 64), np.uint8), "fp8_e4m3", 16, 64, layout="direct_b_k8")
+    assert W.WeightArtifact.from_storage(np.zeros((16, 128), np.uint8), "fp8_e4m3", 16, 128,
+                                         layout="direct_b_k8").shape == (16, 128)
     with pytest.raises(_capi.AsterGemmError, match="N % 16"):
         W.WeightArtifact.from_storage(np.zeros((8, 32), np.uint16), "bf16", 8, 32, layout="direct_b")
     with pytest.raises(ValueError, match="scale plane"):
@@ -135,6 +137,7 @@ def test_packing_rules():
                                                 ("f16", "lds", 40, 264, 256), ("fp8_e4m3", "lds", 16, 512, 4096),
                                                 ("fp8_e4m3", "lds", 300, 256, 512), ("mxfp4", "lds", 64, 256, 1024),
                                                 ("fp8_e4m3", "direct_b", 16, 528, 4096),
+                                                ("fp8_e4m3", "direct_b_k8", 264, 528, 1152),
                                                 ("mxfp4", "direct_b", 9, 528, 8192),
                                                 ("mxfp4", "direct_b_k8", 264, 576, 2048)])
 def test_artifact_to_gemm_matches_the_oracle(tmp_path, dtype, layout, M, N, K):
@@ -161,7 +164,7 @@ def test_artifact_to_gemm_matches_the_oracle(tmp_path, dtype, layout, M, N, K):
         xs, sx = F.quantize_fp8_tensor(x)
         wq, sw = F.quantize_fp8_tensor(w)
         stored = np.asarray(art.payload).reshape(N, K)
-        assert np.array_equal(stored, shuffle_weight_bytes(wq) if layout == "direct_b" else wq)
+        assert np.array_equal(stored, wq if layout == "lds" else shuffle_weight_bytes(wq))
         assert art.tensor_scale == sw
         d_sx = GpuBuffer(4); d_sx.copy_from_host(np.array([sx], np.float32))
         kw["scale_x"] = d_sx.ptr_value
