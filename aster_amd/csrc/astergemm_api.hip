@@ -210,7 +210,13 @@ const Variant* choose(const astergemm_config& c, int* index_out) {
         // split K (rank 4) only passes its check where it was measured ahead of every
         // unsplit kernel: few output tiles, long rows
         if (x->rank == 4) return 3;
-        if (area >= 256 * 256 && fp4 && c.K < 4096 && c.K % 512 == 0) return -1;
+        // (not the tile walk and the whole-rounds form, rank 3, which pay that prologue once per
+        // workgroup, from about two tiles of K = 2048 per CU on: 8192 x 8192 x 1024 51 against
+        // 57 us, 16384 x 16384 x 1024 180 against 210, 8192 x 8192 x 2048 74 against 84,
+        // 4096 x 8192 x 2048 42 against 45; below that level or behind: 4096 x 8192 x 1024 30.6
+        // against 29.8, 4096 x 6144 x 1024 24.0 against 21.8)
+        const bool walk_pays = x->rank == 3 && wgs(x) * c.K >= (int64_t)512 * 2048;
+        if (area >= 256 * 256 && fp4 && c.K < 4096 && c.K % 512 == 0 && !walk_pays) return -1;
         if (area >= 256 * 256) return wgs(x) >= thr256 ? 2 : -1;
         return wgs(x) >= ((x->rank >= 2) ? thr128s : 448) ? 1 : 0;
       };

@@ -38,6 +38,7 @@ MEASURED_TRAFFIC_BYTES = {
     "stream_bf16_256x256_w2x4_bf16": 1.746e9,   # 8192^3: 1.61e9 read + 1.34e8 written
     "stream_fp8_256x256_w2x4_bf16": 9.40e8,     # 8192^3: 8.06e8 read + 1.34e8 written
     "stream_fp8_256x256_w2x4_walk_bf16": 9.47e8,  # 8192^3 as a tile walk: 8.12e8 read + 1.35e8 written
+    "streamdb_fp8_128x256_w1x4_bf16": 1.203e9,  # 8192^3, weights pre-shuffled: 1.069e9 read + 1.34e8 written
     "stream_mxfp4_256x256_w2x2_bf16": 3.22e8,   # 4096x14336x4096: 2.05e8 read + 1.17e8 written
     "stream_mxfp4_256x256_w2x4_tail128_bf16": 3.10e8,  # the same shape: 1.92e8 read + 1.18e8 written
     "streamdb_mxfp4_128x256_w1x4_bf16": 3.13e8,  # the same shape, weights pre-shuffled: 1.96e8 + 1.17e8
@@ -412,28 +413,29 @@ def main() -> int:
                            "traffic": MEASURED_TRAFFIC_BYTES.get(p.info.name.decode()),
                            "mfma_rate_measured_on_this_data": round(ceil_tf, 1),
                            "frac_of_measured_mfma_rate": round(tf / ceil_tf, 4)})
-            if dt == "mxfp4":
-                # the same product with the weights pre-shuffled (payload in step order, e8m0
-                # plane in lane order: operand_path direct_b_k8), the way the reference's best
-                # kernel takes its B; shuffled once, on the device (astergemm_preshuffle)
-                from aster_amd import quantize as Q
-                bs, sbs = torch.empty_like(b), torch.empty_like(keep["mx_b"])
-                torch.cuda.synchronize()
-                Q.preshuffle_device(b.data_ptr(), bs.data_ptr(), n, k, dt, "direct_b_k8",
-                                    d_mx_src=keep["mx_b"].data_ptr(), d_mx_dst=sbs.data_ptr())
-                torch.cuda.synchronize()
-                pd = AG.GemmPlan.create(m, n, k, dt, "bf16", operand_path="direct_b_k8")
-                c2 = torch.empty_like(c)
-                keep_d = {"mx_a": keep["mx_a"], "mx_b": sbs}
-                p50d, _, _ = event_timed_p50(pd, a, bs, c2, keep_d, 100, 20)
-                tfd = pd.info.flops / p50d * 1e-3
-                others[-1].update({"kernel_weights_pre_shuffled": pd.info.name.decode(),
-                                   "p50_us_weights_pre_shuffled": round(p50d / 1e3, 2),
-                                   "tflops_weights_pre_shuffled": round(tfd, 1),
-                                   "frac_weights_pre_shuffled": round(tfd / PEAK_TFLOPS[dt], 4),
-                                   "traffic_weights_pre_shuffled": MEASURED_TRAFFIC_BYTES.get(pd.info.name.decode()),
-                                   "same_bits_as_row_major_weights": bool(torch.equal(c, c2))})
-                del bs, sbs, c2
+            # the same product with the weights pre-shuffled (operand_path direct_b_k8: payload
+            # in step order, the MXFP4 e8m0 plane in lane order), the way the reference's best
+            # kernel takes its B; shuffled once, on the device (astergemm_preshuffle)
+            from aster_amd import quantize as Q
+            bs = torch.empty_like(b)
+            sbs = torch.empty_like(keep["mx_b"]) if dt == "mxfp4" else None
+            torch.cuda.synchronize()
+            Q.preshuffle_device(b.data_ptr(), bs.data_ptr(), n, k, dt, "direct_b_k8",
+                                d_mx_src=keep["mx_b"].data_ptr() if sbs is not None else None,
+                                d_mx_dst=sbs.data_ptr() if sbs is not None else None)
+            torch.cuda.synchronize()
+            pd = AG.GemmPlan.create(m, n, k, dt, "bf16", operand_path="direct_b_k8")
+            c2 = torch.empty_like(c)
+            keep_d = dict(keep, mx_b=sbs) if sbs is not None else keep
+            p50d, _, _ = event_timed_p50(pd, a, bs, c2, keep_d, 100, 20)
+            tfd = pd.info.flops / p50d * 1e-3
+            others[-1].update({"kernel_weights_pre_shuffled": pd.info.name.decode(),
+                               "p50_us_weights_pre_shuffled": round(p50d / 1e3, 2),
+                               "tflops_weights_pre_shuffled": round(tfd, 1),
+                               "frac_weights_pre_shuffled": round(tfd / PEAK_TFLOPS[dt], 4),
+                               "traffic_weights_pre_shuffled": MEASURED_TRAFFIC_BYTES.get(pd.info.name.decode()),
+                               "same_bits_as_row_major_weights": bool(torch.equal(c, c2))})
+            del bs, sbs, c2
         # the two gfx950 shapes the reference publishes its own kernels' numbers for (f16
         # operands, fp32 output; contrib/kittens/test/bench/best_known.json, quoted, not re-run)
         for (m, n, k, quoted) in ((4096, 4096, 4096, 1007.0), (2048, 4096, 4096, 846.3)):

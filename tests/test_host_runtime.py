@@ -48,6 +48,11 @@ def test_select_headline_configs():
     assert gemm.GemmPlan.create(4096, 14336, 4096, "mxfp4", "bf16").info.name.decode().startswith("stream_mxfp4_256")
     assert gemm.GemmPlan.create(96, 4096, 4096, "mxfp4", "bf16").info.name.decode().startswith("stream_mxfp4_128")
     assert gemm.GemmPlan.create(2048, 4096, 4096, "mxfp4", "bf16").info.name.decode().startswith("stream_mxfp4_128")
+    # short rows of MXFP4: the tile walk from about two tiles of K = 2048 per CU on, else 128 x 128
+    assert gemm.GemmPlan.create(8192, 8192, 1024, "mxfp4", "bf16").info.name.decode() == "stream_mxfp4_256x256_w2x4_walk_bf16"
+    assert gemm.GemmPlan.create(4096, 8192, 2048, "mxfp4", "bf16").info.name.decode() == "stream_mxfp4_256x256_w2x4_walk_bf16"
+    assert gemm.GemmPlan.create(4096, 8192, 1024, "mxfp4", "bf16").info.name.decode().startswith("stream_mxfp4_128")
+    assert gemm.GemmPlan.create(8192, 8192, 512, "mxfp4", "bf16").info.name.decode().startswith("stream_mxfp4_128")
     p = gemm.GemmPlan.create(4096, 14336, 4096, "mxfp4", "bf16")
     assert p.info.bytes == 157548544 and p.info.wg_tile_k == 256
     for M, want in ((1, 117477376), (16, 118030336), (64, 119799808)):
