@@ -260,40 +260,45 @@ __device__ __forceinline__ void gemm_stream4db_body(const GemmArgs& p, int bid) 
           if (do_a) issue_a1(k + NSLOT, KM, 3);
         }
         // odd trips: chunk (k + 3) / 2 is fetched behind the barrier that freed its buffer (last
-        // read at m-step 4 of this trip) and written at m-step 11 of the next trip, behind whose
-        // barrier nobody reads that buffer before the barrier of the trip after it
+        // read at m-step 4 of this trip) and written at m-step 4 of the next odd trip, nine
+        // m-steps ahead of the barrier behind which it is first read.  Written there and not
+        // earlier because the compiler's wait for the fetched granule counts only the loads it
+        // sees: one trip after the fetch it would also force the A transfers requested beside
+        // it, two trips after it forces nothing that is not needed by then anyway.
+        if constexpr (ODD && T == 4 && n == 2) {
+          if (STEADY || k + 1 < nk) {
+            if (k > 1) store_scales((k + 1) >> 1);
+          }
+        }
         if constexpr (ODD && T == BAR + 1 && n == 2) {
           if (do_sc) load_scales((k + 3) >> 1);
         }
-        if constexpr (!ODD && T == BAR - 2 && n == 2) {
-          if (STEADY || k + 2 < nk) {
-            if (k > 0) store_scales((k + 2) >> 1);
-          }
-        }
-        // last m-step of a half: tile n of this buffer is done with MFMA (m = 7, n)
+        // last m-step of a half: tile n of this buffer is done with MFMA (m = 7, n).  The B
+        // scales of K-step k + 2 go first in the first half's batch, so that the wait for them
+        // two trips on has this batch and a whole trip of loads behind it.
         if constexpr (m == TM - 1) {
-          if (do_b) load_b1(2 * (k + 2) + U, BIc{}, n);
-          if constexpr (U == 1 && n == TN - 1) {
+          if constexpr (U == 0 && n == 0) {
             if (do_b) load_sb(k + 2, std::integral_constant<int, (KM + 2) % NBUF>{});
           }
+          if (do_b) load_b1(2 * (k + 2) + U, BIc{}, n);
         }
         __builtin_amdgcn_sched_barrier(0);
       });
     });
   };
-  // Loads of a trip in issue order: 4 B loads (first half, m-step 7), the barrier, 4 A transfers
-  // (m-steps 13, 14), on odd trips one A-scale load, 4 B loads and one B-scale load (m-step 15).
+  // Loads of a trip in issue order: one B-scale load and 4 B loads (first half, m-step 7), the
+  // barrier, 4 A transfers (m-steps 13, 14), on odd trips one A-scale load, 4 B loads (m-step 15).
   // Younger than the transfers of A(k+1) at the barrier of trip k, steady state, counted from
-  // below (a smaller count only waits for loads that are older and long complete): 5 behind them
-  // in trip k - 3, 13 in each of the two trips between, 4 of trip k; the A-scale loads of odd
+  // below (a smaller count only waits for loads that are older and long complete): 4 behind them
+  // in trip k - 3, 13 in each of the two trips between, 5 of trip k; the A-scale loads of odd
   // trips are not counted.  Trips 0..2: A(k+1) was requested in the prologue, followed there by
-  // A(k+2..3) and here by 13 loads per earlier trip and 4 of this one.
-  constexpr int VM_STEADY = 5 + 2 * 13 + 4;
+  // A(k+2..3) and here by 13 loads per earlier trip and 5 of this one.
+  constexpr int VM_STEADY = 4 + 2 * 13 + 5;
   auto group = [&](int k0, auto first_c) {
     constexpr bool FIRST = decltype(first_c)::value;
     static_for<0, NSLOT>([&](auto ic) {
       constexpr int I = decltype(ic)::value;
-      constexpr int VM = (FIRST && I <= NSLOT - 2) ? (NSLOT - 2 - I) * LH + 13 * I + 4 : VM_STEADY;
+      constexpr int VM = (FIRST && I <= NSLOT - 2) ? (NSLOT - 2 - I) * LH + 13 * I + 5 : VM_STEADY;
       trip(k0 + I, ic, std::integral_constant<int, VM>{});
     });
   };
