@@ -57,7 +57,12 @@ def _compile(src: str) -> str:
     if not os.path.exists(asm):
         raise RuntimeError(f"hipcc left no device assembly for {src} (expected {asm})")
     with open(asm) as f:
-        found = scan_mfma_hazards(f.read())
+        text = f.read()
+    found = scan_mfma_hazards(text)
+    spilled = scan_spills_beside_asm_loads(text)
+    if spilled:
+        raise RuntimeError(f"{src}: register spills in kernels whose register loads are inline assembly "
+                           f"(the compiler does not wait for those loads): {spilled}")
     for name in os.listdir(OBJ_DIR):  # the other intermediates are large and of no use
         if name.startswith(stem + "-") and name.endswith((".hipi", ".bc", ".out", ".resolution.txt")):
             os.remove(os.path.join(OBJ_DIR, name))
@@ -177,6 +182,37 @@ def scan_mfma_hazards(asm_text: str, wait_states: int = MFMA_WAIT_STATES):
             hist.append((w, written, l, no))
         if len(hist) > 12:
             hist.pop(0)
+    return found
+
+
+def scan_spills_beside_asm_loads(asm_text: str):
+    """[(function, spill instructions)] for every function of gfx9 assembly text that loads
+    registers inside inline-asm blocks (loads the kernel counts by hand: the compiler inserts no
+    wait for them) and also holds register spills: a spill of such a register between the load and
+    the kernel's own wait would store the bytes the register held before."""
+    found = []
+    name, asm_loads, spills, in_asm = None, 0, 0, False
+
+    def close():
+        if name and asm_loads and spills:
+            found.append((name, spills))
+
+    for raw in asm_text.split("\n"):
+        l = raw.strip()
+        if l.startswith(";;#ASMSTART"):
+            in_asm = True
+        elif l.startswith(";;#ASMEND"):
+            in_asm = False
+        elif l.endswith(":") and not l.startswith((".L", ";")):
+            close()
+            name, asm_loads, spills = l[:-1], 0, 0
+        elif l and l[0] not in ";.":
+            op = l.split()[0]
+            if in_asm and op.startswith(("buffer_load_dword", "global_load_dword")) and "_lds_" not in op:
+                asm_loads += 1
+            elif op.startswith(("scratch_store", "scratch_load")):
+                spills += 1
+    close()
     return found
 
 

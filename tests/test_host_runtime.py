@@ -376,3 +376,18 @@ def test_build_scan_finds_a_register_copy_in_front_of_an_inline_asm_mfma():
     assert len(scan_mfma_hazards("\tv_readlane_b32 s4, v127, 3\n\tv_readlane_b32 s5, v127, 4\n" + g2s)) == 2
     assert scan_mfma_hazards("\tv_readlane_b32 s4, v127, 3\n\ts_nop 3\n" + g2s) == []
     assert scan_mfma_hazards("\ts_add_u32 s4, s6, s7\n" + g2s) == []
+
+
+def test_spills_beside_hand_counted_loads_are_found():
+    # a kernel that loads registers in inline assembly counts those loads itself; the compiler,
+    # which inserts no wait for them, must not spill in such a kernel (aster_amd/build.py)
+    from aster_amd.build import scan_spills_beside_asm_loads
+    load = "\t;;#ASMSTART\n\tbuffer_load_dwordx4 v[8:11], v123, s[16:19], s66 offen\n\t;;#ASMEND\n"
+    lds = "\t;;#ASMSTART\n\tglobal_load_lds_dwordx4 v98, s[56:57]\n\t;;#ASMEND\n"
+    spill = "\tscratch_store_dwordx4 off, v[8:11], off ; 16-byte Folded Spill\n"
+    assert scan_spills_beside_asm_loads("k1:\n" + load + spill) == [("k1", 1)]
+    assert scan_spills_beside_asm_loads("k1:\n" + load + "k2:\n" + spill) == []
+    assert scan_spills_beside_asm_loads("k1:\n" + lds + spill) == []       # transfers into LDS write no register
+    assert scan_spills_beside_asm_loads("k1:\n.LBB0_1:\n" + load + ".LBB0_2:\n" + spill + spill) == [("k1", 2)]
+    assert scan_spills_beside_asm_loads("k1:\n\tbuffer_load_dwordx4 v[8:11], v1, s[0:3], 0 offen\n" + spill) == []
+
