@@ -1503,6 +1503,55 @@ def test_random_shapes_through_auto_selection(gpu, dt, out_dt, M, N, K, with_bia
         assert np.isnan(tail).all() if out_dt == "f32" else (tail == 0x7FC1).all()
 
 
+def _random_pre_shuffled_cases(n_cases=36, seed=77):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for i in range(n_cases):
+        dt = ("bf16", "f16", "fp8_e4m3", "mxfp4")[i % 4]
+        M = int(rng.integers(1, 160)) * 8
+        N = int(rng.integers(1, 24)) * 64
+        K = int(rng.integers(1, 12)) * 512 if dt == "mxfp4" else int(rng.integers(1, 40)) * 128
+        out = ("f32", "bf16", "f16")[int(rng.integers(0, 3))]
+        cases.append((dt, out, M, N, K, bool(rng.integers(0, 2)), int(rng.integers(0, 3)) * 8))
+    return cases
+
+
+@pytest.mark.parametrize("dt,out_dt,M,N,K,with_bias,pad", _random_pre_shuffled_cases())
+def test_random_shapes_with_pre_shuffled_weights(gpu, dt, out_dt, M, N, K, with_bias, pad):
+    """The stream kernels that load pre-shuffled B straight into MFMA operands (operand_path
+    direct_b_k8: 16-bit, fp8, MXFP4) on seeded random shapes with edge tiles in M and N and every
+    residue of the K-step count: the oracle's result, pad columns untouched."""
+    from aster_amd.kittens_helpers import shuffle_scales_e8m0_lanes, shuffle_weight_bytes, shuffle_weight_k8
+    a, b, extra = operands(M, N, K, dt, seed=3000 + M + N + K, b_std=0.05)
+    bias = np.random.default_rng(6).standard_normal(N).astype(np.float32) if with_bias else None
+    dev = dict(extra)
+    if dt in ("bf16", "f16"):
+        b_dev = shuffle_weight_k8(np.ascontiguousarray(b).view(np.uint16))
+    else:
+        b_dev = shuffle_weight_bytes(b)
+        if dt == "mxfp4":
+            dev["mx_b"] = shuffle_scales_e8m0_lanes(extra["mx_b"])
+    out, name = run_gemm(a, b_dev, M, N, K, dt, out_dt, bias=bias, ldc=N + pad if pad else 0,
+                         operand_path="direct_b_k8", **dev)
+    assert name.startswith("streamdb_")
+    if dt == "fp8_e4m3":
+        want = G.gemm_fp8(a, b, extra["scale_a"], extra["scale_b"], out_dtype=_DT[out_dt], bias=bias)
+    elif dt == "mxfp4":
+        want = G.gemm_mxfp4(a, extra["mx_a"], b, extra["mx_b"], out_dtype=_DT[out_dt], bias=bias)
+    else:
+        want = G.gemm(a, b, _DT[dt], _DT[out_dt], bias=bias)
+    got, ref = G.output_to_f32(out[:, :N], _DT[out_dt]), G.output_to_f32(want, _DT[out_dt])
+    assert not np.isnan(got).any(), name
+    ulp = {"f32": 2.0 ** -20, "bf16": 2.0 ** -7, "f16": 2.0 ** -10}[out_dt]
+    tol = 2 * ulp * np.abs(ref) + 2e-4 * np.abs(ref).max()
+    assert np.all(np.abs(got - ref) <= tol), (name, float(np.abs(got - ref).max()))
+    bar = REL_L2_BAR if out_dt != "f32" else (1e-4 if dt == "fp8_e4m3" else 1e-5)
+    assert G.rel_l2(got, ref) <= bar, name
+    if pad:
+        tail = out[:, N:]
+        assert np.isnan(tail).all() if out_dt == "f32" else (tail == 0x7FC1).all()
+
+
 @pytest.mark.parametrize("M,N,K,dt", [(512, 768, 1024, "bf16"), (16, 520, 4096, "bf16"), (300, 200, 512, "fp8_e4m3")])
 def test_tune_returns_a_runnable_variant_that_matches_the_oracle(gpu, M, N, K, dt):
     a, b, extra = operands(M, N, K, dt, seed=91, b_std=0.05)
