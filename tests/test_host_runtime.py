@@ -182,6 +182,22 @@ def test_descriptor_says_when_the_mapping_is_not_honoured(tmp_path):
         assert "operand_path" not in rep.not_honoured
 
 
+def test_direct_b_mapping_selects_a_stream_kernel_for_every_operand_type():
+    # the reference's best mapping (128 x 256 tile, 1 x 4 waves, B pre-shuffled and loaded straight
+    # into MFMA operands) on a compute-bound shape: a kernel of that geometry exists for 16-bit,
+    # fp8 and MXFP4 operands, and nothing of the request is reported as dropped
+    from aster_amd.gemm_config import OperandPath
+    for dt, kernel in (("bf16", "streamdb_bf16_128x256_w1x4"), ("f16", "streamdb_f16_128x256_w1x4"),
+                       ("fp8_e4m3", "streamdb_fp8_128x256_w1x4"), ("mxfp4", "streamdb_mxfp4_128x256_w1x4")):
+        cfg = make_instance(512, 768, 1024, dtype_ab=dt, wg_tile=(128, 256), waves=(1, 4),
+                            operand_path=OperandPath.DIRECT_B)
+        c, info = gemm.select_for_instance(cfg)
+        assert info.name.decode().startswith(kernel), (dt, info.name)
+        assert c.operand_path == _capi.OPERAND_DIRECT_B_K8
+        rep = gemm.mapping_report(cfg, c, info)
+        assert rep.honoured and not rep.not_honoured, (dt, rep.not_honoured)
+
+
 def test_execute_checks_host_operand_sizes_before_touching_the_gpu(tmp_path):
     cfg = make_instance(256, 256, 256)
     path, _ = gemm.compile_gemm(cfg, str(tmp_path / "k.hsaco"))
