@@ -59,6 +59,12 @@ __device__ __forceinline__ void gemm_stream8_body(const GemmArgs& p, int bid, in
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wm = wave / WN, wn = wave % WN;
+  // Eight waves: waves w and w + 4 share a SIMD.  The upper four get the higher issue priority,
+  // so that of the two the same one wins whenever both are ready (measured on 8192^3: 350-352 us
+  // without, 343-346 with; no difference for the 16-bit and MXFP4 kernels, which do not do it).
+  if constexpr (NW == 8) {
+    if (wave >= 4) __builtin_amdgcn_s_setprio(1);
+  }
 
   // ---- global -> LDS: identical to the 16-bit stream kernel --------------------------------
   const int lane = threadIdx.x & 63;
