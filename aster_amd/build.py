@@ -10,10 +10,12 @@ tree.  `python -m aster_amd.build` rebuilds it.
 from __future__ import annotations
 
 import os
-import re
 import subprocess
 import sys
 from concurrent.futures import ThreadPoolExecutor
+
+from .asm_scan import (MFMA_WAIT_STATES, VMEM_SGPR_WAIT_STATES, scan_mfma_hazards,  # noqa: F401
+                       scan_spills_beside_asm_loads)
 
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(PKG_DIR)
@@ -61,7 +63,8 @@ def _compile(src: str) -> str:
     found = scan_mfma_hazards(text)
     spilled = scan_spills_beside_asm_loads(text)
     if spilled:
-        raise RuntimeError(f"{src}: register spills in kernels whose register loads are inline assembly "
+        raise RuntimeError(f"{src}: register spills (scratch, accumulation registers or the metadata's "
+                           f"spill counts) in kernels whose register loads are inline assembly "
                            f"(the compiler does not wait for those loads): {spilled}")
     for name in os.listdir(OBJ_DIR):  # the other intermediates are large and of no use
         if name.startswith(stem + "-") and name.endswith((".hipi", ".bc", ".out", ".resolution.txt")):
@@ -73,147 +76,6 @@ def _compile(src: str) -> str:
                            f"wrote too few wait states earlier (MFMA sources: {MFMA_WAIT_STATES}, scalar "
                            f"bases of vector-memory instructions: {VMEM_SGPR_WAIT_STATES}):\n{lines}")
     return obj
-
-
-# ---- a hazard the compiler cannot see -----------------------------------------------------
-#
-# The stream kernels write some MFMAs as inline asm (to tie the accumulator to the accumulation
-# registers).  The compiler's hazard recogniser does not look inside inline asm: where register
-# allocation places a copy (v_mov, v_accvgpr_mov, v_and ...) into a source register right in front
-# of such an MFMA, it inserts no wait states and the MFMA reads the register before the copy has
-# landed: wrong sums, no error (seen on gfx950 with one v_mov_b64 directly in front of a
-# v_mfma_scale_f32_16x16x128_f8f6f4).  The kernels keep such copies out of their K loops and put
-# `s_nop 1` in front of the MFMAs elsewhere; this scan of the generated assembly is the proof.
-
-MFMA_WAIT_STATES = 2
-# The same blind spot for the transfers (global_load_lds_* / buffer_load_* written as inline asm with
-# a scalar base): an SGPR written by a VALU instruction (v_readlane restoring a spilled SGPR,
-# v_readfirstlane, a compare into an SGPR pair) must not be read by a vector-memory instruction
-# for five wait states.
-VMEM_SGPR_WAIT_STATES = 5
-
-_REG_RANGE = re.compile(r"([va])\[(\d+):(\d+)\]$")
-_REG_ONE = re.compile(r"([va])(\d+)$")
-
-
-_SREG_RANGE = re.compile(r"s\[(\d+):(\d+)\]$")
-_SREG_ONE = re.compile(r"s(\d+)$")
-
-
-def _sregs(tok: str) -> set:
-    tok = tok.strip().rstrip(",")
-    m = _SREG_RANGE.match(tok)
-    if m:
-        return {("s", i) for i in range(int(m.group(1)), int(m.group(2)) + 1)}
-    m = _SREG_ONE.match(tok)
-    return {("s", int(m.group(1)))} if m else set()
-
-
-def _regs(tok: str) -> set:
-    tok = tok.strip().rstrip(",")
-    m = _REG_RANGE.match(tok)
-    if m:
-        return {(m.group(1), i) for i in range(int(m.group(2)), int(m.group(3)) + 1)}
-    m = _REG_ONE.match(tok)
-    return {(m.group(1), int(m.group(2)))} if m else set()
-
-
-def scan_mfma_hazards(asm_text: str, wait_states: int = MFMA_WAIT_STATES):
-    """[(line, instruction text, writer line, writer text)] for every MFMA inside an inline-asm block
-    of gfx9 assembly text whose A, B, C or scale registers were written by a VALU instruction fewer
-    than `wait_states` wait states earlier (an instruction is one wait state, `s_nop n` is n + 1),
-    and for every vector-memory instruction inside an inline-asm block whose SGPR operands were
-    written by a VALU instruction fewer than VMEM_SGPR_WAIT_STATES wait states earlier."""
-    found = []
-    hist = []      # (wait states, registers written by a VALU instruction, text, line)
-    in_asm = False
-    for no, raw in enumerate(asm_text.split("\n"), 1):
-        l = raw.strip()
-        if l.startswith(";;#ASMSTART"):
-            in_asm = True
-            continue
-        if l.startswith(";;#ASMEND"):
-            in_asm = False
-            continue
-        if not l or l[0] in ";." :
-            continue
-        if l.endswith(":"):
-            if not l.startswith(".L"):
-                hist = []          # a new function
-            continue
-        op = l.split()[0]
-        args = l[len(op):].split(";")[0]
-        toks = [t for t in re.split(r",\s*", args.strip()) if t]
-        if op.startswith("v_mfma") or op.startswith("v_smfmac"):
-            if in_asm:
-                srcs = set()
-                for t in toks[1:]:
-                    if t.split():
-                        srcs |= _regs(t.split()[0])
-                ws = 0
-                for (w, written, text, wno) in reversed(hist):
-                    if ws >= wait_states:
-                        break
-                    if written & srcs:
-                        found.append((no, l[:110], wno, text[:90]))
-                    ws += w
-            hist.append((1, set(), l, no))
-        else:
-            w, written = 1, set()
-            if op == "s_nop":
-                w = int(toks[0], 0) + 1 if toks else 1
-            elif op.startswith(("v_readlane", "v_readfirstlane")) or \
-                    (op.startswith("v_cmp") and toks and toks[0].startswith("s")):
-                written = _sregs(toks[0]) if toks else set()
-            elif op.startswith("v_") and not op.startswith("v_cmp"):
-                written = _regs(toks[0]) if toks else set()
-            if in_asm and op.startswith(("global_load", "global_store", "buffer_load", "buffer_store")):
-                srcs = set()
-                for t in toks:
-                    if t.split():
-                        srcs |= _sregs(t.split()[0])
-                ws = 0
-                for (w2, written2, text, wno) in reversed(hist):
-                    if ws >= VMEM_SGPR_WAIT_STATES:
-                        break
-                    if written2 & srcs:
-                        found.append((no, l[:110], wno, text[:90]))
-                    ws += w2
-            hist.append((w, written, l, no))
-        if len(hist) > 12:
-            hist.pop(0)
-    return found
-
-
-def scan_spills_beside_asm_loads(asm_text: str):
-    """[(function, spill instructions)] for every function of gfx9 assembly text that loads
-    registers inside inline-asm blocks (loads the kernel counts by hand: the compiler inserts no
-    wait for them) and also holds register spills: a spill of such a register between the load and
-    the kernel's own wait would store the bytes the register held before."""
-    found = []
-    name, asm_loads, spills, in_asm = None, 0, 0, False
-
-    def close():
-        if name and asm_loads and spills:
-            found.append((name, spills))
-
-    for raw in asm_text.split("\n"):
-        l = raw.strip()
-        if l.startswith(";;#ASMSTART"):
-            in_asm = True
-        elif l.startswith(";;#ASMEND"):
-            in_asm = False
-        elif l.endswith(":") and not l.startswith((".L", ";")):
-            close()
-            name, asm_loads, spills = l[:-1], 0, 0
-        elif l and l[0] not in ";.":
-            op = l.split()[0]
-            if in_asm and op.startswith(("buffer_load_dword", "global_load_dword")) and "_lds_" not in op:
-                asm_loads += 1
-            elif op.startswith(("scratch_store", "scratch_load")):
-                spills += 1
-    close()
-    return found
 
 
 def _genco(src: str) -> str:

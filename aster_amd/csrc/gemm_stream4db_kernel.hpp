@@ -106,7 +106,9 @@ __device__ __forceinline__ void gemm_stream4db_body(const GemmArgs& p, int bid) 
   };
 
   // ---- B: global -> registers.  One buffer resource over the payload and one over the scale
-  // plane; a load is resource + scalar offset + per-lane offset. ------------------------------------
+  // plane; a load is resource + scalar offset + per-lane offset.  The hardware's range check does
+  // not cover the scalar offset, so the block indices of an edge tile are clamped to the last
+  // 16-row block of B and the last 64-row group of the plane (those columns are never stored). ------
   const unsigned chunk_row = (unsigned)(p.K >> 7) * 1024u;  // bytes of 16 rows of B (K/2 per row)
   const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(
       (void*)p.B, 0, (int)((unsigned)(p.N >> 4) * chunk_row), 0x00020000);
@@ -114,9 +116,15 @@ __device__ __forceinline__ void gemm_stream4db_body(const GemmArgs& p, int bid) 
       (void*)p.mx_b, 0, (int)((unsigned)(p.N >> 6) * (unsigned)nk * 512u), 0x00020000);
   unsigned b_tile[TN];
 #pragma unroll
-  for (int n = 0; n < TN; ++n)
-    b_tile[n] = __builtin_amdgcn_readfirstlane((unsigned)((col0 >> 4) + wn * TN + n) * chunk_row);
-  const unsigned s_tile = __builtin_amdgcn_readfirstlane((unsigned)((col0 >> 6) + wn) * (unsigned)nk * 512u);
+  for (int n = 0; n < TN; ++n) {
+    int nb = (col0 >> 4) + wn * TN + n;
+    const int last = (p.N >> 4) - 1;
+    nb = nb < last ? nb : last;
+    b_tile[n] = __builtin_amdgcn_readfirstlane((unsigned)nb * chunk_row);
+  }
+  int sg = (col0 >> 6) + wn;
+  sg = sg < (p.N >> 6) - 1 ? sg : (p.N >> 6) - 1;
+  const unsigned s_tile = __builtin_amdgcn_readfirstlane((unsigned)sg * (unsigned)nk * 512u);
   const unsigned b_lane = (unsigned)lane * 16, s_lane = (unsigned)lane * 8;
   i32x4 fb[NBUF][TN];
   int sbk[NBUF][2];  // scales of K-step k in sbk[k mod 4]

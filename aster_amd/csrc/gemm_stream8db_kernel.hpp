@@ -73,17 +73,22 @@ __device__ __forceinline__ void gemm_stream8db_body(const GemmArgs& p, int bid) 
         lds + slot * SLOT + (j * NW + wave) * 8 * kRowBytes);
   };
 
-  // ---- B: global -> registers.  A raw buffer over the payload (loads past its end return
-  // zeros: the columns of an edge tile); a load is resource + scalar offset + lane offset +
-  // the chunk's immediate. ---------------------------------------------------------------------------
+  // ---- B: global -> registers.  A raw buffer over the payload; a load is resource + scalar
+  // offset + lane offset + the chunk's immediate.  The hardware's range check covers the lane
+  // offset and the immediate only, not the scalar offset, so the 16-row block index of an edge
+  // tile is clamped to the last block of B here (those columns are never stored). ------------------
   const unsigned chunk_row = (unsigned)nk * 2048u;  // bytes of 16 rows of B
   const uint64_t b_addr = (uint64_t)(uintptr_t)p.B;
   const i32x4 b_rsrc = {(int)(unsigned)b_addr, (int)((unsigned)(b_addr >> 32) & 0xffffu),
                         (int)((unsigned)(p.N >> 4) * chunk_row), 0x00020000};
   unsigned b_tile[TN];
 #pragma unroll
-  for (int n = 0; n < TN; ++n)
-    b_tile[n] = __builtin_amdgcn_readfirstlane((unsigned)((col0 >> 4) + wn * TN + n) * chunk_row);
+  for (int n = 0; n < TN; ++n) {
+    int nb = (col0 >> 4) + wn * TN + n;
+    const int last = (p.N >> 4) - 1;
+    nb = nb < last ? nb : last;
+    b_tile[n] = __builtin_amdgcn_readfirstlane((unsigned)nb * chunk_row);
+  }
   const unsigned b_lane = (unsigned)lane * 16;
   i32x4 fbl[NBUF][TN][2];
   auto load_b1 = [&](int k, auto buf, auto nc) {

@@ -376,7 +376,7 @@ def test_build_scan_finds_a_register_copy_in_front_of_an_inline_asm_mfma():
             "v32, v95 op_sel_hi:[0,0,0] cbsz:4 blgp:4\n\t;;#ASMEND\n")
     copy = "\tv_mov_b64_e32 v[38:39], v[36:37]\n\tv_mov_b64_e32 v[36:37], v[34:35]\n"
     found = scan_mfma_hazards(copy + mfma.format(pre=""))
-    assert [(f[0], f[2]) for f in found] == [(4, 2), (4, 1)]
+    assert sorted((f[0], f[2]) for f in found) == [(4, 1), (4, 2)]
     # two wait states in between, of any kind, are enough
     assert scan_mfma_hazards(copy + mfma.format(pre="\ts_nop 1\n")) == []
     assert scan_mfma_hazards(copy + "\ts_add_u32 s0, s1, s2\n\ts_nop 0\n" + mfma.format(pre="")) == []
@@ -394,16 +394,87 @@ def test_build_scan_finds_a_register_copy_in_front_of_an_inline_asm_mfma():
     assert scan_mfma_hazards("\ts_add_u32 s4, s6, s7\n" + g2s) == []
 
 
+def test_build_scan_follows_the_back_edge_of_a_loop():
+    # a VALU write at the bottom of a loop and an inline-asm MFMA at its head are neighbours in
+    # execution order although the text has them far apart
+    from aster_amd.build import scan_mfma_hazards
+    mfma = ("\t;;#ASMSTART\n\tv_mfma_f32_16x16x32_bf16 a[0:3], v[36:39], v[4:7], a[0:3]\n\t;;#ASMEND\n")
+    filler = "\ts_add_u32 s0, s1, s2\n" * 6
+    loop = ("kern:                                   ; @kern\n" + filler + ".LBB0_1:    ; =>This Inner Loop\n" + mfma +
+            filler + "\tv_mov_b32_e32 v5, v9\n\ts_cbranch_scc1 .LBB0_1\n" + "\ts_endpgm\n")
+    found = scan_mfma_hazards(loop)
+    assert len(found) == 1 and "v_mov_b32_e32 v5" in found[0][3]
+    # the branch itself is one wait state: one more instruction in between is enough
+    ok = loop.replace("\tv_mov_b32_e32 v5, v9\n", "\tv_mov_b32_e32 v5, v9\n\ts_nop 0\n")
+    assert scan_mfma_hazards(ok) == []
+    # a forward branch over the wait states brings the write next to the MFMA as well
+    skip = ("kern:\n\tv_mov_b32_e32 v5, v9\n\ts_cbranch_scc1 .LBB0_2\n" + filler + ".LBB0_2:\n" + mfma)
+    assert len(scan_mfma_hazards(skip)) == 1
+    # nothing falls through an unconditional branch
+    dead = ("kern:\n\ts_branch .LBB0_3\n\tv_mov_b32_e32 v5, v9\n.LBB0_3:\n" + mfma)
+    assert scan_mfma_hazards(dead) == []
+
+
 def test_spills_beside_hand_counted_loads_are_found():
     # a kernel that loads registers in inline assembly counts those loads itself; the compiler,
-    # which inserts no wait for them, must not spill in such a kernel (aster_amd/build.py)
+    # which inserts no wait for them, must not spill in such a kernel (aster_amd/asm_scan.py)
     from aster_amd.build import scan_spills_beside_asm_loads
     load = "\t;;#ASMSTART\n\tbuffer_load_dwordx4 v[8:11], v123, s[16:19], s66 offen\n\t;;#ASMEND\n"
     lds = "\t;;#ASMSTART\n\tglobal_load_lds_dwordx4 v98, s[56:57]\n\t;;#ASMEND\n"
     spill = "\tscratch_store_dwordx4 off, v[8:11], off ; 16-byte Folded Spill\n"
     assert scan_spills_beside_asm_loads("k1:\n" + load + spill) == [("k1", 1)]
+    # function labels as the compiler writes them, with a trailing comment
+    assert scan_spills_beside_asm_loads("k1:        ; @k1\n" + load + spill) == [("k1", 1)]
     assert scan_spills_beside_asm_loads("k1:\n" + load + "k2:\n" + spill) == []
     assert scan_spills_beside_asm_loads("k1:\n" + lds + spill) == []       # transfers into LDS write no register
     assert scan_spills_beside_asm_loads("k1:\n.LBB0_1:\n" + load + ".LBB0_2:\n" + spill + spill) == [("k1", 2)]
     assert scan_spills_beside_asm_loads("k1:\n\tbuffer_load_dwordx4 v[8:11], v1, s[0:3], 0 offen\n" + spill) == []
+    # gfx950 spills vector registers into accumulation registers first: a copy of a register that
+    # an inline-asm load writes counts, a copy of any other register does not
+    assert scan_spills_beside_asm_loads("k1:\n" + load + "\tv_accvgpr_write_b32 a200, v9\n") == [("k1", 1)]
+    assert scan_spills_beside_asm_loads("k1:\n" + load + "\tv_accvgpr_write_b32 a200, v12\n") == []
+    assert scan_spills_beside_asm_loads("k1:\n" + load + "\tv_accvgpr_write_b32 a0, 0\n") == []
+    # and the allocator's own account in the kernel metadata
+    meta = ("\t.amdgpu_metadata\n---\namdhsa.kernels:\n  - .agpr_count:     0\n    .args:\n"
+            "      - .name:           p\n        .size: 8\n    .name:           {name}\n"
+            "    .sgpr_spill_count: {s}\n    .symbol:         {name}.kd\n    .vgpr_spill_count: {v}\n"
+            "...\n\t.end_amdgpu_metadata\n")
+    assert scan_spills_beside_asm_loads("k1:\n" + load + meta.format(name="k1", s=0, v=0)) == []
+    assert scan_spills_beside_asm_loads("k1:\n" + load + meta.format(name="k1", s=3, v=1)) == [("k1", 4)]
+    assert scan_spills_beside_asm_loads("k1:\n" + load + meta.format(name="k2", s=3, v=1)) == []
 
+
+def test_direct_b_loads_of_edge_tiles_stay_inside_the_payload():
+    # The pre-shuffled-B stream kernels address B as buffer resource + scalar offset (16-row block
+    # and K-step) + lane offset (+ 1 KiB immediate); the hardware checks only the lane offset and
+    # the immediate against the resource, so the scalar part must never leave the payload.  This
+    # models the offset arithmetic of gemm_stream8db / gemm_stream4db / gemm_streamdb_kernel.hpp
+    # (block index clamped to the last block of B) over edge shapes.
+    def extent(N, K, bytes_per_k_num, bytes_per_k_den, group, clamp):
+        row_bytes = K * bytes_per_k_num // bytes_per_k_den
+        chunk_row = 16 * row_bytes                     # bytes of a 16-row block
+        steps_bytes = row_bytes * 16                   # a block's K-steps lie back to back
+        worst = 0
+        for col0 in range(0, N, 256):
+            for wn in range(4):
+                for n in range(4):
+                    nb = (col0 >> 4) + wn * 4 + n
+                    if clamp:
+                        nb = min(nb, (N >> 4) - 1)
+                    worst = max(worst, nb * chunk_row + steps_bytes)   # one past the block's last byte
+        return worst
+    for N in (16, 64, 80, 192, 272, 1000 // 16 * 16, 4096 + 64):
+        for K in (128, 512, 4096):
+            payload = N * K                               # fp8: one byte per element
+            assert extent(N, K, 1, 1, 16, clamp=True) <= payload
+            if N % 256:
+                assert extent(N, K, 1, 1, 16, clamp=False) > payload   # what the clamp is for
+    for N in (64, 128, 192, 320, 4096 + 64):
+        for K in (512, 4096):
+            payload = N * K // 2
+            assert extent(N, K, 1, 2, 16, clamp=True) <= payload
+            # lane-order scale plane: 64-row groups of (K / 256) * 512 bytes
+            groups = N >> 6
+            plane = groups * (K // 256) * 512
+            worst = max(min((col0 >> 6) + wn, groups - 1) + 1 for col0 in range(0, N, 256) for wn in range(4))
+            assert worst * (K // 256) * 512 <= plane
