@@ -22,7 +22,9 @@ SCALE_NONE, SCALE_TENSOR, SCALE_MX32 = 0, 1, 2
 # astergemm_kernel_family
 KERNEL_AUTO, KERNEL_TILE, KERNEL_SKINNY = 0, 1, 2
 OPERAND_LDS, OPERAND_DIRECT_B, OPERAND_DIRECT_B_K8 = 0, 1, 2
-ABI_VERSION = 2
+# astergemm_mx_layout
+MX_ROWS, MX_LANES128 = 0, 1
+ABI_VERSION = 3
 NOALLOC_SCRATCH_BYTES = 16 << 20
 
 DTYPE_NAMES = {"f16": F16, "bf16": BF16, "fp8_e4m3": FP8_E4M3, "mxfp4": MXFP4, "f32": F32}
@@ -47,7 +49,8 @@ class Config(C.Structure):
         ("waves_m", C.c_int32), ("waves_n", C.c_int32),
         ("variant", C.c_int32),
         ("operand_path", C.c_int32),
-        ("reserved", C.c_int32 * 5),
+        ("mx_a_layout", C.c_int32),
+        ("reserved", C.c_int32 * 4),
     ]
 
 
@@ -124,6 +127,11 @@ SIGNATURES = {
     "astergemm_shuffle_weight_8": (C.c_int, [_P, _P, C.c_int64, C.c_int64]),
     "astergemm_shuffle_scales_e8m0": (C.c_int, [_P, _P, C.c_int64, C.c_int64]),
     "astergemm_shuffle_scales_e8m0_lanes": (C.c_int, [_P, _P, C.c_int64, C.c_int64]),
+    "astergemm_mx_lanes128_bytes": (C.c_int64, [C.c_int64, C.c_int64]),
+    "astergemm_shuffle_scales_e8m0_lanes128": (C.c_int, [_P, _P, C.c_int64, C.c_int64]),
+    "astergemm_preshuffle_scales_a": (C.c_int, [C.c_int64, C.c_int64, _P, _P, _P]),
+    "astergemm_quantize_mxfp4_ex": (C.c_int, [_P, C.c_int, C.c_int64, C.c_int64, C.c_int64, _P, _P,
+                                              C.c_int, _P]),
     "astergemm_preshuffle": (C.c_int, [C.c_int, C.c_int, C.c_int64, C.c_int64, _P, _P, _P, _P, _P]),
     "astergemm_weight_crc32": (C.c_uint32, [_P, C.c_size_t]),
     "astergemm_weight_header_init": (C.c_int, [C.POINTER(WeightHeader), C.c_int, C.c_int, C.c_int64,

@@ -76,7 +76,8 @@ const Variant* variant_at(int index) {
 }
 
 bool variant_matches_types(const Variant& v, const astergemm_config& c) {
-  return v.dtype_ab == c.dtype_ab && v.dtype_c == c.dtype_c && v.operand_path == c.operand_path;
+  return v.dtype_ab == c.dtype_ab && v.dtype_c == c.dtype_c && v.operand_path == c.operand_path &&
+         v.mx_a_layout == c.mx_a_layout;
 }
 
 const char* validate_problem(const astergemm_config& c) {
@@ -89,6 +90,9 @@ const char* validate_problem(const astergemm_config& c) {
     return "bad scale_mode";
   if (c.operand_path < ASTERGEMM_OPERAND_LDS || c.operand_path > ASTERGEMM_OPERAND_DIRECT_B_K8)
     return "bad operand_path";
+  if (c.mx_a_layout != ASTERGEMM_MX_ROWS &&
+      (c.mx_a_layout != ASTERGEMM_MX_LANES128 || c.dtype_ab != ASTERGEMM_MXFP4))
+    return "bad mx_a_layout (LANES128 goes with MXFP4 operands)";
   if ((c.dtype_ab == ASTERGEMM_MXFP4) != (c.scale_mode == ASTERGEMM_SCALE_MX32))
     return "MXFP4 operands and SCALE_MX32 go together";
   if (c.dtype_ab == ASTERGEMM_MXFP4 && c.K % 32 != 0) return "MXFP4 needs K % 32 == 0";
@@ -313,6 +317,10 @@ int build_args(const Variant& v, const astergemm_config& c, const astergemm_oper
   }
   if (c.scale_mode == ASTERGEMM_SCALE_MX32 && (!ops.dMxA || !ops.dMxB)) {
     set_error("astergemm: SCALE_MX32 needs dMxA and dMxB");
+    return ASTERGEMM_EINVAL;
+  }
+  if (c.mx_a_layout == ASTERGEMM_MX_LANES128 && (((uintptr_t)ops.dMxA) & 15)) {
+    set_error("astergemm: dMxA in lane order must be 16-byte aligned");
     return ASTERGEMM_EINVAL;
   }
   if (c.scale_mode == ASTERGEMM_SCALE_MX32 && ((((uintptr_t)ops.dMxA) | ((uintptr_t)ops.dMxB)) & 7)) {
@@ -754,6 +762,32 @@ int astergemm_shuffle_scales_e8m0_lanes(const uint8_t* src, uint8_t* dst, int64_
           for (int t = 0; t < 4; ++t)
             for (int h = 0; h < 2; ++h)
               *o++ = src[(nb4 * 64 + t * 16 + i) * ld + st * 8 + 4 * h + q];
+  return 0;
+}
+
+int64_t astergemm_mx_lanes128_bytes(int64_t M, int64_t K) {
+  if (M < 0 || K < 0) return 0;
+  return ((M + 127) / 128) * (K / 256) * 1024;
+}
+
+int astergemm_shuffle_scales_e8m0_lanes128(const uint8_t* src, uint8_t* dst, int64_t M, int64_t K) {
+  if (!src || !dst || M < 0 || K < 0 || K % 256 != 0) {
+    set_error("astergemm_shuffle_scales_e8m0_lanes128: need K %% 256 == 0");
+    return ASTERGEMM_EINVAL;
+  }
+  // dst order (group g, step, lane group q, row i, tile t, half h) <- src (g, t, i, step, 4 h + q);
+  // rows past M: 127
+  const int64_t steps = K / 256, ld = K / 32;
+  uint8_t* o = dst;
+  for (int64_t g = 0; g < (M + 127) / 128; ++g)
+    for (int64_t st = 0; st < steps; ++st)
+      for (int q = 0; q < 4; ++q)
+        for (int i = 0; i < 16; ++i)
+          for (int t = 0; t < 8; ++t)
+            for (int h = 0; h < 2; ++h) {
+              const int64_t row = g * 128 + t * 16 + i;
+              *o++ = row < M ? src[row * ld + st * 8 + 4 * h + q] : (uint8_t)127;
+            }
   return 0;
 }
 

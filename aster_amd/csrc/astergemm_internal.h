@@ -68,6 +68,8 @@ struct Variant {
   // Grid the launcher uses when it is not the number of output tiles (persistent kernels);
   // `cus` = compute units of the current device.  nullptr = tiles (times splits).
   int (*grid)(const astergemm_config& c, int cus) = nullptr;
+  // Layout of A's e8m0 plane this variant reads (astergemm_mx_layout); row-major by default.
+  int mx_a_layout = 0;
 };
 
 // Compute units of the current device (0 when there is none), cached per device ordinal.

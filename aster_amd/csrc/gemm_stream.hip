@@ -84,10 +84,10 @@ const char* check_streamdb(const astergemm_config& c) {
 
 // ---- MXFP4, B pre-shuffled (payload in step order, scale plane in lane order) and loaded
 // straight into MFMA operands: 128 x 256 tiles, four waves (gemm_stream4db_kernel.hpp) ---------
-template <int DT, int OUT>
+template <int DT, int OUT, bool SAL>
 int launch_stream4db(const GemmArgs& a, int grid, hipStream_t s) {
   constexpr int lds = 4 * 128 * kRowBytes + 2 * 128 * 16;
-  auto k = gemm_stream4db_kernel<DT, OUT>;
+  auto k = gemm_stream4db_kernel<DT, OUT, SAL>;
   static std::atomic<uint64_t> attr_devs{0};
   if (int e = lds_attr_once(attr_devs, (const void*)k, lds)) return e;
   // what the kernel's indexing assumes: whole 64-row groups of B, an even number of whole
@@ -110,12 +110,14 @@ const char* check_stream4db(const astergemm_config& c) {
   return nullptr;
 }
 
-#define AG_STREAM4DB(name, DT, OUT)                                              \
+#define AG_STREAM4DB(name, DT, OUT, SAL)                                         \
   Variant {                                                                      \
     name, ASTERGEMM_KERNEL_TILE, DT, OUT, 128, 256, kRowBytes, 1, 4, 4, 2,       \
         4 * 128 * kRowBytes + 2 * 128 * 16,                                      \
-        (const void*)gemm_stream4db_kernel<DT, OUT>, launch_stream4db<DT, OUT>,  \
-        check_stream4db, ASTERGEMM_OPERAND_DIRECT_B_K8                           \
+        (const void*)gemm_stream4db_kernel<DT, OUT, SAL>,                        \
+        launch_stream4db<DT, OUT, SAL>, check_stream4db,                         \
+        ASTERGEMM_OPERAND_DIRECT_B_K8, nullptr, nullptr,                         \
+        SAL ? ASTERGEMM_MX_LANES128 : ASTERGEMM_MX_ROWS                          \
   }
 
 // ---- fp8, B pre-shuffled into step order and loaded straight into MFMA operands: 128 x 256
@@ -579,15 +581,19 @@ const Variant kStreamVariants[] = {
     AG_STREAM4_WALK("stream_mxfp4_256x256_w2x4_walk_bf16", ASTERGEMM_MXFP4, ASTERGEMM_BF16),
     AG_STREAM4_WALK("stream_mxfp4_256x256_w2x4_walk_f32", ASTERGEMM_MXFP4, ASTERGEMM_F32),
     AG_STREAM4_WALK("stream_mxfp4_256x256_w2x4_walk_f16", ASTERGEMM_MXFP4, ASTERGEMM_F16),
-    AG_STREAM4DB("streamdb_mxfp4_128x256_w1x4_bf16", ASTERGEMM_MXFP4, ASTERGEMM_BF16),
-    AG_STREAM4DB("streamdb_mxfp4_128x256_w1x4_f32", ASTERGEMM_MXFP4, ASTERGEMM_F32),
-    AG_STREAM4DB("streamdb_mxfp4_128x256_w1x4_f16", ASTERGEMM_MXFP4, ASTERGEMM_F16),
+    AG_STREAM4DB("streamdb_mxfp4_128x256_w1x4_bf16", ASTERGEMM_MXFP4, ASTERGEMM_BF16, false),
+    AG_STREAM4DB("streamdb_mxfp4_128x256_w1x4_f32", ASTERGEMM_MXFP4, ASTERGEMM_F32, false),
+    AG_STREAM4DB("streamdb_mxfp4_128x256_w1x4_f16", ASTERGEMM_MXFP4, ASTERGEMM_F16, false),
     AG_STREAM8DB("streamdb_fp8_128x256_w1x4_bf16", ASTERGEMM_FP8_E4M3, ASTERGEMM_BF16),
     AG_STREAM8DB("streamdb_fp8_128x256_w1x4_f32", ASTERGEMM_FP8_E4M3, ASTERGEMM_F32),
     AG_STREAM8DB("streamdb_fp8_128x256_w1x4_f16", ASTERGEMM_FP8_E4M3, ASTERGEMM_F16),
     AG_STREAM4_128("stream_mxfp4_128x128_w2x2_bf16", ASTERGEMM_MXFP4, ASTERGEMM_BF16),
     AG_STREAM4_128("stream_mxfp4_128x128_w2x2_f32", ASTERGEMM_MXFP4, ASTERGEMM_F32),
     AG_STREAM4_128("stream_mxfp4_128x128_w2x2_f16", ASTERGEMM_MXFP4, ASTERGEMM_F16),
+    // the same with A's e8m0 plane in lane order (mx_a_layout = ASTERGEMM_MX_LANES128)
+    AG_STREAM4DB("streamdb_mxfp4_128x256_w1x4_sal_bf16", ASTERGEMM_MXFP4, ASTERGEMM_BF16, true),
+    AG_STREAM4DB("streamdb_mxfp4_128x256_w1x4_sal_f32", ASTERGEMM_MXFP4, ASTERGEMM_F32, true),
+    AG_STREAM4DB("streamdb_mxfp4_128x256_w1x4_sal_f16", ASTERGEMM_MXFP4, ASTERGEMM_F16, true),
 };
 
 }  // namespace

@@ -160,7 +160,9 @@ __global__ __launch_bounds__(256) void quantize_fp8_kernel(const void* __restric
 // block maximum goes round the 8 lanes with three exchanges; every lane then encodes its 4
 // elements (2 bytes out) and lane 0 of the group writes the scale byte.  CONTIG: ld == K, so
 // block t sits at element 32 t and no (row, column) split is needed.
-template <int SRC, bool CONTIG>
+// LANES: the scale byte of block c of row r goes where astergemm_shuffle_scales_e8m0_lanes128 puts
+// it (groups of 128 rows, one KiB per group and 8-block step).
+template <int SRC, bool CONTIG, bool LANES = false>
 __global__ __launch_bounds__(256) void quantize_mxfp4_kernel(const void* __restrict__ src,
                                                              int64_t nblocks, unsigned bpr,
                                                              int64_t ld,
@@ -221,7 +223,16 @@ __global__ __launch_bounds__(256) void quantize_mxfp4_kernel(const void* __restr
       }
       if (live[u]) {
         *(unsigned short*)(packed + t[u] * 16 + l8 * 2) = (unsigned short)w;
-        if (l8 == 0) scales[t[u]] = bad ? (uint8_t)0xFF : (uint8_t)sbyte;
+        if (l8 == 0) {
+          int64_t so = t[u];
+          if constexpr (LANES) {
+            const unsigned r = (unsigned)t[u] / bpr, c = (unsigned)t[u] - r * bpr;
+            // (group, step, q, i, tile, h): block c = 8 step + 4 h + q, row r = 128 group + 16 tile + i
+            so = ((int64_t)(r >> 7) * (bpr >> 3) + (c >> 3)) * 1024 +
+                 (((c & 3) * 16 + (r & 15)) * 16 + ((r >> 4) & 7) * 2 + ((c >> 2) & 1));
+          }
+          scales[so] = bad ? (uint8_t)0xFF : (uint8_t)sbyte;
+        }
       }
     }
   }
@@ -291,15 +302,18 @@ extern "C" int astergemm_quantize_fp8_tensor(const void* dSrc, int src_dtype, in
   return 0;
 }
 
-extern "C" int astergemm_quantize_mxfp4(const void* dSrc, int src_dtype, int64_t rows, int64_t K,
-                                        int64_t ld_src, uint8_t* dPacked, uint8_t* dScales,
-                                        void* stream) {
+extern "C" int astergemm_quantize_mxfp4_ex(const void* dSrc, int src_dtype, int64_t rows, int64_t K,
+                                           int64_t ld_src, uint8_t* dPacked, uint8_t* dScales,
+                                           int scales_layout, void* stream) {
   if (ld_src == 0) ld_src = K;
+  const bool lanes = scales_layout == ASTERGEMM_MX_LANES128;
   if (rows < 0 || K < 0 || K % 32 != 0 || ld_src < K || ld_src % 8 != 0 || !src_ok(src_dtype) ||
       ((rows > 0 && K > 0) && (!dSrc || !dPacked || !dScales)) || (((uintptr_t)dSrc) & 15) ||
-      (((uintptr_t)dPacked) & 15)) {
+      (((uintptr_t)dPacked) & 15) || (!lanes && scales_layout != ASTERGEMM_MX_ROWS) ||
+      (lanes && (K % 256 != 0 || (((uintptr_t)dScales) & 15)))) {
     set_error("astergemm_quantize_mxfp4: need a source of F32, BF16 or F16, K %% 32 == 0, "
-              "ld_src >= K, ld_src %% 8 == 0, dSrc and dPacked 16-byte aligned");
+              "ld_src >= K, ld_src %% 8 == 0, dSrc and dPacked 16-byte aligned; scales in lane "
+              "order: K %% 256 == 0 and dScales 16-byte aligned");
     return ASTERGEMM_EINVAL;
   }
   if (rows == 0 || K == 0) return 0;
@@ -312,17 +326,27 @@ extern "C" int astergemm_quantize_mxfp4(const void* dSrc, int src_dtype, int64_t
   (void)hipGetLastError();
   with_src(src_dtype, [&](auto T) {
     constexpr int SRC = decltype(T)::value;
-    if (ld_src == K)
-      hipLaunchKernelGGL((quantize_mxfp4_kernel<SRC, true>), grid, dim3(256), 0,
-                         (hipStream_t)stream, dSrc, nblocks, (unsigned)(K / 32), ld_src, dPacked,
-                         dScales);
-    else
-      hipLaunchKernelGGL((quantize_mxfp4_kernel<SRC, false>), grid, dim3(256), 0,
-                         (hipStream_t)stream, dSrc, nblocks, (unsigned)(K / 32), ld_src, dPacked,
-                         dScales);
+    auto go = [&](auto kern) {
+      hipLaunchKernelGGL(kern, grid, dim3(256), 0, (hipStream_t)stream, dSrc, nblocks,
+                         (unsigned)(K / 32), ld_src, dPacked, dScales);
+    };
+    if (lanes) {
+      if (ld_src == K) go(quantize_mxfp4_kernel<SRC, true, true>);
+      else go(quantize_mxfp4_kernel<SRC, false, true>);
+    } else {
+      if (ld_src == K) go(quantize_mxfp4_kernel<SRC, true, false>);
+      else go(quantize_mxfp4_kernel<SRC, false, false>);
+    }
   });
   AG_HIP(hipGetLastError());
   return 0;
+}
+
+extern "C" int astergemm_quantize_mxfp4(const void* dSrc, int src_dtype, int64_t rows, int64_t K,
+                                        int64_t ld_src, uint8_t* dPacked, uint8_t* dScales,
+                                        void* stream) {
+  return astergemm_quantize_mxfp4_ex(dSrc, src_dtype, rows, K, ld_src, dPacked, dScales,
+                                     ASTERGEMM_MX_ROWS, stream);
 }
 
 // ---- pre-shuffle of weights on the device ----------------------------------------------------
@@ -365,13 +389,27 @@ __global__ __launch_bounds__(256) void preshuffle_kernel(const uint8_t* __restri
     const int n = (int)(t & 15);
     const int64_t st = (t >> 4) % steps, nb = (t >> 4) / steps;
     *(uint2*)(dst + t * 8) = *(const uint2*)(src + (nb * 16 + n) * rb + st * 8);
-  } else {
+  } else if constexpr (MODE == 4) {
     // dst (nb4, step, q, i, tile, h) <- src (nb4, tile, i, step, 4h + q), bytes; rb = K / 32 bytes
     const int64_t steps = rb / 8;
     const int h = (int)(t & 1), tl = (int)((t >> 1) & 3), i = (int)((t >> 3) & 15), q = (int)((t >> 7) & 3);
     const int64_t st = (t >> 9) % steps, nb4 = (t >> 9) / steps;
     dst[t] = src[(nb4 * 64 + tl * 16 + i) * rb + st * 8 + 4 * h + q];
   }
+}
+
+// A's plane into lane order in groups of 128 rows: dst (g, step, q, i, tile, h) <- src (g, tile, i,
+// step, 4h + q), one byte per thread; rows past `rows` get 127 (scale 1)
+__global__ __launch_bounds__(256) void preshuffle_scales_a_kernel(const uint8_t* __restrict__ src,
+                                                                  uint8_t* __restrict__ dst,
+                                                                  int64_t units, int64_t rb, int64_t rows) {
+  const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (t >= units) return;
+  const int64_t steps = rb / 8;
+  const int h = (int)(t & 1), tl = (int)((t >> 1) & 7), i = (int)((t >> 4) & 15), q = (int)((t >> 8) & 3);
+  const int64_t st = (t >> 10) % steps, g = (t >> 10) / steps;
+  const int64_t row = g * 128 + tl * 16 + i;
+  dst[t] = row < rows ? src[row * rb + st * 8 + 4 * h + q] : (uint8_t)127;
 }
 
 template <int MODE>
@@ -428,4 +466,25 @@ extern "C" int astergemm_preshuffle(int dtype_ab, int operand_path, int64_t N, i
   if (rc != 0 || !fp4) return rc;
   return k8 ? preshuffle_launch<4>(dMxSrc, dMxDst, N * (K / 32), 1, K / 32, s)
             : preshuffle_launch<3>(dMxSrc, dMxDst, N * (K / 32), 8, K / 32, s);
+}
+
+extern "C" int astergemm_preshuffle_scales_a(int64_t M, int64_t K, const uint8_t* dMxSrc,
+                                             uint8_t* dMxDst, void* stream) {
+  using namespace astergemm;
+  if (M < 0 || K < 0 || K % 256 != 0 || (M > 0 && K > 0 && (!dMxSrc || !dMxDst || dMxSrc == dMxDst)) ||
+      ((((uintptr_t)dMxSrc) | ((uintptr_t)dMxDst)) & 15)) {
+    set_error("astergemm_preshuffle_scales_a: need K %% 256 == 0 and distinct 16-byte aligned planes");
+    return ASTERGEMM_EINVAL;
+  }
+  const int64_t units = astergemm_mx_lanes128_bytes(M, K);
+  if (units == 0) return 0;
+  if ((units + 255) / 256 >= (int64_t)1 << 31) {
+    set_error("astergemm_preshuffle_scales_a: plane too large");
+    return ASTERGEMM_EINVAL;
+  }
+  (void)hipGetLastError();
+  hipLaunchKernelGGL(preshuffle_scales_a_kernel, dim3((unsigned)((units + 255) / 256)), dim3(256), 0,
+                     (hipStream_t)stream, dMxSrc, dMxDst, units, K / 32, M);
+  AG_HIP(hipGetLastError());
+  return 0;
 }

@@ -199,14 +199,18 @@ class GemmPlan:
     def create(cls, M: int, N: int, K: int, dtype_ab: str = "bf16", dtype_c: str = "bf16", *,
                scale_mode: Optional[str] = None, has_bias: bool = False, lda: int = 0,
                ldb: int = 0, ldc: int = 0, family: int = _capi.KERNEL_AUTO, wg_tile=(0, 0),
-               variant: int = 0, operand_path: str = "lds") -> "GemmPlan":
+               variant: int = 0, operand_path: str = "lds", mx_a_layout: str = "rows") -> "GemmPlan":
         """`operand_path` follows GemmMappingSpec.operand_path of the reference: "lds" = B is
         plain row-major [N, ldb]; "direct_b" = B was pre-shuffled with `shuffle_weight` (the
         reference's order, read by the decode kernels; fp8 / MXFP4: `shuffle_weight_bytes`, the
         MXFP4 plane with `shuffle_scales_e8m0`); "direct_b_k8" = pre-shuffled for the stream
         kernels: 16-bit operands with `shuffle_weight_k8`, fp8 with `shuffle_weight_bytes`, MXFP4
-        with `shuffle_weight_bytes` and the scale plane with `shuffle_scales_e8m0_lanes`."""
+        with `shuffle_weight_bytes` and the scale plane with `shuffle_scales_e8m0_lanes`.
+        `mx_a_layout` = "rows" (A's e8m0 plane [M, K/32]) or "lanes128" (in the order of
+        `shuffle_scales_e8m0_lanes128` / `quantize_mxfp4_device(..., scales_layout="lanes128")`,
+        read by the "direct_b_k8" MXFP4 stream kernel without a pass through LDS)."""
         c = _capi.Config()
+        c.mx_a_layout = {"rows": _capi.MX_ROWS, "lanes128": _capi.MX_LANES128}[mx_a_layout]
         c.operand_path = _OPERAND_PATH_ID[operand_path]
         c.M, c.N, c.K = M, N, K
         c.lda, c.ldb, c.ldc = lda, ldb, ldc

@@ -166,3 +166,34 @@ def unshuffle_scales_e8m0_lanes(Ss: np.ndarray) -> np.ndarray:
     N, nb = Ss.shape
     view = np.ascontiguousarray(Ss).reshape(N // 64, nb // 8, 4, 16, 4, 2)
     return np.ascontiguousarray(view.transpose(0, 4, 3, 1, 5, 2)).reshape(N, nb)
+
+
+def mx_lanes128_bytes(M: int, K: int) -> int:
+    """Bytes of an activation e8m0 plane in lane order: whole groups of 128 rows."""
+    return ((M + 127) // 128) * (K // 256) * 1024
+
+
+def shuffle_scales_e8m0_lanes128(S: np.ndarray) -> np.ndarray:
+    """The e8m0 plane S[M, K/32] of MXFP4 ACTIVATIONS in lane order, for the stream kernel whose
+    waves multiply eight 16-row tiles of A each: rows padded to whole groups of 128 with the byte
+    127 (scale 1), viewed as (group, tile t=8, row i=16, step, half h=2, lane group q=4) and
+    stored (group, step, q, i, t, h): lane 16 q + i finds in its 16 bytes of the KiB (group,
+    step) the scales of blocks q (h = 0) and 4 + q (h = 1) of its row in each of the eight
+    tiles.  Returns a flat array of `mx_lanes128_bytes(M, K)` bytes."""
+    S = np.ascontiguousarray(S, dtype=np.uint8)
+    M, nb = S.shape
+    if nb % 8 != 0:
+        raise AssertionError(f"{nb} scale bytes per row are not whole 256-element steps")
+    G = (M + 127) // 128
+    pad = np.full((G * 128, nb), 127, np.uint8)
+    pad[:M] = S
+    view = pad.reshape(G, 8, 16, nb // 8, 2, 4)
+    return np.ascontiguousarray(view.transpose(0, 3, 5, 2, 1, 4)).reshape(-1)
+
+
+def unshuffle_scales_e8m0_lanes128(flat: np.ndarray, M: int, K: int) -> np.ndarray:
+    """Inverse of `shuffle_scales_e8m0_lanes128`: the row-major plane [M, K/32]."""
+    nb = K // 32
+    G = (M + 127) // 128
+    view = np.ascontiguousarray(flat, dtype=np.uint8).reshape(G, nb // 8, 4, 16, 8, 2)
+    return np.ascontiguousarray(view.transpose(0, 4, 3, 1, 5, 2)).reshape(G * 128, nb)[:M]

@@ -45,12 +45,24 @@ def quantize_fp8_tensor_device(d_src: int, n: int, d_dst: int, d_scale: int, *,
 
 
 def quantize_mxfp4_device(d_src: int, rows: int, K: int, d_packed: int, d_scales: int, *,
-                          src_dtype: str = "f32", ld_src: int = 0,
+                          src_dtype: str = "f32", ld_src: int = 0, scales_layout: str = "rows",
                           stream: Optional[int] = None) -> None:
-    """rows x K elements -> packed e2m1 [rows, K/2] and e8m0 scale bytes [rows, K/32]."""
-    _capi.check(_capi.load().astergemm_quantize_mxfp4(
+    """rows x K elements -> packed e2m1 [rows, K/2] and e8m0 scale bytes [rows, K/32]; with
+    `scales_layout="lanes128"` the scale bytes go into the lane order of
+    `kittens_helpers.shuffle_scales_e8m0_lanes128` (`mx_lanes128_bytes(rows, K)` bytes), what a
+    plan with `mx_a_layout="lanes128"` reads for its activations."""
+    layout = {"rows": _capi.MX_ROWS, "lanes128": _capi.MX_LANES128}[scales_layout]
+    _capi.check(_capi.load().astergemm_quantize_mxfp4_ex(
         ctypes.c_void_p(d_src), _src(src_dtype), rows, K, ld_src, ctypes.c_void_p(d_packed),
-        ctypes.c_void_p(d_scales), _s(stream)))
+        ctypes.c_void_p(d_scales), layout, _s(stream)))
+
+
+def preshuffle_scales_a_device(d_mx_src: int, d_mx_dst: int, M: int, K: int, *,
+                               stream: Optional[int] = None) -> None:
+    """The e8m0 plane [M, K/32] of quantised activations, device to device, into the lane order
+    of `kittens_helpers.shuffle_scales_e8m0_lanes128`."""
+    _capi.check(_capi.load().astergemm_preshuffle_scales_a(
+        M, K, ctypes.c_void_p(d_mx_src), ctypes.c_void_p(d_mx_dst), _s(stream)))
 
 
 def preshuffle_device(d_src: int, d_dst: int, N: int, K: int, dtype_ab: str, operand_path: str, *,

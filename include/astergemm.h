@@ -42,7 +42,7 @@
 extern "C" {
 #endif
 
-#define ASTERGEMM_ABI_VERSION 2
+#define ASTERGEMM_ABI_VERSION 3
 
 /* ---- error codes ------------------------------------------------------ */
 #define ASTERGEMM_OK 0
@@ -107,6 +107,21 @@ typedef enum astergemm_operand_path {
                                      kernel, N % 16 == 0, K % 64 == 0)       */
 } astergemm_operand_path;
 
+/* Layout of the e8m0 plane of the ACTIVATIONS (A) of an MXFP4 GEMM.  The
+ * reference has no scaled-MFMA GEMM; the operand form being matched is the
+ * scale register of v_mfma_scale_f32_16x16x128_f8f6f4
+ * (test/Dialect/AMDGCN/cdna4-scaled-mfma.mlir:37-47). */
+typedef enum astergemm_mx_layout {
+  ASTERGEMM_MX_ROWS = 0,     /* [M, K/32] bytes, row-major                      */
+  ASTERGEMM_MX_LANES128 = 1  /* lane order in groups of 128 rows, padded to
+                                whole groups: astergemm_shuffle_scales_e8m0_lanes128
+                                / astergemm_quantize_mxfp4_ex.  Read by the
+                                ASTERGEMM_OPERAND_DIRECT_B_K8 MXFP4 stream
+                                kernel with one 16-byte load per wave and
+                                256-element step, instead of a pass through
+                                LDS                                            */
+} astergemm_mx_layout;
+
 /* ---- problem + mapping --------------------------------------------------
  * C[M,N] = epilogue( sum_k A[M,K] * B[N,K] )      (B is stored N x K, i.e.
  * "column-major K x N"; reference: gemm_config.py:94, 109).
@@ -129,7 +144,9 @@ typedef struct astergemm_config {
   int32_t variant;       /* explicit variant id from astergemm_variant_*,
                             or 0                                             */
   int32_t operand_path;  /* astergemm_operand_path: how B is stored         */
-  int32_t reserved[5];
+  int32_t mx_a_layout;   /* astergemm_mx_layout: how A's e8m0 plane is stored
+                            (SCALE_MX32 only; B's follows operand_path)      */
+  int32_t reserved[4];
 } astergemm_config;
 
 /* What astergemm_select() reports back; the reference gets the same facts by
@@ -291,6 +308,17 @@ int astergemm_shuffle_scales_e8m0(const uint8_t* src, uint8_t* dst, int64_t N, i
  * reference (it has no scaled MFMA kernels). */
 int astergemm_shuffle_scales_e8m0_lanes(const uint8_t* src, uint8_t* dst, int64_t N, int64_t K);
 
+/* The e8m0 plane of MXFP4 ACTIVATIONS [M, K/32] in lane order
+ * (ASTERGEMM_MX_LANES128): rows in groups of 128 (the eight 16-row tiles a wave
+ * of the 128 x 256 stream kernel multiplies), per group and 256-element step one
+ * KiB in which lane L = 16 q + i finds, at byte 16 L + 2 t + h, the scale of
+ * block 4 h + q of row 128 g + 16 t + i.  M need not be a multiple of 128: the
+ * destination holds astergemm_mx_lanes128_bytes(M, K) = ceil(M / 128) * (K / 256)
+ * * 1024 bytes and the rows past M get the byte 127 (scale 1).  K % 256 == 0.
+ * No counterpart in the reference (it has no scaled MFMA kernels). */
+int64_t astergemm_mx_lanes128_bytes(int64_t M, int64_t K);
+int astergemm_shuffle_scales_e8m0_lanes128(const uint8_t* src, uint8_t* dst, int64_t M, int64_t K);
+
 /* ---- operand quantisers (device to device, on `stream`) -------------------
  * They write the bytes the fp8 / MXFP4 GEMM paths read (dtype_ab
  * ASTERGEMM_FP8_E4M3 / ASTERGEMM_MXFP4), so that a caller holding activations
@@ -326,6 +354,15 @@ int astergemm_quantize_fp8_tensor(const void* dSrc, int src_dtype, int64_t n, ui
 int astergemm_quantize_mxfp4(const void* dSrc, int src_dtype, int64_t rows, int64_t K,
                              int64_t ld_src, uint8_t* dPacked, uint8_t* dScales,
                              void* stream);
+/* The same with the scale plane written in `scales_layout` (astergemm_mx_layout):
+ * ASTERGEMM_MX_ROWS = astergemm_quantize_mxfp4; ASTERGEMM_MX_LANES128 = dScales
+ * holds astergemm_mx_lanes128_bytes(rows, K) bytes in the order of
+ * astergemm_shuffle_scales_e8m0_lanes128 (K % 256 == 0; the bytes of rows past
+ * `rows` in the last group are left as they are: those rows are never stored).
+ * The packed elements are the same bytes either way. */
+int astergemm_quantize_mxfp4_ex(const void* dSrc, int src_dtype, int64_t rows, int64_t K,
+                                int64_t ld_src, uint8_t* dPacked, uint8_t* dScales,
+                                int scales_layout, void* stream);
 
 /* The pre-shuffles above on the device (device to device, on `stream`), for a
  * caller whose weights are already in HBM (e.g. straight out of the quantisers):
@@ -341,6 +378,11 @@ int astergemm_quantize_mxfp4(const void* dSrc, int src_dtype, int64_t rows, int6
  * (test_102_gemm_python_multitile_g2s_directb_cdna4.py:446-467).             */
 int astergemm_preshuffle(int dtype_ab, int operand_path, int64_t N, int64_t K, const void* dSrc,
                          void* dDst, const uint8_t* dMxSrc, uint8_t* dMxDst, void* stream);
+/* astergemm_shuffle_scales_e8m0_lanes128 on the device, for activations that are
+ * already quantised: dMxSrc[M, K/32] row-major -> dMxDst (astergemm_mx_lanes128_bytes
+ * (M, K) bytes, rows past M get 127).  Distinct, 16-byte aligned planes. */
+int astergemm_preshuffle_scales_a(int64_t M, int64_t K, const uint8_t* dMxSrc, uint8_t* dMxDst,
+                                  void* stream);
 
 /* ---- weight artefact files (host side) -------------------------------------
  * A weight matrix B[N, K] on disk in the bytes the kernels stream, so that

@@ -29,12 +29,12 @@ _OUT_NP = {"f32": np.float32, "bf16": np.uint16, "f16": np.uint16}
 
 def run_gemm(a, b, M, N, K, dtype_ab, dtype_c, *, scale_a=None, scale_b=None, mx_a=None, mx_b=None,
              bias=None, lda=0, ldb=0, ldc=0, family=_capi.KERNEL_AUTO, wg_tile=(0, 0),
-             operand_path="lds", variant=0):
+             operand_path="lds", variant=0, mx_a_layout="rows"):
     """Upload, launch once through astergemm_run, download.  Returns the raw
     output storage [M, ldc or N] and the kernel name."""
     plan = AG.GemmPlan.create(M, N, K, dtype_ab, dtype_c, has_bias=bias is not None, lda=lda,
                               ldb=ldb, ldc=ldc, family=family, wg_tile=wg_tile,
-                              operand_path=operand_path, variant=variant)
+                              operand_path=operand_path, variant=variant, mx_a_layout=mx_a_layout)
     ldc_eff = ldc or N
     out = np.full((M, ldc_eff), 0x7FC1 if dtype_c != "f32" else np.nan, dtype=_OUT_NP[dtype_c])
     bufs = []
@@ -921,17 +921,22 @@ def test_every_tile_variant(gpu, vid, name, dtype_ab, dtype_c):
     a, b, ex = operands(M, N, K, dtype_ab, seed=11, a_std=1.0, b_std=1.0 if dtype_ab != "bf16" else 0.05)
     bias = np.random.default_rng(12).standard_normal(N).astype(np.float32)
     path, b_dev, ex_dev = "lds", b, ex
+    mxl = "rows"
     if name.startswith("streamdb_mxfp4"):  # payload in step order, scale plane in lane order
-        from aster_amd.kittens_helpers import shuffle_scales_e8m0_lanes, shuffle_weight_bytes
+        from aster_amd.kittens_helpers import (shuffle_scales_e8m0_lanes, shuffle_scales_e8m0_lanes128,
+                                               shuffle_weight_bytes)
         path, b_dev = "direct_b_k8", shuffle_weight_bytes(b)
         ex_dev = dict(ex, mx_b=shuffle_scales_e8m0_lanes(ex["mx_b"]))
+        if "_sal_" in name:    # and A's plane in lane order as well
+            mxl, ex_dev["mx_a"] = "lanes128", shuffle_scales_e8m0_lanes128(ex["mx_a"])
     elif name.startswith("streamdb_fp8"):  # byte rows in step order
         from aster_amd.kittens_helpers import shuffle_weight_bytes
         path, b_dev = "direct_b_k8", shuffle_weight_bytes(b)
     elif name.startswith("streamdb"):  # B pre-shuffled in K8 order
         from aster_amd.kittens_helpers import shuffle_weight_k8
         path, b_dev = "direct_b_k8", shuffle_weight_k8(np.ascontiguousarray(b).view(np.uint16))
-    plan = AG.GemmPlan.create(M, N, K, dtype_ab, dtype_c, has_bias=True, variant=vid, operand_path=path)
+    plan = AG.GemmPlan.create(M, N, K, dtype_ab, dtype_c, has_bias=True, variant=vid, operand_path=path,
+                              mx_a_layout=mxl)
     assert plan.info.name.decode() == name
     out = np.zeros((M, N), dtype=_OUT_NP[dtype_c])
     bufs = {}
@@ -1240,6 +1245,69 @@ def test_mxfp4_stream_direct_b(gpu, M, N, K, dtype_c):
                                  family=_capi.KERNEL_TILE)
     if lds_name.startswith("stream_mxfp4"):   # the same products in the same order
         assert np.array_equal(out.view(np.uint8), lds_out.view(np.uint8))
+    # A's e8m0 plane in lane order (groups of 128 rows, padded): one 16-byte load per wave and
+    # K-step instead of the pass through LDS; the same bits
+    from aster_amd.kittens_helpers import shuffle_scales_e8m0_lanes128
+    sal, sal_name = run_gemm(a, shuffle_weight_bytes(b), M, N, K, "mxfp4", dtype_c, bias=bias,
+                             mx_a=shuffle_scales_e8m0_lanes128(mxa), mx_b=shuffle_scales_e8m0_lanes(mxb),
+                             operand_path="direct_b_k8", mx_a_layout="lanes128")
+    assert sal_name == f"streamdb_mxfp4_128x256_w1x4_sal_{dtype_c}"
+    assert np.array_equal(sal.view(np.uint8), out.view(np.uint8))
+
+
+def test_mxfp4_lane_order_activation_scales_are_refused_where_no_kernel_reads_them(gpu):
+    with pytest.raises(_capi.AsterGemmError):      # row-major weights: the LDS kernels read rows
+        AG.GemmPlan.create(512, 512, 4096, "mxfp4", "bf16", mx_a_layout="lanes128")
+    with pytest.raises(_capi.AsterGemmError):      # not an MXFP4 problem
+        AG.GemmPlan.create(512, 512, 4096, "bf16", "bf16", mx_a_layout="lanes128")
+    p = AG.GemmPlan.create(512, 512, 4096, "mxfp4", "bf16", operand_path="direct_b_k8", mx_a_layout="lanes128")
+    assert p.info.name.decode() == "streamdb_mxfp4_128x256_w1x4_sal_bf16"
+
+
+def test_mxfp4_quantise_into_lane_order_then_gemm_full_size(gpu):
+    """Configuration 5 at the size the bench times with everything made on the device: activations
+    quantised straight into (payload, lane-order plane), weights quantised and pre-shuffled, GEMM
+    through the lane-order kernel.  The plane equals the host shuffle of the row-major plane, and
+    the product equals the row-major path's bit for bit and the oracle's on sampled rows."""
+    from aster_amd.kittens_helpers import mx_lanes128_bytes, shuffle_scales_e8m0_lanes128
+    from aster_amd.quantize import preshuffle_device, preshuffle_scales_a_device, quantize_mxfp4_device
+    M, N, K = 4096, 14336, 4096
+    rng = np.random.default_rng(5)
+    xa = rng.standard_normal((M, K)).astype(np.float32)
+    xb = rng.standard_normal((N, K)).astype(np.float32)
+    a, mxa = F.quantize_mxfp4(xa)
+    b, mxb = F.quantize_mxfp4(xb)
+    bufs = {k: GpuBuffer(n) for k, n in dict(xa=xa.nbytes, xb=xb.nbytes, a=M * K // 2, b=N * K // 2,
+                                             bs=N * K // 2, sa=mx_lanes128_bytes(M, K), sa2=mx_lanes128_bytes(M, K),
+                                             sar=M * K // 32, sb=N * K // 32, sbs=N * K // 32, c=M * N * 2).items()}
+    bufs["xa"].copy_from_host(xa)
+    bufs["xb"].copy_from_host(xb)
+    quantize_mxfp4_device(bufs["xa"].ptr_value, M, K, bufs["a"].ptr_value, bufs["sa"].ptr_value,
+                          scales_layout="lanes128")
+    quantize_mxfp4_device(bufs["xa"].ptr_value, M, K, bufs["a"].ptr_value, bufs["sar"].ptr_value)
+    preshuffle_scales_a_device(bufs["sar"].ptr_value, bufs["sa2"].ptr_value, M, K)
+    quantize_mxfp4_device(bufs["xb"].ptr_value, N, K, bufs["b"].ptr_value, bufs["sb"].ptr_value)
+    preshuffle_device(bufs["b"].ptr_value, bufs["bs"].ptr_value, N, K, "mxfp4", "direct_b_k8",
+                      d_mx_src=bufs["sb"].ptr_value, d_mx_dst=bufs["sbs"].ptr_value)
+    got_sa, got_sa2 = np.empty(mx_lanes128_bytes(M, K), np.uint8), np.empty(mx_lanes128_bytes(M, K), np.uint8)
+    bufs["sa"].copy_to_host(got_sa)
+    bufs["sa2"].copy_to_host(got_sa2)
+    assert np.array_equal(got_sa, shuffle_scales_e8m0_lanes128(mxa))
+    assert np.array_equal(got_sa2, got_sa)
+    out = np.zeros((M, N), np.uint16)
+    plan = AG.GemmPlan.create(M, N, K, "mxfp4", "bf16", operand_path="direct_b_k8", mx_a_layout="lanes128")
+    assert plan.info.name.decode() == "streamdb_mxfp4_128x256_w1x4_sal_bf16"
+    print("launch", plan.info.name.decode(), flush=True)
+    plan.run(bufs["a"].ptr_value, bufs["bs"].ptr_value, bufs["c"].ptr_value, mx_a=bufs["sa"].ptr_value,
+             mx_b=bufs["sbs"].ptr_value)
+    bufs["c"].copy_to_host(out)
+    for bf in bufs.values():
+        bf.free()
+    rows, cols = _sampled_rows_and_cols(M, N)
+    check(out[rows], G.gemm_mxfp4(a[rows], mxa[rows], b, mxb, out_dtype=G.BF16), "bf16", N)
+    check(out[:, cols], G.gemm_mxfp4(a, mxa, b[cols], mxb[cols], out_dtype=G.BF16), "bf16", len(cols))
+    plain, _ = run_gemm(a, b, M, N, K, "mxfp4", "bf16", mx_a=mxa, mx_b=mxb)
+    assert np.array_equal(out, plain)
 
 
 def test_mxfp4_stream_direct_b_full_size_row_sample(gpu):

@@ -305,3 +305,32 @@ def test_shuffle_scales_e8m0_lanes_is_what_a_lane_of_the_stream_kernel_loads():
     assert lib.astergemm_shuffle_scales_e8m0_lanes(mx.ctypes.data, out.ctypes.data, N, K + 32) != 0
     with pytest.raises(AssertionError):
         shuffle_scales_e8m0_lanes(mx[:48])
+
+
+def test_shuffle_scales_e8m0_lanes128_is_what_a_lane_of_the_stream_kernel_loads():
+    # activations: groups of 128 rows (padded with the byte 127), per group and step one KiB in
+    # which lane L = 16 q + i finds at byte 16 L + 2 t + h the scale of block 4 h + q of row
+    # 128 g + 16 t + i (gemm_stream4db_kernel.hpp, A scales in lane order)
+    from aster_amd import _capi
+    from aster_amd.kittens_helpers import (mx_lanes128_bytes, shuffle_scales_e8m0_lanes128,
+                                           unshuffle_scales_e8m0_lanes128)
+    M, K = 328, 1024           # two whole groups and 72 rows of a third
+    rng = np.random.default_rng(3)
+    mx = rng.integers(0, 255, (M, K // 32), dtype=np.uint8)
+    sh = shuffle_scales_e8m0_lanes128(mx)
+    assert sh.shape == (mx_lanes128_bytes(M, K),) and mx_lanes128_bytes(M, K) == 3 * 4 * 1024
+    steps = K // 256
+    for g, s_, L, t, h in [(0, 0, 0, 0, 0), (1, 2, 37, 5, 1), (2, 3, 63, 7, 1), (2, 1, 8, 4, 0), (2, 0, 9, 4, 0)]:
+        q, i = L // 16, L % 16
+        row = 128 * g + 16 * t + i
+        want = mx[row, 8 * s_ + 4 * h + q] if row < M else 127
+        assert sh[(g * steps + s_) * 1024 + 16 * L + 2 * t + h] == want
+    assert np.array_equal(unshuffle_scales_e8m0_lanes128(sh, M, K), mx)
+    lib = _capi.load()
+    out = np.zeros_like(sh)
+    assert lib.astergemm_mx_lanes128_bytes(M, K) == sh.size
+    _capi.check(lib.astergemm_shuffle_scales_e8m0_lanes128(mx.ctypes.data, out.ctypes.data, M, K))
+    assert np.array_equal(out, sh)
+    assert lib.astergemm_shuffle_scales_e8m0_lanes128(mx.ctypes.data, out.ctypes.data, M, K + 32) != 0
+    with pytest.raises(AssertionError):
+        shuffle_scales_e8m0_lanes128(mx[:, :-1])
