@@ -24,8 +24,17 @@ LIB_DIR = os.path.join(PKG_DIR, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libastergemm.so")
 OBJ_DIR = os.path.join(ROOT, "build", "obj")
 
-SOURCES = ["gemm_tile.hip", "gemm_stream.hip", "gemm_skinny.hip", "astergemm_api.hip", "quantize.hip",
-           "weight_artifact.hip", "diag_mfma_rate.hip"]
+# (object stem, source file, extra flags).  gemm_stream.hip holds the variant table of the stream
+# kernels in three parts (16-bit, fp8, MXFP4 operands) and is compiled once per part.
+UNITS = [("gemm_stream_p2", "gemm_stream.hip", ["-DAG_STREAM_PART=2"]),
+         ("gemm_stream_p0", "gemm_stream.hip", ["-DAG_STREAM_PART=0"]),
+         ("gemm_stream_p1", "gemm_stream.hip", ["-DAG_STREAM_PART=1"]),
+         ("gemm_skinny", "gemm_skinny.hip", []),
+         ("gemm_tile", "gemm_tile.hip", []),
+         ("astergemm_api", "astergemm_api.hip", []),
+         ("quantize", "quantize.hip", []),
+         ("weight_artifact", "weight_artifact.hip", []),
+         ("diag_mfma_rate", "diag_mfma_rate.hip", [])]
 HSACO_SOURCE = "hsaco_kernels.hip"
 HSACO_PATH = os.path.join(LIB_DIR, "astergemm_kernels.hsaco")
 REPLAY_PATH = os.path.join(LIB_DIR, "astergemm_replay")
@@ -46,16 +55,20 @@ COMMON_FLAGS = [
 ]
 
 
-def _compile(src: str) -> str:
-    """Compile one source; the device assembly is kept beside the object and checked for the
+def _compile(unit) -> str:
+    """Compile one unit; the device assembly is kept beside the object and checked for the
     hazard `scan_mfma_hazards` describes."""
-    stem = os.path.splitext(src)[0]
-    obj = os.path.join(OBJ_DIR, stem + ".o")
-    cmd = [HIPCC, *COMMON_FLAGS, "-save-temps=obj", "-c", os.path.join(CSRC, src), "-o", obj]
+    stem, src, extra = unit
+    # a directory per unit: the intermediates kept by -save-temps are named after the source file
+    udir = os.path.join(OBJ_DIR, stem)
+    os.makedirs(udir, exist_ok=True)
+    obj = os.path.join(udir, stem + ".o")
+    cmd = [HIPCC, *COMMON_FLAGS, *extra, "-save-temps=obj", "-c", os.path.join(CSRC, src), "-o", obj]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError(f"hipcc failed on {src}:\n{proc.stdout}\n{proc.stderr}")
-    asm = os.path.join(OBJ_DIR, stem + "-hip-amdgcn-amd-amdhsa-gfx950.s")
+    sstem = os.path.splitext(src)[0]
+    asm = os.path.join(udir, sstem + "-hip-amdgcn-amd-amdhsa-gfx950.s")
     if not os.path.exists(asm):
         raise RuntimeError(f"hipcc left no device assembly for {src} (expected {asm})")
     with open(asm) as f:
@@ -66,9 +79,9 @@ def _compile(src: str) -> str:
         raise RuntimeError(f"{src}: register spills (scratch, accumulation registers or the metadata's "
                            f"spill counts) in kernels whose register loads are inline assembly "
                            f"(the compiler does not wait for those loads): {spilled}")
-    for name in os.listdir(OBJ_DIR):  # the other intermediates are large and of no use
-        if name.startswith(stem + "-") and name.endswith((".hipi", ".bc", ".out", ".resolution.txt")):
-            os.remove(os.path.join(OBJ_DIR, name))
+    for name in os.listdir(udir):  # the other intermediates are large and of no use
+        if name.startswith(sstem + "-") and name.endswith((".hipi", ".bc", ".out", ".resolution.txt")):
+            os.remove(os.path.join(udir, name))
     if found:
         lines = "\n".join(f"  {asm}:{no}: {mfma}\n      written at line {wno}: {writer}"
                           for (no, mfma, wno, writer) in found[:20])
@@ -88,15 +101,24 @@ def _genco(src: str) -> str:
     return HSACO_PATH
 
 
-def build_library(verbose: bool = False) -> str:
+def build_library(verbose: bool = False, only=None) -> str:
     """Compile every HIP source, link libastergemm.so and build the code object
-    astergemm_kernels.hsaco; returns the library path."""
+    astergemm_kernels.hsaco; returns the library path.  `only` (a list of unit names, for work
+    on one kernel file) recompiles just those and links them with the objects already there."""
     os.makedirs(OBJ_DIR, exist_ok=True)
     os.makedirs(LIB_DIR, exist_ok=True)
-    with ThreadPoolExecutor(max_workers=4) as pool:
-        hsaco = pool.submit(_genco, HSACO_SOURCE)
-        objs = list(pool.map(_compile, SOURCES))
-        hsaco.result()
+    with ThreadPoolExecutor(max_workers=6) as pool:
+        if only:
+            todo = [u for u in UNITS if u[0] in only]
+            list(pool.map(_compile, todo))
+            objs = [os.path.join(OBJ_DIR, u[0], u[0] + ".o") for u in UNITS]
+            missing = [o for o in objs if not os.path.exists(o)]
+            if missing:
+                raise RuntimeError(f"objects missing for a partial build: {missing}")
+        else:
+            hsaco = pool.submit(_genco, HSACO_SOURCE)
+            objs = list(pool.map(_compile, UNITS))
+            hsaco.result()
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC",
            "-Wno-unused-command-line-argument", *objs, "-o", LIB_PATH]
     proc = subprocess.run(cmd, capture_output=True, text=True)
@@ -115,5 +137,5 @@ def build_library(verbose: bool = False) -> str:
 
 
 if __name__ == "__main__":
-    build_library(verbose=True)
+    build_library(verbose=True, only=sys.argv[1:] or None)
     sys.exit(0)

@@ -1,11 +1,14 @@
 // Stream kernels (whole-ring, hand-scheduled MFMA loops) for f16 / bf16, fp8 and MXFP4:
 // launchers, shape checks and the variant table.  Kept apart from gemm_tile.hip so that the
 // two halves of the kernel set compile side by side.
+#include <vector>
+
 #include "gemm_stream_kernel.hpp"
 #include "gemm_stream8_kernel.hpp"
 #include "gemm_stream4_kernel.hpp"
 #include "gemm_streamdb_kernel.hpp"
 #include "gemm_stream4db_kernel.hpp"
+#include "gemm_stream4dbl_kernel.hpp"
 #include "gemm_stream8db_kernel.hpp"
 
 namespace astergemm {
@@ -86,8 +89,11 @@ const char* check_streamdb(const astergemm_config& c) {
 // straight into MFMA operands: 128 x 256 tiles, four waves (gemm_stream4db_kernel.hpp) ---------
 template <int DT, int OUT, bool SAL>
 int launch_stream4db(const GemmArgs& a, int grid, hipStream_t s) {
-  constexpr int lds = 4 * 128 * kRowBytes + 2 * 128 * 16;
-  auto k = gemm_stream4db_kernel<DT, OUT, SAL>;
+  // SAL: A's e8m0 plane in lane order as well (gemm_stream4dbl_kernel.hpp), nothing but A in LDS
+  constexpr int lds = 4 * 128 * kRowBytes + (SAL ? 0 : 2 * 128 * 16);
+  void (*k)(const GemmArgs);
+  if constexpr (SAL) k = gemm_stream4dbl_kernel<DT, OUT>;
+  else k = gemm_stream4db_kernel<DT, OUT>;
   static std::atomic<uint64_t> attr_devs{0};
   if (int e = lds_attr_once(attr_devs, (const void*)k, lds)) return e;
   // what the kernel's indexing assumes: whole 64-row groups of B, an even number of whole
@@ -113,8 +119,9 @@ const char* check_stream4db(const astergemm_config& c) {
 #define AG_STREAM4DB(name, DT, OUT, SAL)                                         \
   Variant {                                                                      \
     name, ASTERGEMM_KERNEL_TILE, DT, OUT, 128, 256, kRowBytes, 1, 4, 4, 2,       \
-        4 * 128 * kRowBytes + 2 * 128 * 16,                                      \
-        (const void*)gemm_stream4db_kernel<DT, OUT, SAL>,                        \
+        4 * 128 * kRowBytes + (SAL ? 0 : 2 * 128 * 16),                          \
+        SAL ? (const void*)gemm_stream4dbl_kernel<DT, OUT>                       \
+            : (const void*)gemm_stream4db_kernel<DT, OUT>,                       \
         launch_stream4db<DT, OUT, SAL>, check_stream4db,                         \
         ASTERGEMM_OPERAND_DIRECT_B_K8, nullptr, nullptr,                         \
         SAL ? ASTERGEMM_MX_LANES128 : ASTERGEMM_MX_ROWS                          \
@@ -534,14 +541,17 @@ int grid_stream_tail(const astergemm_config& c, int cus) {
       AG_STREAM(prefix "_128x128_w2x2_f32", DT, ASTERGEMM_F32, 128, 128, 2, 2),          \
       AG_STREAM(prefix "_128x128_w2x2_f16", DT, ASTERGEMM_F16, 128, 128, 2, 2)
 
+// The table is compiled in three parts (this file once per AG_STREAM_PART: 16-bit, fp8 and MXFP4
+// operands), so that the parts build side by side and work on one family recompiles one part.
+#ifndef AG_STREAM_PART
+#error "compile with -DAG_STREAM_PART=0, 1 or 2"
+#endif
+
 const Variant kStreamVariants[] = {
+#if AG_STREAM_PART == 0
     AG_STREAM_SET("stream_bf16", ASTERGEMM_BF16),
     AG_STREAM_SPLITK_SET("splitk_bf16", 0, ASTERGEMM_BF16, 5 * 128 * kRowBytes, gemm_stream_splitk_kernel),
     AG_STREAM_SPLITK_SET("splitk_f16", 0, ASTERGEMM_F16, 5 * 128 * kRowBytes, gemm_stream_splitk_kernel),
-    AG_STREAM_SPLITK_SET("splitk_fp8", 1, ASTERGEMM_FP8_E4M3, 5 * 128 * kRowBytes,
-                         gemm_stream8_splitk_kernel),
-    AG_STREAM_SPLITK_SET("splitk_mxfp4", 2, ASTERGEMM_MXFP4, 4 * 128 * kRowBytes + 4 * 128 * 16,
-                         gemm_stream4_splitk_kernel),
     AG_STREAM_SET("stream_f16", ASTERGEMM_F16),
     AG_STREAMDB("streamdb_bf16_256x256_w2x4_bf16", ASTERGEMM_BF16, ASTERGEMM_BF16, 5, 5, 2, 2),
     AG_STREAMDB("streamdb_bf16_256x256_w2x4_f32", ASTERGEMM_BF16, ASTERGEMM_F32, 5, 5, 2, 2),
@@ -559,10 +569,11 @@ const Variant kStreamVariants[] = {
                        gemm_stream_kernel),
     AG_STREAM_TAIL_SET("stream_f16_256x256_w2x4_tail128", 0, ASTERGEMM_F16, 2, 4, 5 * 256 * kRowBytes,
                        gemm_stream_kernel),
+#elif AG_STREAM_PART == 1
+    AG_STREAM_SPLITK_SET("splitk_fp8", 1, ASTERGEMM_FP8_E4M3, 5 * 128 * kRowBytes,
+                         gemm_stream8_splitk_kernel),
     AG_STREAM_TAIL_SET("stream_fp8_256x256_w2x4_tail128", 1, ASTERGEMM_FP8_E4M3, 2, 4,
                        5 * 256 * kRowBytes, gemm_stream8_kernel),
-    AG_STREAM_TAIL_SET("stream_mxfp4_256x256_w2x4_tail128", 2, ASTERGEMM_MXFP4, 2, 4,
-                       4 * 256 * kRowBytes + 4 * 256 * 16, gemm_stream4_kernel),
     AG_STREAM8("stream_fp8_256x256_w2x4_bf16", ASTERGEMM_FP8_E4M3, ASTERGEMM_BF16),
     AG_STREAM8("stream_fp8_256x256_w2x4_f32", ASTERGEMM_FP8_E4M3, ASTERGEMM_F32),
     AG_STREAM8("stream_fp8_256x256_w2x4_f16", ASTERGEMM_FP8_E4M3, ASTERGEMM_F16),
@@ -572,6 +583,14 @@ const Variant kStreamVariants[] = {
     AG_STREAM8_128("stream_fp8_128x128_w2x2_bf16", ASTERGEMM_FP8_E4M3, ASTERGEMM_BF16),
     AG_STREAM8_128("stream_fp8_128x128_w2x2_f32", ASTERGEMM_FP8_E4M3, ASTERGEMM_F32),
     AG_STREAM8_128("stream_fp8_128x128_w2x2_f16", ASTERGEMM_FP8_E4M3, ASTERGEMM_F16),
+    AG_STREAM8DB("streamdb_fp8_128x256_w1x4_bf16", ASTERGEMM_FP8_E4M3, ASTERGEMM_BF16),
+    AG_STREAM8DB("streamdb_fp8_128x256_w1x4_f32", ASTERGEMM_FP8_E4M3, ASTERGEMM_F32),
+    AG_STREAM8DB("streamdb_fp8_128x256_w1x4_f16", ASTERGEMM_FP8_E4M3, ASTERGEMM_F16),
+#else
+    AG_STREAM_SPLITK_SET("splitk_mxfp4", 2, ASTERGEMM_MXFP4, 4 * 128 * kRowBytes + 4 * 128 * 16,
+                         gemm_stream4_splitk_kernel),
+    AG_STREAM_TAIL_SET("stream_mxfp4_256x256_w2x4_tail128", 2, ASTERGEMM_MXFP4, 2, 4,
+                       4 * 256 * kRowBytes + 4 * 256 * 16, gemm_stream4_kernel),
     AG_STREAM4("stream_mxfp4_256x256_w2x2_bf16", ASTERGEMM_MXFP4, ASTERGEMM_BF16),
     AG_STREAM4("stream_mxfp4_256x256_w2x2_f32", ASTERGEMM_MXFP4, ASTERGEMM_F32),
     AG_STREAM4("stream_mxfp4_256x256_w2x2_f16", ASTERGEMM_MXFP4, ASTERGEMM_F16),
@@ -584,9 +603,6 @@ const Variant kStreamVariants[] = {
     AG_STREAM4DB("streamdb_mxfp4_128x256_w1x4_bf16", ASTERGEMM_MXFP4, ASTERGEMM_BF16, false),
     AG_STREAM4DB("streamdb_mxfp4_128x256_w1x4_f32", ASTERGEMM_MXFP4, ASTERGEMM_F32, false),
     AG_STREAM4DB("streamdb_mxfp4_128x256_w1x4_f16", ASTERGEMM_MXFP4, ASTERGEMM_F16, false),
-    AG_STREAM8DB("streamdb_fp8_128x256_w1x4_bf16", ASTERGEMM_FP8_E4M3, ASTERGEMM_BF16),
-    AG_STREAM8DB("streamdb_fp8_128x256_w1x4_f32", ASTERGEMM_FP8_E4M3, ASTERGEMM_F32),
-    AG_STREAM8DB("streamdb_fp8_128x256_w1x4_f16", ASTERGEMM_FP8_E4M3, ASTERGEMM_F16),
     AG_STREAM4_128("stream_mxfp4_128x128_w2x2_bf16", ASTERGEMM_MXFP4, ASTERGEMM_BF16),
     AG_STREAM4_128("stream_mxfp4_128x128_w2x2_f32", ASTERGEMM_MXFP4, ASTERGEMM_F32),
     AG_STREAM4_128("stream_mxfp4_128x128_w2x2_f16", ASTERGEMM_MXFP4, ASTERGEMM_F16),
@@ -594,11 +610,39 @@ const Variant kStreamVariants[] = {
     AG_STREAM4DB("streamdb_mxfp4_128x256_w1x4_sal_bf16", ASTERGEMM_MXFP4, ASTERGEMM_BF16, true),
     AG_STREAM4DB("streamdb_mxfp4_128x256_w1x4_sal_f32", ASTERGEMM_MXFP4, ASTERGEMM_F32, true),
     AG_STREAM4DB("streamdb_mxfp4_128x256_w1x4_sal_f16", ASTERGEMM_MXFP4, ASTERGEMM_F16, true),
+#endif
 };
 
 }  // namespace
 
-int num_stream_variants() { return (int)(sizeof(kStreamVariants) / sizeof(kStreamVariants[0])); }
-const Variant* stream_variants() { return kStreamVariants; }
+#define AG_CAT_(a, b) a##b
+#define AG_CAT(a, b) AG_CAT_(a, b)
+const Variant* AG_CAT(stream_variants_part, AG_STREAM_PART)(int* count) {
+  *count = (int)(sizeof(kStreamVariants) / sizeof(kStreamVariants[0]));
+  return kStreamVariants;
+}
+
+#if AG_STREAM_PART == 0
+const Variant* stream_variants_part1(int* count);
+const Variant* stream_variants_part2(int* count);
+
+// the three parts as one table, in part order
+static const std::vector<Variant>& all_stream_variants() {
+  static const std::vector<Variant> all = [] {
+    std::vector<Variant> v;
+    int n = 0;
+    const Variant* p = stream_variants_part0(&n);
+    v.insert(v.end(), p, p + n);
+    p = stream_variants_part1(&n);
+    v.insert(v.end(), p, p + n);
+    p = stream_variants_part2(&n);
+    v.insert(v.end(), p, p + n);
+    return v;
+  }();
+  return all;
+}
+int num_stream_variants() { return (int)all_stream_variants().size(); }
+const Variant* stream_variants() { return all_stream_variants().data(); }
+#endif
 
 }  // namespace astergemm

@@ -26,12 +26,6 @@
 // (waves 2 and 3 repeat what waves 0 and 1 do, which keeps the loop free of branches), so that
 // only the A tile transfers are counted by hand.
 //
-// SAL (A scales in lane order, astergemm_shuffle_scales_e8m0_lanes128): the caller hands over A's
-// plane in 1 KiB chunks, chunk (g * steps + s) for rows 128 g .. 128 g + 127 and step s holding at
-// byte 16 L + 2 t + h of lane L = 16 q + i the scale of block 4 h + q of row 128 g + 16 t + i.
-// One 16-byte load per wave and K-step then brings the scales of the wave's eight A tiles, two
-// K-steps ahead like B's, and nothing of the scales passes through LDS.
-//
 // MFMA order is m-outer per half K-step: m-step T = 8 u + m multiplies A fragment (m, u), read
 // from LDS three m-steps ahead into a ring of four, with the four B fragments of half u.
 // One barrier per K-step, three m-steps before its end: it certifies A(k+1) and, all reads of
@@ -42,7 +36,7 @@
 namespace astergemm {
 namespace {
 
-template <int DT, int OUT, bool SAL>
+template <int DT, int OUT>
 __device__ __forceinline__ void gemm_stream4db_body(const GemmArgs& p, int bid) {
   constexpr int BM = 128, BN = 256, WM = 1, WN = 4;
   constexpr int NW = WM * WN;
@@ -93,7 +87,7 @@ __device__ __forceinline__ void gemm_stream4db_body(const GemmArgs& p, int bid) 
   // row 64 (w & 1) + L, re-packed into pairs {b[8h+q], b[8h+4+q]} (h = K-step parity) -------------
   int sc_row = row0 + (wave & 1) * 64 + lane;
   sc_row = sc_row < p.M ? sc_row : p.M - 1;  // rows past the end of an edge tile re-read the last
-  const uint8_t* sc_src = p.mx_a + (SAL ? 0 : (int64_t)sc_row * p.mx_ld);
+  const uint8_t* sc_src = p.mx_a + (int64_t)sc_row * p.mx_ld;
   uint8_t* sc_dst = lds + SC_A + ((wave & 1) * 64 + lane) * 8;
   i32x4 sc_raw = {0, 0, 0, 0};
   auto load_scales = [&](int c) { sc_raw = *(const i32x4*)(sc_src + c * 16); };
@@ -134,11 +128,6 @@ __device__ __forceinline__ void gemm_stream4db_body(const GemmArgs& p, int bid) 
   const unsigned b_lane = (unsigned)lane * 16, s_lane = (unsigned)lane * 8;
   i32x4 fb[NBUF][TN];
   int sbk[NBUF][2];  // scales of K-step k in sbk[k mod 4]
-  // SAL: A's plane holds whole 128-row groups (padded past M), group tile_m is this tile's
-  const __amdgpu_buffer_rsrc_t sa_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)p.mx_a, 0, SAL ? (int)((unsigned)p.tiles_m * (unsigned)nk * 1024u) : 0, 0x00020000);
-  const unsigned sa_tile = __builtin_amdgcn_readfirstlane((unsigned)tile_m * (unsigned)nk * 1024u);
-  int sak[NBUF][4];  // SAL: A scales of K-step k in sak[k mod 4], tiles 2 d, 2 d + 1 in dword d
   typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
   typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
   auto load_b1 = [&](int j, auto buf, int n) {  // substep j = 2 k + u
@@ -146,15 +135,6 @@ __device__ __forceinline__ void gemm_stream4db_body(const GemmArgs& p, int bid) 
     const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, (int)b_lane,
                                                           (int)(b_tile[n] + (unsigned)j * 1024u), 0);
     fb[BI][n] = __builtin_bit_cast(i32x4, v);
-  };
-  auto load_sa = [&](int k, auto buf) {
-    constexpr int KB = decltype(buf)::value;
-    const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(sa_rsrc, (int)b_lane,
-                                                          (int)(sa_tile + (unsigned)k * 1024u), 0);
-    sak[KB][0] = (int)v.x;
-    sak[KB][1] = (int)v.y;
-    sak[KB][2] = (int)v.z;
-    sak[KB][3] = (int)v.w;
   };
   auto load_sb = [&](int k, auto buf) {
     constexpr int KB = decltype(buf)::value;
@@ -185,7 +165,7 @@ __device__ __forceinline__ void gemm_stream4db_body(const GemmArgs& p, int bid) 
     constexpr int T = decltype(tt)::value;
     constexpr int OFF = KS * SLOT + (T % TM) * 16 * kRowBytes;
     fa[T % RA] = *(lvec_t)(size_t)(rd_addr[T / TM] + (unsigned)OFF);
-    if constexpr (T < TM && !SAL) {
+    if constexpr (T < TM) {
       constexpr int SOFF = ((KS >> 1) & 1) * BM * 16 + (KS & 1) * BM * 8 + T * 16 * 8;
       sa[T] = *(lu16_t)(size_t)(sc_addr + (unsigned)SOFF);
     }
@@ -210,16 +190,11 @@ __device__ __forceinline__ void gemm_stream4db_body(const GemmArgs& p, int bid) 
   });
   load_sb(0, std::integral_constant<int, 0>{});
   load_sb(1, std::integral_constant<int, 1>{});
-  if constexpr (SAL) {
-    load_sa(0, std::integral_constant<int, 0>{});
-    load_sa(1, std::integral_constant<int, 1>{});
-  } else {
-    load_scales(0);
-    store_scales(0);
-    if (nk > 2) {
-      load_scales(1);
-      store_scales(1);
-    }
+  load_scales(0);
+  store_scales(0);
+  if (nk > 2) {
+    load_scales(1);
+    store_scales(1);
   }
   asm volatile("" ::: "memory");
 #pragma unroll
@@ -270,24 +245,14 @@ __device__ __forceinline__ void gemm_stream4db_body(const GemmArgs& p, int bid) 
         constexpr int n = decltype(nc)::value;
         // scale bytes: A pair {q, 4+q} in bytes 0, 1 of sa[m] -> byte U; B pairs of tiles
         // 2 d, 2 d + 1 in the four bytes of sbk[KM][d] -> byte 2 (n & 1) + U
-        // SAL: A pairs of tiles 2 d, 2 d + 1 in the four bytes of sak[KM][d] -> byte 2 (m & 1) + U
 #define AG_MFMA4DB(SEL)                                                                     \
   asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 " SEL " cbsz:4 blgp:4" \
                : "+a"(acc[m][n])                                                            \
-               : "v"(fb[BI][n]), "v"(fa[T % RA]), "v"(sbk[KM][n >> 1]),                     \
-                 "v"(SAL ? sak[KM][m >> 1] : sa[m]))
-        constexpr bool AH = SAL && (m & 1) != 0;  // high half of the A scale register
-        if constexpr (!AH) {
-          if constexpr (U == 0 && (n & 1) == 0) AG_MFMA4DB("op_sel:[0,0,0] op_sel_hi:[0,0,0]");
-          else if constexpr (U == 0) AG_MFMA4DB("op_sel:[0,0,0] op_sel_hi:[1,0,0]");
-          else if constexpr ((n & 1) == 0) AG_MFMA4DB("op_sel:[1,1,0] op_sel_hi:[0,0,0]");
-          else AG_MFMA4DB("op_sel:[1,1,0] op_sel_hi:[1,0,0]");
-        } else {
-          if constexpr (U == 0 && (n & 1) == 0) AG_MFMA4DB("op_sel:[0,0,0] op_sel_hi:[0,1,0]");
-          else if constexpr (U == 0) AG_MFMA4DB("op_sel:[0,0,0] op_sel_hi:[1,1,0]");
-          else if constexpr ((n & 1) == 0) AG_MFMA4DB("op_sel:[1,1,0] op_sel_hi:[0,1,0]");
-          else AG_MFMA4DB("op_sel:[1,1,0] op_sel_hi:[1,1,0]");
-        }
+               : "v"(fb[BI][n]), "v"(fa[T % RA]), "v"(sbk[KM][n >> 1]), "v"(sa[m]))
+        if constexpr (U == 0 && (n & 1) == 0) AG_MFMA4DB("op_sel:[0,0,0] op_sel_hi:[0,0,0]");
+        else if constexpr (U == 0) AG_MFMA4DB("op_sel:[0,0,0] op_sel_hi:[1,0,0]");
+        else if constexpr ((n & 1) == 0) AG_MFMA4DB("op_sel:[1,1,0] op_sel_hi:[0,0,0]");
+        else AG_MFMA4DB("op_sel:[1,1,0] op_sel_hi:[1,0,0]");
 #undef AG_MFMA4DB
         // ---- at most two side instructions behind an MFMA ---------------------------------------
         if constexpr (n == 0) {
@@ -308,12 +273,12 @@ __device__ __forceinline__ void gemm_stream4db_body(const GemmArgs& p, int bid) 
         // earlier because the compiler's wait for the fetched granule counts only the loads it
         // sees: one trip after the fetch it would also force the A transfers requested beside
         // it, two trips after it forces nothing that is not needed by then anyway.
-        if constexpr (!SAL && ODD && T == 4 && n == 2) {
+        if constexpr (ODD && T == 4 && n == 2) {
           if (STEADY || k + 1 < nk) {
             if (k > 1) store_scales((k + 1) >> 1);
           }
         }
-        if constexpr (!SAL && ODD && T == BAR + 1 && n == 2) {
+        if constexpr (ODD && T == BAR + 1 && n == 2) {
           if (do_sc) load_scales((k + 3) >> 1);
         }
         // last m-step of a half: tile n of this buffer is done with MFMA (m = 7, n).  The B
@@ -322,9 +287,6 @@ __device__ __forceinline__ void gemm_stream4db_body(const GemmArgs& p, int bid) 
         if constexpr (m == TM - 1) {
           if constexpr (U == 0 && n == 0) {
             if (do_b) load_sb(k + 2, std::integral_constant<int, (KM + 2) % NBUF>{});
-          }
-          if constexpr (SAL && U == 0 && n == 1) {
-            if (do_b) load_sa(k + 2, std::integral_constant<int, (KM + 2) % NBUF>{});
           }
           if (do_b) load_b1(2 * (k + 2) + U, BIc{}, n);
         }
@@ -339,14 +301,12 @@ __device__ __forceinline__ void gemm_stream4db_body(const GemmArgs& p, int bid) 
   // in trip k - 3, 13 in each of the two trips between, 5 of trip k; the A-scale loads of odd
   // trips are not counted.  Trips 0..2: A(k+1) was requested in the prologue, followed there by
   // A(k+2..3) and here by 13 loads per earlier trip and 5 of this one.
-  // SAL: one more load (A's scales) in the first half's batch of every trip, none on odd trips.
-  constexpr int TL = SAL ? 14 : 13, TB = SAL ? 6 : 5;
-  constexpr int VM_STEADY = 4 + 2 * TL + TB;
+  constexpr int VM_STEADY = 4 + 2 * 13 + 5;
   auto group = [&](int k0, auto first_c) {
     constexpr bool FIRST = decltype(first_c)::value;
     static_for<0, NSLOT>([&](auto ic) {
       constexpr int I = decltype(ic)::value;
-      constexpr int VM = (FIRST && I <= NSLOT - 2) ? (NSLOT - 2 - I) * LH + TL * I + TB : VM_STEADY;
+      constexpr int VM = (FIRST && I <= NSLOT - 2) ? (NSLOT - 2 - I) * LH + 13 * I + 5 : VM_STEADY;
       trip(k0 + I, ic, std::integral_constant<int, VM>{});
     });
   };
@@ -371,9 +331,9 @@ __device__ __forceinline__ void gemm_stream4db_body(const GemmArgs& p, int bid) 
   stream_epilogue<OUT, BM, BN, WM, WN>(p, acc, lds, wave, row0, col0);
 }
 
-template <int DT, int OUT, bool SAL = false>
+template <int DT, int OUT>
 __global__ __launch_bounds__(256, 2) void gemm_stream4db_kernel(const GemmArgs p) {
-  gemm_stream4db_body<DT, OUT, SAL>(p, blockIdx.x);
+  gemm_stream4db_body<DT, OUT>(p, blockIdx.x);
 }
 
 }  // namespace
