@@ -12,6 +12,12 @@
 //                    [--variant ID] [--flush BYTES] [--bias] [--json] [--calib BYTES]
 //                    [--direct-b | --direct-b-k8]   (B taken as pre-shuffled in the reference's order /
 //                                    in K8 order; timing only, the fill is random)
+//                    [--normal]      (operands as the benchmark makes them: N(0,1) sources, for
+//                                    bf16 / f16 times 0.02, for fp8 / MXFP4 quantised on the device
+//                                    and, with --direct-b-k8, pre-shuffled on the device: valid
+//                                    operands, so that counters describe what the benchmark times)
+//                    [--mx-a-lanes]  (MXFP4: A's e8m0 plane in lane order, mx_a_layout LANES128;
+//                                    needs --normal and --direct-b-k8)
 //   astergemm_replay --quantize fp8|mxfp4 --m ROWS --k K --iters 100
 //                    (operand quantiser on a ROWS x K fp32 source instead of a GEMM)
 //
@@ -84,6 +90,30 @@ static void fill(std::vector<uint8_t>& buf, int dtype, uint64_t seed) {
 }
 
 
+// N(0,1) * scale by Box-Muller over xorshift64 (synthetic data, not the benchmark's generator)
+static std::vector<float> normal(size_t n, uint64_t seed, float scale) {
+  std::vector<float> out(n);
+  uint64_t x = seed * 0x9E3779B97F4A7C15ull + 88172645463325252ull;
+  auto uni = [&]() {
+    x ^= x << 13;
+    x ^= x >> 7;
+    x ^= x << 17;
+    return ((double)(x >> 11) + 0.5) * (1.0 / 9007199254740992.0);  // (0, 1)
+  };
+  for (size_t i = 0; i < n; i += 2) {
+    const double r = sqrt(-2.0 * log(uni())), t = 6.283185307179586 * uni();
+    out[i] = (float)(r * cos(t)) * scale;
+    if (i + 1 < n) out[i + 1] = (float)(r * sin(t)) * scale;
+  }
+  return out;
+}
+
+static uint16_t bf16_rne(float f) {
+  uint32_t u;
+  memcpy(&u, &f, 4);
+  return (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
+}
+
 // --quantize: time astergemm_quantize_fp8_tensor / astergemm_quantize_mxfp4 on a rows x K
 // fp32 source, one event pair per call on the null stream.
 static int run_quantize(const char* kind, long long rows, long long K, int iters, int warmup) {
@@ -130,7 +160,7 @@ int main(int argc, char** argv) {
   cfg.M = cfg.N = cfg.K = 8192;
   cfg.dtype_ab = ASTERGEMM_BF16;
   cfg.dtype_c = ASTERGEMM_BF16;
-  int iters = 100, warmup = 20, json = 0;
+  int iters = 100, warmup = 20, json = 0, use_normal = 0;
   long long flush = 0, calib = 0;
   const char* quantize = nullptr;
   for (int i = 1; i < argc; ++i) {
@@ -156,6 +186,8 @@ int main(int argc, char** argv) {
     else if (a == "--direct-b") cfg.operand_path = ASTERGEMM_OPERAND_DIRECT_B;
     else if (a == "--direct-b-k8") cfg.operand_path = ASTERGEMM_OPERAND_DIRECT_B_K8;
     else if (a == "--bias") cfg.has_bias = 1;
+    else if (a == "--normal") use_normal = 1;
+    else if (a == "--mx-a-lanes") cfg.mx_a_layout = ASTERGEMM_MX_LANES128;
     else if (a == "--json") json = 1;
     else if (a == "--quantize") quantize = val();
     else if (a == "--family") {
@@ -169,6 +201,15 @@ int main(int argc, char** argv) {
   }
   if (cfg.dtype_ab == ASTERGEMM_FP8_E4M3) cfg.scale_mode = ASTERGEMM_SCALE_TENSOR;
   if (cfg.dtype_ab == ASTERGEMM_MXFP4) cfg.scale_mode = ASTERGEMM_SCALE_MX32;
+  if (cfg.mx_a_layout == ASTERGEMM_MX_LANES128 &&
+      (!use_normal || cfg.operand_path != ASTERGEMM_OPERAND_DIRECT_B_K8 || cfg.dtype_ab != ASTERGEMM_MXFP4)) {
+    fprintf(stderr, "--mx-a-lanes needs --ab mxfp4 --normal --direct-b-k8\n");
+    return 2;
+  }
+  if (use_normal && cfg.dtype_ab == ASTERGEMM_F16) {
+    fprintf(stderr, "--normal covers bf16, fp8 and mxfp4\n");
+    return 2;
+  }
   if (iters <= warmup) {
     fprintf(stderr, "--iters must exceed --warmup\n");
     return 2;
@@ -188,38 +229,84 @@ int main(int argc, char** argv) {
   const int bits = cfg.dtype_ab == ASTERGEMM_MXFP4 ? 4 : cfg.dtype_ab == ASTERGEMM_FP8_E4M3 ? 8 : 16;
   const size_t a_bytes = (size_t)cfg.M * cfg.K * bits / 8, b_bytes = (size_t)cfg.N * cfg.K * bits / 8;
   const size_t c_bytes = (size_t)cfg.M * cfg.N * (cfg.dtype_c == ASTERGEMM_F32 ? 4 : 2);
-  std::vector<uint8_t> ha(a_bytes), hb(b_bytes);
-  fill(ha, cfg.dtype_ab, 42);
-  fill(hb, cfg.dtype_ab, 43);
-
   astergemm_operands ops;
   memset(&ops, 0, sizeof(ops));
   void *dA, *dB, *dC;
   CHECK(aster_rt_malloc(&dA, a_bytes));
   CHECK(aster_rt_malloc(&dB, b_bytes));
   CHECK(aster_rt_malloc(&dC, c_bytes));
-  CHECK(aster_rt_memcpy_h2d(dA, ha.data(), a_bytes));
-  CHECK(aster_rt_memcpy_h2d(dB, hb.data(), b_bytes));
   ops.dA = dA;
   ops.dB = dB;
   ops.dC = dC;
-  if (cfg.scale_mode == ASTERGEMM_SCALE_TENSOR) {
-    const float s[2] = {0.01f, 0.02f};
-    void* ds;
-    CHECK(aster_rt_malloc(&ds, 256));
-    CHECK(aster_rt_memcpy_h2d(ds, s, sizeof(s)));
-    ops.dScaleA = (const float*)ds;
-    ops.dScaleB = (const float*)ds + 1;
-  }
-  if (cfg.scale_mode == ASTERGEMM_SCALE_MX32) {
-    std::vector<uint8_t> sa((size_t)cfg.M * cfg.K / 32, 122), sb((size_t)cfg.N * cfg.K / 32, 123);
-    void *da, *db;
-    CHECK(aster_rt_malloc(&da, sa.size()));
-    CHECK(aster_rt_malloc(&db, sb.size()));
-    CHECK(aster_rt_memcpy_h2d(da, sa.data(), sa.size()));
-    CHECK(aster_rt_memcpy_h2d(db, sb.data(), sb.size()));
-    ops.dMxA = (const uint8_t*)da;
-    ops.dMxB = (const uint8_t*)db;
+  if (!use_normal) {
+    std::vector<uint8_t> ha(a_bytes), hb(b_bytes);
+    fill(ha, cfg.dtype_ab, 42);
+    fill(hb, cfg.dtype_ab, 43);
+    CHECK(aster_rt_memcpy_h2d(dA, ha.data(), a_bytes));
+    CHECK(aster_rt_memcpy_h2d(dB, hb.data(), b_bytes));
+    if (cfg.scale_mode == ASTERGEMM_SCALE_TENSOR) {
+      const float s[2] = {0.01f, 0.02f};
+      void* ds;
+      CHECK(aster_rt_malloc(&ds, 256));
+      CHECK(aster_rt_memcpy_h2d(ds, s, sizeof(s)));
+      ops.dScaleA = (const float*)ds;
+      ops.dScaleB = (const float*)ds + 1;
+    }
+    if (cfg.scale_mode == ASTERGEMM_SCALE_MX32) {
+      std::vector<uint8_t> sa((size_t)cfg.M * cfg.K / 32, 122), sb((size_t)cfg.N * cfg.K / 32, 123);
+      void *da, *db;
+      CHECK(aster_rt_malloc(&da, sa.size()));
+      CHECK(aster_rt_malloc(&db, sb.size()));
+      CHECK(aster_rt_memcpy_h2d(da, sa.data(), sa.size()));
+      CHECK(aster_rt_memcpy_h2d(db, sb.data(), sb.size()));
+      ops.dMxA = (const uint8_t*)da;
+      ops.dMxB = (const uint8_t*)db;
+    }
+  } else {
+    // the benchmark's operands: N(0,1) sources (16-bit: times 0.02), quantised on the device
+    const bool is16 = cfg.dtype_ab == ASTERGEMM_BF16;
+    for (int side = 0; side < 2; ++side) {
+      const int64_t rows = side == 0 ? cfg.M : cfg.N;
+      const size_t n = (size_t)rows * (size_t)cfg.K;
+      void* dst = side == 0 ? dA : dB;
+      std::vector<float> src = normal(n, 42 + (uint64_t)side, is16 ? 0.02f : 1.0f);
+      if (is16) {
+        std::vector<uint16_t> h(n);
+        for (size_t i = 0; i < n; ++i) h[i] = bf16_rne(src[i]);
+        CHECK(aster_rt_memcpy_h2d(dst, h.data(), n * 2));
+        continue;
+      }
+      void* dsrc;
+      CHECK(aster_rt_malloc(&dsrc, n * 4));
+      CHECK(aster_rt_memcpy_h2d(dsrc, src.data(), n * 4));
+      const bool shuffle = side == 1 && cfg.operand_path != ASTERGEMM_OPERAND_LDS;
+      void* payload = dst;
+      if (shuffle) CHECK(aster_rt_malloc(&payload, side == 0 ? a_bytes : b_bytes));
+      if (cfg.dtype_ab == ASTERGEMM_FP8_E4M3) {
+        void* ds;
+        CHECK(aster_rt_malloc(&ds, 256));
+        CHECK(astergemm_quantize_fp8_tensor(dsrc, ASTERGEMM_F32, (int64_t)n, (uint8_t*)payload, (float*)ds, nullptr));
+        (side == 0 ? ops.dScaleA : ops.dScaleB) = (const float*)ds;
+        if (shuffle)
+          CHECK(astergemm_preshuffle(cfg.dtype_ab, cfg.operand_path, rows, cfg.K, payload, dst, nullptr, nullptr, nullptr));
+      } else {
+        const bool lanes = side == 0 && cfg.mx_a_layout == ASTERGEMM_MX_LANES128;
+        const size_t plane = lanes ? (size_t)astergemm_mx_lanes128_bytes(rows, cfg.K) : n / 32;
+        void *sc, *sc2 = nullptr;
+        CHECK(aster_rt_malloc(&sc, plane));
+        CHECK(astergemm_quantize_mxfp4_ex(dsrc, ASTERGEMM_F32, rows, cfg.K, 0, (uint8_t*)payload, (uint8_t*)sc,
+                                          lanes ? ASTERGEMM_MX_LANES128 : ASTERGEMM_MX_ROWS, nullptr));
+        if (shuffle) {
+          CHECK(aster_rt_malloc(&sc2, plane));
+          CHECK(astergemm_preshuffle(cfg.dtype_ab, cfg.operand_path, rows, cfg.K, payload, dst, (const uint8_t*)sc,
+                                     (uint8_t*)sc2, nullptr));
+        }
+        (side == 0 ? ops.dMxA : ops.dMxB) = (const uint8_t*)(shuffle ? sc2 : sc);
+      }
+      CHECK(aster_rt_device_synchronize());
+      CHECK(aster_rt_free(dsrc));
+      if (shuffle) CHECK(aster_rt_free(payload));
+    }
   }
   if (cfg.has_bias) {
     std::vector<float> hbias((size_t)cfg.N, 0.5f);

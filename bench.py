@@ -42,6 +42,8 @@ MEASURED_TRAFFIC_BYTES = {
     "stream_mxfp4_256x256_w2x2_bf16": 3.22e8,   # 4096x14336x4096: 2.05e8 read + 1.17e8 written
     "stream_mxfp4_256x256_w2x4_tail128_bf16": 3.10e8,  # the same shape: 1.92e8 read + 1.18e8 written
     "streamdb_mxfp4_128x256_w1x4_bf16": 3.13e8,  # the same shape, weights pre-shuffled: 1.96e8 + 1.17e8
+    # the same shape, both e8m0 planes in lane order, operands quantised from N(0,1): 1.99e8 + 1.17e8
+    "streamdb_mxfp4_128x256_w1x4_sal_bf16": 3.17e8,
 }
 
 
@@ -464,6 +466,29 @@ def main() -> int:
                                "frac_weights_pre_shuffled": round(tfd / PEAK_TFLOPS[dt], 4),
                                "traffic_weights_pre_shuffled": MEASURED_TRAFFIC_BYTES.get(pd.info.name.decode()),
                                "same_bits_as_row_major_weights": bool(torch.equal(c, c2))})
+            if dt == "mxfp4":
+                # and with the activations' e8m0 plane in lane order as well (mx_a_layout lanes128:
+                # what the device quantiser writes with scales_layout="lanes128"; here made from the
+                # row-major plane by the device pre-shuffle), no scale traffic through LDS
+                from aster_amd.kittens_helpers import mx_lanes128_bytes
+                sal = torch.empty(mx_lanes128_bytes(m, k), device=dev, dtype=torch.uint8)
+                torch.cuda.synchronize()
+                Q.preshuffle_scales_a_device(keep["mx_a"].data_ptr(), sal.data_ptr(), m, k)
+                torch.cuda.synchronize()
+                pl = AG.GemmPlan.create(m, n, k, dt, "bf16", operand_path="direct_b_k8", mx_a_layout="lanes128")
+                c3 = torch.empty_like(c)
+                keep_l = dict(mx_a=sal, mx_b=sbs)
+                pre_l = preheat(pl, a, bs, c3, keep_l, others_preheat_ms)
+                p50l, _, _ = event_timed_p50(pl, a, bs, c3, keep_l, 100, 20)
+                tfl = pl.info.flops / p50l * 1e-3
+                others[-1].update({"kernel_scales_in_lane_order": pl.info.name.decode(),
+                                   "preheat_launches_scales_in_lane_order": pre_l,
+                                   "p50_us_scales_in_lane_order": round(p50l / 1e3, 2),
+                                   "tflops_scales_in_lane_order": round(tfl, 1),
+                                   "frac_scales_in_lane_order": round(tfl / PEAK_TFLOPS[dt], 4),
+                                   "traffic_scales_in_lane_order": MEASURED_TRAFFIC_BYTES.get(pl.info.name.decode()),
+                                   "scales_in_lane_order_same_bits": bool(torch.equal(c, c3))})
+                del sal, c3
             del bs, sbs, c2
         # the two gfx950 shapes the reference publishes its own kernels' numbers for (f16
         # operands, fp32 output; contrib/kittens/test/bench/best_known.json, quoted, not re-run)
