@@ -199,6 +199,14 @@ __global__ __launch_bounds__(KW * 64) void gemm_skinny_kernel(const GemmArgs p) 
 //
 // SPB = 128-byte steps per wave and block = K / 512; a unit of work is four steps
 // (eight loads, eight MFMAs) and two units are kept in flight per wave.
+//
+// Rows of 4 KiB (SPB = 4: a unit is a wave's whole 512-byte slice of 16 rows) are fetched as
+// 2 rows x 512 contiguous bytes per instruction instead of 8 rows x 128 bytes: measured back to
+// back over rotating weight sets, M = 16, 8 rows x 128 -> 2 rows x 512: fp8 14336 x 4096 14.2 ->
+// 12.7 us, fp8 28672 x 4096 25.5 -> 22.1, bf16 28672 x 2048 25.4 -> 22.7.  On longer rows, where a
+// unit is half or a quarter of the slice, the same change loses 3-5 % (bf16 14336 x 4096 20.6 ->
+// 21.6 us, x 8192 38.0 -> 39.2, fp8 x 8192 20.9 -> 21.5), and so does one row x 1 KiB per
+// instruction with a block per LDS pass (bf16 14336 x 4096 21.6): they keep 8 rows x 128 bytes.
 template <int DT, int OUT, int SPB>
 __global__ __launch_bounds__(512) void gemm_skinny_reg_kernel(const GemmArgs p) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t slds[];
@@ -224,10 +232,24 @@ __global__ __launch_bounds__(512) void gemm_skinny_reg_kernel(const GemmArgs p) 
   // load: lane -> row (lane >> 3) of an 8-row half block, 16-byte piece (lane & 7)
   const int lrow = lane >> 3, lpiece = lane & 7;
   const uint8_t* wbase = p.B + wave * slice + lpiece * 16;
+  constexpr bool CONTIG = UPB == 1;              // 2 rows x 512 contiguous bytes per instruction
+  const int hi = lane >> 5, p32 = lane & 31;     // CONTIG: row of the pair, piece of its 512 bytes
   auto issue = [&](int j, i32x4(&dst)[8]) {      // flat index j = block * UPB + t
     int blk = j / UPB;
     const int t = j % UPB;
     blk = blk < nblk ? blk : nblk - 1;
+    if constexpr (CONTIG) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {              // instruction i: rows 2 i and 2 i + 1 of the block
+        const int nh = r0 + blk * 16 + 2 * i;
+        int n = nh + hi;
+        n = n < r1 ? n : r1 - 1;
+        const uint8_t* src = p.B + wave * slice + (int64_t)n * p.ldb_bytes + p32 * 16;
+        if (j >= total || nh >= r1) src = p.A + lpiece * 16;  // nothing to fetch: a line that stays in L2
+        dst[i] = __builtin_nontemporal_load((const i32x4*)src);
+      }
+      return;
+    }
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       const int nh = r0 + blk * 16 + h * 8;
@@ -249,6 +271,19 @@ __global__ __launch_bounds__(512) void gemm_skinny_reg_kernel(const GemmArgs p) 
 #pragma unroll
     for (int i = 0; i < 8; ++i)
       *(i32x4*)(tbuf + (i >> 1) * 2048 + (i & 1) * 1024 + wr_off) = src[i];
+  };
+  // the same LDS layout from the CONTIG load pattern: register i holds, for row r = 2 i + hi,
+  // piece p32 of the 512 bytes = piece (p32 & 7) of step (p32 >> 3)
+  const int wr_c = (p32 >> 3) * 2048 + hi * 128;
+  const int pch = ((p32 & 7) ^ hi) << 4;
+  auto stash_w = [&](const i32x4(&src)[8]) {
+    if constexpr (CONTIG) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        *(i32x4*)(tbuf + wr_c + (i >> 2) * 1024 + (i & 3) * 256 + (pch ^ ((i & 3) << 5))) = src[i];
+    } else {
+      stash(src);
+    }
   };
   auto operand = [&](int s, int u) {             // MFMA operand (row li, K piece 4u + lq) of step s
     return *(const i32x4*)(tbuf + s * 2048 + rd_off + (((4 * u + lq) ^ (li & 7)) << 4));
@@ -357,13 +392,13 @@ __global__ __launch_bounds__(512) void gemm_skinny_reg_kernel(const GemmArgs p) 
       constexpr int i = decltype(I)::value * 2;
       // each register set is refilled as soon as its unit has been written to LDS;
       // the scheduler must not move the loads across the units they overlap with
-      stash(w0);
+      stash_w(w0);
       __builtin_amdgcn_sched_barrier(0);
       issue(j + i + 2, w0);
       __builtin_amdgcn_sched_barrier(0);
       mma(blk + i / UPB, std::integral_constant<int, i % UPB>{});
       __builtin_amdgcn_sched_barrier(0);
-      stash(w1);
+      stash_w(w1);
       __builtin_amdgcn_sched_barrier(0);
       issue(j + i + 3, w1);
       __builtin_amdgcn_sched_barrier(0);
@@ -372,7 +407,7 @@ __global__ __launch_bounds__(512) void gemm_skinny_reg_kernel(const GemmArgs p) 
     });
   }
   if (j < total) {  // UPB == 1, odd block count
-    stash(w0);
+    stash_w(w0);
     mma(j / UPB, std::integral_constant<int, 0>{});
   }
 }
@@ -427,12 +462,28 @@ __global__ __launch_bounds__(512) void gemm_skinny_fp4_kernel(const GemmArgs p) 
   const int lrow = lane >> 3, lpiece = lane & 7;
   const uint8_t* wbase = p.B + wave * slice + lpiece * 16;
   const uint8_t* sbase = p.mx_b + wave * (SPB * 8);       // this wave's scale bytes of a row
+  // a unit that is the wave's whole slice of a row (UPB == 1) is fetched as R rows x SU * 128
+  // contiguous bytes per instruction instead of 8 rows x 128 bytes (see gemm_skinny_reg_kernel)
+  constexpr bool CONTIG = UPB == 1;
+  constexpr int R = 16 / NL, LPR = 64 / R;       // rows per instruction, lanes (pieces) per row
+  const int rsel = lane / LPR, pidx = lane % LPR;
   auto issue = [&](int j, i32x4(&dst)[NL], i32x2(&sc)[SU]) {  // flat index j = block * UPB + t
     int blk = j / UPB;
     const int t = j % UPB;
     blk = blk < nblk ? blk : nblk - 1;
+    if constexpr (CONTIG) {
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
+      for (int i = 0; i < NL; ++i) {             // instruction i: rows R i .. R i + R - 1 of the block
+        const int nh = r0 + blk * 16 + R * i;
+        int n = nh + rsel;
+        n = n < r1 ? n : r1 - 1;
+        const uint8_t* src = p.B + wave * slice + (int64_t)n * p.ldb_bytes + pidx * 16;
+        if (j >= total || nh >= r1) src = p.A + lpiece * 16;  // nothing to fetch: a line that stays in L2
+        dst[i] = __builtin_nontemporal_load((const i32x4*)src);
+      }
+    }
+#pragma unroll
+    for (int h = 0; h < (CONTIG ? 0 : 2); ++h) {
       const int nh = r0 + blk * 16 + h * 8;
       int n = nh + lrow;
       n = n < r1 ? n : r1 - 1;
@@ -455,6 +506,21 @@ __global__ __launch_bounds__(512) void gemm_skinny_fp4_kernel(const GemmArgs p) 
 #pragma unroll
     for (int i = 0; i < NL; ++i)
       *(i32x4*)(tbuf + (i >> 1) * 2048 + (i & 1) * 1024 + wr_off) = src[i];
+  };
+  // the same LDS layout from the CONTIG load pattern: register i holds, for row r = R i + rsel,
+  // piece (pidx & 7) of step (pidx >> 3)
+  const int wr_c = (pidx >> 3) * 2048 + rsel * 128;
+  const int pch = ((pidx & 7) ^ rsel) << 4;
+  auto stash_w = [&](const i32x4(&src)[NL]) {
+    if constexpr (CONTIG) {
+#pragma unroll
+      for (int i = 0; i < NL; ++i) {
+        const int rr = R * i;                    // compile time after unrolling
+        *(i32x4*)(tbuf + wr_c + (rr >> 3) * 1024 + (rr & 7) * 128 + (pch ^ ((rr & 7) << 4))) = src[i];
+      }
+    } else {
+      stash(src);
+    }
   };
   auto operand = [&](int s, int u) {             // piece 4u + lq of step s, row li
     return *(const i32x4*)(tbuf + s * 2048 + rd_off + (((4 * u + lq) ^ (li & 7)) << 4));
@@ -554,14 +620,14 @@ __global__ __launch_bounds__(512) void gemm_skinny_fp4_kernel(const GemmArgs p) 
     const int blk = j / UPB;
     static_for<0, TRIP / 2>([&](auto I) {
       constexpr int i = decltype(I)::value * 2;
-      stash(w0);
+      stash_w(w0);
       take_scales(s0, sc);
       __builtin_amdgcn_sched_barrier(0);
       issue(j + i + 2, w0, s0);
       __builtin_amdgcn_sched_barrier(0);
       mma(blk + i / UPB, std::integral_constant<int, i % UPB>{}, sc);
       __builtin_amdgcn_sched_barrier(0);
-      stash(w1);
+      stash_w(w1);
       take_scales(s1, sc);
       __builtin_amdgcn_sched_barrier(0);
       issue(j + i + 3, w1, s1);
@@ -571,7 +637,7 @@ __global__ __launch_bounds__(512) void gemm_skinny_fp4_kernel(const GemmArgs p) 
     });
   }
   if (j < total) {  // UPB == 1, odd block count
-    stash(w0);
+    stash_w(w0);
     take_scales(s0, sc);
     mma(j / UPB, std::integral_constant<int, 0>{}, sc);
   }
@@ -756,6 +822,11 @@ __global__ __launch_bounds__(512) void gemm_skinny_fp4m_kernel(const GemmArgs p)
   const int lrow = lane >> 3, lpiece = lane & 7;
   const uint8_t* wbase = p.B + koff + wave * slice + lpiece * 16;
   const uint8_t* sbase = p.mx_b + koff / 16 + wave * (SPB * 8);  // this wave's scale bytes of a row
+  // a unit that is the wave's whole slice of a row (UPB == 1): R rows x SU * 128 contiguous bytes
+  // per instruction instead of 8 rows x 128 bytes (see gemm_skinny_reg_kernel)
+  constexpr bool CONTIG = UPB == 1;
+  constexpr int R = 16 / NL, LPR = 64 / R;       // rows per instruction, lanes (pieces) per row
+  const int rsel = lane / LPR, pidx = lane % LPR;
   auto issue = [&](int j, i32x4(&dst)[NL], i32x2(&sc)[SU]) {  // flat index j = block * UPB + t
     int blk = j / UPB;
     const int t = j % UPB;
@@ -767,8 +838,19 @@ __global__ __launch_bounds__(512) void gemm_skinny_fp4m_kernel(const GemmArgs p)
       for (int s = 0; s < SU; ++s) sc[s] = i32x2{0x7F7F7F7F, 0x7F7F7F7F};
       return;
     }
+    if constexpr (CONTIG) {
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
+      for (int i = 0; i < NL; ++i) {             // instruction i: rows R i .. R i + R - 1 of the block
+        const int nh = r0 + blk * 16 + R * i;
+        int n = nh + rsel;
+        n = n < r1 ? n : r1 - 1;
+        const uint8_t* src = p.B + koff + wave * slice + (int64_t)n * p.ldb_bytes + pidx * 16;
+        if (j >= total || nh >= r1) src = p.A + lpiece * 16;  // nothing to fetch: a line that stays in L2
+        dst[i] = __builtin_nontemporal_load((const i32x4*)src);
+      }
+    }
+#pragma unroll
+    for (int h = 0; h < (CONTIG ? 0 : 2); ++h) {
       const int nh = r0 + blk * 16 + h * 8;
       int n = nh + lrow;
       n = n < r1 ? n : r1 - 1;
@@ -791,6 +873,19 @@ __global__ __launch_bounds__(512) void gemm_skinny_fp4m_kernel(const GemmArgs p)
 #pragma unroll
     for (int i = 0; i < NL; ++i)
       *(i32x4*)(tbuf + (i >> 1) * 2048 + (i & 1) * 1024 + wr_off) = src[i];
+  };
+  const int wr_c = (pidx >> 3) * 2048 + rsel * 128;
+  const int pch = ((pidx & 7) ^ rsel) << 4;
+  auto stash_w = [&](const i32x4(&src)[NL]) {
+    if constexpr (CONTIG) {
+#pragma unroll
+      for (int i = 0; i < NL; ++i) {
+        const int rr = R * i;                    // compile time after unrolling
+        *(i32x4*)(tbuf + wr_c + (rr >> 3) * 1024 + (rr & 7) * 128 + (pch ^ ((rr & 7) << 4))) = src[i];
+      }
+    } else {
+      stash(src);
+    }
   };
   auto operand = [&](int s, int u) {             // piece 4u + lq of step s, row li
     return *(const i32x4*)(tbuf + s * 2048 + rd_off + (((4 * u + lq) ^ (li & 7)) << 4));
@@ -912,14 +1007,14 @@ __global__ __launch_bounds__(512) void gemm_skinny_fp4m_kernel(const GemmArgs p)
     const int blk = j / UPB;
     static_for<0, TRIP / 2>([&](auto I) {
       constexpr int i = decltype(I)::value * 2;
-      stash(w0);
+      stash_w(w0);
       take_scales(s0, sc);
       __builtin_amdgcn_sched_barrier(0);
       issue(j + i + 2, w0, s0);
       __builtin_amdgcn_sched_barrier(0);
       mma(blk + i / UPB, std::integral_constant<int, i % UPB>{}, sc);
       __builtin_amdgcn_sched_barrier(0);
-      stash(w1);
+      stash_w(w1);
       take_scales(s1, sc);
       __builtin_amdgcn_sched_barrier(0);
       issue(j + i + 3, w1, s1);
@@ -929,7 +1024,7 @@ __global__ __launch_bounds__(512) void gemm_skinny_fp4m_kernel(const GemmArgs p)
     });
   }
   if (j < total) {  // UPB == 1, odd block count
-    stash(w0);
+    stash_w(w0);
     take_scales(s0, sc);
     mma(j / UPB, std::integral_constant<int, 0>{}, sc);
   }
@@ -1059,6 +1154,10 @@ __global__ __launch_bounds__(512) void gemm_skinny_regm_kernel(const GemmArgs p)
 
   const int lrow = lane >> 3, lpiece = lane & 7;
   const uint8_t* wbase = p.B + koff + wave * slice + lpiece * 16;
+  // a unit that is the wave's whole slice of a row (UPB == 1): 2 rows x 512 contiguous bytes per
+  // instruction instead of 8 rows x 128 bytes (see gemm_skinny_reg_kernel)
+  constexpr bool CONTIG = UPB == 1;
+  const int hi = lane >> 5, p32 = lane & 31;
   auto issue = [&](int j, i32x4(&dst)[8]) {      // flat index j = block * UPB + t
     int blk = j / UPB;
     const int t = j % UPB;
@@ -1066,6 +1165,18 @@ __global__ __launch_bounds__(512) void gemm_skinny_regm_kernel(const GemmArgs p)
     if (dead) {                                    // zeros, so that nothing non-finite gets in
 #pragma unroll
       for (int i = 0; i < 8; ++i) dst[i] = i32x4{0, 0, 0, 0};
+      return;
+    }
+    if constexpr (CONTIG) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {              // instruction i: rows 2 i and 2 i + 1 of the block
+        const int nh = r0 + blk * 16 + 2 * i;
+        int n = nh + hi;
+        n = n < r1 ? n : r1 - 1;
+        const uint8_t* src = p.B + koff + wave * slice + (int64_t)n * p.ldb_bytes + p32 * 16;
+        if (j >= total || nh >= r1) src = p.A + lpiece * 16;  // nothing to fetch: a line that stays in L2
+        dst[i] = __builtin_nontemporal_load((const i32x4*)src);
+      }
       return;
     }
 #pragma unroll
@@ -1087,6 +1198,17 @@ __global__ __launch_bounds__(512) void gemm_skinny_regm_kernel(const GemmArgs p)
 #pragma unroll
     for (int i = 0; i < 8; ++i)
       *(i32x4*)(tbuf + (i >> 1) * 2048 + (i & 1) * 1024 + wr_off) = src[i];
+  };
+  const int wr_c = (p32 >> 3) * 2048 + hi * 128;
+  const int pch = ((p32 & 7) ^ hi) << 4;
+  auto stash_w = [&](const i32x4(&src)[8]) {
+    if constexpr (CONTIG) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        *(i32x4*)(tbuf + wr_c + (i >> 2) * 1024 + (i & 3) * 256 + (pch ^ ((i & 3) << 5))) = src[i];
+    } else {
+      stash(src);
+    }
   };
   auto operand = [&](int s, int u) {
     return *(const i32x4*)(tbuf + s * 2048 + rd_off + (((4 * u + lq) ^ (li & 7)) << 4));
@@ -1207,13 +1329,13 @@ __global__ __launch_bounds__(512) void gemm_skinny_regm_kernel(const GemmArgs p)
     const int blk = j / UPB;
     static_for<0, TRIP / 2>([&](auto I) {
       constexpr int i = decltype(I)::value * 2;
-      stash(w0);
+      stash_w(w0);
       __builtin_amdgcn_sched_barrier(0);
       issue(j + i + 2, w0);
       __builtin_amdgcn_sched_barrier(0);
       mma(blk + i / UPB, std::integral_constant<int, i % UPB>{});
       __builtin_amdgcn_sched_barrier(0);
-      stash(w1);
+      stash_w(w1);
       __builtin_amdgcn_sched_barrier(0);
       issue(j + i + 3, w1);
       __builtin_amdgcn_sched_barrier(0);
@@ -1222,7 +1344,7 @@ __global__ __launch_bounds__(512) void gemm_skinny_regm_kernel(const GemmArgs p)
     });
   }
   if (j < total) {  // UPB == 1, odd block count
-    stash(w0);
+    stash_w(w0);
     mma(j / UPB, std::integral_constant<int, 0>{});
   }
 }
