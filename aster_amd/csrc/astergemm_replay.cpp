@@ -16,6 +16,10 @@
 //                                    bf16 / f16 times 0.02, for fp8 / MXFP4 quantised on the device
 //                                    and, with --direct-b-k8, pre-shuffled on the device: valid
 //                                    operands, so that counters describe what the benchmark times)
+//                    [--same-rows]   (with --normal, 16-bit operands: every row of A and of B a copy of
+//                                    its first row: the operand values a kernel sees do not change
+//                                    when all its transfers are pointed at one row, so the cost of
+//                                    the memory path can be told from the cost of the operand bits)
 //                    [--mx-a-lanes]  (MXFP4: A's e8m0 plane in lane order, mx_a_layout LANES128;
 //                                    needs --normal and --direct-b-k8)
 //   astergemm_replay --quantize fp8|mxfp4 --m ROWS --k K --iters 100
@@ -160,7 +164,7 @@ int main(int argc, char** argv) {
   cfg.M = cfg.N = cfg.K = 8192;
   cfg.dtype_ab = ASTERGEMM_BF16;
   cfg.dtype_c = ASTERGEMM_BF16;
-  int iters = 100, warmup = 20, json = 0, use_normal = 0;
+  int iters = 100, warmup = 20, json = 0, use_normal = 0, same_rows = 0;
   long long flush = 0, calib = 0;
   const char* quantize = nullptr;
   for (int i = 1; i < argc; ++i) {
@@ -187,6 +191,7 @@ int main(int argc, char** argv) {
     else if (a == "--direct-b-k8") cfg.operand_path = ASTERGEMM_OPERAND_DIRECT_B_K8;
     else if (a == "--bias") cfg.has_bias = 1;
     else if (a == "--normal") use_normal = 1;
+    else if (a == "--same-rows") same_rows = 1;
     else if (a == "--mx-a-lanes") cfg.mx_a_layout = ASTERGEMM_MX_LANES128;
     else if (a == "--json") json = 1;
     else if (a == "--quantize") quantize = val();
@@ -272,7 +277,7 @@ int main(int argc, char** argv) {
       std::vector<float> src = normal(n, 42 + (uint64_t)side, is16 ? 0.02f : 1.0f);
       if (is16) {
         std::vector<uint16_t> h(n);
-        for (size_t i = 0; i < n; ++i) h[i] = bf16_rne(src[i]);
+        for (size_t i = 0; i < n; ++i) h[i] = bf16_rne(src[same_rows ? i % (size_t)cfg.K : i]);
         CHECK(aster_rt_memcpy_h2d(dst, h.data(), n * 2));
         continue;
       }
