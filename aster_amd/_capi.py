@@ -114,6 +114,7 @@ SIGNATURES = {
     "astergemm_variant_info": (C.c_int, [C.c_int, C.POINTER(Config), C.POINTER(KernelInfo)]),
     "astergemm_run": (C.c_int, [C.POINTER(Config), C.POINTER(Operands), _P]),
     "astergemm_run_noalloc": (C.c_int, [C.POINTER(Config), C.POINTER(Operands), _P]),
+    "astergemm_prepare": (C.c_int, [C.POINTER(Config)]),
     "astergemm_workspace_bytes": (C.c_int, [C.POINTER(Config), C.POINTER(C.c_size_t)]),
     "astergemm_bench_rotate": (C.c_int, [C.POINTER(Config), C.POINTER(Operands), C.c_int, C.c_int,
                                          C.POINTER(C.c_int64), C.c_void_p]),

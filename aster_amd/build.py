@@ -91,6 +91,25 @@ def _compile(unit) -> str:
     return obj
 
 
+PLAN_HEADER = os.path.join(CSRC, "stream_load_plan.inc")
+
+
+def write_generated_sources() -> None:
+    """The stream kernels' staging constants come from the cooperative load plan of
+    `aster_amd.coop` (the host-side mirror of the reference's make_coop_load_plan): the header the
+    kernels include is written from it, so a change of the plan changes the kernels."""
+    from .coop import stream_load_plan_header
+
+    text = stream_load_plan_header()
+    old = None
+    if os.path.exists(PLAN_HEADER):
+        with open(PLAN_HEADER) as f:
+            old = f.read()
+    if old != text:
+        with open(PLAN_HEADER, "w") as f:
+            f.write(text)
+
+
 def _genco(src: str) -> str:
     """Device-only code object for module launchers (hipModuleLoadData)."""
     flags = [f for f in COMMON_FLAGS if f != "-fPIC"]
@@ -107,6 +126,7 @@ def build_library(verbose: bool = False, only=None) -> str:
     on one kernel file) recompiles just those and links them with the objects already there."""
     os.makedirs(OBJ_DIR, exist_ok=True)
     os.makedirs(LIB_DIR, exist_ok=True)
+    write_generated_sources()
     with ThreadPoolExecutor(max_workers=6) as pool:
         if only:
             todo = [u for u in UNITS if u[0] in only]

@@ -124,3 +124,59 @@ def stream_kernel_load_plan(wid: int, *, tile_rows: int, num_waves: int,
     l = Layout((tiles, 1), (STREAM_TILE_ROWS * STREAM_ROW_BYTES, STREAM_TILE_ROWS * STREAM_ROW_BYTES * tiles))
     return make_coop_load_plan(wid, num_waves=num_waves, wg_tile_global=g, wg_tile_lds=l,
                                interleave=True)
+
+
+# (tile rows, waves) of every instantiation of the stream kernels' staging.
+STREAM_PLAN_CONFIGS = [(256, 8), (256, 4), (128, 4)]
+
+
+def stream_load_plan_header() -> str:
+    """Text of `aster_amd/csrc/stream_load_plan.inc`: for every (tile rows, waves) the stream
+    kernels are built with, the constants of `stream_kernel_load_plan` as a C++ struct the
+    kernels take their transfer count, operand rows and LDS offsets from.  The plan of wave w is
+    affine in (w, transfer j) - checked here - so four numbers describe it: transfers per wave,
+    tiles between the first tiles of neighbouring waves, tiles between a wave's consecutive
+    transfers, and the tile (rows, LDS bytes)."""
+    out = ["// Generated by aster_amd.coop.stream_load_plan_header() (python -m aster_amd.build writes it);",
+           "// do not edit.  The staging of one operand half of one K-step in the stream kernels as the",
+           "// cooperative load plan of the reference (make_coop_load_plan,",
+           "// contrib/kittens/test/coop.py:50-94): transfer j of wave w covers operand rows",
+           "// first_row(w, j) .. + TILE_ROWS - 1 and lands at lds_offset(w, j) of the ring slot.",
+           "#pragma once",
+           "",
+           "namespace astergemm {",
+           "",
+           "template <int TILE_ROWS_OF_SLOT, int NUM_WAVES>",
+           "struct StreamLoadPlan;",
+           ""]
+    ld = 1 << 20      # any pitch: the plan is linear in it
+    for rows, nw in STREAM_PLAN_CONFIGS:
+        plans = [stream_kernel_load_plan(w, tile_rows=rows, num_waves=nw, ld_bytes=ld) for w in range(nw)]
+        lh = plans[0].global_layout.sizes[0]
+        t = [p_.transfers() for p_ in plans]
+        row = lambda w, j: t[w][j][0] // ld
+        assert all(t[w][j][0] % ld == 0 for w in range(nw) for j in range(lh))
+        wave_step_rows = row(1, 0) - row(0, 0)
+        xfer_step_rows = row(0, 1) - row(0, 0) if lh > 1 else nw * STREAM_TILE_ROWS
+        tile_lds = STREAM_TILE_ROWS * STREAM_ROW_BYTES
+        for w in range(nw):
+            for j in range(lh):
+                assert row(w, j) == w * wave_step_rows + j * xfer_step_rows
+                assert t[w][j][1] * STREAM_TILE_ROWS == row(w, j) * tile_lds   # LDS follows the rows
+        assert wave_step_rows % STREAM_TILE_ROWS == 0 and xfer_step_rows % STREAM_TILE_ROWS == 0
+        out += [f"template <>",
+                f"struct StreamLoadPlan<{rows}, {nw}> {{",
+                f"  static constexpr int LH = {lh};                 // transfers per wave and slot",
+                f"  static constexpr int TILE_ROWS = {STREAM_TILE_ROWS};          // operand rows of one transfer",
+                f"  static constexpr int TILE_LDS_BYTES = {tile_lds};  // its bytes in the slot",
+                f"  static constexpr int WAVE_STEP_TILES = {wave_step_rows // STREAM_TILE_ROWS};    // from wave w to w + 1",
+                f"  static constexpr int XFER_STEP_TILES = {xfer_step_rows // STREAM_TILE_ROWS};    // from transfer j to j + 1",
+                "  __host__ __device__ static constexpr int tile(int w, int j) {",
+                "    return w * WAVE_STEP_TILES + j * XFER_STEP_TILES;",
+                "  }",
+                "  __host__ __device__ static constexpr int first_row(int w, int j) { return tile(w, j) * TILE_ROWS; }",
+                "  __host__ __device__ static constexpr int lds_offset(int w, int j) { return tile(w, j) * TILE_LDS_BYTES; }",
+                "};",
+                ""]
+    out += ["}  // namespace astergemm", ""]
+    return "\n".join(out)

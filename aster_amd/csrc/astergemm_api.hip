@@ -29,6 +29,31 @@ int hip_fail(hipError_t e, const char* what, const char* file, int line) {
   return ASTERGEMM_EHIP;
 }
 
+LaunchContext& launch_context() {
+  static thread_local LaunchContext ctx;
+  return ctx;
+}
+
+// Sets the launch context for the launcher calls of one entry point and clears it on return.
+struct LaunchScope {
+  explicit LaunchScope(void* stream, bool prepare_only = false) {
+    launch_context().stream = (hipStream_t)stream;
+    launch_context().prepare_only = prepare_only;
+  }
+  ~LaunchScope() { launch_context() = LaunchContext{}; }
+};
+
+// The error text of a launcher's status; a first launch refused inside a capture says what to do.
+int launch_fail(int e, const char* name, const char* file, int line) {
+  if ((hipError_t)e == hipErrorStreamCaptureUnsupported) {
+    set_error("%s: the first launch of a kernel on a device sets a function attribute, which cannot "
+              "happen while the stream is being captured; call astergemm_prepare(cfg) (or launch "
+              "once eagerly) before the capture", name);
+    return ASTERGEMM_EHIP;
+  }
+  return hip_fail((hipError_t)e, name, file, line);
+}
+
 // Compute units of the current device (0 when there is none), cached per device ordinal.
 int device_cus() {
   static std::atomic<int> cus[64];
@@ -488,8 +513,45 @@ int astergemm_run(const astergemm_config* cfg, const astergemm_operands* ops, vo
   GemmArgs a;
   if (int rc = build_args(*v, *cfg, *ops, &a)) return rc;
   (void)hipGetLastError();  // the launchers report hipGetLastError(): drop what an earlier call left
+  LaunchScope scope(stream);
   const int e = v->launch(a, grid_of(*v, *cfg), (hipStream_t)stream);
-  if (e != 0) return hip_fail((hipError_t)e, v->name, __FILE__, __LINE__);
+  if (e != 0) return launch_fail(e, v->name, __FILE__, __LINE__);
+  return 0;
+}
+
+int astergemm_prepare(const astergemm_config* cfg) {
+  if (!cfg) {
+    set_error("astergemm_prepare: null argument");
+    return ASTERGEMM_EINVAL;
+  }
+  int index = -1;
+  const Variant* v = choose(*cfg, &index);
+  if (!v) return g_choose_rc;
+  if (device_cus() <= 0) {
+    set_error("astergemm_prepare: no HIP device");
+    return ASTERGEMM_ENODEV;
+  }
+  void* scratch_ptr = scratch_address();
+  if (!scratch_ptr) return ASTERGEMM_EHIP;
+  if (cfg->M == 0 || cfg->N == 0) return 0;
+  // The launcher runs with every one-time step (function attributes, cached device facts) and
+  // without the kernel launches; the operands are never read.  Partial sums, where the config
+  // has any, point at the built-in scratch when they fit, so that nothing is allocated either.
+  GemmArgs a;
+  astergemm_operands o;
+  memset(&o, 0, sizeof(o));
+  o.dA = o.dB = o.dC = scratch_ptr;
+  o.dScaleA = o.dScaleB = o.dBias = (const float*)scratch_ptr;
+  o.dMxA = o.dMxB = (const uint8_t*)scratch_ptr;
+  if (workspace_need(*v, *cfg) <= (size_t)ASTERGEMM_NOALLOC_SCRATCH_BYTES) {
+    o.dWorkspace = scratch_ptr;
+    o.workspace_bytes = (size_t)ASTERGEMM_NOALLOC_SCRATCH_BYTES;
+  }
+  if (int rc = build_args(*v, *cfg, o, &a)) return rc;
+  (void)hipGetLastError();
+  LaunchScope scope(nullptr, /*prepare_only=*/true);
+  const int e = v->launch(a, grid_of(*v, *cfg), nullptr);
+  if (e != 0) return launch_fail(e, v->name, __FILE__, __LINE__);
   return 0;
 }
 
@@ -534,8 +596,9 @@ int astergemm_run_noalloc(const astergemm_config* cfg, const astergemm_operands*
   GemmArgs a;
   if (int rc = build_args(*v, *cfg, o, &a)) return rc;
   (void)hipGetLastError();
+  LaunchScope scope(stream);
   const int e = v->launch(a, grid_of(*v, *cfg), (hipStream_t)stream);
-  if (e != 0) return hip_fail((hipError_t)e, v->name, __FILE__, __LINE__);
+  if (e != 0) return launch_fail(e, v->name, __FILE__, __LINE__);
   return 0;
 }
 
@@ -554,6 +617,7 @@ int astergemm_bench_rotate(const astergemm_config* cfg, const astergemm_operands
   for (int i = 0; i < n_ops; ++i)
     if (int rc = build_args(*v, *cfg, ops[i], &args[(size_t)i])) return rc;
   hipStream_t s = (hipStream_t)stream;
+  LaunchScope scope(stream);
   const int grid = grid_of(*v, *cfg);
   EventPair ev;
   AG_HIP(ev.create());
@@ -582,6 +646,7 @@ int astergemm_tune(const astergemm_config* cfg, const astergemm_operands* ops, i
   *best_variant = 0;
   if (best_ns) *best_ns = 0;
   hipStream_t s = (hipStream_t)stream;
+  LaunchScope scope(stream);
   EventPair ev;
   AG_HIP(ev.create());
   hipEvent_t e0 = ev.e0, e1 = ev.e1;
@@ -598,6 +663,9 @@ int astergemm_tune(const astergemm_config* cfg, const astergemm_operands* ops, i
       *best_variant = i + 1;
       break;
     }
+    // a caller's workspace too small for this variant's K ranges: the variant is skipped, the
+    // tune goes on with the others
+    if (ops->dWorkspace && ops->workspace_bytes < workspace_need(*v, *cfg)) continue;
     GemmArgs a;
     if ((rc = build_args(*v, *cfg, *ops, &a)) != 0) break;
     const int grid = grid_of(*v, *cfg);
@@ -644,6 +712,7 @@ int astergemm_bench(const astergemm_config* cfg, const astergemm_operands* ops, 
   GemmArgs a;
   if (int rc = build_args(*v, *cfg, *ops, &a)) return rc;
   hipStream_t s = (hipStream_t)stream;
+  LaunchScope scope(stream);
   const int grid = grid_of(*v, *cfg);
 
   DeviceBuffer flush_buf;

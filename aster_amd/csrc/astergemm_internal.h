@@ -75,13 +75,37 @@ struct Variant {
 // Compute units of the current device (0 when there is none), cached per device ordinal.
 int device_cus();
 
+// State of the launcher call in progress on this thread, set by the entry points in
+// astergemm_api.hip: the stream the kernels go to, and whether this is astergemm_prepare (every
+// one-time step of the launcher runs, the kernels themselves are not launched).
+struct LaunchContext {
+  hipStream_t stream = nullptr;
+  bool prepare_only = false;
+};
+LaunchContext& launch_context();
+
+// Every GEMM kernel launch of the library goes through this macro.
+#define AG_LAUNCH_KERNEL(...)                                                   \
+  do {                                                                          \
+    if (!::astergemm::launch_context().prepare_only) hipLaunchKernelGGL(__VA_ARGS__); \
+  } while (0)
+
 // Raises a kernel's dynamic-LDS limit once per device; `devs` is a static of the launcher with
-// one bit per device ordinal.  Returns 0 or a hipError_t.
+// one bit per device ordinal.  Returns 0 or a hipError_t.  Changing a function attribute is not
+// a stream operation: when the kernel's first launch on a device arrives while the stream is
+// being captured into a graph, the launcher refuses (hipErrorStreamCaptureUnsupported) instead
+// of touching the runtime from inside the capture; astergemm_prepare does this step ahead of time.
 inline int lds_attr_once(std::atomic<uint64_t>& devs, const void* func, int lds_bytes) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return (int)hipGetLastError();
   const uint64_t bit = (uint64_t)1 << (dev & 63);
   if (devs.load(std::memory_order_acquire) & bit) return 0;
+  hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(launch_context().stream, &st) != hipSuccess ||
+      st != hipStreamCaptureStatusNone) {
+    (void)hipGetLastError();
+    return (int)hipErrorStreamCaptureUnsupported;
+  }
   const hipError_t e = hipFuncSetAttribute(func, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
   if (e != hipSuccess) return (int)e;
   devs.fetch_or(bit, std::memory_order_release);

@@ -422,7 +422,7 @@ int launch_skinny_reg_t(const GemmArgs& a, hipStream_t s) {
   if (cus <= 0) return (int)hipErrorNoDevice;
   const int nblocks = (int)((a.N + 15) / 16);
   const int g = nblocks < cus ? nblocks : cus;
-  hipLaunchKernelGGL(k, dim3(g), dim3(512), lds, s, a);
+  AG_LAUNCH_KERNEL(k, dim3(g), dim3(512), lds, s, a);
   return (int)hipGetLastError();
 }
 
@@ -653,7 +653,7 @@ int launch_skinny_fp4_t(const GemmArgs& a, hipStream_t s) {
   if (cus <= 0) return (int)hipErrorNoDevice;
   const int nblocks = (int)((a.N + 15) / 16);
   const int g = nblocks < cus ? nblocks : cus;
-  hipLaunchKernelGGL(k, dim3(g), dim3(512), lds, s, a);
+  AG_LAUNCH_KERNEL(k, dim3(g), dim3(512), lds, s, a);
   return (int)hipGetLastError();
 }
 
@@ -729,7 +729,7 @@ template <int OUT>
 void launch_splitk_reduce(const GemmArgs& a, int S, hipStream_t s) {
   const int64_t total = (int64_t)a.M * ((a.N + 3) / 4);
   const int rg = (int)((total + 255) / 256 < 2048 ? (total + 255) / 256 : 2048);
-  hipLaunchKernelGGL(skinny_splitk_reduce_kernel<OUT>, dim3(rg), dim3(256), 0, s, a.workspace, S,
+  AG_LAUNCH_KERNEL(skinny_splitk_reduce_kernel<OUT>, dim3(rg), dim3(256), 0, s, a.workspace, S,
                      a.M, a.N, a.ldc, a.scale_a, a.scale_b, a.bias, a.C);
 }
 
@@ -1055,7 +1055,9 @@ int launch_skinny_fp4m_t(const GemmArgs& a0, int S, hipStream_t s) {
   if (S > 1 && !a.workspace) {
     if (int rc = splitk_workspace((size_t)S * a.M * a.N * sizeof(float), s, &a.workspace)) return rc;
   }
-  hipLaunchKernelGGL(k, dim3(kg.grid), dim3(512), lds, s, a);
+  AG_LAUNCH_KERNEL(k, dim3(kg.grid), dim3(512), lds, s, a);
+  // the partial sums must exist before anything adds them: a failed launch ends here
+  if (const hipError_t e = hipGetLastError(); e != hipSuccess) return (int)e;
   if (S > 1) launch_splitk_reduce<OUT>(a, S, s);
   return (int)hipGetLastError();
 }
@@ -1395,7 +1397,9 @@ int launch_skinny_regm_t(const GemmArgs& a0, int S, hipStream_t s) {
   if (S > 1 && !a.workspace) {
     if (int rc = splitk_workspace((size_t)S * a.M * a.N * sizeof(float), s, &a.workspace)) return rc;
   }
-  hipLaunchKernelGGL(k, dim3(kg.grid), dim3(512), lds, s, a);
+  AG_LAUNCH_KERNEL(k, dim3(kg.grid), dim3(512), lds, s, a);
+  // the partial sums must exist before anything adds them: a failed launch ends here
+  if (const hipError_t e = hipGetLastError(); e != hipSuccess) return (int)e;
   if (S > 1) launch_splitk_reduce<OUT>(a, S, s);
   return (int)hipGetLastError();
 }
@@ -1635,7 +1639,7 @@ int launch_skinny_direct_t(const GemmArgs& a, hipStream_t s) {
   if (cus <= 0) return (int)hipErrorNoDevice;
   const int nblocks = (int)((a.N + 15) / 16);
   const int g = nblocks < cus ? nblocks : cus;
-  hipLaunchKernelGGL(k, dim3(g), dim3(512), lds, s, a);
+  AG_LAUNCH_KERNEL(k, dim3(g), dim3(512), lds, s, a);
   return (int)hipGetLastError();
 }
 
@@ -1865,7 +1869,7 @@ int launch_skinny_directb_t(const GemmArgs& a, hipStream_t s) {
     return (int)hipErrorInvalidValue;
   const int nblocks = (int)(a.N / 16);
   const int g = nblocks < cus ? nblocks : cus;
-  hipLaunchKernelGGL(k, dim3(g), dim3(512), lds, s, a);
+  AG_LAUNCH_KERNEL(k, dim3(g), dim3(512), lds, s, a);
   return (int)hipGetLastError();
 }
 
@@ -1900,7 +1904,7 @@ const char* check_skinny_directb(const astergemm_config& c) {
 
 template <int DT, int OUT, int MT, int NB, int KW, int U>
 int launch_skinny(const GemmArgs& a, int grid, hipStream_t s) {
-  hipLaunchKernelGGL((gemm_skinny_kernel<DT, OUT, MT, NB, KW, U>), dim3(grid), dim3(KW * 64), 0,
+  AG_LAUNCH_KERNEL((gemm_skinny_kernel<DT, OUT, MT, NB, KW, U>), dim3(grid), dim3(KW * 64), 0,
                      s, a);
   return (int)hipGetLastError();
 }

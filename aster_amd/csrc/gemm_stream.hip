@@ -20,7 +20,7 @@ int launch_stream(const GemmArgs& a, int grid, hipStream_t s) {
   auto k = gemm_stream_kernel<DT, OUT, BM, BN, WM, WN>;
   static std::atomic<uint64_t> attr_devs{0};
   if (int e = lds_attr_once(attr_devs, (const void*)k, lds)) return e;
-  hipLaunchKernelGGL(k, dim3(grid), dim3(WM * WN * 64), lds, s, a);
+  AG_LAUNCH_KERNEL(k, dim3(grid), dim3(WM * WN * 64), lds, s, a);
   return (int)hipGetLastError();
 }
 
@@ -62,7 +62,7 @@ int launch_streamdb(const GemmArgs& a, int grid, hipStream_t s) {
   if (a.N % 16 != 0 || a.N < 16 || a.M < 8 || a.M % 8 != 0 || a.K % 64 != 0 || a.tail_granules != 0 ||
       a.ldb_bytes != (int64_t)a.K * 2)
     return (int)hipErrorInvalidValue;
-  hipLaunchKernelGGL(k, dim3(grid), dim3(WM * 256), lds, s, a);
+  AG_LAUNCH_KERNEL(k, dim3(grid), dim3(WM * 256), lds, s, a);
   return (int)hipGetLastError();
 }
 
@@ -102,7 +102,7 @@ int launch_stream4db(const GemmArgs& a, int grid, hipStream_t s) {
       a.ldb_bytes != (int64_t)a.K / 2 || (((uintptr_t)a.mx_a | (uintptr_t)a.mx_b) & 15) != 0 ||
       a.mx_ld % 16 != 0)
     return (int)hipErrorInvalidValue;
-  hipLaunchKernelGGL(k, dim3(grid), dim3(256), lds, s, a);
+  AG_LAUNCH_KERNEL(k, dim3(grid), dim3(256), lds, s, a);
   return (int)hipGetLastError();
 }
 
@@ -139,7 +139,7 @@ int launch_stream8db(const GemmArgs& a, int grid, hipStream_t s) {
   if (a.N % 16 != 0 || a.N < 16 || a.M < 8 || a.M % 8 != 0 || a.K % 128 != 0 || a.tail_granules != 0 ||
       a.ldb_bytes != (int64_t)a.K)
     return (int)hipErrorInvalidValue;
-  hipLaunchKernelGGL(k, dim3(grid), dim3(256), lds, s, a);
+  AG_LAUNCH_KERNEL(k, dim3(grid), dim3(256), lds, s, a);
   return (int)hipGetLastError();
 }
 
@@ -191,7 +191,7 @@ int launch_stream_splitk(const GemmArgs& a0, int grid, hipStream_t s) {
   part.ksteps = a.ksteps / S;
   part.ldc = a.N;
   part.scale_a = part.scale_b = part.bias = nullptr;
-  hipLaunchKernelGGL(k, dim3(tiles * S), dim3(256), lds, s, part);
+  AG_LAUNCH_KERNEL(k, dim3(tiles * S), dim3(256), lds, s, part);
   return splitk_reduce(OUT, a, S, s);
 }
 
@@ -235,7 +235,7 @@ int launch_stream8(const GemmArgs& a, int grid, hipStream_t s) {
   auto k = gemm_stream8_kernel<DT, OUT, BM, BN, WM, WN>;
   static std::atomic<uint64_t> attr_devs{0};
   if (int e = lds_attr_once(attr_devs, (const void*)k, lds)) return e;
-  hipLaunchKernelGGL(k, dim3(grid), dim3(WM * WN * 64), lds, s, a);
+  AG_LAUNCH_KERNEL(k, dim3(grid), dim3(WM * WN * 64), lds, s, a);
   return (int)hipGetLastError();
 }
 
@@ -254,7 +254,7 @@ int launch_stream8_walk(const GemmArgs& a, int grid, hipStream_t s) {
   const int cus = device_cus();
   if (cus <= 0) return (int)hipErrorNoDevice;
   const int tiles = a.tiles_m * a.tiles_n;
-  hipLaunchKernelGGL(k, dim3(tiles < cus ? tiles : cus), dim3(512), lds, s, a);
+  AG_LAUNCH_KERNEL(k, dim3(tiles < cus ? tiles : cus), dim3(512), lds, s, a);
   return (int)hipGetLastError();
 }
 
@@ -307,7 +307,7 @@ int launch_stream4(const GemmArgs& a, int grid, hipStream_t s) {
   auto k = gemm_stream4_kernel<DT, OUT, BM, BN, WM, WN>;
   static std::atomic<uint64_t> attr_devs{0};
   if (int e = lds_attr_once(attr_devs, (const void*)k, lds)) return e;
-  hipLaunchKernelGGL(k, dim3(grid), dim3(WM * WN * 64), lds, s, a);
+  AG_LAUNCH_KERNEL(k, dim3(grid), dim3(WM * WN * 64), lds, s, a);
   return (int)hipGetLastError();
 }
 
@@ -356,7 +356,7 @@ int launch_stream4_walk(const GemmArgs& a, int grid, hipStream_t s) {
   const int cus = device_cus();
   if (cus <= 0) return (int)hipErrorNoDevice;
   const int tiles = a.tiles_m * a.tiles_n;
-  hipLaunchKernelGGL(k, dim3(tiles < cus ? tiles : cus), dim3(512), lds, s, a);
+  AG_LAUNCH_KERNEL(k, dim3(tiles < cus ? tiles : cus), dim3(512), lds, s, a);
   return (int)hipGetLastError();
 }
 

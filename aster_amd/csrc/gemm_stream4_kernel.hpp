@@ -49,7 +49,9 @@ __device__ __forceinline__ void gemm_stream4_body(const GemmArgs& p, int bid, in
   constexpr int TM = BM / WM / 16;
   constexpr int TN = BN / WN / 16;
   constexpr int SLOT = BM * kRowBytes;  // 32 KiB: one operand half of one K-step
-  constexpr int LH = BM / 8 / NW;       // 1 KiB transfers per wave and slot
+  using Plan = StreamLoadPlan<BM, NW>;  // the staging as a cooperative load plan (stream_load_plan.inc)
+  constexpr int LH = Plan::LH;       // 1 KiB transfers per wave and slot
+  static_assert(Plan::TILE_ROWS == 8 && Plan::TILE_LDS_BYTES == 8 * kRowBytes, "transfer tile");
   constexpr int NMF = TM * TN;          // slots per trip (two MFMAs each)
   constexpr int BAR = (TN - 2) * TM + 4;  // slots of a trip issued ahead of its barrier
   constexpr int NSR = BM / 64;          // scale transfers per operand and chunk (64 rows each)
@@ -96,8 +98,8 @@ __device__ __forceinline__ void gemm_stream4_body(const GemmArgs& p, int bid, in
       t.a[0] = p.A + (int64_t)(t.row0 + wave * 8) * p.lda_bytes;
       t.b[0] = p.B + (int64_t)(t.col0 + wave * 8) * p.ldb_bytes;
     } else {
-      group_bases<LH, NW>(p.A, p.lda_bytes, t.row0 + wave * 8, p.M, t.a);
-      group_bases<LH, NW>(p.B, p.ldb_bytes, t.col0 + wave * 8, p.N, t.b);
+      group_bases<Plan>(p.A, p.lda_bytes, t.row0, wave, p.M, t.a);
+      group_bases<Plan>(p.B, p.ldb_bytes, t.col0, wave, p.N, t.b);
     }
     // scales: transfer x = wave + i * NW (0..7): x < 4 covers A rows [64x, +64), else B rows
     // [64(x-4), +64); lane L brings the 16 scale bytes of row L for chunk c (K-steps 2c and
@@ -127,11 +129,11 @@ __device__ __forceinline__ void gemm_stream4_body(const GemmArgs& p, int bid, in
   // K-step k of tile t into ring slot `slot` (A: 0..1, B: 2..3)
   auto issue_a1 = [&](const Src& t, int k, int slot, int j) {
     const uint8_t* base = WALK ? t.a[0] + (int64_t)j * (8 * NW) * p.lda_bytes : t.a[j];
-    g2s(base + (int64_t)k * kRowBytes, a_off, lds + slot * SLOT + (j * NW + wave) * 8 * kRowBytes);
+    g2s(base + (int64_t)k * kRowBytes, a_off, lds + slot * SLOT + Plan::lds_offset(wave, j));
   };
   auto issue_b1 = [&](const Src& t, int k, int slot, int j) {
     const uint8_t* base = WALK ? t.b[0] + (int64_t)j * (8 * NW) * p.ldb_bytes : t.b[j];
-    g2s(base + (int64_t)k * kRowBytes, b_off, lds + slot * SLOT + (j * NW + wave) * 8 * kRowBytes);
+    g2s(base + (int64_t)k * kRowBytes, b_off, lds + slot * SLOT + Plan::lds_offset(wave, j));
   };
   // scale chunk c of tile t into scale buffer `buf`
   auto issue_scales = [&](const Src& t, int c, int buf) {

@@ -42,7 +42,9 @@ __device__ __forceinline__ void gemm_stream8_body(const GemmArgs& p, int bid, in
   constexpr int TM = BM / WM / 16;
   constexpr int TN = BN / WN / 16;
   constexpr int SLOT = BM * kRowBytes;  // 32 KiB: one operand half of one K-step
-  constexpr int LH = BM / 8 / NW;       // 1 KiB transfers per wave and slot
+  using Plan = StreamLoadPlan<BM, NW>;  // the staging as a cooperative load plan (stream_load_plan.inc)
+  constexpr int LH = Plan::LH;       // 1 KiB transfers per wave and slot
+  static_assert(Plan::TILE_ROWS == 8 && Plan::TILE_LDS_BYTES == 8 * kRowBytes, "transfer tile");
   constexpr int NMF = TM * TN;
   // MFMAs of a trip issued ahead of its barrier: behind the last read of B(k), at MFMA
   // (TN-2)*TM, and not behind the first read of K-step k+1, at MFMA (TN-1)*TM
@@ -85,8 +87,8 @@ __device__ __forceinline__ void gemm_stream8_body(const GemmArgs& p, int bid, in
       a_base[0] = p.A + (int64_t)(row0 + wave * 8) * p.lda_bytes;
       b_base[0] = p.B + (int64_t)(col0 + wave * 8) * p.ldb_bytes;
     } else {
-      group_bases<LH, NW>(p.A, p.lda_bytes, row0 + wave * 8, p.M, a_base);
-      group_bases<LH, NW>(p.B, p.ldb_bytes, col0 + wave * 8, p.N, b_base);
+      group_bases<Plan>(p.A, p.lda_bytes, row0, wave, p.M, a_base);
+      group_bases<Plan>(p.B, p.ldb_bytes, col0, wave, p.N, b_base);
     }
   };
   set_tile(bid);
@@ -101,11 +103,11 @@ __device__ __forceinline__ void gemm_stream8_body(const GemmArgs& p, int bid, in
   };
   auto issue_a1 = [&](int k, int slot, int j) {  // slot: 0..2
     const uint8_t* base = WALK ? a_base[0] + (int64_t)j * (8 * NW) * p.lda_bytes : a_base[j];
-    g2s(base + (int64_t)k * kRowBytes, a_off, lds + slot * SLOT + (j * NW + wave) * 8 * kRowBytes);
+    g2s(base + (int64_t)k * kRowBytes, a_off, lds + slot * SLOT + Plan::lds_offset(wave, j));
   };
   auto issue_b1 = [&](int k, int slot, int j) {  // slot: 3..4
     const uint8_t* base = WALK ? b_base[0] + (int64_t)j * (8 * NW) * p.ldb_bytes : b_base[j];
-    g2s(base + (int64_t)k * kRowBytes, b_off, lds + slot * SLOT + (j * NW + wave) * 8 * kRowBytes);
+    g2s(base + (int64_t)k * kRowBytes, b_off, lds + slot * SLOT + Plan::lds_offset(wave, j));
   };
   auto issue_a = [&](int k, int slot) {
 #pragma unroll

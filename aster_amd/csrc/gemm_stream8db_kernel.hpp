@@ -35,7 +35,9 @@ __device__ __forceinline__ void gemm_stream8db_body(const GemmArgs& p, int bid) 
   constexpr int SLOT = BM * kRowBytes;  // 16 KiB: A rows of one K-step
   constexpr int NSLOT = 4;              // A ring
   constexpr int NBUF = 2;               // B register buffers of one K-step each
-  constexpr int LH = BM / 8 / NW;       // 4 transfers of 1 KiB per wave and slot
+  using Plan = StreamLoadPlan<BM, NW>;  // the staging as a cooperative load plan (stream_load_plan.inc)
+  constexpr int LH = Plan::LH;       // 4 transfers of 1 KiB per wave and slot
+  static_assert(Plan::TILE_ROWS == 8 && Plan::TILE_LDS_BYTES == 8 * kRowBytes, "transfer tile");
   constexpr int RA = 4;                 // A fragment ring
   constexpr int MS = TM;                // m-steps per K-step
   constexpr int BAR = MS - (RA - 1);    // m-step whose first MFMA follows the barrier
@@ -60,7 +62,7 @@ __device__ __forceinline__ void gemm_stream8db_body(const GemmArgs& p, int bid) 
   const int g_lane = (lane & 7) ^ (((wave * 8 + lrow) >> 1) & 7);
   const unsigned a_off = (unsigned)(lrow * (int)p.lda_bytes + g_lane * 16);
   const uint8_t* a_base[LH];
-  group_bases<LH, NW>(p.A, p.lda_bytes, row0 + wave * 8, p.M, a_base);
+  group_bases<Plan>(p.A, p.lda_bytes, row0, wave, p.M, a_base);
   auto g2s = [&](const uint8_t* base, unsigned voff, uint8_t* dst) {
     const unsigned m0v = (unsigned)(size_t)AG_LDS(dst);
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
@@ -70,7 +72,7 @@ __device__ __forceinline__ void gemm_stream8db_body(const GemmArgs& p, int bid) 
   };
   auto issue_a1 = [&](int k, int slot, int j) {
     g2s(a_base[j] + (int64_t)k * kRowBytes, a_off,
-        lds + slot * SLOT + (j * NW + wave) * 8 * kRowBytes);
+        lds + slot * SLOT + Plan::lds_offset(wave, j));
   };
 
   // ---- B: global -> registers.  A raw buffer over the payload; a load is resource + scalar

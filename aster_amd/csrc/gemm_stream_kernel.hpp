@@ -31,6 +31,7 @@
 #include <type_traits>
 
 #include "gemm_tile_kernel.hpp"
+#include "stream_load_plan.inc"
 
 namespace astergemm {
 namespace {
@@ -55,13 +56,13 @@ __device__ __forceinline__ void static_for(Fn&& f) {
 // transfers.  Operand heights are multiples of 8, so a group lies either inside the matrix or
 // wholly past its end; the latter re-read the last 8 rows (their products land in output rows
 // or columns the epilogue does not store).
-template <int LH, int NW>
-__device__ __forceinline__ void group_bases(const uint8_t* mat, int64_t ld_bytes, int first_row,
-                                            int rows, const uint8_t* (&out)[LH]) {
+template <class Plan>
+__device__ __forceinline__ void group_bases(const uint8_t* mat, int64_t ld_bytes, int tile_row0, int wave,
+                                            int rows, const uint8_t* (&out)[Plan::LH]) {
 #pragma unroll
-  for (int j = 0; j < LH; ++j) {
-    int r = first_row + j * 8 * NW;
-    r = r < rows - 8 ? r : rows - 8;
+  for (int j = 0; j < Plan::LH; ++j) {
+    int r = tile_row0 + Plan::first_row(wave, j);
+    r = r < rows - Plan::TILE_ROWS ? r : rows - Plan::TILE_ROWS;
     out[j] = mat + (int64_t)r * ld_bytes;
   }
 }
@@ -261,7 +262,9 @@ __device__ __forceinline__ void gemm_stream_body(const GemmArgs& p, int bid) {
   constexpr int TN = BN / WN / 16;
   constexpr int SLOT = BM * kRowBytes;  // 32 KiB: one operand half of one K-step
   constexpr int NSLOT = 5;
-  constexpr int LH = BM / 8 / NW;       // 1 KiB (8 rows x 128 B) transfers per wave and slot
+  using Plan = StreamLoadPlan<BM, NW>;  // the staging as a cooperative load plan (stream_load_plan.inc)
+  constexpr int LH = Plan::LH;       // 1 KiB (8 rows x 128 B) transfers per wave and slot
+  static_assert(Plan::TILE_ROWS == 8 && Plan::TILE_LDS_BYTES == 8 * kRowBytes, "transfer tile");
   constexpr bool AX = NW == 4;          // one wave per SIMD: accumulators in accumulation registers
   static_assert(BM == BN, "the ring holds equal A and B halves");
   static_assert(DT == ASTERGEMM_BF16 || DT == ASTERGEMM_F16, "16-bit operands");
@@ -289,8 +292,8 @@ __device__ __forceinline__ void gemm_stream_body(const GemmArgs& p, int bid) {
   const unsigned b_off = (unsigned)(lrow * (int)p.ldb_bytes + g_lane * 16);
   const uint8_t* a_base[LH];
   const uint8_t* b_base[LH];
-  group_bases<LH, NW>(p.A, p.lda_bytes, row0 + wave * 8, p.M, a_base);
-  group_bases<LH, NW>(p.B, p.ldb_bytes, col0 + wave * 8, p.N, b_base);
+  group_bases<Plan>(p.A, p.lda_bytes, row0, wave, p.M, a_base);
+  group_bases<Plan>(p.B, p.ldb_bytes, col0, wave, p.N, b_base);
   const int nk = p.ksteps - (p.tail_granules ? 1 : 0);  // whole 128-byte steps
 
   // 64 lanes x 16 bytes from (scalar base + per-lane offset) to LDS at M0 + lane*16.
@@ -305,11 +308,11 @@ __device__ __forceinline__ void gemm_stream_body(const GemmArgs& p, int bid) {
   // transfer j (0..LH-1) of this wave for the A / B half of K-step k
   auto issue_a1 = [&](int k, int slot, int j) {
     g2s(a_base[j] + (int64_t)k * kRowBytes, a_off,
-        lds + slot * SLOT + (j * NW + wave) * 8 * kRowBytes);
+        lds + slot * SLOT + Plan::lds_offset(wave, j));
   };
   auto issue_b1 = [&](int k, int slot, int j) {
     g2s(b_base[j] + (int64_t)k * kRowBytes, b_off,
-        lds + slot * SLOT + (j * NW + wave) * 8 * kRowBytes);
+        lds + slot * SLOT + Plan::lds_offset(wave, j));
   };
   auto issue_a = [&](int k, int slot) {
 #pragma unroll

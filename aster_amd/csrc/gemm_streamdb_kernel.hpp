@@ -45,7 +45,9 @@ __device__ __forceinline__ void gemm_streamdb_body(const GemmArgs& p, int bid) {
   constexpr int TM = BM / WM / 16;      // 8
   constexpr int TN = BN / WN / 16;      // 4
   constexpr int SLOT = BM * kRowBytes;  // 32 (16) KiB: A rows of one K-step
-  constexpr int LH = BM / 8 / NW;       // 4 transfers of 1 KiB per wave and slot
+  using Plan = StreamLoadPlan<BM, NW>;  // the staging as a cooperative load plan (stream_load_plan.inc)
+  constexpr int LH = Plan::LH;       // 4 transfers of 1 KiB per wave and slot
+  static_assert(Plan::TILE_ROWS == 8 && Plan::TILE_LDS_BYTES == 8 * kRowBytes, "transfer tile");
   // NSLOT A slots in LDS, NBUF B register buffers of one MFMA substep each; the loop is unrolled
   // over NSLOT trips, after which slot and buffer numbers repeat
   static_assert(NBUF == NSLOT || NBUF == 2 * NSLOT, "buffer numbers repeat with the slots");
@@ -78,7 +80,7 @@ __device__ __forceinline__ void gemm_streamdb_body(const GemmArgs& p, int bid) {
   const int g_lane = (lane & 7) ^ (((wave * 8 + lrow) >> 1) & 7);
   const unsigned a_off = (unsigned)(lrow * (int)p.lda_bytes + g_lane * 16);
   const uint8_t* a_base[LH];
-  group_bases<LH, NW>(p.A, p.lda_bytes, row0 + wave * 8, p.M, a_base);
+  group_bases<Plan>(p.A, p.lda_bytes, row0, wave, p.M, a_base);
   auto g2s = [&](const uint8_t* base, unsigned voff, uint8_t* dst) {
     const unsigned m0v = (unsigned)(size_t)AG_LDS(dst);
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
@@ -88,7 +90,7 @@ __device__ __forceinline__ void gemm_streamdb_body(const GemmArgs& p, int bid) {
   };
   auto issue_a1 = [&](int k, int slot, int j) {
     g2s(a_base[j] + (int64_t)k * kRowBytes, a_off,
-        lds + slot * SLOT + (j * NW + wave) * 8 * kRowBytes);
+        lds + slot * SLOT + Plan::lds_offset(wave, j));
   };
 
   // ---- B: global -> registers.  Scalar base of the wave's n-tile `n` (16 rows of B, clamped to

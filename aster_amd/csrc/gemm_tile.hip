@@ -12,7 +12,7 @@ int launch_tile(const GemmArgs& a, int grid, hipStream_t s) {
   auto k = gemm_tile_kernel<DT, OUT, BM, BN, WM, WN>;
   static std::atomic<uint64_t> attr_devs{0};
   if (int e = lds_attr_once(attr_devs, (const void*)k, lds)) return e;
-  hipLaunchKernelGGL(k, dim3(grid), dim3(WM * WN * 64), lds, s, a);
+  AG_LAUNCH_KERNEL(k, dim3(grid), dim3(WM * WN * 64), lds, s, a);
   return (int)hipGetLastError();
 }
 

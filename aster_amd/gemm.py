@@ -234,6 +234,12 @@ class GemmPlan:
         ops.dWorkspace, ops.workspace_bytes = workspace, workspace_bytes
         return ops
 
+    def prepare(self) -> None:
+        """Everything a first launch of this plan's kernel does on the current device apart from
+        launching (function attributes, cached device facts): call before capturing launches
+        of the plan into a HIP graph."""
+        _capi.check(_capi.load().astergemm_prepare(ctypes.byref(self.config)))
+
     def workspace_bytes(self) -> int:
         """Bytes of fp32 workspace a launch of this plan needs (0 unless its rows are cut into
         K ranges); pass a buffer of that size as `workspace` to `run`, or leave it to the

@@ -233,10 +233,27 @@ int astergemm_workspace_bytes(const astergemm_config* cfg, size_t* bytes);
  * its stream: calls that overlap on one device race (calls on one stream are
  * ordered and safe).  Nothing in the array has to start at zero: every launch
  * writes all the planes it later adds.  The array's address is looked up on
- * the first call on a device, or by aster_rt_init for the current device.     */
+ * the first call on a device, or by aster_rt_init / astergemm_prepare for the
+ * current device.  A kernel's FIRST launch on a device also sets a function
+ * attribute and is refused while the stream is being captured: call
+ * astergemm_prepare(cfg) (below) or launch the config once eagerly before
+ * capturing it.                                                              */
 #define ASTERGEMM_NOALLOC_SCRATCH_BYTES (16u << 20)
 int astergemm_run_noalloc(const astergemm_config* cfg, const astergemm_operands* ops,
                           void* stream);
+
+/* Does, for the kernel `cfg` selects on the current device, everything a first
+ * launch does apart from launching: raises the kernel's dynamic-LDS limit
+ * (hipFuncSetAttribute), caches the device's compute-unit count and looks up
+ * the address of the built-in scratch.  None of these is a stream operation,
+ * so they must not happen inside a stream capture: astergemm_run and
+ * astergemm_run_noalloc REFUSE a kernel's first launch on a device when the
+ * stream is being captured (ASTERGEMM_EHIP, the message names this function).
+ * Call it once per config and device before capturing (an eager launch of the
+ * same config does the same).  Allocates nothing when the config's partial
+ * sums fit the built-in scratch; reads no operand.  No counterpart in the
+ * reference, whose kernels carry their LDS size in the code object. */
+int astergemm_prepare(const astergemm_config* cfg);
 
 /* Replaces execute_fn's timed loop (execution/core.py:690-703): `iters`
  * launches, each bracketed by its own HIP event pair on `stream`;

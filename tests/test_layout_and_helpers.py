@@ -1,6 +1,7 @@
 """Layout algebra, swizzles, B pre-shuffle and the cooperative split."""
 import ctypes
 import itertools
+import os
 import math
 
 import numpy as np
@@ -236,6 +237,34 @@ def test_stream_kernel_staging_is_the_interleaved_coop_plan(tile_rows, num_waves
     # the slot is filled exactly once: every 1 KiB of it, every 8-row group of the tile
     assert sorted(lo for _, lo in everything) == [t * 1024 for t in range(tile_rows // 8)]
     assert sorted(go for go, _ in everything) == [t * 8 * ld for t in range(tile_rows // 8)]
+
+
+def test_stream_kernels_are_compiled_from_the_coop_plan():
+    """The header the stream kernels take LH, their operand rows and their LDS offsets from is the
+    text the plan generator writes (the build rewrites it before compiling), its constants are
+    the plan's, and no kernel source restates the staging formula."""
+    import glob
+    import re
+    from aster_amd.build import CSRC, PLAN_HEADER
+    from aster_amd.coop import STREAM_PLAN_CONFIGS, stream_kernel_load_plan, stream_load_plan_header
+    with open(PLAN_HEADER) as f:
+        text = f.read()
+    assert text == stream_load_plan_header()
+    for rows, nw in STREAM_PLAN_CONFIGS:
+        body = text[text.index(f"struct StreamLoadPlan<{rows}, {nw}>"):]
+        body = body[:body.index("};")]
+        const = {k: int(v) for k, v in re.findall(r"static constexpr int (\w+) = (\d+);", body)}
+        for w in range(nw):
+            plan = stream_kernel_load_plan(w, tile_rows=rows, num_waves=nw, ld_bytes=4096)
+            assert const["LH"] == plan.global_layout.sizes[0]
+            for j, (go, lo) in enumerate(plan.transfers()):
+                tile = w * const["WAVE_STEP_TILES"] + j * const["XFER_STEP_TILES"]
+                assert go == tile * const["TILE_ROWS"] * 4096 and lo == tile * const["TILE_LDS_BYTES"]
+    for path in glob.glob(os.path.join(CSRC, "gemm_stream*_kernel.hpp")):
+        with open(path) as f:
+            src = f.read()
+        assert "StreamLoadPlan<BM, NW>" in src, path
+        assert "j * NW + wave" not in src and "BM / 8 / NW" not in src, path
 
 
 def test_shuffle_weight_bytes_is_the_operand_order_of_the_16x16x128_mfma():

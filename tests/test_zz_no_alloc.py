@@ -7,6 +7,7 @@ one that needs more than the array holds are covered as well, and so is a HIP gr
 two launches of it and is replayed on fresh activations.
 """
 import ctypes
+import os
 
 import numpy as np
 import pytest
@@ -173,3 +174,77 @@ def test_noalloc_launches_replay_from_a_graph(gpu):
         _capi.check(rt.aster_rt_stream_destroy(stream))
         for bf in (dx, dw1, dw2, dh, dy):
             bf.free()
+
+
+_CAPTURE_CHILD = r"""
+import ctypes, sys
+import numpy as np
+from aster_amd import _capi, gemm as AG
+from aster_amd.execution import GpuBuffer
+
+lib = _capi.load()
+for name, args in (("hipStreamBeginCapture", [ctypes.c_void_p, ctypes.c_int]),
+                   ("hipStreamEndCapture", [ctypes.c_void_p, ctypes.POINTER(ctypes.c_void_p)]),
+                   ("hipGraphInstantiate", [ctypes.POINTER(ctypes.c_void_p), ctypes.c_void_p,
+                                            ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t]),
+                   ("hipGraphLaunch", [ctypes.c_void_p, ctypes.c_void_p])):
+    fn = getattr(lib, name)
+    fn.argtypes, fn.restype = args, ctypes.c_int
+_capi.check(lib.aster_rt_init())
+M, N, K = 16, 4096, 14336                      # rows cut into K ranges: partial sums in the scratch
+rng = np.random.default_rng(3)
+x = (rng.standard_normal((M, K)).astype(np.float32)).view(np.uint32) >> 16
+w = (rng.standard_normal((N, K)).astype(np.float32) * 0.02).view(np.uint32) >> 16
+x, w = x.astype(np.uint16), w.astype(np.uint16)
+dx, dw, dy = GpuBuffer(x.nbytes), GpuBuffer(w.nbytes), GpuBuffer(M * N * 2)
+dx.copy_from_host(x)
+dw.copy_from_host(w)
+plan = AG.GemmPlan.create(M, N, K, "bf16", "bf16")
+stream, graph, gexec = ctypes.c_void_p(), ctypes.c_void_p(), ctypes.c_void_p()
+_capi.check(lib.aster_rt_stream_create(ctypes.byref(stream)))
+
+# 1. nothing of this config has run in this process: its first launch inside a capture is refused
+assert lib.hipStreamBeginCapture(stream, 0) == 0
+try:
+    plan.run_noalloc(dx.ptr_value, dw.ptr_value, dy.ptr_value, stream=stream.value)
+    refused = None
+except _capi.AsterGemmError as exc:
+    refused = str(exc)
+rc = lib.hipStreamEndCapture(stream, ctypes.byref(graph))
+assert refused and "astergemm_prepare" in refused, refused
+print("refused:", refused, flush=True)
+
+# 2. after astergemm_prepare the same capture goes through, and the replay gives the eager bits
+plan.prepare()
+assert lib.hipStreamBeginCapture(stream, 0) == 0
+plan.run_noalloc(dx.ptr_value, dw.ptr_value, dy.ptr_value, stream=stream.value)
+assert lib.hipStreamEndCapture(stream, ctypes.byref(graph)) == 0 and graph.value
+assert lib.hipGraphInstantiate(ctypes.byref(gexec), graph, None, None, 0) == 0
+got = []
+for _ in range(2):
+    dy.copy_from_host(np.full((M, N), 0x7FC1, np.uint16))
+    assert lib.hipGraphLaunch(gexec, stream) == 0
+    _capi.check(lib.aster_rt_stream_synchronize(stream))
+    y = np.zeros((M, N), np.uint16)
+    dy.copy_to_host(y)
+    got.append(y)
+plan.run(dx.ptr_value, dw.ptr_value, dy.ptr_value)
+_capi.check(lib.aster_rt_device_synchronize())
+eager = np.zeros((M, N), np.uint16)
+dy.copy_to_host(eager)
+assert np.array_equal(got[0], eager) and np.array_equal(got[1], eager)
+print("CAPTURE-OK", flush=True)
+"""
+
+
+def test_first_launch_inside_a_capture_is_refused_until_prepared(gpu):
+    # in a process of its own, so that no earlier test has launched the kernel: the first launch of
+    # a kernel on a device sets a function attribute, which must not happen inside a capture; the
+    # library refuses it and astergemm_prepare does that step ahead of time
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    print("child process: capture before / after astergemm_prepare", flush=True)
+    proc = subprocess.run([sys.executable, "-c", _CAPTURE_CHILD], cwd=root, capture_output=True, text=True,
+                          timeout=110)
+    assert proc.returncode == 0 and "CAPTURE-OK" in proc.stdout, proc.stdout[-2000:] + proc.stderr[-2000:]
