@@ -8,7 +8,9 @@ Mirrors the parts of the reference's bench harness that define what is measured
 `run_single` :1738-1850) and the `BENCH_RESULT_JSON:` line
 (tools/perf_bench_results_io.py:15, 113-144).  The compile pool, GPU workers and
 tiered config search of that file drive the reference's compiler and have no
-counterpart here.
+counterpart here; `bench_perf_sweep` is the sweep in this build's terms: mappings -> select ->
+time -> result lines -> registry dashboard, in one process and one command
+(`python -m aster_amd.bench_harness --m ... --n ... --k ...`).
 """
 
 from __future__ import annotations
@@ -280,3 +282,147 @@ def run_single(cfg, compile_fn, args, execute_fn, *, bench: str = "unknown", out
                 os.unlink(tmp.name)
             except OSError:
                 pass
+
+
+def mapping_candidates(M: int, N: int, K: int, *, dtype_ab: str = "bf16", dtype_c: str = "bf16"):
+    """The mappings a sweep over one problem tries: every workgroup tile / wave grid the pre-built
+    stream kernels have, on both operand paths, that divides the problem (the weak-scale rule of
+    `make_instance`).  The reference enumerates a much larger grid of compiler knobs
+    (bench_perf_102_gemm_python_multitile_g2s_directb_cdna4.py:170-290); here a mapping can only
+    steer the tile, the wave grid and the operand path, and mappings that resolve to the same
+    kernel are timed once."""
+    from .gemm_config import OperandPath, make_instance
+
+    out = []
+    for (tile, waves) in (((256, 256), (2, 4)), ((256, 256), (2, 2)), ((128, 256), (1, 4)), ((128, 128), (2, 2))):
+        if M % tile[0] or N % tile[1]:
+            continue
+        for path in (OperandPath.LDS, OperandPath.DIRECT_B):
+            try:
+                out.append(make_instance(M, N, K, dtype_ab=dtype_ab, dtype_c=dtype_c, wg_tile=tile,
+                                         waves=waves, operand_path=path))
+            except (AssertionError, ValueError):
+                continue
+    return out
+
+
+def bench_perf_sweep(configs, compile_fn, execute_fn, repro_cmd_fn=None, *, mcpu: str = "gfx950",
+                     bench: str = "unknown", iterations: Optional[int] = None,
+                     init_mode=INIT_DEFAULT, results_file: Optional[str] = None,
+                     best_known_file: Optional[str] = None, apply: bool = False, out=sys.stdout):
+    """Every config of `configs` through compile (select) -> timed launches -> one
+    `BENCH_RESULT_JSON:` line each, then the lines against the best-known registry
+    (OK / IMPROVE / REGRESS per size; `apply` writes new winners back).  Same interface idea as
+    the reference's `bench_perf_sweep_pipelined` (bench_harness.py:1271-1501: configs, compile_fn,
+    repro_cmd_fn, bench label, iterations, results file) without its process pools: nothing is
+    compiled at run time, so one process does the whole sweep.  Configs that select the same
+    pre-built kernel for the same problem are timed once and listed as aliases.
+
+    Returns (results, selected): results = [(cfg, PerfStats)] sorted by p50, selected =
+    {"label|operand path": kernel name}."""
+    import json as _json
+    import os
+    import tempfile
+
+    from . import perf_registry as R
+    from .execution import system_has_gpu
+
+    iterations = iterations or NUM_ITERATIONS
+    configs = list(configs)
+    selected, groups, failed = {}, {}, []
+    tmpdir = tempfile.mkdtemp(prefix="astergemm_sweep_")
+    for cfg in configs:
+        path = os.path.join(tmpdir, f"{len(selected)}.hsaco")
+        try:
+            compile_fn(cfg, path)
+            with open(path) as f:
+                desc = _json.load(f)
+        except Exception as exc:  # a mapping no kernel takes: reported, the sweep goes on
+            failed.append((cfg, f"compile: {str(exc).splitlines()[0][:200]}"))
+            continue
+        selected[f"{cfg.label}|{cfg.mapping.operand_path.value}"] = desc["kernel"]
+        key = (desc["kernel"], tuple(cfg.spec.gemm_size))
+        groups.setdefault(key, []).append((cfg, path, desc))
+    print(f"Sweep: {len(configs)} configs -> {len(groups)} distinct kernels, "
+          f"{len(failed)} refused, {iterations} iterations each", file=out)
+    results = []
+    have_gpu = system_has_gpu(mcpu)
+    if not have_gpu:
+        print("No GPUs detected -- execution skipped.", file=out)
+    for (kernel, size), members in (groups.items() if have_gpu else ()):
+        # the mapping the kernel honours stands for the group; the others ran the same code
+        members.sort(key=lambda m: not m[2].get("mapping_honoured", False))
+        cfg, path, desc = members[0]
+        try:
+            A, B = make_inputs(cfg, init_mode)
+            _, times_ns = execute_fn(cfg, path, iterations, A, B, skip_gpu_check=True)
+            s = _compute_stats(times_ns[WARMUP_ITERATIONS:], cfg.total_flops,
+                               peak_tflops(cfg.mapping.mcpu, cfg.spec.dtype_ab))
+            if s is None:
+                raise RuntimeError("no valid timings")
+        except Exception as exc:
+            failed.append((cfg, f"exec: {str(exc).splitlines()[0][:200]}"))
+            continue
+        # the reference's labels do not name the operand path: a run on pre-shuffled B, like a
+        # mapping that was not honoured, is recorded under the name of the kernel that ran
+        plain = cfg.mapping.operand_path.value == "lds"
+        label = cfg.label if desc.get("mapping_honoured", False) and plain else kernel
+        results.append((cfg, s))
+        if results_file:
+            with open(results_file, "a") as rs:
+                emit_one_result(rs, bench, cfg, s, label=label)
+        aliases = [m[0].label for m in members[1:]]
+        print(f"  {s.p50_tf:8.1f} TF p50 ({s.p50_pct:5.1f} % peak)  {kernel}  <- {label}"
+              + (f"  (+{len(aliases)} mappings that select the same kernel)" if aliases else ""), file=out)
+    results.sort(key=lambda r: -r[1].p50_tf)
+    for cfg, why in failed:
+        print(f"  FAILED {cfg.label}: {why}"
+              + (f"   repro: {repro_cmd_fn(cfg)}" if repro_cmd_fn else ""), file=out)
+    if results and results_file and best_known_file is not None:
+        data = R.load(best_known_file) if os.path.exists(best_known_file) else {}
+        with open(results_file) as f:
+            records = [r for r in R.parse_jsonl_results(f) if r.key.bench == bench]
+        rows = R.dashboard_rows(data, records, mcpu=mcpu, bench=bench)
+        print(R.render(rows), file=out)
+        print(R.summarize(rows, allow_missing=True)[0], file=out)
+        if apply:
+            n = R.update_top_n(data, records)
+            R.save(data, best_known_file)
+            print(f"{n} slot(s) updated in {best_known_file}", file=out)
+    return results, selected
+
+
+def main(argv=None) -> int:
+    """`python -m aster_amd.bench_harness --m M --n N --k K [--dtype bf16] ...`: the one-command
+    sweep over the mappings of one problem."""
+    import argparse
+
+    from . import gemm as AG
+    from . import perf_registry as R
+
+    ap = argparse.ArgumentParser(description="Sweep the mappings of one GEMM problem through the pre-built kernels")
+    ap.add_argument("--m", type=int, required=True)
+    ap.add_argument("--n", type=int, required=True)
+    ap.add_argument("--k", type=int, required=True)
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "f16"])
+    ap.add_argument("--out-dtype", default="bf16", choices=["bf16", "f16", "f32"])
+    ap.add_argument("--iterations", type=int, default=NUM_ITERATIONS)
+    ap.add_argument("--results-file", default="sweep_results.jsonl")
+    ap.add_argument("--best-known-file", default=R.DEFAULT_PATH)
+    ap.add_argument("--apply", action="store_true", help="write new winners into the registry")
+    args = ap.parse_args(argv)
+    bench = f"astergemm_{args.dtype}"
+    configs = mapping_candidates(args.m, args.n, args.k, dtype_ab=args.dtype, dtype_c=args.out_dtype)
+    if not configs:
+        print("no mapping divides this problem (M, N multiples of 128 are the smallest tile)")
+        return 2
+    results, _ = bench_perf_sweep(
+        configs, AG.compile_gemm, AG.execute_gemm_hsaco,
+        lambda cfg: f"python -m aster_amd.bench_harness --m {args.m} --n {args.n} --k {args.k}  # {cfg.label}",
+        bench=bench, iterations=args.iterations, results_file=args.results_file,
+        best_known_file=args.best_known_file, apply=args.apply)
+    return 0 if results else 1
+
+
+if __name__ == "__main__":
+    sys.exit(main())

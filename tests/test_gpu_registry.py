@@ -70,3 +70,26 @@ def test_unhonoured_mapping_is_recorded_under_the_kernel_that_ran(gpu, tmp_path)
     rec = next(R.parse_jsonl_results(open(results)))
     desc_kernel = AG.select_for_instance(cfg)[1].name.decode()
     assert rec.label == desc_kernel != cfg.label
+
+
+def test_one_command_sweep_over_mappings(gpu, tmp_path):
+    """Mappings of one problem -> select -> timed launches -> result lines -> registry, the shape
+    of the reference's `bench_perf_sweep_pipelined` (bench_harness.py:1271-1501) in one process:
+    mappings that select the same kernel are timed once, every timed kernel leaves a result line,
+    and `--apply` puts the fastest into the registry, which the next run reads as OK."""
+    results = tmp_path / "sweep.jsonl"
+    registry = tmp_path / "best_known.json"
+    argv = ["--m", "1024", "--n", "1024", "--k", "2048", "--iterations", "40",
+            "--results-file", str(results), "--best-known-file", str(registry)]
+    assert BH.main(argv + ["--apply"]) == 0
+    records = list(R.parse_jsonl_results(open(results)))
+    cfgs = BH.mapping_candidates(1024, 1024, 2048)
+    kernels = {AG.select_for_instance(c)[1].name.decode() for c in cfgs}
+    assert len(records) == len(kernels) >= 4          # 256x256 (2x4, 2x2), 128x256, 128x128, two paths
+    assert len({r.label for r in records}) == len(records)
+    assert all(10.0 < r.tflops_median < 2500.0 for r in records)
+    data = R.load(str(registry))
+    best = R.best_known(data, "gfx950", "astergemm_bf16", 1024, 1024, 2048)
+    assert best == max(records, key=lambda r: r.tflops_median).label
+    # the same measurements against the registry they produced: nothing regresses
+    assert R.main(["--measurements", str(results), "--best-known-file", str(registry)]) == 0
