@@ -192,6 +192,8 @@ int launch_stream_splitk(const GemmArgs& a0, int grid, hipStream_t s) {
   part.ldc = a.N;
   part.scale_a = part.scale_b = part.bias = nullptr;
   AG_LAUNCH_KERNEL(k, dim3(tiles * S), dim3(256), lds, s, part);
+  // the partial sums must exist before anything adds them: a failed launch ends here
+  if (const hipError_t e = hipGetLastError(); e != hipSuccess) return (int)e;
   return splitk_reduce(OUT, a, S, s);
 }
 
