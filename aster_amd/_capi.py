@@ -10,7 +10,9 @@ call fails, an exception is raised.
 from __future__ import annotations
 
 import ctypes as C
+import importlib.util
 import os
+import sys
 from typing import Optional
 
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libastergemm.so")
@@ -182,11 +184,33 @@ def library_path() -> str:
     return _LIB_PATH
 
 
+def _bind_one_hip_runtime() -> None:
+    """PyTorch's ROCm wheels carry a HIP runtime of their own (torch/lib/libamdhip64.so,
+    SONAME libamdhip64.so.7) and ask for it under the file name, not the SONAME.  Loaded after
+    the system's copy, which libastergemm.so would pull in when it comes first, the process holds
+    two runtimes, and the one that initialises second reports that it finds no device.  When
+    PyTorch is installed and not yet imported, its copy is therefore loaded first: the
+    library's request for libamdhip64.so.7 then resolves to it, and so does PyTorch's later.
+    A process without PyTorch keeps the system's runtime."""
+    if "torch" in sys.modules:
+        return
+    try:
+        spec = importlib.util.find_spec("torch")
+    except (ImportError, ValueError):
+        spec = None
+    if spec is None or not spec.origin:
+        return
+    path = os.path.join(os.path.dirname(spec.origin), "lib", "libamdhip64.so")
+    if os.path.exists(path):
+        C.CDLL(path, mode=C.RTLD_GLOBAL)
+
+
 def load() -> C.CDLL:
     """Load libastergemm.so and attach the prototypes. Raises if it is not built."""
     global _lib
     if _lib is not None:
         return _lib
+    _bind_one_hip_runtime()
     if not os.path.exists(_LIB_PATH):
         raise FileNotFoundError(
             f"{_LIB_PATH} is not built; run `python -m aster_amd.build` "

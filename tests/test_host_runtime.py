@@ -478,3 +478,18 @@ def test_direct_b_loads_of_edge_tiles_stay_inside_the_payload():
             plane = groups * (K // 256) * 512
             worst = max(min((col0 >> 6) + wn, groups - 1) + 1 for col0 in range(0, N, 256) for wn in range(4))
             assert worst * (K // 256) * 512 <= plane
+
+
+def test_library_and_pytorch_share_one_hip_runtime_whichever_loads_first():
+    """Loading the library before `import torch` must not leave two copies of the HIP runtime
+    in the process: the one initialised second finds no device."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = ("from aster_amd import _capi; _capi.load(); import torch\n"
+            "for name in ('libamdhip64', 'libhsa-runtime64'):\n"
+            "    paths = {l.split()[-1] for l in open('/proc/self/maps') if name in l}\n"
+            "    assert len(paths) == 1, paths\n"
+            "print('one runtime')\n")
+    out = subprocess.run([sys.executable, "-c", code], cwd=root, capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0 and "one runtime" in out.stdout, out.stderr[-2000:]
