@@ -23,7 +23,7 @@ F16, BF16, FP8_E4M3, MXFP4, F32 = 0, 1, 2, 3, 4
 SCALE_NONE, SCALE_TENSOR, SCALE_MX32 = 0, 1, 2
 # astergemm_kernel_family
 KERNEL_AUTO, KERNEL_TILE, KERNEL_SKINNY = 0, 1, 2
-OPERAND_LDS, OPERAND_DIRECT_B, OPERAND_DIRECT_B_K8 = 0, 1, 2
+OPERAND_LDS, OPERAND_DIRECT_B, OPERAND_DIRECT_B_K8, OPERAND_DIRECT_AB = 0, 1, 2, 3
 # astergemm_mx_layout
 MX_ROWS, MX_LANES128 = 0, 1
 ABI_VERSION = 3

@@ -286,7 +286,7 @@ def run_single(cfg, compile_fn, args, execute_fn, *, bench: str = "unknown", out
 
 def mapping_candidates(M: int, N: int, K: int, *, dtype_ab: str = "bf16", dtype_c: str = "bf16"):
     """The mappings a sweep over one problem tries: every workgroup tile / wave grid the pre-built
-    stream kernels have, on both operand paths, that divides the problem (the weak-scale rule of
+    stream kernels have, on every operand path, that divides the problem (the weak-scale rule of
     `make_instance`).  The reference enumerates a much larger grid of compiler knobs
     (bench_perf_102_gemm_python_multitile_g2s_directb_cdna4.py:170-290); here a mapping can only
     steer the tile, the wave grid and the operand path, and mappings that resolve to the same
@@ -297,7 +297,9 @@ def mapping_candidates(M: int, N: int, K: int, *, dtype_ab: str = "bf16", dtype_
     for (tile, waves) in (((256, 256), (2, 4)), ((256, 256), (2, 2)), ((128, 256), (1, 4)), ((128, 128), (2, 2))):
         if M % tile[0] or N % tile[1]:
             continue
-        for path in (OperandPath.LDS, OperandPath.DIRECT_B):
+        for path in (OperandPath.LDS, OperandPath.DIRECT_B, OperandPath.DIRECT_AB):
+            if path == OperandPath.DIRECT_AB and dtype_ab not in ("bf16", "f16"):
+                continue
             try:
                 out.append(make_instance(M, N, K, dtype_ab=dtype_ab, dtype_c=dtype_c, wg_tile=tile,
                                          waves=waves, operand_path=path))

@@ -113,7 +113,7 @@ const char* validate_problem(const astergemm_config& c) {
     return "dtype_c must be F32, BF16 or F16";
   if (c.scale_mode < ASTERGEMM_SCALE_NONE || c.scale_mode > ASTERGEMM_SCALE_MX32)
     return "bad scale_mode";
-  if (c.operand_path < ASTERGEMM_OPERAND_LDS || c.operand_path > ASTERGEMM_OPERAND_DIRECT_B_K8)
+  if (c.operand_path < ASTERGEMM_OPERAND_LDS || c.operand_path > ASTERGEMM_OPERAND_DIRECT_AB)
     return "bad operand_path";
   if (c.mx_a_layout != ASTERGEMM_MX_ROWS &&
       (c.mx_a_layout != ASTERGEMM_MX_LANES128 || c.dtype_ab != ASTERGEMM_MXFP4))
@@ -181,6 +181,7 @@ const Variant* choose(const astergemm_config& c, int* index_out) {
   }
   if (c.operand_path == ASTERGEMM_OPERAND_DIRECT_B) family = ASTERGEMM_KERNEL_SKINNY;
   if (c.operand_path == ASTERGEMM_OPERAND_DIRECT_B_K8) family = ASTERGEMM_KERNEL_TILE;
+  if (c.operand_path == ASTERGEMM_OPERAND_DIRECT_AB) family = ASTERGEMM_KERNEL_TILE;
 
   const Variant* best = nullptr;
   int best_index = -1;
@@ -207,6 +208,17 @@ const Variant* choose(const astergemm_config& c, int* index_out) {
       else if (!fits) better = v->tile_m > best->tile_m;
       else if (v->rank >= 2 || best->rank >= 2) better = v->rank > best->rank;
       else better = v->tile_m < best->tile_m || (v->tile_m == best->tile_m && v->rank > best->rank);
+    } else if (c.operand_path == ASTERGEMM_OPERAND_DIRECT_AB) {
+      // both operands straight into registers: the 256 x 256 form (128 x 128 per wave, half the
+      // L1 requests per MFMA) once it nearly fills the chip, else the 128 x 256 form (bf16 8192^3
+      // 776 against 950 us, 4096^3 125 against 144, 4096 x 14336 x 4096 456 against 495;
+      // 2048^3, 64 tiles: 52.7 against 36.0)
+      auto wgs = [&](const Variant* x) {
+        return ((c.M + x->tile_m - 1) / x->tile_m) * ((c.N + x->tile_n - 1) / x->tile_n);
+      };
+      const Variant* big = v->tile_m > best->tile_m ? v : best;
+      const Variant* want = wgs(big) >= 200 ? big : (big == v ? best : v);
+      better = want == v;
     } else if (c.operand_path == ASTERGEMM_OPERAND_DIRECT_B_K8) {
       // pre-shuffled B straight into operands: the 128 x 256 form (four waves side by side, two
       // workgroups per CU, no B line fetched by two waves) is ahead of the 256 x 256 form on

@@ -10,8 +10,9 @@
 //   astergemm_replay --m 8192 --n 8192 --k 8192 --ab bf16 --c bf16 --iters 100
 //                    [--warmup 20] [--tile 256] [--family tile|skinny|auto]
 //                    [--variant ID] [--flush BYTES] [--bias] [--json] [--calib BYTES]
-//                    [--direct-b | --direct-b-k8]   (B taken as pre-shuffled in the reference's order /
-//                                    in K8 order; timing only, the fill is random)
+//                    [--direct-b | --direct-b-k8 | --direct-ab]   (B taken as pre-shuffled in the
+//                                    reference's order / in K8 order / A and B both in the
+//                                    reference's order; timing only, the fill is random)
 //                    [--normal]      (operands as the benchmark makes them: N(0,1) sources, for
 //                                    bf16 / f16 times 0.02, for fp8 / MXFP4 quantised on the device
 //                                    and, with --direct-b-k8, pre-shuffled on the device: valid
@@ -189,6 +190,7 @@ int main(int argc, char** argv) {
     else if (a == "--calib") calib = atoll(val());
     else if (a == "--direct-b") cfg.operand_path = ASTERGEMM_OPERAND_DIRECT_B;
     else if (a == "--direct-b-k8") cfg.operand_path = ASTERGEMM_OPERAND_DIRECT_B_K8;
+    else if (a == "--direct-ab") cfg.operand_path = ASTERGEMM_OPERAND_DIRECT_AB;
     else if (a == "--bias") cfg.has_bias = 1;
     else if (a == "--normal") use_normal = 1;
     else if (a == "--same-rows") same_rows = 1;

@@ -10,6 +10,7 @@
 #include "gemm_stream4db_kernel.hpp"
 #include "gemm_stream4dbl_kernel.hpp"
 #include "gemm_stream8db_kernel.hpp"
+#include "gemm_directab_kernel.hpp"
 
 namespace astergemm {
 namespace {
@@ -84,6 +85,47 @@ const char* check_streamdb(const astergemm_config& c) {
         launch_streamdb<DT, OUT, NSLOT, NBUF, WM>, check_streamdb,               \
         ASTERGEMM_OPERAND_DIRECT_B_K8                                            \
   }
+
+// ---- A and B pre-shuffled, both loaded straight into MFMA operands, no LDS
+// (gemm_directab_kernel.hpp) --------------------------------------------------------------------
+template <int DT, int OUT, int TM, int TN, int WM, int WN, int NB>
+int launch_directab(const GemmArgs& a, int grid, hipStream_t s) {
+  auto k = gemm_directab_kernel<DT, OUT, TM, TN, WM, WN, NB>;
+  // what the kernel's indexing assumes: whole 16-row blocks of both operands, whole 32-element
+  // chunk columns, both operands packed
+  if (a.M % 16 != 0 || a.M < 16 || a.N % 16 != 0 || a.N < 16 || a.K % 32 != 0 || a.K < 32 ||
+      a.lda_bytes != (int64_t)a.K * 2 || a.ldb_bytes != (int64_t)a.K * 2)
+    return (int)hipErrorInvalidValue;
+  AG_LAUNCH_KERNEL(k, dim3(grid), dim3(WM * WN * 64), 0, s, a);
+  return (int)hipGetLastError();
+}
+
+const char* check_directab(const astergemm_config& c) {
+  if (c.M % 16 != 0 || c.M < 16) return "pre-shuffled A needs M % 16 == 0";
+  if (c.N % 16 != 0 || c.N < 16) return "pre-shuffled B needs N % 16 == 0";
+  if (c.K % 32 != 0) return "pre-shuffled operands need K % 32 == 0";
+  if (c.lda != 0 && c.lda != c.K) return "pre-shuffled A is packed (lda = K)";
+  if (c.ldb != 0 && c.ldb != c.K) return "pre-shuffled B is packed (ldb = K)";
+  if (c.ldc % 4 != 0) return "ldc must be a multiple of 4 elements";
+  if (c.M * c.K * 2 >= ((int64_t)1 << 32) || c.N * c.K * 2 >= ((int64_t)1 << 32))
+    return "pre-shuffled operands must stay below 4 GiB each";
+  return nullptr;
+}
+
+#define AG_DIRECTAB(name, DT, OUT, TM, TN, WM, WN, NB, RANK)                     \
+  Variant {                                                                      \
+    name, ASTERGEMM_KERNEL_TILE, DT, OUT, TM * 16 * WM, TN * 16 * WN, 64, WM, WN, NB, RANK, 0, \
+        (const void*)gemm_directab_kernel<DT, OUT, TM, TN, WM, WN, NB>,          \
+        launch_directab<DT, OUT, TM, TN, WM, WN, NB>, check_directab,            \
+        ASTERGEMM_OPERAND_DIRECT_AB                                              \
+  }
+#define AG_DIRECTAB_SET(prefix, DT)                                                        \
+  AG_DIRECTAB(prefix "_128x256_w1x4_bf16", DT, ASTERGEMM_BF16, 8, 4, 1, 4, 4, 1),          \
+      AG_DIRECTAB(prefix "_128x256_w1x4_f32", DT, ASTERGEMM_F32, 8, 4, 1, 4, 4, 1),        \
+      AG_DIRECTAB(prefix "_128x256_w1x4_f16", DT, ASTERGEMM_F16, 8, 4, 1, 4, 4, 1),        \
+      AG_DIRECTAB(prefix "_256x256_w2x2_bf16", DT, ASTERGEMM_BF16, 8, 8, 2, 2, 3, 2),      \
+      AG_DIRECTAB(prefix "_256x256_w2x2_f32", DT, ASTERGEMM_F32, 8, 8, 2, 2, 3, 2),        \
+      AG_DIRECTAB(prefix "_256x256_w2x2_f16", DT, ASTERGEMM_F16, 8, 8, 2, 2, 3, 2)
 
 // ---- MXFP4, B pre-shuffled (payload in step order, scale plane in lane order) and loaded
 // straight into MFMA operands: 128 x 256 tiles, four waves (gemm_stream4db_kernel.hpp) ---------
@@ -571,6 +613,8 @@ const Variant kStreamVariants[] = {
                        gemm_stream_kernel),
     AG_STREAM_TAIL_SET("stream_f16_256x256_w2x4_tail128", 0, ASTERGEMM_F16, 2, 4, 5 * 256 * kRowBytes,
                        gemm_stream_kernel),
+    AG_DIRECTAB_SET("directab_bf16", ASTERGEMM_BF16),
+    AG_DIRECTAB_SET("directab_f16", ASTERGEMM_F16),
 #elif AG_STREAM_PART == 1
     AG_STREAM_SPLITK_SET("splitk_fp8", 1, ASTERGEMM_FP8_E4M3, 5 * 128 * kRowBytes,
                          gemm_stream8_splitk_kernel),

@@ -441,8 +441,11 @@ extern "C" int astergemm_preshuffle(int dtype_ab, int operand_path, int64_t N, i
     set_error("astergemm_preshuffle: dtype_ab must be F16, BF16, FP8_E4M3 or MXFP4");
     return ASTERGEMM_EINVAL;
   }
+  // DIRECT_AB: one call per operand (A [M, K] or B [N, K]), both in DIRECT_B's 16-bit order
+  if (operand_path == ASTERGEMM_OPERAND_DIRECT_AB && is16) operand_path = ASTERGEMM_OPERAND_DIRECT_B;
   if (operand_path != ASTERGEMM_OPERAND_DIRECT_B && operand_path != ASTERGEMM_OPERAND_DIRECT_B_K8) {
-    set_error("astergemm_preshuffle: operand_path must be DIRECT_B or DIRECT_B_K8");
+    set_error("astergemm_preshuffle: operand_path must be DIRECT_B, DIRECT_B_K8 or (16-bit "
+              "operands) DIRECT_AB");
     return ASTERGEMM_EINVAL;
   }
   const bool k8 = operand_path == ASTERGEMM_OPERAND_DIRECT_B_K8;

@@ -33,7 +33,7 @@ _DTYPE_ID = {"f16": _capi.F16, "bf16": _capi.BF16, "fp8_e4m3": _capi.FP8_E4M3,
 _SCALE_ID = {"none": _capi.SCALE_NONE, "tensor": _capi.SCALE_TENSOR, "mx32": _capi.SCALE_MX32}
 _OUT_NP = {"f32": np.float32, "bf16": np.uint16, "f16": np.float16}
 _OPERAND_PATH_ID = {"lds": _capi.OPERAND_LDS, "direct_b": _capi.OPERAND_DIRECT_B,
-                    "direct_b_k8": _capi.OPERAND_DIRECT_B_K8}
+                    "direct_b_k8": _capi.OPERAND_DIRECT_B_K8, "direct_ab": _capi.OPERAND_DIRECT_AB}
 _OPERAND_PATH_NAME = {v: k for k, v in _OPERAND_PATH_ID.items()}
 
 
@@ -117,11 +117,16 @@ def select_for_instance(cfg: WeakScaledMappedGemmInstance) -> Tuple[_capi.Config
     `shuffle_weight` order, else the stream kernels in `shuffle_weight_k8` order (fp8: step
     order; MXFP4: step order with the scale plane in lane order) (the
     returned config's `operand_path` says which; `execute_gemm_hsaco` shuffles accordingly) --
-    and falls back to plain row-major B otherwise."""
-    want_direct = cfg.mapping.direct_b and not cfg.mapping.direct_a
-    paths = [_capi.OPERAND_DIRECT_B] if want_direct else []
-    if want_direct:
-        paths.append(_capi.OPERAND_DIRECT_B_K8)          # the stream kernels
+    and falls back to plain row-major B otherwise.  A `direct_ab` mapping gets the kernel that
+    reads A and B both pre-shuffled with `shuffle_weight` (16-bit operands, M and N multiples of
+    16), else plain row-major operands."""
+    want_direct = cfg.mapping.direct_b
+    if cfg.mapping.direct_a:                             # both operands pre-shuffled, no LDS
+        paths = [_capi.OPERAND_DIRECT_AB]
+    elif want_direct:                                    # decode kernels, then the stream kernels
+        paths = [_capi.OPERAND_DIRECT_B, _capi.OPERAND_DIRECT_B_K8]
+    else:
+        paths = []
     for use_mapping in (True, False):
         for path in paths + [_capi.OPERAND_LDS]:
             if not use_mapping and path == _capi.OPERAND_LDS and not want_direct:
@@ -205,7 +210,8 @@ class GemmPlan:
         reference's order, read by the decode kernels; fp8 / MXFP4: `shuffle_weight_bytes`, the
         MXFP4 plane with `shuffle_scales_e8m0`); "direct_b_k8" = pre-shuffled for the stream
         kernels: 16-bit operands with `shuffle_weight_k8`, fp8 with `shuffle_weight_bytes`, MXFP4
-        with `shuffle_weight_bytes` and the scale plane with `shuffle_scales_e8m0_lanes`.
+        with `shuffle_weight_bytes` and the scale plane with `shuffle_scales_e8m0_lanes`;
+        "direct_ab" = 16-bit A [M, K] and B [N, K] both pre-shuffled with `shuffle_weight`.
         `mx_a_layout` = "rows" (A's e8m0 plane [M, K/32]) or "lanes128" (in the order of
         `shuffle_scales_e8m0_lanes128` / `quantize_mxfp4_device(..., scales_layout="lanes128")`,
         read by the "direct_b_k8" MXFP4 stream kernel without a pass through LDS)."""
@@ -399,6 +405,11 @@ def execute_gemm_hsaco(cfg: WeakScaledMappedGemmInstance, hsaco_path: str, num_i
                 sc_shuffle = (shuffle_scales_e8m0 if c.operand_path == _capi.OPERAND_DIRECT_B
                               else shuffle_scales_e8m0_lanes)
                 mx_b = sc_shuffle(np.asarray(mx_b, dtype=np.uint8).reshape(N, K // 32))
+        elif c.operand_path == _capi.OPERAND_DIRECT_AB:
+            # both operands, as the reference's execute_fn does for `direct_a`
+            # (test_perf_001_gemm_fp16_weak_scaled.py:252-254)
+            A = shuffle_weight(np.ascontiguousarray(A).reshape(M, K))
+            B = shuffle_weight(np.ascontiguousarray(B).reshape(N, K))
         else:
             shuffle = shuffle_weight if c.operand_path == _capi.OPERAND_DIRECT_B else shuffle_weight_k8
             B = shuffle(np.ascontiguousarray(B).reshape(N, K))

@@ -72,7 +72,8 @@ def preshuffle_device(d_src: int, d_dst: int, N: int, K: int, dtype_ab: str, ope
     ("direct_b" / "direct_b_k8") names for `dtype_ab`, device to device; for MXFP4 the e8m0
     plane goes from `d_mx_src` to `d_mx_dst` in the matching order (the device form of
     `kittens_helpers.shuffle_weight*` / `shuffle_scales_e8m0*`)."""
-    path = {"direct_b": _capi.OPERAND_DIRECT_B, "direct_b_k8": _capi.OPERAND_DIRECT_B_K8}[operand_path]
+    path = {"direct_b": _capi.OPERAND_DIRECT_B, "direct_b_k8": _capi.OPERAND_DIRECT_B_K8,
+            "direct_ab": _capi.OPERAND_DIRECT_AB}[operand_path]
     _capi.check(_capi.load().astergemm_preshuffle(
         _capi.DTYPE_NAMES[dtype_ab], path, N, K, ctypes.c_void_p(d_src), ctypes.c_void_p(d_dst),
         ctypes.c_void_p(d_mx_src) if d_mx_src else None,

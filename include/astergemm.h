@@ -89,7 +89,7 @@ typedef enum astergemm_operand_path {
                                      (MXFP4: dMxB pre-shuffled as well, with
                                      astergemm_shuffle_scales_e8m0).  The
                                      decode kernels, M <= 16                 */
-  ASTERGEMM_OPERAND_DIRECT_B_K8 = 2 /* B packed [N, K] and pre-shuffled for the
+  ASTERGEMM_OPERAND_DIRECT_B_K8 = 2, /* B packed [N, K] and pre-shuffled for the
                                      stream kernels that load B straight into
                                      MFMA operands.  MXFP4: payload with
                                      astergemm_shuffle_weight_8, dMxB with
@@ -105,6 +105,15 @@ typedef enum astergemm_operand_path {
                                      16x16x32 MFMA and of 16-byte LDS reads
                                      (the 128 x 256 and 256 x 256 stream
                                      kernel, N % 16 == 0, K % 64 == 0)       */
+  ASTERGEMM_OPERAND_DIRECT_AB = 3 /* 16-bit operands: A packed [M, K] AND B
+                                     packed [N, K], both pre-shuffled with
+                                     astergemm_shuffle_weight_16 (the
+                                     reference's order: its direct_ab
+                                     template shuffles both operands alike,
+                                     test_perf_001_gemm_fp16_weak_scaled.py:
+                                     252-254); neither passes through LDS
+                                     (M % 16 == 0, N % 16 == 0,
+                                     K % 32 == 0)                             */
 } astergemm_operand_path;
 
 /* Layout of the e8m0 plane of the ACTIVATIONS (A) of an MXFP4 GEMM.  The
@@ -143,7 +152,8 @@ typedef struct astergemm_config {
   int32_t waves_n;       /* num_waves_per_workgroup[N]                      */
   int32_t variant;       /* explicit variant id from astergemm_variant_*,
                             or 0                                             */
-  int32_t operand_path;  /* astergemm_operand_path: how B is stored         */
+  int32_t operand_path;  /* astergemm_operand_path: how B (DIRECT_AB: and A)
+                            is stored                                       */
   int32_t mx_a_layout;   /* astergemm_mx_layout: how A's e8m0 plane is stored
                             (SCALE_MX32 only; B's follows operand_path)      */
   int32_t reserved[4];
@@ -388,7 +398,9 @@ int astergemm_quantize_mxfp4_ex(const void* dSrc, int src_dtype, int64_t rows, i
  * astergemm_shuffle_weight_8 (fp8, MXFP4; dMxSrc -> dMxDst in
  * astergemm_shuffle_scales_e8m0 order); DIRECT_B_K8 =
  * astergemm_shuffle_weight_k8_16 (16-bit) or astergemm_shuffle_weight_8 (fp8;
- * MXFP4, with the plane in astergemm_shuffle_scales_e8m0_lanes order).  The same
+ * MXFP4, with the plane in astergemm_shuffle_scales_e8m0_lanes order);
+ * DIRECT_AB (16-bit only) = DIRECT_B's order, one call per operand (A with
+ * N = M).  The same
  * size rules as the host functions; source and destination distinct and
  * 16-byte aligned (scale planes 8-byte; ignored unless MXFP4).  The reference
  * shuffles on the host on every call

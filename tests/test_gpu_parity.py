@@ -935,12 +935,18 @@ def test_every_tile_variant(gpu, vid, name, dtype_ab, dtype_c):
     elif name.startswith("streamdb"):  # B pre-shuffled in K8 order
         from aster_amd.kittens_helpers import shuffle_weight_k8
         path, b_dev = "direct_b_k8", shuffle_weight_k8(np.ascontiguousarray(b).view(np.uint16))
+    a_dev = a
+    if name.startswith("directab"):  # A and B both in the reference's shuffle_weight order
+        from aster_amd.kittens_helpers import shuffle_weight
+        path = "direct_ab"
+        a_dev = shuffle_weight(np.ascontiguousarray(a).view(np.uint16))
+        b_dev = shuffle_weight(np.ascontiguousarray(b).view(np.uint16))
     plan = AG.GemmPlan.create(M, N, K, dtype_ab, dtype_c, has_bias=True, variant=vid, operand_path=path,
                               mx_a_layout=mxl)
     assert plan.info.name.decode() == name
     out = np.zeros((M, N), dtype=_OUT_NP[dtype_c])
     bufs = {}
-    for key, arr in dict(a=a, b=b_dev, c=out, bias=bias, **{k: np.asarray(v) for k, v in ex_dev.items()}).items():
+    for key, arr in dict(a=a_dev, b=b_dev, c=out, bias=bias, **{k: np.asarray(v) for k, v in ex_dev.items()}).items():
         arr = np.ascontiguousarray(arr if arr.ndim else arr.reshape(1).astype(np.float32))
         bufs[key] = GpuBuffer(arr.nbytes)
         bufs[key].copy_from_host(arr)
@@ -1439,6 +1445,100 @@ def test_direct_b_mapping_of_a_compute_bound_fp8_shape(gpu, tmp_path):
     a, b, ex = operands(M, N, K, "fp8_e4m3", seed=93, b_std=0.05)
     c_flat, times = AG.execute_gemm_hsaco(cfg, path, 2, a, b, **ex)
     check(c_flat.reshape(M, N), G.gemm(a, b, G.FP8_E4M3, G.F32, **ex), "f32", N, bar=1e-4)
+
+
+# ---- direct_ab: A and B both pre-shuffled, neither through LDS ---------------------------------
+
+@pytest.mark.parametrize("M,N,K", [(16, 16, 32), (128, 256, 64), (128, 256, 96), (144, 272, 128),
+                                   (256, 512, 160), (512, 768, 224), (1008, 1040, 256),
+                                   (128, 1024, 576), (2048, 2048, 4096)])
+@pytest.mark.parametrize("dtype_ab,dtype_c", [("bf16", "bf16"), ("f16", "f32"), ("bf16", "f16")])
+@pytest.mark.parametrize("tile,waves", [((128, 256), "1x4"), ((256, 256), "2x2")])
+def test_direct_ab(gpu, M, N, K, dtype_ab, dtype_c, tile, waves):
+    """Both operands in the reference's `shuffle_weight` order, straight into MFMA operands
+    (reference template: gemm_16x32_f16_k_loop_helpers_direct_ab.mlir; execute side
+    test_perf_001_gemm_fp16_weak_scaled.py:252-254).  Chunk-column counts 1, 2, 3, 4 (one whole
+    ring of the 128 x 256 form), 5, 7, 8, 18, 128; edge tiles in M and N (multiples of 16); N(0,1)
+    data, so a wrong lane or K order fails.  Both geometries: 128 x 64 per wave with a ring of four
+    chunk columns, 128 x 128 per wave with a ring of three."""
+    from aster_amd.kittens_helpers import shuffle_weight
+    a, b, _ = operands(M, N, K, dtype_ab)
+    bias = np.random.default_rng(4).standard_normal(N).astype(np.float32)
+    out, name = run_gemm(shuffle_weight(a), shuffle_weight(b), M, N, K, dtype_ab, dtype_c, bias=bias,
+                         operand_path="direct_ab", wg_tile=tile)
+    assert name.startswith(f"directab_{dtype_ab}_{tile[0]}x{tile[1]}_w{waves}_")
+    check(out, G.gemm(a, b, _DT[dtype_ab], _DT[dtype_c], bias=bias), dtype_c, N)
+
+
+def test_direct_ab_output_pitch_and_no_bias(gpu):
+    from aster_amd.kittens_helpers import shuffle_weight
+    M, N, K, ldc = 272, 528, 352, 540
+    a, b, _ = operands(M, N, K, "bf16")
+    out, _ = run_gemm(shuffle_weight(a), shuffle_weight(b), M, N, K, "bf16", "bf16", ldc=ldc,
+                      operand_path="direct_ab")
+    check(out, G.gemm(a, b, G.BF16, G.BF16), "bf16", N)
+    assert (out[:, N:] == 0x7FC1).all()          # the padding of the rows is not written
+
+
+def test_direct_ab_full_size_row_sample_with_device_preshuffle(gpu, big):
+    """8192^3 with both operands shuffled on the device (`astergemm_preshuffle`, one call per
+    operand); the device order equals the host's, rows and columns sampled against the oracle."""
+    import torch
+    from aster_amd import quantize as Q
+    from aster_amd.kittens_helpers import shuffle_weight
+    M, N, K, a, b = big
+    dev = torch.device("cuda:0")
+    ta = torch.from_numpy(a.view(np.int16)).to(dev)
+    tb = torch.from_numpy(b.view(np.int16)).to(dev)
+    sa, sb = torch.empty_like(ta), torch.empty_like(tb)
+    tc = torch.zeros(M, N, dtype=torch.int16, device=dev)
+    torch.cuda.synchronize()
+    Q.preshuffle_device(ta.data_ptr(), sa.data_ptr(), M, K, "bf16", "direct_ab")
+    Q.preshuffle_device(tb.data_ptr(), sb.data_ptr(), N, K, "bf16", "direct_ab")
+    plan = AG.GemmPlan.create(M, N, K, "bf16", "bf16", operand_path="direct_ab")
+    assert plan.info.name.decode() == "directab_bf16_256x256_w2x2_bf16"
+    print(f"launch {plan.info.name.decode()} M={M} N={N} K={K}", flush=True)
+    plan.run(sa.data_ptr(), sb.data_ptr(), tc.data_ptr())
+    torch.cuda.synchronize()
+    assert np.array_equal(sa[:64].cpu().numpy().view(np.uint16), shuffle_weight(a[:64]))
+    out = tc.cpu().numpy().view(np.uint16)
+    rows, cols = _sampled_rows_and_cols(M, N)
+    check(out[rows], G.gemm(a[rows], b, G.BF16, G.BF16), "bf16", N)
+    check(out[:, cols], G.gemm(a, b[cols], G.BF16, G.BF16), "bf16", len(cols))
+
+
+def test_direct_ab_mapping_through_the_harness_seam(gpu, tmp_path):
+    # a DIRECT_AB mapping: compile_gemm selects the kernel without LDS, execute_gemm_hsaco shuffles
+    # the row-major A and B it is given (the reference's single point of truth)
+    M, N, K = 512, 768, 640
+    cfg = make_instance(M, N, K, wg_tile=(128, 256), waves=(1, 4), operand_path=OperandPath.DIRECT_AB)
+    path, asm = AG.compile_gemm(cfg, str(tmp_path / "k.hsaco"))
+    desc = json.load(open(path))
+    assert desc["kernel"] == "directab_bf16_128x256_w1x4_bf16" and desc["operand_path"] == "direct_ab"
+    assert desc["mapping_honoured"] is True and desc["lds_bytes"] == 0
+    a, b, _ = operands(M, N, K, "bf16")
+    c_flat, times = AG.execute_gemm_hsaco(cfg, path, 3, a, b)
+    assert len(times) == 3
+    check(c_flat.reshape(M, N), G.gemm(a, b, G.BF16, G.BF16), "bf16", N)
+    # rows that do not fill 32-element chunks: the LDS kernels run and the descriptor says so
+    cfg = make_instance(512, 768, 264, operand_path=OperandPath.DIRECT_AB)
+    path, _ = AG.compile_gemm(cfg, str(tmp_path / "k2.hsaco"))
+    desc = json.load(open(path))
+    assert desc["operand_path"] == "lds"
+    assert desc["mapping_not_honoured"]["operand_path"] == {"requested": "direct_ab", "kernel": "lds"}
+    a, b, _ = operands(512, 768, 264, "bf16")
+    c_flat, _ = AG.execute_gemm_hsaco(cfg, path, 1, a, b)
+    check(c_flat.reshape(512, 768), G.gemm(a, b, G.BF16, G.BF16), "bf16", 768)
+
+
+def test_direct_ab_is_refused_where_it_is_not_implemented(gpu):
+    for kw in (dict(M=120, N=256, K=512), dict(M=128, N=264, K=512), dict(M=128, N=256, K=528)):
+        with pytest.raises(_capi.AsterGemmError):
+            AG.GemmPlan.create(kw["M"], kw["N"], kw["K"], "bf16", "bf16", operand_path="direct_ab")
+    with pytest.raises(_capi.AsterGemmError):
+        AG.GemmPlan.create(128, 256, 512, "fp8_e4m3", "bf16", operand_path="direct_ab")
+    with pytest.raises(_capi.AsterGemmError):
+        AG.GemmPlan.create(128, 256, 512, "bf16", "bf16", operand_path="direct_ab", lda=520)
 
 
 def test_direct_b_is_refused_where_it_is_not_implemented(gpu):

@@ -198,6 +198,34 @@ def test_direct_b_mapping_selects_a_stream_kernel_for_every_operand_type():
         assert rep.honoured and not rep.not_honoured, (dt, rep.not_honoured)
 
 
+def test_direct_ab_mapping_selects_the_kernel_without_lds():
+    # reference: operand_path = direct_ab (contrib/kittens/gemm_config.py:213-276) -- A and B both
+    # pre-shuffled; here a 16-bit kernel of the 128 x 256, 1 x 4 geometry with no LDS at all
+    from aster_amd.gemm_config import OperandPath
+    for dt in ("bf16", "f16"):
+        cfg = make_instance(512, 768, 640, dtype_ab=dt, wg_tile=(128, 256), waves=(1, 4),
+                            operand_path=OperandPath.DIRECT_AB)
+        c, info = gemm.select_for_instance(cfg)
+        assert info.name.decode().startswith(f"directab_{dt}_128x256_w1x4_"), info.name
+        assert c.operand_path == _capi.OPERAND_DIRECT_AB and info.lds_bytes == 0
+        assert info.grid_x == 4 * 3 and info.block_x == 256
+        rep = gemm.mapping_report(cfg, c, info)
+        assert rep.honoured and not rep.not_honoured
+    # a row length that does not fill 32-element chunks falls back to the LDS kernels, and says so
+    cfg = make_instance(512, 768, 264, operand_path=OperandPath.DIRECT_AB)
+    c, info = gemm.select_for_instance(cfg)
+    assert c.operand_path == _capi.OPERAND_LDS
+    assert gemm.mapping_report(cfg, c, info).not_honoured["operand_path"] == {
+        "requested": "direct_ab", "kernel": "lds"}
+    # byte operands have no such kernel; M, N in 16-row blocks; packed operands
+    for args, kw in (((128, 256, 512, "fp8_e4m3", "bf16"), {}), ((120, 256, 512, "bf16", "bf16"), {}),
+                     ((128, 264, 512, "bf16", "bf16"), {}), ((128, 256, 528, "bf16", "bf16"), {}),
+                     ((128, 256, 512, "bf16", "bf16"), dict(lda=520)),
+                     ((128, 256, 512, "bf16", "bf16"), dict(ldb=520))):
+        with pytest.raises(_capi.AsterGemmError):
+            gemm.GemmPlan.create(*args, operand_path="direct_ab", **kw)
+
+
 def test_execute_checks_host_operand_sizes_before_touching_the_gpu(tmp_path):
     cfg = make_instance(256, 256, 256)
     path, _ = gemm.compile_gemm(cfg, str(tmp_path / "k.hsaco"))
