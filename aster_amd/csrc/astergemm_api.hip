@@ -233,13 +233,14 @@ const Variant* choose(const astergemm_config& c, int* index_out) {
       auto wgs = [&](const Variant* x) {
         return ((c.M + x->tile_m - 1) / x->tile_m) * ((c.N + x->tile_n - 1) / x->tile_n);
       };
-      // 256 x 256 from 230 workgroups on; already from 140 on when the last round of the
+      // 256 x 256 from 220 workgroups on (bf16 1024 x 14336 x 4096, 224 tiles: 85.6 us against
+      // 103.9 for 896 tiles of 128 x 128); already from 140 on when the last round of the
       // 128 x 128 stream kernel (512 workgroups fill the chip) would be less than about a
       // third full.  The 128 x 128 stream kernel from 200 workgroups on,
       // from 128 on when rows are long (8 KiB and more: few prologues per byte streamed).
       const int64_t g128 = ((c.M + 127) / 128) * ((c.N + 127) / 128);
       const bool ragged_128 = g128 > 512 && g128 % 512 != 0 && g128 % 512 < 180;
-      const int thr256 = ragged_128 ? 140 : 230;
+      const int thr256 = ragged_128 ? 140 : 220;
       // MXFP4: the generic tile kernels are weak next to the stream kernels, so the 128 x 128
       // stream kernel from 16 workgroups on when K >= 4096, and instead of the 256 x 256 one
       // (long prologue: two K-steps and their scales) when K < 4096

@@ -15,10 +15,10 @@
 namespace astergemm {
 namespace {
 
-template <int DT, int OUT, int BM, int BN, int WM, int WN>
+template <int DT, int OUT, int BM, int BN, int WM, int WN, int NSLOT = 5>
 int launch_stream(const GemmArgs& a, int grid, hipStream_t s) {
-  constexpr int lds = 5 * BM * kRowBytes;
-  auto k = gemm_stream_kernel<DT, OUT, BM, BN, WM, WN>;
+  constexpr int lds = NSLOT * BM * kRowBytes;
+  auto k = gemm_stream_kernel<DT, OUT, BM, BN, WM, WN, NSLOT>;
   static std::atomic<uint64_t> attr_devs{0};
   if (int e = lds_attr_once(attr_devs, (const void*)k, lds)) return e;
   AG_LAUNCH_KERNEL(k, dim3(grid), dim3(WM * WN * 64), lds, s, a);
@@ -51,6 +51,34 @@ const char* check_stream_whole_k(const astergemm_config& c) {
         launch_stream<DT, OUT, BM, BN, WM, WN>,                                  \
         (WM * WN == 8 || BM == 128) ? check_stream : check_stream_whole_k        \
   }
+
+// The 128 x 128 kernel with a ring of nine slots (144 KiB of LDS, one workgroup per CU): four
+// K-steps requested ahead instead of two.  For grids of at most one workgroup per CU with two or
+// more tile rows, where nothing else covers a workgroup's waits (bf16, five -> nine slots:
+// 256 x 14336 x 4096 37.7-38.7 -> 33.7-34.4 us, 384 x 8192 x 4096 34.4 -> 31.0, 2048^3 23.3 ->
+// 21.2, 1024 x 4096 x 4096 36.9 -> 35.5; one tile row, which is HBM-bound on B alone, loses:
+// 128 x 28672 x 4096 39.8 -> 41.8; eight waves instead of four: level).
+const char* check_stream_ring9(const astergemm_config& c) {
+  if (const char* why = check_stream(c)) return why;
+  int cus = device_cus();
+  if (cus <= 0) cus = 256;  // no device to ask: describe the MI355X
+  const int64_t tm = (c.M + 127) / 128, tn = (c.N + 127) / 128;
+  if (tm < 2) return "the nine-slot ring pays from two tile rows on";
+  if (tm * tn > cus) return "the nine-slot ring takes the LDS of a CU: at most one workgroup per CU";
+  if (row_bytes(c.dtype_ab, c.K) < 16 * kRowBytes) return "the nine-slot ring needs 16 K-steps or more";
+  return nullptr;
+}
+#define AG_STREAM_RING9(name, DT, OUT)                                           \
+  Variant {                                                                      \
+    name, ASTERGEMM_KERNEL_TILE, DT, OUT, 128, 128, kRowBytes, 2, 2, 5, 3,       \
+        9 * 128 * kRowBytes,                                                     \
+        (const void*)gemm_stream_kernel<DT, OUT, 128, 128, 2, 2, 9>,             \
+        launch_stream<DT, OUT, 128, 128, 2, 2, 9>, check_stream_ring9            \
+  }
+#define AG_STREAM_RING9_SET(prefix, DT)                                          \
+  AG_STREAM_RING9(prefix "_128x128_w2x2_ring9_bf16", DT, ASTERGEMM_BF16),        \
+      AG_STREAM_RING9(prefix "_128x128_w2x2_ring9_f32", DT, ASTERGEMM_F32),      \
+      AG_STREAM_RING9(prefix "_128x128_w2x2_ring9_f16", DT, ASTERGEMM_F16)
 
 // ---- B pre-shuffled, loaded straight into MFMA operands (gemm_streamdb_kernel.hpp) ---------
 template <int DT, int OUT, int NSLOT, int NBUF, int WM>
@@ -613,6 +641,8 @@ const Variant kStreamVariants[] = {
                        gemm_stream_kernel),
     AG_STREAM_TAIL_SET("stream_f16_256x256_w2x4_tail128", 0, ASTERGEMM_F16, 2, 4, 5 * 256 * kRowBytes,
                        gemm_stream_kernel),
+    AG_STREAM_RING9_SET("stream_bf16", ASTERGEMM_BF16),
+    AG_STREAM_RING9_SET("stream_f16", ASTERGEMM_F16),
     AG_DIRECTAB_SET("directab_bf16", ASTERGEMM_BF16),
     AG_DIRECTAB_SET("directab_f16", ASTERGEMM_F16),
 #elif AG_STREAM_PART == 1

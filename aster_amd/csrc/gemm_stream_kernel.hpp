@@ -255,13 +255,18 @@ __device__ __forceinline__ void stream_mma(const i32x4& a, const i32x4& b, f32x4
   }
 }
 
-template <int DT, int OUT, int BM, int BN, int WM, int WN>
+template <int DT, int OUT, int BM, int BN, int WM, int WN, int NSLOT = 5>
 __device__ __forceinline__ void gemm_stream_body(const GemmArgs& p, int bid) {
   constexpr int NW = WM * WN;
   constexpr int TM = BM / WM / 16;
   constexpr int TN = BN / WN / 16;
   constexpr int SLOT = BM * kRowBytes;  // 32 KiB: one operand half of one K-step
-  constexpr int NSLOT = 5;
+  // Ring of NSLOT = 2 D + 1 slots: A(k) in slot 2k mod NSLOT, B(k) in slot 2k + 1 mod NSLOT; while
+  // K-step k is multiplied, B(k + D) and A(k + D + 1) are requested.  Five slots (D = 2) fill the
+  // LDS of a CU at 256 x 256; the 128 x 128 form is also built with nine (D = 4, 144 KiB) for
+  // grids of at most one workgroup per CU, where the bytes in flight per CU bound the speed.
+  static_assert(NSLOT % 2 == 1 && NSLOT >= 5, "odd ring");
+  constexpr int D = (NSLOT - 1) / 2;
   using Plan = StreamLoadPlan<BM, NW>;  // the staging as a cooperative load plan (stream_load_plan.inc)
   constexpr int LH = Plan::LH;       // 1 KiB (8 rows x 128 B) transfers per wave and slot
   static_assert(Plan::TILE_ROWS == 8 && Plan::TILE_LDS_BYTES == 8 * kRowBytes, "transfer tile");
@@ -332,7 +337,7 @@ __device__ __forceinline__ void gemm_stream_body(const GemmArgs& p, int bid) {
   const unsigned a_rd = (unsigned)(wm * TM * 16 * kRowBytes);
   const unsigned b_rd = (unsigned)(wn * TN * 16 * kRowBytes);
 
-  // KM = k mod 5 fixes the ring slots of K-step k at compile time.
+  // KM = k mod NSLOT fixes the ring slots of K-step k at compile time.
   i32x4 fa[2][TM], fb[2][TN];
   auto read_frags = [&](auto kmod, auto sub) {
     constexpr int KM = decltype(kmod)::value;
@@ -384,18 +389,24 @@ __device__ __forceinline__ void gemm_stream_body(const GemmArgs& p, int bid) {
   using S0 = std::integral_constant<int, 0>;
   using S1 = std::integral_constant<int, 1>;
 
-  // ---- prologue: A(0) B(0) A(1) B(1) A(2) in flight, both fragment sets of K-step 0
+  // ---- prologue: A(0) B(0) ... A(D-1) B(D-1) A(D) in flight, both fragment sets of K-step 0
   // read, first substep multiplied -----------------------------------------------------------
-  issue_a(0, 0);
-  issue_b(0, 1);
-  if (nk > 1) {
-    issue_a(1, 2);
-    issue_b(1, 3);
+  static_for<0, D>([&](auto ic) {
+    constexpr int I = decltype(ic)::value;
+    if (nk > I) {
+      issue_a(I, (2 * I) % NSLOT);
+      issue_b(I, (2 * I + 1) % NSLOT);
+    }
+  });
+  if (nk > D) issue_a(D, (2 * D) % NSLOT);
+  {
+    // groups of LH transfers issued; all but the first two (A(0), B(0)) may stay in flight
+    const int groups = 2 * (nk < D ? nk : D) + (nk > D ? 1 : 0);
+    static_for<2, 2 * D + 2>([&](auto gc) {
+      constexpr int G = decltype(gc)::value;
+      if (groups == G) __builtin_amdgcn_s_waitcnt(waitcnt_imm((G - 2) * LH, 15));
+    });
   }
-  if (nk > 2) issue_a(2, 4);
-  if (nk > 2) __builtin_amdgcn_s_waitcnt(waitcnt_imm(3 * LH, 15));
-  else if (nk > 1) __builtin_amdgcn_s_waitcnt(waitcnt_imm(2 * LH, 15));
-  else __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
   using K0 = std::integral_constant<int, 0>;
@@ -408,14 +419,14 @@ __device__ __forceinline__ void gemm_stream_body(const GemmArgs& p, int bid) {
   // ---- K loop ------------------------------------------------------------------------------
   // One trip finishes K-step k (substep 1) and starts K-step k+1 (substep 0).  It
   // begins with a wait and a barrier: A(k+1) and B(k+1) have landed for everybody
-  // (only A(k+2) may still be in flight) and every fragment of K-step k is in
-  // registers, which frees its two slots for B(k+2) and A(k+3).
+  // (only A(k+2) ... A(k+D) may still be in flight) and every fragment of K-step k is in
+  // registers, which frees its two slots for B(k+D) and A(k+D+1).
   // Inside a trip nothing is issued in bursts: a wave that is stuck pushing loads
   // into a full address queue, or reads into a full LDS queue, cannot issue MFMAs.
   // So every MFMA is followed by at most one LDS read or one global->LDS transfer:
   // block 1 (substep 1 of K-step k) carries the reads of substep 0 of K-step k+1 and
-  // the transfers of B(k+2), which is needed first; block 2 carries the reads of
-  // substep 1 and the transfers of A(k+3).
+  // the transfers of B(k+D), which is needed first; block 2 carries the reads of
+  // substep 1 and the transfers of A(k+D+1).
   auto trip = [&](int k, auto kmod, auto steady) {
     constexpr int KM = decltype(kmod)::value;
     constexpr bool STEADY = decltype(steady)::value;
@@ -423,18 +434,19 @@ __device__ __forceinline__ void gemm_stream_body(const GemmArgs& p, int bid) {
     constexpr int NF = TM + TN;      // fragments per substep
     constexpr int NMF = TM * TN;     // MFMAs per substep
     static_assert(NF + LH <= NMF, "one side instruction per MFMA");
-    if constexpr (STEADY) __builtin_amdgcn_s_waitcnt(waitcnt_imm(LH, 0));
+    static_assert((2 * D - 3) * LH <= 63, "vmcnt field");
+    if constexpr (STEADY) __builtin_amdgcn_s_waitcnt(waitcnt_imm((2 * D - 3) * LH, 0));
     else __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    const bool do_b = STEADY || k + 2 < nk;
-    const bool do_a = STEADY || k + 3 < nk;
+    const bool do_b = STEADY || k + D < nk;
+    const bool do_a = STEADY || k + D + 1 < nk;
     static_for<0, NMF>([&](auto ic) {
       constexpr int I = decltype(ic)::value;
       constexpr int n = I / TM, m = I % TM;
       stream_mma<DT, AX>(fb[1][n], fa[1][m], acc[m][n]);
       if constexpr (I < LH) {
-        if (do_b) issue_b1(k + 2, (2 * KM) % NSLOT, I);
+        if (do_b) issue_b1(k + D, (2 * KM) % NSLOT, I);
       }
       if constexpr (I >= LH && I < LH + NF) read_one(KN{}, S0{}, std::integral_constant<int, I - LH>{});
       __builtin_amdgcn_sched_barrier(0);
@@ -445,7 +457,7 @@ __device__ __forceinline__ void gemm_stream_body(const GemmArgs& p, int bid) {
       stream_mma<DT, AX>(fb[0][n], fa[0][m], acc[m][n]);
       if constexpr (I < NF) read_one(KN{}, S1{}, std::integral_constant<int, I>{});
       if constexpr (I >= NF && I < NF + LH) {
-        if (do_a) issue_a1(k + 3, (2 * KM + 1) % NSLOT, I - NF);
+        if (do_a) issue_a1(k + D + 1, (2 * KM + 1) % NSLOT, I - NF);
       }
       __builtin_amdgcn_sched_barrier(0);
     });
@@ -453,21 +465,13 @@ __device__ __forceinline__ void gemm_stream_body(const GemmArgs& p, int bid) {
   using T = std::true_type;
   using F = std::false_type;
   int k = 0;
-  // steady: K-steps up to k+4+3 exist for the whole group of five trips
-  for (; k + 8 <= nk; k += 5) {
-    trip(k, std::integral_constant<int, 0>{}, T{});
-    trip(k + 1, std::integral_constant<int, 1>{}, T{});
-    trip(k + 2, std::integral_constant<int, 2>{}, T{});
-    trip(k + 3, std::integral_constant<int, 3>{}, T{});
-    trip(k + 4, std::integral_constant<int, 4>{}, T{});
-  }
-  for (; k + 1 < nk; k += 5) {
-    trip(k, std::integral_constant<int, 0>{}, F{});
-    if (k + 2 < nk) trip(k + 1, std::integral_constant<int, 1>{}, F{});
-    if (k + 3 < nk) trip(k + 2, std::integral_constant<int, 2>{}, F{});
-    if (k + 4 < nk) trip(k + 3, std::integral_constant<int, 3>{}, F{});
-    if (k + 5 < nk) trip(k + 4, std::integral_constant<int, 4>{}, F{});
-  }
+  // steady: K-steps up to k + (NSLOT - 1) + D + 1 exist for the whole group of NSLOT trips
+  for (; k + NSLOT + D + 1 <= nk; k += NSLOT)
+    static_for<0, NSLOT>([&](auto ic) { trip(k + decltype(ic)::value, ic, T{}); });
+  for (; k + 1 < nk; k += NSLOT)
+    static_for<0, NSLOT>([&](auto ic) {
+      if (k + decltype(ic)::value + 1 < nk) trip(k + decltype(ic)::value, ic, F{});
+    });
   __builtin_amdgcn_sched_barrier(0);
   mfmas(S1{});
 
@@ -477,16 +481,16 @@ __device__ __forceinline__ void gemm_stream_body(const GemmArgs& p, int bid) {
   stream_epilogue<OUT, BM, BN, WM, WN>(p, acc, lds, wave, row0, col0);
 }
 
-template <int DT, int OUT, int BM, int BN, int WM, int WN>
+template <int DT, int OUT, int BM, int BN, int WM, int WN, int NSLOT = 5>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_stream_kernel(const GemmArgs p) {
-  gemm_stream_body<DT, OUT, BM, BN, WM, WN>(p, blockIdx.x);
+  gemm_stream_body<DT, OUT, BM, BN, WM, WN, NSLOT>(p, blockIdx.x);
 }
 
 // Split K: the grid is p.split_k copies of the tile grid; copy s multiplies K steps
 // [s * p.ksteps, (s + 1) * p.ksteps) of every row and leaves its fp32 sums in plane s of the
 // workspace [split_k][M][N] (no scale, no bias: the kernel that adds the planes applies them).
 // For few output tiles and long rows, where the tile grid alone leaves most CUs idle.
-template <int DT, int BM, int BN, int WM, int WN>
+template <int DT, int BM, int BN, int WM, int WN, int NSLOT = 5>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_stream_splitk_kernel(const GemmArgs p) {
   const int tiles = p.tiles_m * p.tiles_n;
   const int ks = blockIdx.x / tiles;
@@ -494,7 +498,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_stream_splitk_kernel(const G
   q.A = p.A + (int64_t)ks * p.ksteps * kRowBytes;
   q.B = p.B + (int64_t)ks * p.ksteps * kRowBytes;
   q.C = p.workspace + (int64_t)ks * p.M * p.N;
-  gemm_stream_body<DT, ASTERGEMM_F32, BM, BN, WM, WN>(q, blockIdx.x - ks * tiles);
+  gemm_stream_body<DT, ASTERGEMM_F32, BM, BN, WM, WN, NSLOT>(q, blockIdx.x - ks * tiles);
 }
 
 }  // namespace

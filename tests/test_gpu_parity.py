@@ -637,6 +637,38 @@ def test_stream_kernels_edge_tiles(gpu, M, N, K, dtype_ab, dtype_c):
     assert np.isnan(pad).all() if dtype_c == "f32" else (pad == 0x7FC1).all()
 
 
+@pytest.mark.parametrize("M,N,K", [(256, 256, 1024), (264, 520, 1088), (384, 1000, 1152), (256, 384, 1216),
+                                   (512, 264, 1408), (256, 256, 1472), (264, 256, 1536), (256, 512, 1600),
+                                   (1000, 1024, 1664), (256, 256, 1728), (504, 776, 1800), (256, 128, 2120),
+                                   (2048, 2048, 2048)])
+@pytest.mark.parametrize("dtype_ab,dtype_c", [("bf16", "bf16"), ("f16", "f32")])
+def test_stream_128_with_nine_slot_ring(gpu, M, N, K, dtype_ab, dtype_c):
+    """The 128 x 128 stream kernel with four K-steps requested ahead (nine LDS slots), which AUTO
+    takes for at most one workgroup per CU and two or more tile rows.  K-step counts 16 (the
+    minimum), 17, 18, 19 (one whole steady group of nine trips + prologue depth exactly), 22, 23,
+    24, 25, 26, 27, 28 + a tail of granules, 33 + a tail, 32; edge tiles in M and N.  The same
+    sums as the five-slot kernel (same K order, same accumulation)."""
+    a, b, _ = operands(M, N, K, dtype_ab, seed=61, b_std=0.05)
+    bias = np.random.default_rng(62).standard_normal(N).astype(np.float32)
+    out, name = run_gemm(a, b, M, N, K, dtype_ab, dtype_c, bias=bias, wg_tile=(128, 128),
+                         family=_capi.KERNEL_TILE)
+    assert name == f"stream_{dtype_ab}_128x128_w2x2_ring9_{dtype_c}"
+    check(out, G.gemm(a, b, _DT[dtype_ab], _DT[dtype_c], bias=bias), dtype_c, N,
+          bar=REL_L2_BAR if dtype_c != "f32" else 1e-5)
+    five, five_name = run_gemm(a, b, M, N, K, dtype_ab, dtype_c, bias=bias,
+                               variant=_variant_id(f"stream_{dtype_ab}_128x128_w2x2_{dtype_c}"))
+    assert five_name == f"stream_{dtype_ab}_128x128_w2x2_{dtype_c}"
+    assert np.array_equal(out, five)
+
+
+def test_nine_slot_ring_is_left_to_grids_of_one_workgroup_per_cu(gpu):
+    name = lambda *shape: AG.GemmPlan.create(*shape, "bf16", "bf16").info.name.decode()
+    assert name(256, 14336, 4096) == "stream_bf16_128x128_w2x2_ring9_bf16"      # 224 tiles, two tile rows
+    assert name(128, 28672, 4096) == "stream_bf16_128x128_w2x2_bf16"            # one tile row: HBM-bound
+    assert name(512, 14336, 4096) == "stream_bf16_128x128_w2x2_bf16"            # 448 tiles: two per CU
+    assert AG.GemmPlan.create(256, 14336, 4096, "bf16", "bf16").info.lds_bytes == 9 * 128 * 128
+
+
 # ---- edge cases: ragged M / N, K tails, leading dimensions, epilogue -----------------
 
 @pytest.mark.parametrize("M,N,K", [(1, 1, 8), (65, 16, 8), (130, 257, 72), (300, 520, 776), (129, 1, 64)])
