@@ -120,6 +120,8 @@ SIGNATURES = {
     "astergemm_workspace_bytes": (C.c_int, [C.POINTER(Config), C.POINTER(C.c_size_t)]),
     "astergemm_bench_rotate": (C.c_int, [C.POINTER(Config), C.POINTER(Operands), C.c_int, C.c_int,
                                          C.POINTER(C.c_int64), C.c_void_p]),
+    "astergemm_bench_graph": (C.c_int, [C.POINTER(Config), C.POINTER(Operands), C.c_int, C.c_int,
+                                        C.c_int, C.POINTER(C.c_int64)]),
     "astergemm_bench": (C.c_int, [C.POINTER(Config), C.POINTER(Operands), C.c_int,
                                   C.POINTER(C.c_int64), C.c_int64, _P]),
     "astergemm_tune": (C.c_int, [C.POINTER(Config), C.POINTER(Operands), C.c_int, C.POINTER(C.c_int),

@@ -646,6 +646,63 @@ int astergemm_bench_rotate(const astergemm_config* cfg, const astergemm_operands
   return 0;
 }
 
+int astergemm_bench_graph(const astergemm_config* cfg, const astergemm_operands* ops, int n_ops,
+                          int launches, int replays, int64_t* total_ns) {
+  if (!cfg || !ops || !total_ns || launches <= 0 || launches > 4096 || replays <= 0 || n_ops <= 0) {
+    set_error("astergemm_bench_graph: bad argument");
+    return ASTERGEMM_EINVAL;
+  }
+  int index = -1;
+  const Variant* v = choose(*cfg, &index);
+  if (!v) return g_choose_rc;
+  *total_ns = 0;
+  if (cfg->M == 0 || cfg->N == 0) return 0;
+  std::vector<GemmArgs> args((size_t)n_ops);
+  for (int i = 0; i < n_ops; ++i)
+    if (int rc = build_args(*v, *cfg, ops[i], &args[(size_t)i])) return rc;
+  const int grid = grid_of(*v, *cfg);
+  // a stream of this call's own (default priority), so that the capture sees nothing else
+  hipStream_t s = nullptr;
+  AG_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t exec = nullptr;
+  EventPair ev;
+  int le = (int)ev.create();
+  {
+    LaunchScope scope(s);
+    // one eager launch first: function attributes, and the partial-sum workspace of this stream
+    // where the config has one, are one-time steps that may not happen inside a capture
+    (void)hipGetLastError();
+    if (le == 0) le = v->launch(args[0], grid, s);
+    if (le == 0) le = (int)hipStreamSynchronize(s);
+    if (le == 0) {
+      le = (int)hipStreamBeginCapture(s, hipStreamCaptureModeGlobal);
+      if (le == 0) {
+        int ce = 0;
+        for (int i = 0; i < launches && ce == 0; ++i) ce = v->launch(args[(size_t)(i % n_ops)], grid, s);
+        le = (int)hipStreamEndCapture(s, &graph);  // always ended, also after a refused launch
+        if (ce != 0) le = ce;
+      }
+    }
+  }
+  if (le == 0) le = (int)hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+  if (le == 0) le = (int)hipGraphLaunch(exec, s);  // untimed: the first replay uploads the graph
+  if (le == 0) le = (int)hipStreamSynchronize(s);
+  if (le == 0) le = (int)hipEventRecord(ev.e0, s);
+  for (int r = 0; r < replays && le == 0; ++r) le = (int)hipGraphLaunch(exec, s);
+  if (le == 0) le = (int)hipEventRecord(ev.e1, s);
+  if (le == 0) le = (int)hipEventSynchronize(ev.e1);
+  float ms = 0.f;
+  if (le == 0) le = (int)hipEventElapsedTime(&ms, ev.e0, ev.e1);
+  if (exec) (void)hipGraphExecDestroy(exec);
+  if (graph) (void)hipGraphDestroy(graph);
+  (void)hipStreamSynchronize(s);
+  (void)hipStreamDestroy(s);
+  if (le != 0) return hip_fail((hipError_t)le, v->name, __FILE__, __LINE__);
+  *total_ns = (int64_t)((double)ms * 1e6);
+  return 0;
+}
+
 int astergemm_tune(const astergemm_config* cfg, const astergemm_operands* ops, int iters,
                    int* best_variant, int64_t* best_ns, void* stream) {
   if (!cfg || !ops || !best_variant || iters <= 0) {

@@ -316,6 +316,21 @@ class GemmPlan:
         return total.value
 
 
+    def bench_graph(self, operand_sets, launches: int, replays: int) -> int:
+        """`launches` launches (launch i on operand set i % len(operand_sets), sets as for
+        `bench_rotate`) captured once into a HIP graph on a stream of the call's own and replayed
+        `replays` times between one event pair.  Returns the total time in ns of the
+        launches * replays launches: what a loop that replays a captured decode step pays."""
+        arr = (_capi.Operands * len(operand_sets))()
+        for i, o in enumerate(operand_sets):
+            arr[i] = self._operands(o["dA"], o["dB"], o["dC"], o.get("scale_a"), o.get("scale_b"),
+                                    o.get("mx_a"), o.get("mx_b"), o.get("bias"))
+        total = ctypes.c_int64()
+        _capi.check(_capi.load().astergemm_bench_graph(
+            ctypes.byref(self.config), arr, len(operand_sets), launches, replays, ctypes.byref(total)))
+        return total.value
+
+
 def gemm_device(dA: int, dB: int, dC: int, M: int, N: int, K: int, dtype_ab: str = "bf16",
                 dtype_c: str = "bf16", **kw) -> None:
     """One launch on caller-owned device pointers (integers)."""

@@ -527,6 +527,8 @@ def main() -> int:
             sets = [{"dA": a.data_ptr(), "dB": w.data_ptr(), "dC": c.data_ptr()} for w in wts]
             p.bench_rotate(sets, 40)
             rot_ns = p.bench_rotate(sets, 200) / 200.0
+            # the same 200 launches as 5 replays of a captured HIP graph of 40 kernel nodes
+            graph_ns = p.bench_graph(sets, 40, 5) / 200.0
             del wts, sets
             others.append({"workload": f"bf16 skinny GEMM M={m} N=14336 K=4096 -> bf16, LLC flushed "
                                        "(512 MiB rewritten) before every launch",
@@ -536,7 +538,9 @@ def main() -> int:
                            "p50_us_cache_warm": round(hot / 1e3, 2),
                            "us_back_to_back_8_weight_sets": round(rot_ns / 1e3, 2),
                            "gbps_back_to_back": round(p.info.bytes / rot_ns, 1),
-                           "frac_back_to_back": round(p.info.bytes / rot_ns / PEAK_HBM_GBPS, 4)})
+                           "frac_back_to_back": round(p.info.bytes / rot_ns / PEAK_HBM_GBPS, 4),
+                           "us_graph_replay_8_weight_sets": round(graph_ns / 1e3, 2),
+                           "frac_graph_replay": round(p.info.bytes / graph_ns / PEAK_HBM_GBPS, 4)})
         # the decode shape with quantised weights and activations (same kernel frame)
         for dt in ("fp8_e4m3", "mxfp4"):
             del a, b, c

@@ -285,6 +285,16 @@ int astergemm_bench(const astergemm_config* cfg, const astergemm_operands* ops,
 int astergemm_bench_rotate(const astergemm_config* cfg, const astergemm_operands* ops,
                            int n_ops, int iters, int64_t* total_ns, void* stream);
 
+/* The same launches as nodes of a HIP graph: `launches` launches (launch i on
+ * ops[i % n_ops]) are captured once on a stream of the call's own, after one
+ * eager launch that does the config's one-time steps, and the graph is replayed
+ * `replays` times between one event pair after one untimed replay;
+ * *total_ns covers launches * replays launches.  What a serving loop that
+ * replays a captured decode step pays per GEMM.  No counterpart in the
+ * reference.                                                                  */
+int astergemm_bench_graph(const astergemm_config* cfg, const astergemm_operands* ops,
+                          int n_ops, int launches, int replays, int64_t* total_ns);
+
 /* Measures every variant that can run cfg on the given operands (`iters`
  * back-to-back launches between one event pair each, after two warm-up
  * launches) and returns the fastest: *best_variant is what cfg->variant takes

@@ -1083,6 +1083,41 @@ def test_bench_rotate_uses_every_operand_set(gpu):
         plan.bench_rotate([], 3)
 
 
+@pytest.mark.parametrize("M,N,K", [(16, 512, 2048), (16, 520, 14336), (128, 4096, 14336)])
+def test_bench_graph_replays_the_captured_launches(gpu, M, N, K):
+    """Launches captured once into a HIP graph and replayed (a decode kernel, one in K ranges with
+    the library's partial-sum workspace, split K with its second kernel): every operand set ends
+    up with the product of its own weights, three replays after the untimed one, and the outputs
+    are the bits of eager launches."""
+    a, _, _ = operands(M, N, K, "bf16", seed=31)
+    plan = AG.GemmPlan.create(M, N, K, "bf16", "bf16")
+    bufs, sets, eager = [], [], []
+    da = GpuBuffer(a.nbytes)
+    da.copy_from_host(a)
+    for i in range(3):
+        _, b, _ = operands(M, N, K, "bf16", seed=40 + i, b_std=0.05)
+        db, dc = GpuBuffer(b.nbytes), GpuBuffer(M * N * 2)
+        db.copy_from_host(b)
+        plan.run(da.ptr_value, db.ptr_value, dc.ptr_value)
+        ref = np.zeros((M, N), np.uint16)
+        dc.copy_to_host(ref)
+        eager.append(ref)
+        dc.copy_from_host(np.full((M, N), 0x7FC1, np.uint16))
+        bufs += [db, dc]
+        sets.append({"dA": da.ptr_value, "dB": db.ptr_value, "dC": dc.ptr_value})
+    print(f"graph of 6 launches of {plan.info.name.decode()} M={M} N={N} K={K}", flush=True)
+    total = plan.bench_graph(sets, 6, 3)
+    assert total > 0
+    for i in range(3):
+        out = np.zeros((M, N), np.uint16)
+        bufs[2 * i + 1].copy_to_host(out)
+        assert np.array_equal(out, eager[i])
+    for bf in bufs + [da]:
+        bf.free()
+    with pytest.raises(_capi.AsterGemmError):
+        plan.bench_graph([], 3, 1)
+
+
 @pytest.mark.parametrize("ksteps", [2, 4, 6, 8, 10, 12, 14])
 @pytest.mark.parametrize("tile", [256, 128])
 def test_mxfp4_stream_kernel_every_loop_phase(gpu, ksteps, tile):
