@@ -697,6 +697,7 @@ int astergemm_bench_graph(const astergemm_config* cfg, const astergemm_operands*
   if (exec) (void)hipGraphExecDestroy(exec);
   if (graph) (void)hipGraphDestroy(graph);
   (void)hipStreamSynchronize(s);
+  splitk_workspace_release(s);  // the partial-sum workspace this stream may have been given
   (void)hipStreamDestroy(s);
   if (le != 0) return hip_fail((hipError_t)le, v->name, __FILE__, __LINE__);
   *total_ns = (int64_t)((double)ms * 1e6);

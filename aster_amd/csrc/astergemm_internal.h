@@ -144,6 +144,8 @@ inline int stream_split_of(int64_t tiles, int64_t ksteps, bool even_ranges = fal
 // workspace of a (device, stream), and the kernel that adds `splits` planes [M][N] of
 // a.workspace in index order, applies a's scales and bias and stores a.C in `out_dtype`.
 int splitk_workspace_for(size_t bytes, hipStream_t stream, float** out);
+// Frees the workspace of a (synchronised) stream that is about to be destroyed.
+void splitk_workspace_release(hipStream_t stream);
 int splitk_reduce(int out_dtype, const GemmArgs& a, int splits, hipStream_t stream);
 
 void set_error(const char* fmt, ...);

@@ -765,6 +765,18 @@ int splitk_workspace(size_t bytes, hipStream_t stream, float** out) {
   return 0;
 }
 
+// Gives back the workspace of a stream that is about to be destroyed.  The caller has
+// synchronised the stream: nothing enqueued on it can still use the buffer.
+void splitk_workspace_drop(hipStream_t stream) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return;
+  std::lock_guard<std::mutex> lock(g_ws_mutex);
+  auto it = g_ws.find({dev, stream});
+  if (it == g_ws.end()) return;
+  if (it->second.ptr) (void)hipFree(it->second.ptr);
+  g_ws.erase(it);
+}
+
 // Grid of the K-range decode kernels: S K ranges x R row ranges, one workgroup per CU; with
 // mh = 2 two workgroups share a row range, in whole pairs on each of the 8 XCDs.  The launchers
 // and the description of a variant both come here.
@@ -2002,6 +2014,8 @@ const Variant* skinny_variants() { return kSkinnyVariants; }
 int splitk_workspace_for(size_t bytes, hipStream_t stream, float** out) {
   return splitk_workspace(bytes, stream, out);
 }
+
+void splitk_workspace_release(hipStream_t stream) { splitk_workspace_drop(stream); }
 
 int splitk_reduce(int out_dtype, const GemmArgs& a, int splits, hipStream_t stream) {
   switch (out_dtype) {
