@@ -131,8 +131,53 @@ const char* validate_problem(const astergemm_config& c) {
   return nullptr;
 }
 
+// The last selections of this thread: a serving loop calls the entry points with the same few
+// configs over and over, and walking the variant table with its shape checks costs about 5 us of
+// host time a call.  A selection depends on the config and, through the CU count, on the device.
+struct ChoiceCacheEntry {
+  astergemm_config cfg;
+  int dev;
+  int index;
+};
+constexpr int kChoiceCache = 16;
+thread_local ChoiceCacheEntry g_choice_cache[kChoiceCache];
+thread_local int g_choice_cache_used = 0, g_choice_cache_next = 0;
+
+int current_device_or_minus_one() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    (void)hipGetLastError();
+    dev = -1;
+  }
+  return dev;
+}
+
+const Variant* choose_uncached(const astergemm_config& c, int* index_out);
+
 // Picks the variant for cfg; on failure returns nullptr with the error set.
 const Variant* choose(const astergemm_config& c, int* index_out) {
+  const int dev = current_device_or_minus_one();
+  for (int i = 0; i < g_choice_cache_used; ++i) {
+    const ChoiceCacheEntry& e = g_choice_cache[i];
+    if (e.dev == dev && memcmp(&e.cfg, &c, sizeof(c)) == 0) {
+      if (index_out) *index_out = e.index;
+      return variant_at(e.index);
+    }
+  }
+  int index = -1;
+  const Variant* v = choose_uncached(c, &index);
+  if (!v) return nullptr;  // refusals are not remembered: the message is made again
+  ChoiceCacheEntry& e = g_choice_cache[g_choice_cache_next];
+  memcpy(&e.cfg, &c, sizeof(c));
+  e.dev = dev;
+  e.index = index;
+  g_choice_cache_next = (g_choice_cache_next + 1) % kChoiceCache;
+  if (g_choice_cache_used < kChoiceCache) ++g_choice_cache_used;
+  if (index_out) *index_out = index;
+  return v;
+}
+
+const Variant* choose_uncached(const astergemm_config& c, int* index_out) {
   g_choose_rc = ASTERGEMM_ENOTSUP;
   if (const char* why = validate_problem(c)) {
     set_error("astergemm: invalid config: %s", why);

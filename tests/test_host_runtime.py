@@ -226,6 +226,30 @@ def test_direct_ab_mapping_selects_the_kernel_without_lds():
             gemm.GemmPlan.create(*args, operand_path="direct_ab", **kw)
 
 
+def test_repeated_selection_is_remembered_per_config():
+    # the library remembers a thread's last selections; a config that differs in any field is a
+    # different entry, refusals are never remembered, and more configs than the memory holds
+    # still select correctly
+    lib = _capi.load()
+    names = {}
+    shapes = [(256 * i, 1024 * j, 2048 * j) for i in range(1, 6) for j in range(1, 6)]   # 25 > 16 entries
+    for rnd in range(3):
+        for shape in shapes:
+            for dt in ("bf16", "fp8_e4m3"):
+                name = gemm.GemmPlan.create(*shape, dt, "bf16").info.name.decode()
+                assert names.setdefault((shape, dt), name) == name
+    assert len(set(names.values())) >= 3, set(names.values())
+    for _ in range(2):
+        with pytest.raises(_capi.AsterGemmError) as err:
+            gemm.GemmPlan.create(120, 256, 512, "bf16", "bf16", operand_path="direct_ab")
+        assert "M % 16" in str(err.value)
+    a = gemm.GemmPlan.create(16, 14336, 4096, "bf16", "bf16")
+    b = gemm.GemmPlan.create(16, 14336, 4096, "bf16", "f32")
+    c = gemm.GemmPlan.create(16, 14336, 4096, "bf16", "bf16", has_bias=True)
+    assert a.info.name != b.info.name and a.info.name == c.info.name
+    assert lib.astergemm_variant_count() > 0
+
+
 def test_execute_checks_host_operand_sizes_before_touching_the_gpu(tmp_path):
     cfg = make_instance(256, 256, 256)
     path, _ = gemm.compile_gemm(cfg, str(tmp_path / "k.hsaco"))
