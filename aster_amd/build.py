@@ -25,9 +25,10 @@ LIB_PATH = os.path.join(LIB_DIR, "libastergemm.so")
 OBJ_DIR = os.path.join(ROOT, "build", "obj")
 
 # (object stem, source file, extra flags).  gemm_stream.hip holds the variant table of the stream
-# kernels in three parts (16-bit, fp8, MXFP4 operands) and is compiled once per part.
-UNITS = [("gemm_stream_p2", "gemm_stream.hip", ["-DAG_STREAM_PART=2"]),
-         ("gemm_stream_p0", "gemm_stream.hip", ["-DAG_STREAM_PART=0"]),
+# kernels in four parts (bf16, fp8, MXFP4, f16 operands) and is compiled once per part.
+UNITS = [("gemm_stream_p0", "gemm_stream.hip", ["-DAG_STREAM_PART=0"]),
+         ("gemm_stream_p3", "gemm_stream.hip", ["-DAG_STREAM_PART=3"]),
+         ("gemm_stream_p2", "gemm_stream.hip", ["-DAG_STREAM_PART=2"]),
          ("gemm_stream_p1", "gemm_stream.hip", ["-DAG_STREAM_PART=1"]),
          ("gemm_skinny", "gemm_skinny.hip", []),
          ("gemm_tile", "gemm_tile.hip", []),
@@ -127,7 +128,7 @@ def build_library(verbose: bool = False, only=None) -> str:
     os.makedirs(OBJ_DIR, exist_ok=True)
     os.makedirs(LIB_DIR, exist_ok=True)
     write_generated_sources()
-    with ThreadPoolExecutor(max_workers=6) as pool:
+    with ThreadPoolExecutor(max_workers=8) as pool:
         if only:
             todo = [u for u in UNITS if u[0] in only]
             list(pool.map(_compile, todo))

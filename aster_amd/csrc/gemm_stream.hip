@@ -613,38 +613,33 @@ int grid_stream_tail(const astergemm_config& c, int cus) {
       AG_STREAM(prefix "_128x128_w2x2_f32", DT, ASTERGEMM_F32, 128, 128, 2, 2),          \
       AG_STREAM(prefix "_128x128_w2x2_f16", DT, ASTERGEMM_F16, 128, 128, 2, 2)
 
-// The table is compiled in three parts (this file once per AG_STREAM_PART: 16-bit, fp8 and MXFP4
+// The table is compiled in four parts (this file once per AG_STREAM_PART: bf16, fp8, MXFP4 and f16
 // operands), so that the parts build side by side and work on one family recompiles one part.
 #ifndef AG_STREAM_PART
-#error "compile with -DAG_STREAM_PART=0, 1 or 2"
+#error "compile with -DAG_STREAM_PART=0, 1, 2 or 3"
 #endif
 
 const Variant kStreamVariants[] = {
+#if AG_STREAM_PART == 0 || AG_STREAM_PART == 3
 #if AG_STREAM_PART == 0
-    AG_STREAM_SET("stream_bf16", ASTERGEMM_BF16),
-    AG_STREAM_SPLITK_SET("splitk_bf16", 0, ASTERGEMM_BF16, 5 * 128 * kRowBytes, gemm_stream_splitk_kernel),
-    AG_STREAM_SPLITK_SET("splitk_f16", 0, ASTERGEMM_F16, 5 * 128 * kRowBytes, gemm_stream_splitk_kernel),
-    AG_STREAM_SET("stream_f16", ASTERGEMM_F16),
-    AG_STREAMDB("streamdb_bf16_256x256_w2x4_bf16", ASTERGEMM_BF16, ASTERGEMM_BF16, 5, 5, 2, 2),
-    AG_STREAMDB("streamdb_bf16_256x256_w2x4_f32", ASTERGEMM_BF16, ASTERGEMM_F32, 5, 5, 2, 2),
-    AG_STREAMDB("streamdb_bf16_256x256_w2x4_f16", ASTERGEMM_BF16, ASTERGEMM_F16, 5, 5, 2, 2),
-    AG_STREAMDB("streamdb_f16_256x256_w2x4_bf16", ASTERGEMM_F16, ASTERGEMM_BF16, 5, 5, 2, 2),
-    AG_STREAMDB("streamdb_f16_256x256_w2x4_f32", ASTERGEMM_F16, ASTERGEMM_F32, 5, 5, 2, 2),
-    AG_STREAMDB("streamdb_f16_256x256_w2x4_f16", ASTERGEMM_F16, ASTERGEMM_F16, 5, 5, 2, 2),
-    AG_STREAMDB("streamdb_bf16_128x256_w1x4_bf16", ASTERGEMM_BF16, ASTERGEMM_BF16, 5, 5, 1, 1),
-    AG_STREAMDB("streamdb_bf16_128x256_w1x4_f32", ASTERGEMM_BF16, ASTERGEMM_F32, 5, 5, 1, 1),
-    AG_STREAMDB("streamdb_bf16_128x256_w1x4_f16", ASTERGEMM_BF16, ASTERGEMM_F16, 5, 5, 1, 1),
-    AG_STREAMDB("streamdb_f16_128x256_w1x4_bf16", ASTERGEMM_F16, ASTERGEMM_BF16, 5, 5, 1, 1),
-    AG_STREAMDB("streamdb_f16_128x256_w1x4_f32", ASTERGEMM_F16, ASTERGEMM_F32, 5, 5, 1, 1),
-    AG_STREAMDB("streamdb_f16_128x256_w1x4_f16", ASTERGEMM_F16, ASTERGEMM_F16, 5, 5, 1, 1),
-    AG_STREAM_TAIL_SET("stream_bf16_256x256_w2x4_tail128", 0, ASTERGEMM_BF16, 2, 4, 5 * 256 * kRowBytes,
+#define AG_P16 ASTERGEMM_BF16
+#define AG_N16(x) x "_bf16"
+#else
+#define AG_P16 ASTERGEMM_F16
+#define AG_N16(x) x "_f16"
+#endif
+    AG_STREAM_SET(AG_N16("stream"), AG_P16),
+    AG_STREAM_SPLITK_SET(AG_N16("splitk"), 0, AG_P16, 5 * 128 * kRowBytes, gemm_stream_splitk_kernel),
+    AG_STREAMDB(AG_N16("streamdb") "_256x256_w2x4_bf16", AG_P16, ASTERGEMM_BF16, 5, 5, 2, 2),
+    AG_STREAMDB(AG_N16("streamdb") "_256x256_w2x4_f32", AG_P16, ASTERGEMM_F32, 5, 5, 2, 2),
+    AG_STREAMDB(AG_N16("streamdb") "_256x256_w2x4_f16", AG_P16, ASTERGEMM_F16, 5, 5, 2, 2),
+    AG_STREAMDB(AG_N16("streamdb") "_128x256_w1x4_bf16", AG_P16, ASTERGEMM_BF16, 5, 5, 1, 1),
+    AG_STREAMDB(AG_N16("streamdb") "_128x256_w1x4_f32", AG_P16, ASTERGEMM_F32, 5, 5, 1, 1),
+    AG_STREAMDB(AG_N16("streamdb") "_128x256_w1x4_f16", AG_P16, ASTERGEMM_F16, 5, 5, 1, 1),
+    AG_STREAM_TAIL_SET(AG_N16("stream") "_256x256_w2x4_tail128", 0, AG_P16, 2, 4, 5 * 256 * kRowBytes,
                        gemm_stream_kernel),
-    AG_STREAM_TAIL_SET("stream_f16_256x256_w2x4_tail128", 0, ASTERGEMM_F16, 2, 4, 5 * 256 * kRowBytes,
-                       gemm_stream_kernel),
-    AG_STREAM_RING9_SET("stream_bf16", ASTERGEMM_BF16),
-    AG_STREAM_RING9_SET("stream_f16", ASTERGEMM_F16),
-    AG_DIRECTAB_SET("directab_bf16", ASTERGEMM_BF16),
-    AG_DIRECTAB_SET("directab_f16", ASTERGEMM_F16),
+    AG_STREAM_RING9_SET(AG_N16("stream"), AG_P16),
+    AG_DIRECTAB_SET(AG_N16("directab"), AG_P16),
 #elif AG_STREAM_PART == 1
     AG_STREAM_SPLITK_SET("splitk_fp8", 1, ASTERGEMM_FP8_E4M3, 5 * 128 * kRowBytes,
                          gemm_stream8_splitk_kernel),
@@ -701,13 +696,16 @@ const Variant* AG_CAT(stream_variants_part, AG_STREAM_PART)(int* count) {
 #if AG_STREAM_PART == 0
 const Variant* stream_variants_part1(int* count);
 const Variant* stream_variants_part2(int* count);
+const Variant* stream_variants_part3(int* count);
 
-// the three parts as one table, in part order
+// the four parts as one table: bf16, f16, fp8, MXFP4
 static const std::vector<Variant>& all_stream_variants() {
   static const std::vector<Variant> all = [] {
     std::vector<Variant> v;
     int n = 0;
     const Variant* p = stream_variants_part0(&n);
+    v.insert(v.end(), p, p + n);
+    p = stream_variants_part3(&n);
     v.insert(v.end(), p, p + n);
     p = stream_variants_part1(&n);
     v.insert(v.end(), p, p + n);
