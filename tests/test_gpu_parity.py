@@ -1787,6 +1787,45 @@ def test_random_shapes_with_pre_shuffled_weights(gpu, dt, out_dt, M, N, K, with_
         assert np.isnan(tail).all() if out_dt == "f32" else (tail == 0x7FC1).all()
 
 
+def _random_direct_ab_cases(n_cases=24, seed=313):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for i in range(n_cases):
+        dt = ("bf16", "f16")[i % 2]
+        big = i % 6 == 5          # enough tiles for the 256 x 256 form to be chosen
+        M = int(rng.integers(225, 240) if big else rng.integers(1, 70)) * 16
+        N = int(rng.integers(225, 240) if big else rng.integers(1, 70)) * 16
+        K = int(rng.integers(1, 12 if big else 40)) * 32
+        out = ("f32", "bf16", "f16")[int(rng.integers(0, 3))]
+        cases.append((dt, out, M, N, K, bool(rng.integers(0, 2)), int(rng.integers(0, 3)) * 4))
+    return cases
+
+
+@pytest.mark.parametrize("dt,out_dt,M,N,K,with_bias,pad", _random_direct_ab_cases())
+def test_random_shapes_with_both_operands_pre_shuffled(gpu, dt, out_dt, M, N, K, with_bias, pad):
+    """operand_path direct_ab on seeded random shapes: edge tiles in M and N (multiples of 16),
+    every residue of the chunk-column count against both ring depths, whichever of the two
+    geometries AUTO takes; the oracle's result, pad columns untouched."""
+    from aster_amd.kittens_helpers import shuffle_weight
+    a, b, _ = operands(M, N, K, dt, seed=4000 + M + N + K, b_std=0.05)
+    bias = np.random.default_rng(7).standard_normal(N).astype(np.float32) if with_bias else None
+    out, name = run_gemm(shuffle_weight(np.ascontiguousarray(a).view(np.uint16)),
+                         shuffle_weight(np.ascontiguousarray(b).view(np.uint16)), M, N, K, dt, out_dt,
+                         bias=bias, ldc=N + pad if pad else 0, operand_path="direct_ab")
+    assert name.startswith(f"directab_{dt}_")
+    want = G.gemm(a, b, _DT[dt], _DT[out_dt], bias=bias)
+    got, ref = G.output_to_f32(out[:, :N], _DT[out_dt]), G.output_to_f32(want, _DT[out_dt])
+    assert not np.isnan(got).any(), name
+    ulp = {"f32": 2.0 ** -20, "bf16": 2.0 ** -7, "f16": 2.0 ** -10}[out_dt]
+    tol = 2 * ulp * np.abs(ref) + 2e-4 * np.abs(ref).max()
+    assert np.all(np.abs(got - ref) <= tol), (name, float(np.abs(got - ref).max()))
+    if M * N >= 4096:
+        assert G.rel_l2(got, ref) <= (REL_L2_BAR if out_dt != "f32" else 1e-5), name
+    if pad:
+        tail = out[:, N:]
+        assert np.isnan(tail).all() if out_dt == "f32" else (tail == 0x7FC1).all()
+
+
 @pytest.mark.parametrize("M,N,K,dt", [(512, 768, 1024, "bf16"), (16, 520, 4096, "bf16"), (300, 200, 512, "fp8_e4m3")])
 def test_tune_returns_a_runnable_variant_that_matches_the_oracle(gpu, M, N, K, dt):
     a, b, extra = operands(M, N, K, dt, seed=91, b_std=0.05)
