@@ -1853,3 +1853,27 @@ def test_tune_returns_a_runnable_variant_that_matches_the_oracle(gpu, M, N, K, d
     only_tile = AG.GemmPlan.create(M, N, K, dt, "f32", family=_capi.KERNEL_TILE).tune(
         *(x.ptr_value for x in bufs), iters=3, **kw)
     assert only_tile.info.family == _capi.KERNEL_TILE
+
+
+def test_library_loaded_before_pytorch_still_launches(gpu):
+    """A process that loads the library first and imports PyTorch afterwards must end up with one
+    HIP runtime: with two, the one initialised second reports that it finds no device at the
+    first launch.  Fresh process: library, then torch, then a GEMM on torch-owned memory."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = ("from aster_amd import _capi, gemm as AG\n"
+            "_capi.load()\n"
+            "import torch\n"
+            "a = torch.ones(256, 512, dtype=torch.bfloat16, device='cuda:0')\n"
+            "b = torch.ones(384, 512, dtype=torch.bfloat16, device='cuda:0')\n"
+            "c = torch.zeros(256, 384, dtype=torch.bfloat16, device='cuda:0')\n"
+            "torch.cuda.synchronize()\n"
+            "p = AG.GemmPlan.create(256, 384, 512, 'bf16', 'bf16')\n"
+            "print('launch', p.info.name.decode(), flush=True)\n"
+            "p.run(a.data_ptr(), b.data_ptr(), c.data_ptr())\n"
+            "torch.cuda.synchronize()\n"
+            "assert bool((c == 512).all()), c\n"
+            "print('one runtime, launch ok')\n")
+    out = subprocess.run([sys.executable, "-c", code], cwd=root, capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0 and "launch ok" in out.stdout, out.stderr[-2000:]
