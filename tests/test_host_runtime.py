@@ -250,6 +250,29 @@ def test_repeated_selection_is_remembered_per_config():
     assert lib.astergemm_variant_count() > 0
 
 
+def test_selection_from_many_threads_is_consistent():
+    # the selection memory is per thread: threads that select different configs at the same time
+    # never see each other's entries
+    import threading
+    shapes = [(256 * (i + 1), 1024 * (i % 3 + 1), 2048 * (i % 2 + 1)) for i in range(8)]
+    want = [gemm.GemmPlan.create(*s_, "bf16", "bf16").info.name for s_ in shapes]
+    bad = []
+
+    def worker(i):
+        for _ in range(300):
+            for j in (i, (i + 3) % 8):
+                name = gemm.GemmPlan.create(*shapes[j], "bf16", "bf16").info.name
+                if name != want[j]:
+                    bad.append((i, j, name))
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(8)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not bad, bad[:3]
+
+
 def test_execute_checks_host_operand_sizes_before_touching_the_gpu(tmp_path):
     cfg = make_instance(256, 256, 256)
     path, _ = gemm.compile_gemm(cfg, str(tmp_path / "k.hsaco"))
