@@ -21,6 +21,8 @@
 //                                    its first row: the operand values a kernel sees do not change
 //                                    when all its transfers are pointed at one row, so the cost of
 //                                    the memory path can be told from the cost of the operand bits)
+//                    [--zeros]       (all-zero operands instead of the random fill: what the clock does
+//                                    when the operand bits cost nothing)
 //                    [--mx-a-lanes]  (MXFP4: A's e8m0 plane in lane order, mx_a_layout LANES128;
 //                                    needs --normal and --direct-b-k8)
 //   astergemm_replay --quantize fp8|mxfp4 --m ROWS --k K --iters 100
@@ -165,7 +167,7 @@ int main(int argc, char** argv) {
   cfg.M = cfg.N = cfg.K = 8192;
   cfg.dtype_ab = ASTERGEMM_BF16;
   cfg.dtype_c = ASTERGEMM_BF16;
-  int iters = 100, warmup = 20, json = 0, use_normal = 0, same_rows = 0;
+  int iters = 100, warmup = 20, json = 0, use_normal = 0, same_rows = 0, use_zeros = 0;
   long long flush = 0, calib = 0;
   const char* quantize = nullptr;
   for (int i = 1; i < argc; ++i) {
@@ -194,6 +196,7 @@ int main(int argc, char** argv) {
     else if (a == "--bias") cfg.has_bias = 1;
     else if (a == "--normal") use_normal = 1;
     else if (a == "--same-rows") same_rows = 1;
+    else if (a == "--zeros") use_zeros = 1;
     else if (a == "--mx-a-lanes") cfg.mx_a_layout = ASTERGEMM_MX_LANES128;
     else if (a == "--json") json = 1;
     else if (a == "--quantize") quantize = val();
@@ -247,8 +250,10 @@ int main(int argc, char** argv) {
   ops.dC = dC;
   if (!use_normal) {
     std::vector<uint8_t> ha(a_bytes), hb(b_bytes);
-    fill(ha, cfg.dtype_ab, 42);
-    fill(hb, cfg.dtype_ab, 43);
+    if (!use_zeros) {  // --zeros: all-zero operands (the vectors are value-initialised)
+      fill(ha, cfg.dtype_ab, 42);
+      fill(hb, cfg.dtype_ab, 43);
+    }
     CHECK(aster_rt_memcpy_h2d(dA, ha.data(), a_bytes));
     CHECK(aster_rt_memcpy_h2d(dB, hb.data(), b_bytes));
     if (cfg.scale_mode == ASTERGEMM_SCALE_TENSOR) {
