@@ -109,6 +109,48 @@ OPERANDS = {
 }
 
 
+def board_reading_during(plan, a, b, c, seconds=3.5, sample_at=2.5):
+    """Socket power and per-XCD shader clocks as the board itself reports them (`amd-smi metric
+    --power --clock`, run as a child process) while `plan` runs back to back: the launches go out
+    in one call that returns when they are done; a thread takes the sample `sample_at` seconds in.
+    None when the tool is missing or prints something else."""
+    import re
+    import shutil
+    import subprocess
+    import threading
+
+    tool = shutil.which("amd-smi") or "/opt/rocm/bin/amd-smi"
+    if not os.path.exists(tool):
+        return None
+    sets = [{"dA": a.data_ptr(), "dB": b.data_ptr(), "dC": c.data_ptr()}]
+    per_launch_ns = plan.bench_rotate(sets, 20) / 20.0
+    launches = max(20, int(seconds * 1e9 / per_launch_ns))
+    got = {}
+
+    def sample():
+        time.sleep(sample_at)
+        try:
+            got["text"] = subprocess.run([tool, "metric", "--power", "--clock"], capture_output=True,
+                                         text=True, timeout=20).stdout
+        except Exception as e:  # noqa: BLE001 - the reading is optional
+            got["error"] = repr(e)
+
+    th = threading.Thread(target=sample)
+    th.start()
+    total_ns = plan.bench_rotate(sets, launches)
+    th.join()
+    text = got.get("text", "")
+    power = re.search(r"SOCKET_POWER:\s*([0-9.]+)\s*W", text)
+    clocks = [int(m) for m in re.findall(r"GFX_\d+:\s*\n\s*CLK:\s*(\d+)\s*MHz", text)]
+    if not power or not clocks:
+        return None
+    return {"socket_power_w": float(power.group(1)), "gfx_clk_mhz": clocks, "gfx_max_clk_mhz": 2400,
+            "tflops_during_the_reading": round(plan.info.flops * launches / total_ns * 1e-3, 1),
+            "launches": launches, "sampled_after_s": sample_at,
+            "source": "amd-smi metric --power --clock, as a child process, while the headline kernel "
+                      "runs back to back"}
+
+
 def event_timed_p50(plan, a, b, c, keep, iters, drop, flush_bytes=0):
     kw = {k: v.data_ptr() for k, v in keep.items()}
     times = plan.bench(a.data_ptr(), b.data_ptr(), c.data_ptr(), iters, flush_bytes=flush_bytes, **kw)
@@ -318,6 +360,8 @@ def main() -> int:
                          "warm-up launches (0 = none)")
     ap.add_argument("--no-others", action="store_true", help="skip the secondary shapes")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-board", action="store_true",
+                    help="skip the power / clock reading (3.5 s of back-to-back launches)")
     ap.add_argument("--no-vendor", action="store_true",
                     help="skip timing the vendor library (hipBLASLt through torch) on the same shapes")
     ap.add_argument("--sweep", action="store_true",
@@ -427,6 +471,8 @@ def main() -> int:
     }
     out["roofline"]["mfma_rate_measured_on_this_data"] = round(ceil_tf, 1)
     out["roofline"]["frac_of_measured_mfma_rate"] = round(achieved / ceil_tf, 4)
+    # what the board says while this kernel runs (behind the timed region, so it costs it nothing)
+    out["board"] = None if args.no_board else board_reading_during(plan, a, b, c)
 
     if not args.no_others:
         others = []
